@@ -1,0 +1,86 @@
+/*
+ * spear_btp.h -- C ABI of the MI355X (gfx950) Block Two-Pass kernels.
+ *
+ * This is the drop-in boundary for SPEAR's native BTP extension. The reference binds two
+ * functions from its CUDA extension module `spear._btp`:
+ *
+ *     forward (coeff, x, y, checkpoint, k, wpb)               csrc/btp/_bindings.cu:76-150, 241
+ *     backward(coeff, x, dy, checkpoint, dx, dA, k, wpb)      csrc/btp/_bindings.cu:152-229, 242
+ *
+ * which unpack torch tensors and call the launchers
+ *
+ *     sss::launch_block_two_pass<T, O, WPB>                   csrc/btp/btp-forward.cu:462-527
+ *     sss::launch_btp_backward <T, O, 16, WPB>                csrc/btp/btp-backwards.cu:811-884
+ *
+ * The entry points below take exactly what those launchers take -- raw device pointers, B, H, L,
+ * k and a stream -- plus dtype tags in place of the template parameters. No torch types appear.
+ * `wpb` (warps per block) is an sm90 launch-shape knob with no meaning on CDNA4; the host shim
+ * validates it for compatibility and does not pass it down.
+ *
+ * Tensor layouts (all dense, row-major, caller-allocated; spear/ops/btp/interface.py:136-144,155-158):
+ *     coeff       [B, H, L]          in_dtype   linear-space decay a_t in (0, 1]
+ *     x, dx       [B, H, 16, L]      in_dtype   time is the contiguous axis
+ *     y           [B, H, 16, L]      out_dtype  (in_dtype or fp32)
+ *     dy          [B, H, 16, L]      dy_dtype   (in_dtype or fp32)
+ *     checkpoint  [B, H, L/16, 16]   fp32       slot i-1 = local terminal state of block i-1
+ *     dA          [B, H, L]          fp32       every element is written (no accumulation)
+ *
+ * Requirements: L is a positive multiple of 16; every pointer is 16-byte aligned; k is 1 or 2.
+ * Calls are asynchronous on `stream` (a hipStream_t passed as void*, NULL = default stream),
+ * allocate nothing, keep no state besides a thread-local error string, and are re-entrant.
+ *
+ * Return value: 0 on success, a negative SPEAR_BTP_E* code otherwise; spear_btp_last_error()
+ * then describes the failure. B*H == 0 or L == 0 is a successful no-op, as in the reference
+ * launchers (btp-forward.cu:466, btp-backwards.cu:815).
+ */
+#ifndef SPEAR_BTP_H_
+#define SPEAR_BTP_H_
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* element types (template parameters ElementT / ElementO of the reference launchers) */
+#define SPEAR_BTP_BF16 0
+#define SPEAR_BTP_F16 1
+#define SPEAR_BTP_F32 2
+
+/* flags */
+#define SPEAR_BTP_WRITE_CHECKPOINT 0x1u /* forward: also store the carry checkpoint            */
+#define SPEAR_BTP_PATH_MFMA 0x2u        /* use the bf16-MFMA tile kernels (decay matrix rounded */
+                                        /* to bf16) instead of the exact-fp32 recurrence kernels */
+
+/* error codes */
+#define SPEAR_BTP_EINVAL (-1)  /* bad shape, dtype, k, flag or alignment                       */
+#define SPEAR_BTP_ENULL (-2)   /* a required pointer is NULL                                   */
+#define SPEAR_BTP_ELAUNCH (-3) /* the HIP runtime rejected the launch                          */
+
+/* Replaces spear._btp.forward -> sss::launch_block_two_pass (csrc/btp/_bindings.cu:76-150,
+ * csrc/btp/btp-forward.cu:462-527).  `checkpoint` may be NULL unless SPEAR_BTP_WRITE_CHECKPOINT
+ * is set. */
+int spear_btp_forward(const void* coeff, const void* x, void* y, float* checkpoint, int B, int H,
+                      int L, int k, int in_dtype, int out_dtype, unsigned flags, void* stream);
+
+/* Replaces spear._btp.backward -> sss::launch_btp_backward (csrc/btp/_bindings.cu:152-229,
+ * csrc/btp/btp-backwards.cu:811-884).  `checkpoint` is accepted for signature compatibility and
+ * never read: the carries are recomputed from `coeff` and `x`. */
+int spear_btp_backward(const void* coeff, const void* x, const void* dy, const float* checkpoint,
+                       void* dx, float* dA, int B, int H, int L, int k, int in_dtype, int dy_dtype,
+                       unsigned flags, void* stream);
+
+/* Message for the last failing call on this thread ("" if none).  The reference prints launch
+ * failures and carries on (csrc/btp/btp-forward.cu:501-520); here they are reported. */
+const char* spear_btp_last_error(void);
+
+/* ABI version of this header: bumped whenever a signature above changes. */
+int spear_btp_abi_version(void);
+
+/* Measurement aid, not part of the operator: a plain device-to-device copy kernel of known
+ * traffic (reads `bytes`, writes `bytes`; `bytes` a multiple of 16), used to calibrate hardware
+ * counters and to measure the copy bandwidth the BTP kernels are compared with. */
+int spear_btp_copy(const void* src, void* dst, unsigned long long bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SPEAR_BTP_H_ */

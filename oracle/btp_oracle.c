@@ -1,0 +1,260 @@
+/*
+ * btp_oracle.c -- CPU restatement (fp64, plain C) of SPEAR's Block Two-Pass (BTP) operator.
+ *
+ * THIS FILE IS TEST INFRASTRUCTURE. It is the checker the HIP kernels are compared against.
+ * Nothing in the shipped package may import, link or call it; only tests/, the smoke check and
+ * the cpu_baseline leg of bench.py do.
+ *
+ * What it restates (paths relative to the reference repository):
+ *   - spear/ops/btp/reference.py:55-77   construct_L_ref              -> build_L(mode 0)
+ *   - spear/ops/btp/reference.py:38-52   segsum_stable + exp          -> build_L(mode 1)
+ *   - spear/ops/btp/reference.py:79-90   construct_L_masked_cumprod   -> build_L(mode 2)
+ *   - spear/ops/btp/reference.py:105-139 block_two_pass               -> btp_oracle_forward
+ *   - spear/nn/phalanx/inference.py:75-90 sequential jagged form      -> btp_oracle_forward_sequential
+ *   - csrc/btp/btp-forward.cu:369-373    carry checkpoint layout      -> `ckpt` of btp_oracle_forward
+ *   - csrc/btp/btp-backwards.cu:355-413,466-608 + autograd of reference.py:105-139
+ *                                                                     -> btp_oracle_backward
+ *
+ * Layouts (all contiguous, row-major, double):
+ *   a    [B*H][L]          linear-space decay, a_t
+ *   x    [B*H][16][L]      activations, time is the fastest axis
+ *   y    [B*H][16][L]
+ *   ckpt [B*H][L/16][16]   slot i-1 holds the zero-initialised terminal state of block i-1 as
+ *                          consumed by block i (k == 2 only); the last slot is never written
+ *
+ * Pinning (see tests/test_oracle.py): windowed brute-force sum, the sequential form below,
+ * full linear scan for L <= 32, closed forms (a==1, a==0, geometric), central finite differences
+ * and the adjoint identity for the backward.
+ */
+#include <math.h>
+#include <stddef.h>
+#include <stdlib.h>
+#include <string.h>
+
+#define BL 16
+#define DH 16
+
+/* ---- decay matrix of one block: Lm[r][c] = prod_{j=c+1..r} a[j], 1 on the diagonal, 0 above ---- */
+static void build_L(const double *a, int mode, double Lm[BL][BL]) {
+  for (int r = 0; r < BL; ++r)
+    for (int c = 0; c < BL; ++c) Lm[r][c] = 0.0;
+
+  if (mode == 1) {
+    /* reference.py:38-52: column-wise running sum of log a below the diagonal, then exp */
+    for (int c = 0; c < BL; ++c) {
+      double s = 0.0;
+      Lm[c][c] = 1.0; /* exp(0) */
+      for (int r = c + 1; r < BL; ++r) {
+        s += log(a[r]);
+        Lm[r][c] = exp(s);
+      }
+    }
+    return;
+  }
+  /* mode 0 (reference.py:55-77, explicit product) and mode 2 (reference.py:79-90, column-wise
+   * running product) are the same numbers in exact arithmetic; they differ in the order the
+   * factors are multiplied.  mode 0 multiplies a[c+1..r] left to right afresh for every entry. */
+  for (int c = 0; c < BL; ++c) {
+    Lm[c][c] = 1.0;
+    if (mode == 2) {
+      double p = 1.0;
+      for (int r = c + 1; r < BL; ++r) {
+        p *= a[r];
+        Lm[r][c] = p;
+      }
+    } else {
+      for (int r = c + 1; r < BL; ++r) {
+        double p = 1.0;
+        for (int j = c + 1; j <= r; ++j) p *= a[j];
+        Lm[r][c] = p;
+      }
+    }
+  }
+}
+
+/* Two-pass forward, reference.py:105-139.  k == 1 keeps only the block-local pass. */
+int btp_oracle_forward(const double *a, const double *x, double *y, double *ckpt, long BH, long L,
+                       int k, int l_mode) {
+  if (L % BL != 0 || (k != 1 && k != 2)) return -1;
+  const long NB = L / BL;
+  double Lm[BL][BL];
+  double v[DH][BL];
+  double carry[DH];
+
+  for (long bh = 0; bh < BH; ++bh) {
+    const double *a_row = a + bh * L;
+    const double *x_row = x + bh * DH * L;
+    double *y_row = y + bh * DH * L;
+    for (int d = 0; d < DH; ++d) carry[d] = 0.0;
+
+    for (long i = 0; i < NB; ++i) {
+      const double *ab = a_row + i * BL;
+      build_L(ab, l_mode, Lm);
+      /* first pass: v[d][r] = sum_c L[r][c] * x[d][c]   (einsum "shbij,shdbj->shdbi") */
+      for (int d = 0; d < DH; ++d) {
+        const double *xd = x_row + (long)d * L + i * BL;
+        for (int r = 0; r < BL; ++r) {
+          double s = 0.0;
+          for (int c = 0; c <= r; ++c) s += Lm[r][c] * xd[c];
+          v[d][r] = s;
+        }
+      }
+      /* second pass: rank-1 update with the previous block's local terminal row */
+      for (int d = 0; d < DH; ++d) {
+        double *yd = y_row + (long)d * L + i * BL;
+        for (int r = 0; r < BL; ++r) {
+          double out = v[d][r];
+          if (k == 2 && i > 0) {
+            const double g = ab[0] * Lm[r][0]; /* scale_factors * first_cols, reference.py:129-132 */
+            out = g * carry[d] + out;
+          }
+          yd[r] = out;
+        }
+      }
+      if (k == 2 && i > 0 && ckpt) {
+        double *slot = ckpt + (bh * NB + (i - 1)) * DH;
+        for (int d = 0; d < DH; ++d) slot[d] = carry[d];
+      }
+      for (int d = 0; d < DH; ++d) carry[d] = v[d][BL - 1]; /* local state, NOT the corrected one */
+    }
+  }
+  return 0;
+}
+
+/* Token-by-token statement of the same operator (inference.py:75-90):
+ *   y_loc <- a_t*y_loc + x_t ; r_pref <- a_t*r_pref ; y_t = y_loc + r_pref*c_prev ;
+ *   every 16 steps: c_prev <- y_loc, y_loc <- 0, r_pref <- 1.
+ * Shares no code with btp_oracle_forward, so agreement between the two is a real check. */
+int btp_oracle_forward_sequential(const double *a, const double *x, double *y, long BH, long L,
+                                  int k) {
+  if (k != 1 && k != 2) return -1;
+  for (long bh = 0; bh < BH; ++bh) {
+    for (int d = 0; d < DH; ++d) {
+      const double *ar = a + bh * L;
+      const double *xr = x + (bh * DH + d) * L;
+      double *yr = y + (bh * DH + d) * L;
+      double c_prev = 0.0, y_loc = 0.0, r_pref = 1.0;
+      int in_blk = 0;
+      for (long t = 0; t < L; ++t) {
+        y_loc = ar[t] * y_loc + xr[t];
+        r_pref = ar[t] * r_pref;
+        yr[t] = (k == 2) ? y_loc + r_pref * c_prev : y_loc;
+        if (++in_blk == BL) {
+          c_prev = y_loc;
+          y_loc = 0.0;
+          r_pref = 1.0;
+          in_blk = 0;
+        }
+      }
+    }
+  }
+  return 0;
+}
+
+/* Reverse-mode derivative of btp_oracle_forward (explicit-product L), written out by hand.
+ * dx [B*H][16][L], dA [B*H][L] (gradient w.r.t. the linear-space coefficient a_t).
+ *
+ *   dv_i[r]   = dy_i[r] + [r==15] * dCarry_i ,  dCarry_i[d] = sum_r g_{i+1}[r] * dy_{i+1}[r][d]
+ *   dx_i[c]   = sum_{r>=c} L_i[r][c] * dv_i[r]
+ *   dL_i[r][c]= <dv_i[r], x_i[c]>            (+ a_{i,0} * <dy_i[r], carry_i> on column 0)
+ *   da_{i,0} += sum_r <dy_i[r], carry_i> * L_i[r][0]
+ *   da_j     += sum_{r>=j>c} dL_i[r][c] * prod_{j' in c+1..r, j' != j} a_j'     (no division)
+ */
+int btp_oracle_backward(const double *a, const double *x, const double *dy, double *dx, double *dA,
+                        long BH, long L, int k) {
+  if (L % BL != 0 || (k != 1 && k != 2)) return -1;
+  const long NB = L / BL;
+  double Lm[BL][BL], Ln[BL][BL];
+  double dL[BL][BL];
+  double dv[DH][BL];
+  double carry[DH], dcarry[DH];
+  double *vlast = (double *)malloc(sizeof(double) * (size_t)(NB > 0 ? NB : 1) * DH);
+  if (!vlast) return -2;
+
+  for (long bh = 0; bh < BH; ++bh) {
+    const double *a_row = a + bh * L;
+    const double *x_row = x + bh * DH * L;
+    const double *g_row = dy + bh * DH * L;
+    double *dx_row = dx + bh * DH * L;
+    double *dA_row = dA + bh * L;
+
+    /* local terminal state of every block (the forward carries) */
+    for (long i = 0; i < NB; ++i) {
+      build_L(a_row + i * BL, 0, Lm);
+      for (int d = 0; d < DH; ++d) {
+        const double *xd = x_row + (long)d * L + i * BL;
+        double s = 0.0;
+        for (int c = 0; c < BL; ++c) s += Lm[BL - 1][c] * xd[c];
+        vlast[i * DH + d] = s;
+      }
+    }
+
+    for (long i = 0; i < NB; ++i) {
+      const double *ab = a_row + i * BL;
+      build_L(ab, 0, Lm);
+      const int has_prev = (k == 2 && i > 0);
+      const int has_next = (k == 2 && i + 1 < NB);
+      for (int d = 0; d < DH; ++d) {
+        carry[d] = has_prev ? vlast[(i - 1) * DH + d] : 0.0;
+        dcarry[d] = 0.0;
+      }
+      if (has_next) {
+        const double *an = a_row + (i + 1) * BL;
+        build_L(an, 0, Ln);
+        for (int d = 0; d < DH; ++d) {
+          const double *gd = g_row + (long)d * L + (i + 1) * BL;
+          double s = 0.0;
+          for (int r = 0; r < BL; ++r) s += an[0] * Ln[r][0] * gd[r];
+          dcarry[d] = s;
+        }
+      }
+      for (int d = 0; d < DH; ++d) {
+        const double *gd = g_row + (long)d * L + i * BL;
+        for (int r = 0; r < BL; ++r) dv[d][r] = gd[r];
+        dv[d][BL - 1] += dcarry[d];
+      }
+      /* dx */
+      for (int d = 0; d < DH; ++d) {
+        double *dxd = dx_row + (long)d * L + i * BL;
+        for (int c = 0; c < BL; ++c) {
+          double s = 0.0;
+          for (int r = c; r < BL; ++r) s += Lm[r][c] * dv[d][r];
+          dxd[c] = s;
+        }
+      }
+      /* dL and the direct a_{i,0} term of the carry scale */
+      double da[BL];
+      for (int j = 0; j < BL; ++j) da[j] = 0.0;
+      for (int r = 0; r < BL; ++r)
+        for (int c = 0; c < BL; ++c) dL[r][c] = 0.0;
+      for (int r = 0; r < BL; ++r) {
+        for (int c = 0; c < r; ++c) {
+          double s = 0.0;
+          for (int d = 0; d < DH; ++d) s += dv[d][r] * x_row[(long)d * L + i * BL + c];
+          dL[r][c] = s;
+        }
+        if (has_prev) {
+          double dg = 0.0;
+          for (int d = 0; d < DH; ++d) dg += g_row[(long)d * L + i * BL + r] * carry[d];
+          dL[r][0] += dg * ab[0];
+          da[0] += dg * Lm[r][0];
+        }
+      }
+      /* chain through L[r][c] = prod_{j=c+1..r} a_j */
+      for (int r = 1; r < BL; ++r) {
+        for (int c = 0; c < r; ++c) {
+          if (dL[r][c] == 0.0) continue;
+          for (int j = c + 1; j <= r; ++j) {
+            double p = 1.0;
+            for (int jj = c + 1; jj <= r; ++jj)
+              if (jj != j) p *= ab[jj];
+            da[j] += dL[r][c] * p;
+          }
+        }
+      }
+      for (int j = 0; j < BL; ++j) dA_row[i * BL + j] = da[j];
+    }
+  }
+  free(vlast);
+  return 0;
+}

@@ -1,0 +1,121 @@
+"""numpy front-end of the C oracle (oracle/btp_oracle.c) plus bf16 helpers.
+
+TEST INFRASTRUCTURE ONLY: imported by tests/, by ``__graft_entry__.smoke`` and by the
+``cpu_baseline`` leg of ``bench.py``; the shipped package never imports it.
+
+The protocol mirrors the reference's gold-standard runner (spear/ops/btp/runners.py:111-116):
+inputs are first rounded to the kernel's storage dtype (bf16), then promoted to float64, and the
+whole computation runs in float64.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "libbtp_oracle.so")
+_lib = None
+
+L_PRODUCT, L_LOGSUM, L_CUMPROD = 0, 1, 2
+BL = 16
+DH = 16
+
+
+def build(force: bool = False) -> str:
+    """Compile the C oracle with gcc (a second or so)."""
+    src = os.path.join(_HERE, "btp_oracle.c")
+    if force or not os.path.exists(_LIB_PATH) or os.path.getmtime(_LIB_PATH) < os.path.getmtime(src):
+        subprocess.check_call(["make", "-s", "-C", _HERE, "-B", "libbtp_oracle.so"])
+    return _LIB_PATH
+
+
+def _load():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            build()
+        lib = ctypes.CDLL(_LIB_PATH)
+        dp = ctypes.POINTER(ctypes.c_double)
+        lib.btp_oracle_forward.argtypes = [dp, dp, dp, dp, ctypes.c_long, ctypes.c_long, ctypes.c_int, ctypes.c_int]
+        lib.btp_oracle_forward.restype = ctypes.c_int
+        lib.btp_oracle_forward_sequential.argtypes = [dp, dp, dp, ctypes.c_long, ctypes.c_long, ctypes.c_int]
+        lib.btp_oracle_forward_sequential.restype = ctypes.c_int
+        lib.btp_oracle_backward.argtypes = [dp, dp, dp, dp, dp, ctypes.c_long, ctypes.c_long, ctypes.c_int]
+        lib.btp_oracle_backward.restype = ctypes.c_int
+        _lib = lib
+    return _lib
+
+
+def _dptr(arr: np.ndarray):
+    return arr.ctypes.data_as(ctypes.POINTER(ctypes.c_double))
+
+
+def _as_f64(arr) -> np.ndarray:
+    return np.ascontiguousarray(np.asarray(arr, dtype=np.float64))
+
+
+def bf16_round(arr) -> np.ndarray:
+    """Round float32 values to the nearest bfloat16 (ties to even); result stays float32."""
+    f = np.ascontiguousarray(np.asarray(arr, dtype=np.float32))
+    bits = f.view(np.uint32).astype(np.uint64)
+    rounded = ((bits + 0x7FFF + ((bits >> 16) & 1)) & 0xFFFF0000).astype(np.uint32)
+    out = rounded.view(np.float32).copy()
+    nan = np.isnan(f)
+    out[nan] = np.nan
+    return out.reshape(f.shape)
+
+
+def forward(a, x, k: int = 2, l_mode: int = L_PRODUCT, with_checkpoint: bool = False):
+    """a [B,H,L], x [B,H,16,L] -> y [B,H,16,L] (float64). Optionally also the carry checkpoint."""
+    a64, x64 = _as_f64(a), _as_f64(x)
+    B, H, L = a64.shape
+    assert x64.shape == (B, H, DH, L), (a64.shape, x64.shape)
+    y = np.empty_like(x64)
+    ck = np.full((B, H, max(L // BL, 1), DH), np.nan)
+    rc = _load().btp_oracle_forward(_dptr(a64), _dptr(x64), _dptr(y), _dptr(ck), B * H, L, k, l_mode)
+    if rc != 0:
+        raise ValueError(f"btp_oracle_forward rejected its arguments (rc={rc})")
+    return (y, ck) if with_checkpoint else y
+
+
+def forward_sequential(a, x, k: int = 2):
+    a64, x64 = _as_f64(a), _as_f64(x)
+    B, H, L = a64.shape
+    y = np.empty_like(x64)
+    rc = _load().btp_oracle_forward_sequential(_dptr(a64), _dptr(x64), _dptr(y), B * H, L, k)
+    if rc != 0:
+        raise ValueError(f"btp_oracle_forward_sequential rejected its arguments (rc={rc})")
+    return y
+
+
+def backward(a, x, dy, k: int = 2):
+    """Returns (dx [B,H,16,L], dA [B,H,L]) in float64."""
+    a64, x64, g64 = _as_f64(a), _as_f64(x), _as_f64(dy)
+    B, H, L = a64.shape
+    assert x64.shape == g64.shape == (B, H, DH, L)
+    dx = np.empty_like(x64)
+    dA = np.empty_like(a64)
+    rc = _load().btp_oracle_backward(_dptr(a64), _dptr(x64), _dptr(g64), _dptr(dx), _dptr(dA), B * H, L, k)
+    if rc != 0:
+        raise ValueError(f"btp_oracle_backward rejected its arguments (rc={rc})")
+    return dx, dA
+
+
+def windowed_bruteforce(a, x, k: int = 2) -> np.ndarray:
+    """y_t = sum_{s=w(t)}^{t} (prod_{j=s+1}^{t} a_j) x_s with w(t) the start of the block before
+    t's block (k=2) or of t's own block (k=1).  Pure Python loops: tiny inputs only.  This is the
+    closed form of the operator and shares nothing with the C code."""
+    a64, x64 = _as_f64(a), _as_f64(x)
+    B, H, L = a64.shape
+    y = np.zeros_like(x64)
+    for t in range(L):
+        blk = t // BL
+        w = max(0, (blk - 1) * BL) if k == 2 else blk * BL
+        for s in range(w, t + 1):
+            decay = np.prod(a64[:, :, s + 1 : t + 1], axis=-1)  # empty product = 1
+            y[:, :, :, t] += decay[:, :, None] * x64[:, :, :, s]
+    return y

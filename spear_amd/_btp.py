@@ -1,0 +1,198 @@
+"""Host shim between torch tensors and the C ABI of ``libspear_btp.so``.
+
+Takes the place of the reference's compiled extension module ``spear._btp``
+(csrc/btp/_bindings.cu:240-243): it exports ``forward(coeff, x, y, checkpoint, k, wpb)`` and
+``backward(coeff, x, dy, checkpoint, dx, dA, k, wpb)`` with the same positional arguments, the
+same in-place semantics (the caller allocates every output) and the same argument checks and
+messages (csrc/btp/_bindings.cu:19-60, raised as ``RuntimeError`` like ``TORCH_CHECK``).
+
+The kernels are enqueued on torch's current stream of the tensors' device and the call returns
+without synchronising. There is no fallback: if the library cannot be loaded, every call raises.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import os
+import threading
+
+import torch
+
+__all__ = ["forward", "backward", "library_path", "load_library", "FLAG_WRITE_CHECKPOINT", "FLAG_PATH_MFMA"]
+
+_BF16, _F16, _F32 = 0, 1, 2
+FLAG_WRITE_CHECKPOINT = 0x1
+FLAG_PATH_MFMA = 0x2
+_ABI_VERSION = 1
+_SUPPORTED_WPB = (4, 8, 16, 32)
+
+_lock = threading.Lock()
+_lib: ctypes.CDLL | None = None
+_load_error: str | None = None
+
+
+def library_path() -> str:
+    return os.environ.get(
+        "SPEAR_BTP_LIBRARY",
+        os.path.join(os.path.dirname(os.path.abspath(__file__)), "libspear_btp.so"),
+    )
+
+
+def _declare(lib: ctypes.CDLL) -> None:
+    vp, ci, cu = ctypes.c_void_p, ctypes.c_int, ctypes.c_uint
+    lib.spear_btp_forward.argtypes = [vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, cu, vp]
+    lib.spear_btp_forward.restype = ci
+    lib.spear_btp_backward.argtypes = [vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, cu, vp]
+    lib.spear_btp_backward.restype = ci
+    lib.spear_btp_last_error.argtypes = []
+    lib.spear_btp_last_error.restype = ctypes.c_char_p
+    lib.spear_btp_abi_version.argtypes = []
+    lib.spear_btp_abi_version.restype = ci
+    lib.spear_btp_copy.argtypes = [vp, vp, ctypes.c_ulonglong, vp]
+    lib.spear_btp_copy.restype = ci
+
+
+def load_library() -> ctypes.CDLL:
+    """Load (once) and return the native library; raise ``RuntimeError`` if that is impossible."""
+    global _lib, _load_error
+    if _lib is not None:
+        return _lib
+    with _lock:
+        if _lib is not None:
+            return _lib
+        path = library_path()
+        try:
+            lib = ctypes.CDLL(path)
+            _declare(lib)
+            got = lib.spear_btp_abi_version()
+            if got != _ABI_VERSION:
+                raise OSError(f"ABI version {got}, this package needs {_ABI_VERSION}")
+        except (OSError, AttributeError) as exc:
+            _load_error = f"{path}: {exc}"
+            raise RuntimeError(
+                "spear_amd: the HIP BTP library could not be loaded "
+                f"({_load_error}). Build it with `python -m spear_amd.csrc.build` (needs hipcc); "
+                "there is no CPU fallback for spear_amd.ops.btp.btp."
+            ) from exc
+        _lib = lib
+    return _lib
+
+
+def _check(cond: bool, msg: str) -> None:
+    if not cond:
+        raise RuntimeError(msg)
+
+
+def _tag(dtype: torch.dtype) -> int:
+    if dtype == torch.bfloat16:
+        return _BF16
+    if dtype == torch.float16:
+        return _F16
+    if dtype == torch.float32:
+        return _F32
+    return -1
+
+
+def _check_common(x: torch.Tensor, coeff: torch.Tensor, k: int, wpb: int, wpb_msg: str) -> None:
+    _check(x.dim() == 4, "x must be [B, H, 16, L].")
+    _check(x.size(2) == 16, "Channel dim (DH) must be 16.")
+    _check(k in (1, 2), "k must be 1 or 2.")
+    _check(wpb in _SUPPORTED_WPB, f"{wpb_msg}{wpb}")
+    _check(coeff.dtype in (torch.float16, torch.bfloat16), "coeff must be float16 or bfloat16.")
+    _check(x.dtype == coeff.dtype, "x dtype must match coeff.")
+
+
+def _check_layout(name: str, t: torch.Tensor, shape: tuple[int, ...]) -> None:
+    # The reference reads B*H*L (resp. B*H*16*L) elements without looking at shapes or strides
+    # (csrc/btp/_bindings.cu:80-87); a wrong shape there is an out-of-bounds read. Here it raises.
+    _check(tuple(t.shape) == shape, f"{name} must have shape {list(shape)}, got {list(t.shape)}.")
+    _check(t.is_contiguous(), f"{name} must be contiguous.")
+
+
+def _raise_native(lib: ctypes.CDLL, rc: int) -> None:
+    msg = lib.spear_btp_last_error().decode("utf-8", "replace")
+    raise RuntimeError(msg or f"spear_btp call failed with code {rc}")
+
+
+def _stream_ptr(device: torch.device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def forward(
+    coeff: torch.Tensor,
+    x: torch.Tensor,
+    y: torch.Tensor,
+    checkpoint: torch.Tensor,
+    k: int,
+    wpb: int,
+    flags: int = FLAG_WRITE_CHECKPOINT,
+) -> None:
+    """``y <- btp(coeff, x)`` and ``checkpoint <- carries`` in place (csrc/btp/_bindings.cu:76-150).
+
+    ``flags`` is an extension: drop ``FLAG_WRITE_CHECKPOINT`` to skip the carry store (this
+    package's backward recomputes the carries and never reads them).
+    """
+    _check(coeff.is_cuda and x.is_cuda and y.is_cuda and checkpoint.is_cuda, "All tensors must be CUDA.")
+    _check_common(x, coeff, k, wpb, "Unsupported WPB value: ")
+    _check(y.dtype == torch.float32 or y.dtype == x.dtype, "y must be float32 or match x dtype.")
+    _check(checkpoint.dtype == torch.float32, "checkpoint must be float32.")
+    B, H, _, L = x.shape
+    _check(L % 16 == 0, "Length L must be multiple of 16")
+    _check_layout("coeff", coeff, (B, H, L))
+    _check_layout("x", x, (B, H, 16, L))
+    _check_layout("y", y, (B, H, 16, L))
+    _check_layout("checkpoint", checkpoint, (B, H, L // 16, 16))
+    _check(coeff.device == x.device == y.device == checkpoint.device, "All tensors must be on the same device.")
+
+    lib = load_library()
+    with torch.cuda.device(x.device):
+        rc = lib.spear_btp_forward(
+            coeff.data_ptr(), x.data_ptr(), y.data_ptr(), checkpoint.data_ptr(),
+            B, H, L, int(k), _tag(x.dtype), _tag(y.dtype), int(flags), _stream_ptr(x.device),
+        )
+    if rc != 0:
+        _raise_native(lib, rc)
+
+
+def backward(
+    coeff: torch.Tensor,
+    x: torch.Tensor,
+    dy: torch.Tensor,
+    checkpoint: torch.Tensor,
+    dx: torch.Tensor,
+    dA: torch.Tensor,
+    k: int,
+    wpb: int,
+    flags: int = 0,
+) -> None:
+    """``dx, dA <- vjp of btp at (coeff, x) applied to dy``, in place (csrc/btp/_bindings.cu:152-229).
+
+    Every element of ``dA`` is written, so it need not arrive zero-filled. ``checkpoint`` is
+    accepted for signature compatibility and not read.
+    """
+    _check(
+        coeff.is_cuda and x.is_cuda and dy.is_cuda and checkpoint.is_cuda,
+        "coeff, x, dy, checkpoint must be CUDA.",
+    )
+    _check(dx.is_cuda and dA.is_cuda, "dx and dA must be CUDA.")
+    _check_common(x, coeff, k, wpb, "Unsupported WPB value for backward: ")
+    _check(dx.dtype == x.dtype, "dx dtype must match x.")
+    _check(dA.dtype == torch.float32, "dA must be float32.")
+    _check(dy.dtype == torch.float32 or dy.dtype == x.dtype, "dy must be float32 or match x dtype.")
+    B, H, _, L = x.shape
+    _check(L % 16 == 0, "Length L must be multiple of 16")
+    _check_layout("coeff", coeff, (B, H, L))
+    _check_layout("x", x, (B, H, 16, L))
+    _check_layout("dy", dy, (B, H, 16, L))
+    _check_layout("dx", dx, (B, H, 16, L))
+    _check_layout("dA", dA, (B, H, L))
+    _check(coeff.device == x.device == dy.device == dx.device == dA.device, "All tensors must be on the same device.")
+
+    lib = load_library()
+    with torch.cuda.device(x.device):
+        rc = lib.spear_btp_backward(
+            coeff.data_ptr(), x.data_ptr(), dy.data_ptr(), checkpoint.data_ptr(), dx.data_ptr(), dA.data_ptr(),
+            B, H, L, int(k), _tag(x.dtype), _tag(dy.dtype), int(flags), _stream_ptr(x.device),
+        )
+    if rc != 0:
+        _raise_native(lib, rc)

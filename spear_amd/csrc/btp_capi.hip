@@ -1,0 +1,99 @@
+// C ABI of the BTP library: argument validation, error reporting, dispatch to the kernel
+// launchers. Validation mirrors what the reference's binding checks before launching
+// (csrc/btp/_bindings.cu:19-60) for the properties that are visible at this level (k, dtypes),
+// and adds the ones the reference leaves unchecked (L % 16, alignment, NULL pointers).
+#include <hip/hip_runtime.h>
+#include <stdarg.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include "../../include/spear_btp.h"
+#include "btp_launch.h"
+
+namespace {
+
+thread_local char g_error[256] = "";
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_error, sizeof(g_error), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+int check_common(const char* who, int B, int H, int L, int k, int in_dtype, int io_dtype, const char* io_name,
+                 unsigned flags, unsigned allowed_flags) {
+  if (B < 0 || H < 0 || L < 0) return fail(SPEAR_BTP_EINVAL, "%s: negative dimension (B=%d H=%d L=%d)", who, B, H, L);
+  if (L % 16 != 0) return fail(SPEAR_BTP_EINVAL, "%s: Length L must be multiple of 16 (got %d)", who, L);
+  if (k != 1 && k != 2) return fail(SPEAR_BTP_EINVAL, "%s: k must be 1 or 2.", who);
+  if (in_dtype != SPEAR_BTP_BF16 && in_dtype != SPEAR_BTP_F16)
+    return fail(SPEAR_BTP_EINVAL, "%s: coeff must be float16 or bfloat16.", who);
+  if (io_dtype != SPEAR_BTP_F32 && io_dtype != in_dtype)
+    return fail(SPEAR_BTP_EINVAL, "%s: %s must be float32 or match x dtype.", who, io_name);
+  if (flags & ~allowed_flags) return fail(SPEAR_BTP_EINVAL, "%s: unknown flag bits 0x%x", who, flags & ~allowed_flags);
+  if ((long long)B * H * 16ll * L >= (1ll << 40)) return fail(SPEAR_BTP_EINVAL, "%s: tensor too large", who);
+  return 0;
+}
+
+}  // namespace
+
+extern "C" {
+
+int spear_btp_abi_version(void) { return 1; }
+
+const char* spear_btp_last_error(void) { return g_error; }
+
+int spear_btp_forward(const void* coeff, const void* x, void* y, float* checkpoint, int B, int H, int L, int k,
+                      int in_dtype, int out_dtype, unsigned flags, void* stream) {
+  g_error[0] = '\0';
+  if (int rc = check_common("spear_btp_forward", B, H, L, k, in_dtype, out_dtype, "y", flags,
+                            SPEAR_BTP_WRITE_CHECKPOINT | SPEAR_BTP_PATH_MFMA))
+    return rc;
+  if ((long long)B * H == 0 || L == 0) return 0;
+  const bool want_ckpt = (flags & SPEAR_BTP_WRITE_CHECKPOINT) != 0;
+  if (!coeff || !x || !y || (want_ckpt && !checkpoint))
+    return fail(SPEAR_BTP_ENULL, "spear_btp_forward: NULL tensor pointer");
+  if (!aligned16(coeff) || !aligned16(x) || !aligned16(y) || (want_ckpt && !aligned16(checkpoint)))
+    return fail(SPEAR_BTP_EINVAL, "spear_btp_forward: tensor pointers must be 16-byte aligned");
+  if (flags & SPEAR_BTP_PATH_MFMA)
+    return fail(SPEAR_BTP_EINVAL, "spear_btp_forward: the MFMA path is not built into this library");
+
+  spear_btp::FwdArgs a{coeff, x, y, want_ckpt ? checkpoint : nullptr, B, H, L, k, in_dtype, out_dtype};
+  const hipError_t err = spear_btp::scan_forward(a, static_cast<hipStream_t>(stream));
+  if (err != hipSuccess) return fail(SPEAR_BTP_ELAUNCH, "spear_btp_forward: launch failed: %s", hipGetErrorString(err));
+  return 0;
+}
+
+int spear_btp_backward(const void* coeff, const void* x, const void* dy, const float* checkpoint, void* dx, float* dA,
+                       int B, int H, int L, int k, int in_dtype, int dy_dtype, unsigned flags, void* stream) {
+  (void)checkpoint;  // carries are recomputed from coeff and x
+  g_error[0] = '\0';
+  if (int rc = check_common("spear_btp_backward", B, H, L, k, in_dtype, dy_dtype, "dy", flags, SPEAR_BTP_PATH_MFMA))
+    return rc;
+  if ((long long)B * H == 0 || L == 0) return 0;
+  if (!coeff || !x || !dy || !dx || !dA) return fail(SPEAR_BTP_ENULL, "spear_btp_backward: NULL tensor pointer");
+  if (!aligned16(coeff) || !aligned16(x) || !aligned16(dy) || !aligned16(dx) || !aligned16(dA))
+    return fail(SPEAR_BTP_EINVAL, "spear_btp_backward: tensor pointers must be 16-byte aligned");
+  if (flags & SPEAR_BTP_PATH_MFMA)
+    return fail(SPEAR_BTP_EINVAL, "spear_btp_backward: the MFMA path is not built into this library");
+
+  spear_btp::BwdArgs a{coeff, x, dy, dx, dA, B, H, L, k, in_dtype, dy_dtype};
+  const hipError_t err = spear_btp::scan_backward(a, static_cast<hipStream_t>(stream));
+  if (err != hipSuccess) return fail(SPEAR_BTP_ELAUNCH, "spear_btp_backward: launch failed: %s", hipGetErrorString(err));
+  return 0;
+}
+
+int spear_btp_copy(const void* src, void* dst, unsigned long long bytes, void* stream) {
+  g_error[0] = '\0';
+  if (!src || !dst) return fail(SPEAR_BTP_ENULL, "spear_btp_copy: NULL pointer");
+  if (bytes % 16 != 0 || !aligned16(src) || !aligned16(dst))
+    return fail(SPEAR_BTP_EINVAL, "spear_btp_copy: size and pointers must be multiples of 16 bytes");
+  const hipError_t err = spear_btp::device_copy(src, dst, bytes, static_cast<hipStream_t>(stream));
+  if (err != hipSuccess) return fail(SPEAR_BTP_ELAUNCH, "spear_btp_copy: launch failed: %s", hipGetErrorString(err));
+  return 0;
+}
+
+}  // extern "C"

@@ -1,0 +1,39 @@
+// Host-side argument blocks and launcher entry points shared by the C ABI and the kernel files.
+// They stand where the reference has its templated launchers
+// (csrc/btp/btp-forward.cu:462-527, csrc/btp/btp-backwards.cu:811-884).
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+namespace spear_btp {
+
+// Must match SPEAR_BTP_BF16 / _F16 / _F32 of the public header.
+enum Dtype : int { kBf16 = 0, kF16 = 1, kF32 = 2 };
+
+struct FwdArgs {
+  const void* coeff;
+  const void* x;
+  void* y;
+  float* checkpoint;  // nullptr: do not store the carry checkpoint
+  int B, H, L, k;
+  int in_dtype, out_dtype;
+};
+
+struct BwdArgs {
+  const void* coeff;
+  const void* x;
+  const void* dy;
+  void* dx;
+  float* dA;
+  int B, H, L, k;
+  int in_dtype, dy_dtype;
+};
+
+// Exact-fp32 recurrence kernels (btp_scan.hip).
+hipError_t scan_forward(const FwdArgs& p, hipStream_t s);
+hipError_t scan_backward(const BwdArgs& p, hipStream_t s);
+
+// Plain copy kernel used for bandwidth / counter calibration (btp_scan.hip).
+hipError_t device_copy(const void* src, void* dst, unsigned long long bytes, hipStream_t s);
+
+}  // namespace spear_btp

@@ -1,0 +1,563 @@
+// Exact-fp32 recurrence kernels for the Block Two-Pass operator on gfx950 (MI355X).
+//
+// They replace the reference's sm90 kernels
+//   btp_forward_kernel   csrc/btp/btp-forward.cu:85-457
+//   btp_backward_kernel  csrc/btp/btp-backwards.cu:165-808
+// and compute the same function,
+//   y_t = sum_{s = w(t)}^{t} (prod_{j=s+1..t} a_j) x_s ,  w(t) = first step of the block before
+//   t's block (k = 2) or of t's own block (k = 1),
+// but are organised for CDNA4 rather than translated:
+//
+//   * One wavefront owns a span of 128 consecutive steps (8 blocks) of one (batch, head) row:
+//     a [16 channel x 128 step] slab, 4 KiB in bf16. The slab is moved between HBM and LDS with
+//     16-byte-per-lane accesses in which 16 consecutive lanes cover 256 contiguous bytes of one
+//     channel row (for L = 128 a whole instruction covers 1 KiB of contiguous memory).
+//   * In LDS the slab is stored with its 16-byte chunks XOR-swizzled by the channel index, so
+//     that both the row-major (memory order) and the per-channel (compute order) access patterns
+//     are bank-conflict free without padding.
+//   * For the arithmetic, lane (j, d) = (lane / 16, lane % 16) owns channel d of blocks 2j and
+//     2j+1 of the span and runs the linear recurrence h <- a*h + x in registers. The decay
+//     "matrix" of the reference (16x16 per block, built with exp/log and rounded to bf16 for the
+//     tensor-core MMA, btp-forward.cu:214-274) is never materialised: a block's contribution is
+//     a 16-step recurrence started from zero, and the one-hop carry of the second pass is the
+//     same recurrence started from the previous block's local terminal state. All products are
+//     plain fp32 multiplications in linear space, so there is no log/exp, no 0*Inf and no
+//     cancellation; results agree with a float64 evaluation to fp32 rounding.
+//   * The previous block's terminal state travels between lane groups with one ds_bpermute
+//     (the reference uses shared memory plus a DSMEM bulk copy and cluster barriers,
+//     btp-forward.cu:287-374). At the left edge of a span it is recomputed from the 16 steps
+//     before the span (a halo read that normally hits L2), so spans are fully independent:
+//     no flags, no look-back, no second kernel, and the carry is never dropped at a launch-shape
+//     boundary (the reference drops it at cluster boundaries, btp-forward.cu:359-366).
+//
+// Backward uses, per block i with local index r (g = dy, c = carry into the block,
+// dC = carry of the gradient coming back from block i+1):
+//   v_r  = a_r v_{r-1} + x_r            (v_{-1} = 0)      local forward state
+//   A_r  = g_r + a_{r+1} A_{r+1}        (A_16  = 0)       local reverse state
+//   dx_r = g_r + a_{r+1} dx_{r+1}       (a_16 dx_16 := dC) reverse state with the gradient carry
+//   dC_{i-1} = a_0 A_0                                    what block i sends to block i-1
+//   dA_r = <dx_r, v_{r-1}> + (prod_{j<r} a_j) <A_r, c>    (sum over the 16 channels)
+// which is the derivative the reference assembles from "Part V" and "Part A"
+// (btp-backwards.cu:372-413, 637-796) but needs no division by a_r, no max-shifted exponentials
+// and no special cases: it is finite and correct at a_r = 0.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <type_traits>
+
+#include "btp_device.h"
+#include "btp_launch.h"
+
+namespace spear_btp {
+
+namespace {
+
+// Byte offset, inside a wavefront's LDS image with `kRowBytes` per channel row, of the 16-byte
+// chunk `chunk` of channel row `r`. XOR with the row index permutes chunks inside aligned groups
+// of 16, i.e. inside one 256-byte bank period.
+template <int kRowBytes>
+__device__ __forceinline__ int swz(int r, int chunk) {
+  return r * kRowBytes + ((chunk ^ r) << 4);
+}
+
+__device__ __forceinline__ uint4 zero4() { return make_uint4(0u, 0u, 0u, 0u); }
+
+// Loads the 16 coefficients of one block (32 bytes, wave-uniform address per lane group) and
+// returns them clamped, as floats.
+template <class E>
+__device__ __forceinline__ void load_block_coeffs(const uint16_t* p, float (&a)[16]) {
+  const uint4 q0 = *reinterpret_cast<const uint4*>(p);
+  const uint4 q1 = *reinterpret_cast<const uint4*>(p + 8);
+  unpack8<E>(q0, a);
+  unpack8<E>(q1, a + 8);
+#pragma unroll
+  for (int i = 0; i < 16; ++i) a[i] = clamp_coeff<E>(a[i]);
+}
+
+// ------------------------------------------------------------------------------------------
+// Stage a [16 x 128] slab of 16-bit elements: coalesced global reads -> swizzled LDS image.
+// Lane l of pass `it` handles channel row 4*it + l/16, chunk l%16 (8 steps).
+// ------------------------------------------------------------------------------------------
+__device__ __forceinline__ void slab16_global_to_regs(const uint16_t* slab, long L, int nvalid,
+                                                      int lane, uint4 (&q)[4]) {
+  const int lr = lane >> 4, lp = lane & 15;
+  const bool ok = (lp << 3) < nvalid;
+#pragma unroll
+  for (int it = 0; it < 4; ++it) {
+    const int r = it * 4 + lr;
+    q[it] = ok ? *reinterpret_cast<const uint4*>(slab + (long)r * L + (lp << 3)) : zero4();
+  }
+}
+
+__device__ __forceinline__ void slab16_regs_to_lds(unsigned char* img, int lane, const uint4 (&q)[4]) {
+  const int lr = lane >> 4, lp = lane & 15;
+#pragma unroll
+  for (int it = 0; it < 4; ++it) {
+    const int r = it * 4 + lr;
+    *reinterpret_cast<uint4*>(img + swz<256>(r, lp)) = q[it];
+  }
+}
+
+__device__ __forceinline__ void slab16_lds_to_global(const unsigned char* img, uint16_t* slab, long L,
+                                                     int nvalid, int lane) {
+  const int lr = lane >> 4, lp = lane & 15;
+  const bool ok = (lp << 3) < nvalid;
+#pragma unroll
+  for (int it = 0; it < 4; ++it) {
+    const int r = it * 4 + lr;
+    const uint4 v = *reinterpret_cast<const uint4*>(img + swz<256>(r, lp));
+    if (ok) *reinterpret_cast<uint4*>(slab + (long)r * L + (lp << 3)) = v;
+  }
+}
+
+// Same for a [16 x 128] slab of fp32 (512 B per row, 32 chunks of 4 steps).
+// Lane l of pass `it` handles channel row 2*it + l/32, chunk l%32.
+__device__ __forceinline__ void slab32_global_to_regs(const float* slab, long L, int nvalid, int lane,
+                                                      uint4 (&q)[8]) {
+  const int lr = lane >> 5, lp = lane & 31;
+  const bool ok = (lp << 2) < nvalid;
+#pragma unroll
+  for (int it = 0; it < 8; ++it) {
+    const int r = it * 2 + lr;
+    q[it] = ok ? *reinterpret_cast<const uint4*>(slab + (long)r * L + (lp << 2)) : zero4();
+  }
+}
+
+__device__ __forceinline__ void slab32_regs_to_lds(unsigned char* img, int lane, const uint4 (&q)[8]) {
+  const int lr = lane >> 5, lp = lane & 31;
+#pragma unroll
+  for (int it = 0; it < 8; ++it) {
+    const int r = it * 2 + lr;
+    *reinterpret_cast<uint4*>(img + swz<512>(r, lp)) = q[it];
+  }
+}
+
+__device__ __forceinline__ void slab32_lds_to_global(const unsigned char* img, float* slab, long L,
+                                                     int nvalid, int lane) {
+  const int lr = lane >> 5, lp = lane & 31;
+  const bool ok = (lp << 2) < nvalid;
+#pragma unroll
+  for (int it = 0; it < 8; ++it) {
+    const int r = it * 2 + lr;
+    const uint4 v = *reinterpret_cast<const uint4*>(img + swz<512>(r, lp));
+    if (ok) *reinterpret_cast<uint4*>(slab + (long)r * L + (lp << 2)) = v;
+  }
+}
+
+// Per-channel reads/writes of the lane's own 32 steps (blocks 2j and 2j+1 of channel d).
+template <class E>
+__device__ __forceinline__ void lane_read16(const unsigned char* img, int j, int d, float (&v)[32]) {
+#pragma unroll
+  for (int c = 0; c < 4; ++c) {
+    const uint4 q = *reinterpret_cast<const uint4*>(img + swz<256>(d, 4 * j + c));
+    unpack8<E>(q, v + 8 * c);
+  }
+}
+
+template <class E>
+__device__ __forceinline__ void lane_write16(unsigned char* img, int j, int d, const float (&v)[32]) {
+#pragma unroll
+  for (int c = 0; c < 4; ++c)
+    *reinterpret_cast<uint4*>(img + swz<256>(d, 4 * j + c)) = pack8<E>(v + 8 * c);
+}
+
+__device__ __forceinline__ void lane_read32(const unsigned char* img, int j, int d, float (&v)[32]) {
+#pragma unroll
+  for (int c = 0; c < 8; ++c) {
+    const float4 q = *reinterpret_cast<const float4*>(img + swz<512>(d, 8 * j + c));
+    v[4 * c + 0] = q.x; v[4 * c + 1] = q.y; v[4 * c + 2] = q.z; v[4 * c + 3] = q.w;
+  }
+}
+
+__device__ __forceinline__ void lane_write32(unsigned char* img, int j, int d, const float (&v)[32]) {
+#pragma unroll
+  for (int c = 0; c < 8; ++c)
+    *reinterpret_cast<float4*>(img + swz<512>(d, 8 * j + c)) =
+        make_float4(v[4 * c + 0], v[4 * c + 1], v[4 * c + 2], v[4 * c + 3]);
+}
+
+// Coefficients of the span: 2 per lane from global, clamped, as fp32 into LDS; every lane then
+// reads back the 32 of its own two blocks (a broadcast read for the 16 lanes of a group).
+template <class E>
+__device__ __forceinline__ uint32_t coeff_global_to_reg(const uint16_t* arow, int nvalid, int lane) {
+  return ((lane << 1) < nvalid) ? *reinterpret_cast<const uint32_t*>(arow + (lane << 1)) : 0u;
+}
+
+template <class E>
+__device__ __forceinline__ void coeff_reg_to_lds(float* a_lds, int lane, uint32_t w) {
+  float2 f;
+  f.x = clamp_coeff<E>(E::lo(w));
+  f.y = clamp_coeff<E>(E::hi(w));
+  *reinterpret_cast<float2*>(a_lds + (lane << 1)) = f;
+}
+
+__device__ __forceinline__ void coeff_lane_read(const float* a_lds, int j, float (&a)[32]) {
+#pragma unroll
+  for (int c = 0; c < 8; ++c) {
+    const float4 q = *reinterpret_cast<const float4*>(a_lds + 32 * j + 4 * c);
+    a[4 * c + 0] = q.x; a[4 * c + 1] = q.y; a[4 * c + 2] = q.z; a[4 * c + 3] = q.w;
+  }
+}
+
+struct SpanCoord {
+  long row;    // (batch, head) row index
+  int sp;      // span index inside the row
+  int s0;      // first step of the span
+  int nvalid;  // valid steps in the span (multiple of 16, <= 128)
+};
+
+__device__ __forceinline__ SpanCoord span_coord(long span, int spans_per_row, int L) {
+  SpanCoord c;
+  c.row = span / spans_per_row;
+  c.sp = (int)(span - c.row * spans_per_row);
+  c.s0 = c.sp * kSpan;
+  c.nvalid = min(kSpan, L - c.s0);
+  return c;
+}
+
+// ==========================================================================================
+// Forward
+// ==========================================================================================
+template <class E, class OutT, bool kCheckpoint>
+__global__ __launch_bounds__(64 * kWaves) void btp_fwd_scan_kernel(
+    const uint16_t* __restrict__ coeff, const uint16_t* __restrict__ x, OutT* __restrict__ y,
+    float* __restrict__ ckpt, int L, int spans_per_row, long total_spans, int k) {
+  constexpr bool kOutF32 = std::is_same<OutT, float>::value;
+  constexpr int kImgBytes = kOutF32 ? 8192 : 4096;
+  __shared__ __align__(16) unsigned char lds[kWaves][kImgBytes + 512];
+
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const long span = (long)blockIdx.x * kWaves + wave;
+  if (span >= total_spans) return;  // wave-uniform; no workgroup barrier is used anywhere
+  const SpanCoord sc = span_coord(span, spans_per_row, L);
+
+  unsigned char* img = lds[wave];
+  float* a_lds = reinterpret_cast<float*>(img + kImgBytes);
+  const uint16_t* xslab = x + (sc.row * kChan) * (long)L + sc.s0;
+  const uint16_t* arow = coeff + sc.row * (long)L + sc.s0;
+  const int j = lane >> 4, d = lane & 15;
+
+  // ---- all global reads are issued before anything waits on them
+  uint4 xin[4];
+  slab16_global_to_regs(xslab, L, sc.nvalid, lane, xin);
+  const uint32_t ain = coeff_global_to_reg<E>(arow, sc.nvalid, lane);
+
+  const bool halo = (k == 2) && (sc.sp > 0);  // wave-uniform
+  float c_halo = 0.0f;
+  if (halo && j == 0) {
+    // local terminal state of the block just left of the span, channel d
+    float ah[16], xh[16];
+    load_block_coeffs<E>(arow - kTile, ah);
+    const uint16_t* xp = xslab + (long)d * L - kTile;
+    unpack8<E>(*reinterpret_cast<const uint4*>(xp), xh);
+    unpack8<E>(*reinterpret_cast<const uint4*>(xp + 8), xh + 8);
+    float h = 0.0f;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) h = fmaf(ah[r], h, xh[r]);
+    c_halo = h;
+  }
+
+  slab16_regs_to_lds(img, lane, xin);
+  coeff_reg_to_lds<E>(a_lds, lane, ain);
+  wave_lds_handover();
+
+  float xf[32], a[32];
+  lane_read16<E>(img, j, d, xf);
+  coeff_lane_read(a_lds, j, a);
+
+  // chain 1: zero state at the start of block A, run through both blocks. The first 16 steps
+  // give A's local states (only the terminal one is kept); continuing into B from that terminal
+  // state yields exactly B's outputs for k = 2.
+  float yv[32];
+  float h = 0.0f;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) h = fmaf(a[r], h, xf[r]);
+  const float vA_last = h;
+  h = (k == 2) ? vA_last : 0.0f;
+#pragma unroll
+  for (int r = 16; r < 32; ++r) {
+    h = fmaf(a[r], h, xf[r]);
+    yv[r] = h;
+  }
+  // chain 2: B's local terminal state, needed by the next lane group's block A
+  float vB_last = yv[31];
+  if (k == 2) {
+    float h3 = 0.0f;
+#pragma unroll
+    for (int r = 16; r < 32; ++r) h3 = fmaf(a[r], h3, xf[r]);
+    vB_last = h3;
+  }
+  const float from_left = lane_rotate(vB_last, lane, -16);
+  const float cA = (k == 2) ? (j == 0 ? c_halo : from_left) : 0.0f;
+  // chain 3: block A started from its carry
+  h = cA;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    h = fmaf(a[r], h, xf[r]);
+    yv[r] = h;
+  }
+
+  if constexpr (kCheckpoint) {
+    if (k == 2) {
+      const long nb = L / kTile;
+      const long tA = (long)sc.sp * (kSpan / kTile) + 2 * j;  // block index of A inside the row
+      float* slot = ckpt + (sc.row * nb + tA) * kChan + d;    // slot of block A's own state
+      if (32 * j < sc.nvalid && tA >= 1) slot[-kChan] = cA;   // carry consumed by block A
+      if (32 * j + 16 < sc.nvalid) slot[0] = vA_last;         // carry consumed by block B
+    }
+  }
+
+  // ---- results back through LDS so that the global writes are coalesced
+  wave_lds_handover();
+  if constexpr (kOutF32) {
+    lane_write32(img, j, d, yv);
+    wave_lds_handover();
+    slab32_lds_to_global(img, reinterpret_cast<float*>(y) + (sc.row * kChan) * (long)L + sc.s0, L,
+                         sc.nvalid, lane);
+  } else {
+    lane_write16<E>(img, j, d, yv);
+    wave_lds_handover();
+    slab16_lds_to_global(img, reinterpret_cast<uint16_t*>(y) + (sc.row * kChan) * (long)L + sc.s0, L,
+                         sc.nvalid, lane);
+  }
+}
+
+// ==========================================================================================
+// Backward
+// ==========================================================================================
+template <class E, class GradT>
+__global__ __launch_bounds__(64 * kWaves) void btp_bwd_scan_kernel(
+    const uint16_t* __restrict__ coeff, const uint16_t* __restrict__ x, const GradT* __restrict__ dy,
+    uint16_t* __restrict__ dx, float* __restrict__ dA, int L, int spans_per_row, long total_spans,
+    int k) {
+  constexpr bool kGradF32 = std::is_same<GradT, float>::value;
+  constexpr int kGradBytes = kGradF32 ? 8192 : 4096;
+  __shared__ __align__(16) unsigned char lds[kWaves][4096 + kGradBytes + 512];
+
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const long span = (long)blockIdx.x * kWaves + wave;
+  if (span >= total_spans) return;
+  const SpanCoord sc = span_coord(span, spans_per_row, L);
+
+  unsigned char* img_x = lds[wave];
+  unsigned char* img_g = img_x + 4096;
+  float* a_lds = reinterpret_cast<float*>(img_g + kGradBytes);
+  const long slab_off = (sc.row * kChan) * (long)L + sc.s0;
+  const uint16_t* xslab = x + slab_off;
+  const uint16_t* arow = coeff + sc.row * (long)L + sc.s0;
+  const int j = lane >> 4, d = lane & 15;
+
+  // ---- global reads
+  uint4 xin[4];
+  slab16_global_to_regs(xslab, L, sc.nvalid, lane, xin);
+  uint4 gin[kGradF32 ? 8 : 4];
+  if constexpr (kGradF32) {
+    slab32_global_to_regs(reinterpret_cast<const float*>(dy) + slab_off, L, sc.nvalid, lane, gin);
+  } else {
+    slab16_global_to_regs(reinterpret_cast<const uint16_t*>(dy) + slab_off, L, sc.nvalid, lane, gin);
+  }
+  const uint32_t ain = coeff_global_to_reg<E>(arow, sc.nvalid, lane);
+
+  const bool halo_left = (k == 2) && (sc.sp > 0);              // wave-uniform
+  const bool halo_right = (k == 2) && (sc.s0 + kSpan < L);     // wave-uniform
+  float c_halo = 0.0f, dc_halo = 0.0f;
+  if (halo_left && j == 0) {
+    float ah[16], xh[16];
+    load_block_coeffs<E>(arow - kTile, ah);
+    const uint16_t* xp = xslab + (long)d * L - kTile;
+    unpack8<E>(*reinterpret_cast<const uint4*>(xp), xh);
+    unpack8<E>(*reinterpret_cast<const uint4*>(xp + 8), xh + 8);
+    float h = 0.0f;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) h = fmaf(ah[r], h, xh[r]);
+    c_halo = h;
+  }
+  if (halo_right && j == 3) {
+    // gradient carry sent by the block just right of the span: a_0 * A_0 of that block
+    float ah[16], gh[16];
+    load_block_coeffs<E>(arow + kSpan, ah);
+    if constexpr (kGradF32) {
+      const float* gp = reinterpret_cast<const float*>(dy) + slab_off + (long)d * L + kSpan;
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        const float4 q = *reinterpret_cast<const float4*>(gp + 4 * c);
+        gh[4 * c + 0] = q.x; gh[4 * c + 1] = q.y; gh[4 * c + 2] = q.z; gh[4 * c + 3] = q.w;
+      }
+    } else {
+      const uint16_t* gp = reinterpret_cast<const uint16_t*>(dy) + slab_off + (long)d * L + kSpan;
+      unpack8<E>(*reinterpret_cast<const uint4*>(gp), gh);
+      unpack8<E>(*reinterpret_cast<const uint4*>(gp + 8), gh + 8);
+    }
+    float h = gh[15];
+#pragma unroll
+    for (int r = 14; r >= 0; --r) h = fmaf(ah[r + 1], h, gh[r]);
+    dc_halo = ah[0] * h;
+  }
+
+  slab16_regs_to_lds(img_x, lane, xin);
+  if constexpr (kGradF32) {
+    slab32_regs_to_lds(img_g, lane, gin);
+  } else {
+    uint4 g4[4] = {gin[0], gin[1], gin[2], gin[3]};
+    slab16_regs_to_lds(img_g, lane, g4);
+  }
+  coeff_reg_to_lds<E>(a_lds, lane, ain);
+  wave_lds_handover();
+
+  float xf[32], gf[32], a[32];
+  lane_read16<E>(img_x, j, d, xf);
+  if constexpr (kGradF32) {
+    lane_read32(img_g, j, d, gf);
+  } else {
+    lane_read16<E>(img_g, j, d, gf);
+  }
+  coeff_lane_read(a_lds, j, a);
+
+  // local forward states of both blocks (zero start); v[r] for block A, v[16 + r] for block B
+  float v[32];
+  {
+    float h = 0.0f;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) { h = fmaf(a[r], h, xf[r]); v[r] = h; }
+    h = 0.0f;
+#pragma unroll
+    for (int r = 16; r < 32; ++r) { h = fmaf(a[r], h, xf[r]); v[r] = h; }
+  }
+  // local reverse states (zero start at each block's end)
+  float A[32];
+  {
+    float h = gf[15];
+    A[15] = h;
+#pragma unroll
+    for (int r = 14; r >= 0; --r) { h = fmaf(a[r + 1], h, gf[r]); A[r] = h; }
+    h = gf[31];
+    A[31] = h;
+#pragma unroll
+    for (int r = 30; r >= 16; --r) { h = fmaf(a[r + 1], h, gf[r]); A[r] = h; }
+  }
+
+  const bool two = (k == 2);
+  // carries: forward ones flow to the right, gradient ones to the left
+  const float from_left = lane_rotate(v[31], lane, -16);
+  const float from_right = lane_rotate(a[0] * A[0], lane, +16);
+  const float cA = two ? (j == 0 ? c_halo : from_left) : 0.0f;
+  const float cB = two ? v[15] : 0.0f;
+  const float dcA = two ? a[16] * A[16] : 0.0f;
+  const float dcB = two ? (j == 3 ? dc_halo : from_right) : 0.0f;
+
+  float dxv[32];
+  float e[16];
+  float dA_A, dA_B;
+  {
+    // block A
+    float h = gf[15] + dcA;
+    dxv[15] = h;
+#pragma unroll
+    for (int r = 14; r >= 0; --r) { h = fmaf(a[r + 1], h, gf[r]); dxv[r] = h; }
+    float z = cA;
+    e[0] = A[0] * z;
+#pragma unroll
+    for (int r = 1; r < 16; ++r) {
+      z *= a[r - 1];
+      e[r] = fmaf(dxv[r], v[r - 1], A[r] * z);
+    }
+    dA_A = row_transpose_reduce(e, d);
+  }
+  {
+    // block B
+    float h = gf[31] + dcB;
+    dxv[31] = h;
+#pragma unroll
+    for (int r = 30; r >= 16; --r) { h = fmaf(a[r + 1], h, gf[r]); dxv[r] = h; }
+    float z = cB;
+    e[0] = A[16] * z;
+#pragma unroll
+    for (int r = 1; r < 16; ++r) {
+      z *= a[16 + r - 1];
+      e[r] = fmaf(dxv[16 + r], v[16 + r - 1], A[16 + r] * z);
+    }
+    dA_B = row_transpose_reduce(e, d);
+  }
+
+  float* dArow = dA + sc.row * (long)L + sc.s0 + 32 * j + d;
+  if (32 * j < sc.nvalid) dArow[0] = dA_A;
+  if (32 * j + 16 < sc.nvalid) dArow[16] = dA_B;
+
+  // dx goes back through the x image: every lane overwrites exactly the chunks it read
+  lane_write16<E>(img_x, j, d, dxv);
+  wave_lds_handover();
+  slab16_lds_to_global(img_x, dx + slab_off, L, sc.nvalid, lane);
+}
+
+__global__ __launch_bounds__(256) void copy_kernel(const uint4* __restrict__ src, uint4* __restrict__ dst,
+                                                   unsigned long long n16) {
+  const unsigned long long stride = (unsigned long long)gridDim.x * blockDim.x;
+  for (unsigned long long i = (unsigned long long)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += stride)
+    dst[i] = src[i];
+}
+
+struct Grid {
+  int spans_per_row;
+  long total_spans;
+  unsigned blocks;
+};
+
+inline Grid make_grid(long rows, int L) {
+  Grid g;
+  g.spans_per_row = (L + kSpan - 1) / kSpan;
+  g.total_spans = rows * g.spans_per_row;
+  g.blocks = (unsigned)((g.total_spans + kWaves - 1) / kWaves);
+  return g;
+}
+
+template <class E, class OutT>
+hipError_t launch_fwd(const FwdArgs& p, hipStream_t s) {
+  const Grid g = make_grid((long)p.B * p.H, p.L);
+  const auto* c = static_cast<const uint16_t*>(p.coeff);
+  const auto* x = static_cast<const uint16_t*>(p.x);
+  auto* y = static_cast<OutT*>(p.y);
+  if (p.checkpoint != nullptr) {
+    hipLaunchKernelGGL((btp_fwd_scan_kernel<E, OutT, true>), dim3(g.blocks), dim3(64 * kWaves), 0, s, c, x, y,
+                       p.checkpoint, p.L, g.spans_per_row, g.total_spans, p.k);
+  } else {
+    hipLaunchKernelGGL((btp_fwd_scan_kernel<E, OutT, false>), dim3(g.blocks), dim3(64 * kWaves), 0, s, c, x, y,
+                       static_cast<float*>(nullptr), p.L, g.spans_per_row, g.total_spans, p.k);
+  }
+  return hipGetLastError();
+}
+
+template <class E, class GradT>
+hipError_t launch_bwd(const BwdArgs& p, hipStream_t s) {
+  const Grid g = make_grid((long)p.B * p.H, p.L);
+  hipLaunchKernelGGL((btp_bwd_scan_kernel<E, GradT>), dim3(g.blocks), dim3(64 * kWaves), 0, s,
+                     static_cast<const uint16_t*>(p.coeff), static_cast<const uint16_t*>(p.x),
+                     static_cast<const GradT*>(p.dy), static_cast<uint16_t*>(p.dx), p.dA, p.L, g.spans_per_row,
+                     g.total_spans, p.k);
+  return hipGetLastError();
+}
+
+}  // namespace
+
+hipError_t scan_forward(const FwdArgs& p, hipStream_t s) {
+  const bool bf = p.in_dtype == kBf16, f32 = p.out_dtype == kF32;
+  if (bf) return f32 ? launch_fwd<Bf16, float>(p, s) : launch_fwd<Bf16, uint16_t>(p, s);
+  return f32 ? launch_fwd<Fp16, float>(p, s) : launch_fwd<Fp16, uint16_t>(p, s);
+}
+
+hipError_t scan_backward(const BwdArgs& p, hipStream_t s) {
+  const bool bf = p.in_dtype == kBf16, f32 = p.dy_dtype == kF32;
+  if (bf) return f32 ? launch_bwd<Bf16, float>(p, s) : launch_bwd<Bf16, uint16_t>(p, s);
+  return f32 ? launch_bwd<Fp16, float>(p, s) : launch_bwd<Fp16, uint16_t>(p, s);
+}
+
+hipError_t device_copy(const void* src, void* dst, unsigned long long bytes, hipStream_t s) {
+  const unsigned long long n16 = bytes / 16;
+  if (n16 == 0) return hipSuccess;
+  unsigned long long want = (n16 + 255) / 256;
+  const unsigned blocks = (unsigned)(want < 256ull * 32 ? want : 256ull * 32);
+  hipLaunchKernelGGL(copy_kernel, dim3(blocks), dim3(256), 0, s, static_cast<const uint4*>(src),
+                     static_cast<uint4*>(dst), n16);
+  return hipGetLastError();
+}
+
+}  // namespace spear_btp

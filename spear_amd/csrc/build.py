@@ -1,0 +1,72 @@
+"""Builds ``spear_amd/libspear_btp.so`` (HIP kernels + C ABI) for gfx950 with hipcc.
+
+Usage: ``python -m spear_amd.csrc.build`` or ``spear_amd.csrc.build.build()``. hipcc
+cross-compiles without a GPU present. The CMake target in the repository root builds the same
+library from the same sources.
+"""
+
+from __future__ import annotations
+
+import os
+import shutil
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+PKG = os.path.dirname(HERE)
+LIB_NAME = "libspear_btp.so"
+SOURCES = ["btp_scan.hip", "btp_capi.hip"]
+HEADERS = ["btp_device.h", "btp_launch.h", os.path.join("..", "..", "include", "spear_btp.h")]
+
+# -packed-fp32-ops is switched off on purpose: scalar fp32 code must not be fused into
+# v_pk_*_f32 instructions on this hardware pool.
+HIPCC_FLAGS = [
+    "--offload-arch=gfx950",
+    "-O3",
+    "-std=c++17",
+    "-fPIC",
+    "-shared",
+    "-ffp-contract=off",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wall",
+    "-Wno-unused-command-line-argument",
+]
+
+
+def hipcc_path() -> str:
+    cand = shutil.which("hipcc") or os.path.join(os.environ.get("ROCM_PATH", "/opt/rocm"), "bin", "hipcc")
+    if not os.path.exists(cand):
+        raise RuntimeError("hipcc not found; the BTP library can only be built with the ROCm toolchain")
+    return cand
+
+
+def lib_path() -> str:
+    return os.path.join(PKG, LIB_NAME)
+
+
+def build(verbose: bool = False, extra_flags: list[str] | None = None) -> str:
+    out = lib_path()
+    cmd = [hipcc_path(), *HIPCC_FLAGS, *(extra_flags or []), "-o", out, *[os.path.join(HERE, s) for s in SOURCES]]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    proc = subprocess.run(cmd, cwd=HERE, capture_output=True, text=True)
+    noise = "is not a recognized feature for this target"
+    err = "\n".join(line for line in proc.stderr.splitlines() if noise not in line)
+    if proc.returncode != 0:
+        raise RuntimeError(f"hipcc failed ({proc.returncode}):\n{proc.stdout}\n{err}")
+    if verbose and err.strip():
+        print(err, file=sys.stderr)
+    return out
+
+
+def is_stale() -> bool:
+    out = lib_path()
+    if not os.path.exists(out):
+        return True
+    t = os.path.getmtime(out)
+    deps = [os.path.join(HERE, p) for p in SOURCES + HEADERS]
+    return any(os.path.getmtime(p) > t for p in deps)
+
+
+if __name__ == "__main__":
+    print(build(verbose=True))

@@ -1,0 +1,151 @@
+"""``btp(coeff, x, k=2, wpb=None, output_dtype=None)``: the Block Two-Pass operator on MI355X.
+
+Drop-in for the reference's ``spear.ops.btp.interface`` (spear/ops/btp/interface.py): same public
+function, same constants, the same two custom ops ``torch.ops.spear_btp.forward`` /
+``torch.ops.spear_btp.backward`` (schemas at interface.py:55-120, registered so that
+``torch.compile`` can trace through them), and the same autograd contract
+(interface.py:126-161): backward returns ``(dA fp32 [B,H,L], dx [B,H,16,L] in x.dtype)``.
+
+Differences that do not change results:
+  * the native library is loaded on first use, so importing this module works on a machine
+    without a GPU (the reference imports its extension unconditionally, interface.py:16);
+  * ``dA`` is allocated uninitialised, because the kernel writes every element
+    (the reference zero-fills it, interface.py:158);
+  * the carry checkpoint is allocated (the op schema requires it) but not stored by default,
+    because this backward recomputes the carries; set ``SPEAR_BTP_WRITE_CHECKPOINT=1`` or call
+    ``spear_amd._btp.forward`` directly to have it written.
+"""
+
+from __future__ import annotations
+
+import os
+
+import torch
+import torch.library
+
+from spear_amd import _btp
+
+__all__ = ["btp"]
+
+# Fixed by the kernels (interface.py:23-27).
+DH = 16
+BLK = 16
+SUPPORTED_WPB = [4, 8, 16, 32]
+WPB_K1_DEFAULT = 8
+WPB_K2_DEFAULT = 32
+
+
+def _forward_flags() -> int:
+    return _btp.FLAG_WRITE_CHECKPOINT if os.environ.get("SPEAR_BTP_WRITE_CHECKPOINT", "0") == "1" else 0
+
+
+def _forward_impl(
+    coeff: torch.Tensor, x: torch.Tensor, y: torch.Tensor, checkpoint: torch.Tensor, k: int, wpb: int
+) -> None:
+    _btp.forward(coeff, x, y, checkpoint, k, wpb, flags=_forward_flags())
+
+
+def _forward_fake(
+    coeff: torch.Tensor, x: torch.Tensor, y: torch.Tensor, checkpoint: torch.Tensor, k: int, wpb: int
+) -> None:
+    return None
+
+
+def _backward_impl(
+    coeff: torch.Tensor,
+    x: torch.Tensor,
+    dy: torch.Tensor,
+    checkpoint: torch.Tensor,
+    dx: torch.Tensor,
+    dA: torch.Tensor,
+    k: int,
+    wpb: int,
+) -> None:
+    _btp.backward(coeff, x, dy, checkpoint, dx, dA, k, wpb)
+
+
+def _backward_fake(
+    coeff: torch.Tensor,
+    x: torch.Tensor,
+    dy: torch.Tensor,
+    checkpoint: torch.Tensor,
+    dx: torch.Tensor,
+    dA: torch.Tensor,
+    k: int,
+    wpb: int,
+) -> None:
+    return None
+
+
+def register_traceable_op(
+    lib: torch.library.Library,
+    op_name: str,
+    op_impl,
+    op_fake_impl,
+    *,
+    mutates_args=None,
+    tags=(),
+    dispatch_key: str | None = "CUDA",
+) -> None:
+    """Define ``op_name`` in ``lib`` from the Python signature of ``op_impl``, bind the
+    implementation for ``dispatch_key`` and a shape-only fake for tracing (interface.py:36-52).
+    On ROCm the device dispatch key is still called "CUDA"."""
+    schema = torch.library.infer_schema(op_impl, mutates_args=mutates_args)
+    lib.define(op_name + schema, tags=tags)
+    lib.impl(op_name, op_impl, dispatch_key=dispatch_key)
+    lib._register_fake(op_name, op_fake_impl)
+
+
+lib = torch.library.Library("spear_btp", "DEF")
+register_traceable_op(lib, "forward", _forward_impl, _forward_fake, mutates_args=["y", "checkpoint"])
+register_traceable_op(lib, "backward", _backward_impl, _backward_fake, mutates_args=["dx", "dA"])
+
+
+class _BTPFunction(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, coeff: torch.Tensor, x: torch.Tensor, k: int, output_dtype: torch.dtype, wpb: int):
+        B, H, dh_in, L = x.shape
+        assert dh_in == DH, f"Channel dimension must be {DH}"
+        assert L % BLK == 0, f"Length L must be multiple of {BLK}"
+        assert wpb in SUPPORTED_WPB, f"WPB must be one of {SUPPORTED_WPB}"
+
+        y = torch.empty_like(x, dtype=output_dtype)
+        checkpoint = torch.empty((B, H, L // BLK, DH), device=x.device, dtype=torch.float32)
+        torch.ops.spear_btp.forward(coeff, x, y, checkpoint, int(k), int(wpb))
+
+        ctx.save_for_backward(coeff, x, checkpoint)
+        ctx.k, ctx.wpb, ctx.input_dtype = int(k), int(wpb), x.dtype
+        return y
+
+    @staticmethod
+    def backward(ctx, dy: torch.Tensor):
+        coeff, x, checkpoint = ctx.saved_tensors
+        dy = dy.contiguous()
+        dx = torch.empty_like(x, dtype=ctx.input_dtype)
+        dA = torch.empty_like(coeff, dtype=torch.float32)
+        torch.ops.spear_btp.backward(coeff, x, dy, checkpoint, dx, dA, ctx.k, ctx.wpb)
+        return dA, dx, None, None, None
+
+
+def btp(
+    coeff: torch.Tensor,
+    x: torch.Tensor,
+    k: int = 2,
+    wpb: int | None = None,
+    output_dtype: torch.dtype | None = None,
+) -> torch.Tensor:
+    """Block Two-Pass sliding-window recurrence.
+
+    Args:
+        coeff: ``[B, H, L]`` linear-space decay ``a_t``, bf16 or fp16.
+        x: ``[B, H, 16, L]`` inputs, same dtype as ``coeff``; ``L`` a multiple of 16.
+        k: 1 = block-local only, 2 = local plus the one-hop carry from the previous block.
+        wpb: accepted and validated for compatibility (sm90 warps per block); has no effect.
+        output_dtype: dtype of the result, ``float32`` (default) or ``x.dtype``.
+
+    Returns:
+        ``[B, H, 16, L]`` with ``y_t = sum_{s >= w(t)} (prod_{j=s+1..t} a_j) x_s``.
+    """
+    out_dtype = output_dtype or torch.float32
+    wpb_val = wpb if wpb is not None else (WPB_K2_DEFAULT if k == 2 else WPB_K1_DEFAULT)
+    return _BTPFunction.apply(coeff.contiguous(), x.contiguous(), k, out_dtype, wpb_val)

@@ -1,0 +1,170 @@
+"""Parity of the HIP kernels (called through the C ABI via spear_amd._btp) with the CPU oracle.
+
+Tolerances are the north-star ones: bf16 I/O within 2e-2 (absolute + relative), fp32 outputs of
+the exact-fp32 path within 1e-4, both against the float64 oracle evaluated on the same
+bf16-rounded inputs."""
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import BF16_ATOL, BF16_RTOL, F32_ATOL, F32_RTOL, assert_close, f64, make_inputs
+from oracle import btp_oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+
+
+def run_forward(coeff, x, k=2, out_dtype=torch.bfloat16, checkpoint=False):
+    from spear_amd import _btp
+
+    c, xx = coeff.to(DEV), x.to(DEV)
+    B, H, _, L = x.shape
+    y = torch.full((B, H, 16, L), float("nan"), device=DEV, dtype=out_dtype)
+    ck = torch.full((B, H, L // 16, 16), float("nan"), device=DEV, dtype=torch.float32)
+    _btp.forward(c, xx, y, ck, k, 32, flags=_btp.FLAG_WRITE_CHECKPOINT if checkpoint else 0)
+    torch.cuda.synchronize()
+    return (y.cpu(), ck.cpu()) if checkpoint else y.cpu()
+
+
+def run_backward(coeff, x, dy, k=2):
+    from spear_amd import _btp
+
+    c, xx, g = coeff.to(DEV), x.to(DEV), dy.to(DEV)
+    B, H, _, L = x.shape
+    dx = torch.full((B, H, 16, L), float("nan"), device=DEV, dtype=x.dtype)
+    dA = torch.full((B, H, L), float("nan"), device=DEV, dtype=torch.float32)
+    ck = torch.empty((B, H, L // 16, 16), device=DEV, dtype=torch.float32)
+    _btp.backward(c, xx, g, ck, dx, dA, k, 32)
+    torch.cuda.synchronize()
+    return dx.cpu(), dA.cpu()
+
+
+SHAPES = [(1, 1, 16), (2, 3, 32), (1, 2, 48), (2, 2, 64), (1, 2, 128), (2, 2, 144), (1, 3, 256), (2, 8, 512), (1, 2, 1040), (3, 5, 112)]
+
+
+@pytest.mark.parametrize("k", [2, 1])
+@pytest.mark.parametrize("B,H,L", SHAPES)
+def test_forward_bf16_matches_oracle(B, H, L, k):
+    coeff, x, _ = make_inputs(B, H, L, seed=100 + L + k)
+    print(f"fwd bf16 B={B} H={H} L={L} k={k}", flush=True)
+    y = run_forward(coeff, x, k=k)
+    assert_close(f64(y), orc.forward(f64(coeff), f64(x), k=k), BF16_ATOL, BF16_RTOL, "y")
+
+
+@pytest.mark.parametrize("k", [2, 1])
+@pytest.mark.parametrize("B,H,L", SHAPES)
+def test_forward_fp32_out_matches_oracle_to_1e4(B, H, L, k):
+    coeff, x, _ = make_inputs(B, H, L, seed=200 + L + k)
+    print(f"fwd f32 B={B} H={H} L={L} k={k}", flush=True)
+    y = run_forward(coeff, x, k=k, out_dtype=torch.float32)
+    assert_close(f64(y), orc.forward(f64(coeff), f64(x), k=k), F32_ATOL, F32_RTOL, "y")
+
+
+@pytest.mark.parametrize("k", [2, 1])
+@pytest.mark.parametrize("B,H,L", SHAPES)
+def test_backward_bf16_matches_oracle(B, H, L, k):
+    coeff, x, dy = make_inputs(B, H, L, seed=300 + L + k)
+    print(f"bwd bf16 B={B} H={H} L={L} k={k}", flush=True)
+    dx, dA = run_backward(coeff, x, dy, k=k)
+    rdx, rdA = orc.backward(f64(coeff), f64(x), f64(dy), k=k)
+    assert_close(f64(dx), rdx, BF16_ATOL, BF16_RTOL, "dx")
+    # dA is an fp32 output computed in fp32 from exact inputs: hold it to the fp32 bound
+    assert_close(f64(dA), rdA, F32_ATOL, F32_RTOL, "dA")
+
+
+@pytest.mark.parametrize("B,H,L", [(2, 3, 32), (2, 2, 144), (2, 8, 512)])
+def test_backward_fp32_dy(B, H, L):
+    coeff, x, _ = make_inputs(B, H, L, seed=400 + L)
+    dy = torch.randn(B, H, 16, L, generator=torch.Generator().manual_seed(L))
+    print(f"bwd f32-dy B={B} H={H} L={L}", flush=True)
+    dx, dA = run_backward(coeff, x, dy)
+    rdx, rdA = orc.backward(f64(coeff), f64(x), f64(dy))
+    assert_close(f64(dx), rdx, BF16_ATOL, BF16_RTOL, "dx")
+    assert_close(f64(dA), rdA, F32_ATOL, F32_RTOL, "dA")
+
+
+@pytest.mark.parametrize("B,H,L", [(2, 3, 64), (1, 2, 400)])
+def test_fp16_inputs(B, H, L):
+    coeff, x, dy = make_inputs(B, H, L, seed=500 + L, dtype=torch.float16)
+    print(f"fp16 B={B} H={H} L={L}", flush=True)
+    y = run_forward(coeff, x, out_dtype=torch.float16)
+    assert_close(f64(y), orc.forward(f64(coeff), f64(x)), 2e-3, 2e-3, "y fp16")
+    dx, dA = run_backward(coeff, x, dy)
+    rdx, rdA = orc.backward(f64(coeff), f64(x), f64(dy))
+    assert_close(f64(dx), rdx, 2e-3, 2e-3, "dx fp16")
+    assert_close(f64(dA), rdA, F32_ATOL, F32_RTOL, "dA")
+
+
+@pytest.mark.parametrize("L", [64, 272])
+def test_checkpoint_matches_oracle(L):
+    coeff, x, _ = make_inputs(2, 3, L, seed=600 + L)
+    print(f"checkpoint L={L}", flush=True)
+    y, ck = run_forward(coeff, x, checkpoint=True)
+    ry, rck = orc.forward(f64(coeff), f64(x), with_checkpoint=True)
+    assert_close(f64(y), ry, BF16_ATOL, BF16_RTOL, "y")
+    nb = L // 16
+    assert_close(f64(ck)[:, :, : nb - 1], rck[:, :, : nb - 1], F32_ATOL, F32_RTOL, "checkpoint")
+    assert torch.isnan(ck[:, :, nb - 1]).all(), "the last checkpoint slot must stay untouched"
+
+
+@pytest.mark.parametrize("stress", [2.5, 4.0])
+def test_stressed_gates(stress):
+    # sigmoid(N(0, stress)) coefficients as in the reference's stress sweeps (tests/btp/test_numerics.py:104-166)
+    coeff, x, dy = make_inputs(2, 4, 512, seed=321, stress=stress)
+    print(f"stress={stress}", flush=True)
+    y = run_forward(coeff, x, out_dtype=torch.float32)
+    assert_close(f64(y), orc.forward(f64(coeff), f64(x)), F32_ATOL, F32_RTOL, "y")
+    dx, dA = run_backward(coeff, x, dy)
+    rdx, rdA = orc.backward(f64(coeff), f64(x), f64(dy))
+    assert_close(f64(dx), rdx, BF16_ATOL, BF16_RTOL, "dx")
+    assert_close(f64(dA), rdA, F32_ATOL, F32_RTOL, "dA")
+
+
+def test_log_space_stress_mixture():
+    # per head either exp(U[-20,-5]) (near-total forgetting) or exp(U[-1e-4,0]) (near-identity)
+    coeff, x, dy = make_inputs(2, 8, 2048, seed=1236, gate="mixed")
+    print("mixed gates", flush=True)
+    y = run_forward(coeff, x)
+    assert_close(f64(y), orc.forward(f64(coeff), f64(x)), BF16_ATOL, BF16_RTOL, "y")
+    dx, dA = run_backward(coeff, x, dy)
+    rdx, rdA = orc.backward(f64(coeff), f64(x), f64(dy))
+    assert_close(f64(dx), rdx, BF16_ATOL, BF16_RTOL, "dx")
+    assert_close(f64(dA), rdA, F32_ATOL, F32_RTOL, "dA")
+
+
+def test_zero_negative_and_tiny_coefficients():
+    # at or below 1e-9 (and negative) counts as exactly zero, as in the reference kernels
+    coeff, x, dy = make_inputs(1, 2, 160, seed=7)
+    coeff[0, 0, [0, 5, 16, 33, 127, 128]] = 0.0
+    coeff[0, 1, [3, 47, 48]] = -0.5
+    coeff[0, 1, [100]] = 1e-12
+    ref_coeff = f64(coeff).copy()
+    ref_coeff[ref_coeff <= 1e-9] = 0.0
+    print("zero coefficients", flush=True)
+    y = run_forward(coeff, x, out_dtype=torch.float32)
+    assert_close(f64(y), orc.forward(ref_coeff, f64(x)), F32_ATOL, F32_RTOL, "y")
+    dx, dA = run_backward(coeff, x, dy)
+    rdx, rdA = orc.backward(ref_coeff, f64(x), f64(dy))
+    assert_close(f64(dx), rdx, BF16_ATOL, BF16_RTOL, "dx")
+    assert_close(f64(dA), rdA, F32_ATOL, F32_RTOL, "dA")
+
+
+def test_outputs_are_deterministic():
+    coeff, x, dy = make_inputs(2, 4, 256, seed=11)
+    y1, y2 = run_forward(coeff, x), run_forward(coeff, x)
+    assert torch.equal(y1, y2)
+    (dx1, dA1), (dx2, dA2) = run_backward(coeff, x, dy), run_backward(coeff, x, dy)
+    assert torch.equal(dx1, dx2) and torch.equal(dA1, dA2)
+
+
+def test_empty_batch_is_a_noop():
+    from spear_amd import _btp
+
+    coeff = torch.empty(0, 4, 64, device=DEV, dtype=torch.bfloat16)
+    x = torch.empty(0, 4, 16, 64, device=DEV, dtype=torch.bfloat16)
+    y = torch.empty_like(x)
+    ck = torch.empty(0, 4, 4, 16, device=DEV, dtype=torch.float32)
+    _btp.forward(coeff, x, y, ck, 2, 32)
+    torch.cuda.synchronize()
