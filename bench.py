@@ -1,0 +1,236 @@
+#!/usr/bin/env python3
+"""Benchmark of the BTP hot path: forward + backward at B=1024, L=128, dim=512 (H=32) bf16.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c3|c4|c5] [--no-cpu-baseline]
+
+A step is one forward plus one backward launch through the C ABI on one batch of synthetic
+input that is already resident in HBM. Buffers rotate over several independent sets so that a
+step never finds its inputs in the 256 MiB last-level cache left there by the previous step.
+Prints ONE JSON line (see the keys below).
+
+Algorithmic bytes per (token, head): forward 66 (coeff 2 + x 32 read, y 32 written), backward 102
+(coeff 2 + x 32 + dy 32 read, dx 32 + dA 4 written), together 168; per token multiply by H.
+"""
+
+from __future__ import annotations
+
+import argparse
+import ctypes
+import json
+import os
+import statistics
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
+FWD_BYTES, BWD_BYTES = 66, 102  # per (token, head), bf16 y / dy
+
+CONFIGS = {
+    # name: (B, H, L, seed, x_std, gate)
+    "c3": (1024, 32, 128, 1234, 0.25, "sigmoid"),
+    "c4": (16, 64, 8192, 1235, 0.25, "sigmoid"),
+    "c5": (64, 128, 2048, 1236, 1.0, "mixed"),
+}
+
+
+def synth(B, H, L, seed, x_std, gate):
+    import torch
+
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    x = (torch.randn(B, H, 16, L, generator=g) * x_std).to(torch.bfloat16)
+    if gate == "sigmoid":
+        coeff = torch.exp(-torch.nn.functional.softplus(torch.randn(B, H, L, generator=g)))
+    else:
+        forget = torch.rand(B, H, 1, generator=g) < 0.5
+        lo = -20.0 + 15.0 * torch.rand(B, H, L, generator=g)
+        hi = -1e-4 * torch.rand(B, H, L, generator=g)
+        coeff = torch.exp(torch.where(forget, lo, hi))
+    dy = torch.randn(B, H, 16, L, generator=g).to(torch.bfloat16)
+    return coeff.to(torch.bfloat16), x, dy
+
+
+def cpu_baseline(B, H, L, seed, x_std, gate, budget_s=20.0):
+    """Times the PyTorch restatement of the reference's CPU path (block_two_pass_log, forward +
+    backward through autograd, bf16 tensors) on a bounded sample of the workload's batch."""
+    import torch
+
+    from spear_amd.ops.btp.reference import block_two_pass_log
+
+    threads = torch.get_num_threads()
+
+    def once(bs):
+        coeff, x, dy = synth(bs, H, L, seed, x_std, gate)
+        coeff.requires_grad_(True)
+        x.requires_grad_(True)
+        t0 = time.perf_counter()
+        y = block_two_pass_log(coeff, x, 16)
+        y.backward(dy)
+        return time.perf_counter() - t0
+
+    once(max(1, min(B, 4)))  # warm-up (thread pool, allocator)
+    bs, t = max(1, min(B, 8)), 0.0
+    while True:  # grow the sample until one run is long enough to extrapolate from
+        t = once(bs)
+        if t >= 0.5 or bs >= B:
+            break
+        bs = min(B, bs * 4)
+    bs = int(max(1, min(B, bs * (budget_s / 4.0) / max(t, 1e-6))))
+    times = [once(bs) for _ in range(3)]
+    med = statistics.median(times)
+    return {
+        "value": bs * L / med,
+        "unit": "tokens/s",
+        "cores": threads,
+        "kind": "port",
+        "sample": f"block_two_pass_log fwd+bwd (autograd), bf16, first {bs} of {B} batch rows, H={H}, L={L}; median of 3 after 1 warm-up; {med:.3f} s",
+    }
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--config", choices=sorted(CONFIGS), default="c3")
+    ap.add_argument("--sets", type=int, default=4, help="independent buffer sets to rotate over")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+
+    if args.gpus != 1:
+        print(
+            "bench.py: this build measures one GPU only (the op shards over batch and heads with no "
+            "communication; see DESIGN.md). Run with --gpus 1.",
+            file=sys.stderr,
+        )
+        return 2
+
+    import torch
+
+    from spear_amd import _btp
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        return 1
+    lib = _btp.load_library()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    B, H, L, seed, x_std, gate = CONFIGS[args.config]
+    coeff, x, dy = synth(B, H, L, seed, x_std, gate)
+    sets = []
+    for _ in range(args.sets):
+        s = {
+            "coeff": coeff.to(dev),
+            "x": x.to(dev),
+            "dy": dy.to(dev),
+            "y": torch.empty(B, H, 16, L, device=dev, dtype=torch.bfloat16),
+            "dx": torch.empty(B, H, 16, L, device=dev, dtype=torch.bfloat16),
+            "dA": torch.empty(B, H, L, device=dev, dtype=torch.float32),
+        }
+        sets.append(s)
+    del coeff, x, dy
+    stream = torch.cuda.current_stream(dev)
+    sp = ctypes.c_void_p(stream.cuda_stream)
+
+    def fwd(s):
+        rc = lib.spear_btp_forward(s["coeff"].data_ptr(), s["x"].data_ptr(), s["y"].data_ptr(), None,
+                                   B, H, L, 2, 0, 0, 0, sp)
+        assert rc == 0, lib.spear_btp_last_error()
+
+    def bwd(s):
+        rc = lib.spear_btp_backward(s["coeff"].data_ptr(), s["x"].data_ptr(), s["dy"].data_ptr(), None,
+                                    s["dx"].data_ptr(), s["dA"].data_ptr(), B, H, L, 2, 0, 0, 0, sp)
+        assert rc == 0, lib.spear_btp_last_error()
+
+    def step(i):
+        s = sets[i % len(sets)]
+        fwd(s)
+        bwd(s)
+
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(i)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed * 1e3 / args.steps
+
+    # per-kernel average launch duration, HIP events on the launch stream, same rotation
+    def kernel_ms(fn):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        for i in range(min(args.warmup, 10)):
+            fn(sets[i % len(sets)])
+        torch.cuda.synchronize()
+        e0.record(stream)
+        for i in range(args.steps):
+            fn(sets[i % len(sets)])
+        e1.record(stream)
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / args.steps
+
+    fwd_ms, bwd_ms = kernel_ms(fwd), kernel_ms(bwd)
+
+    # copy kernel of the same footprint as a practical ceiling (reads n, writes n)
+    nbytes = sets[0]["x"].numel() * 2
+    def copy(s):
+        lib.spear_btp_copy(s["x"].data_ptr(), s["dx"].data_ptr(), ctypes.c_ulonglong(nbytes), sp)
+    copy_ms = kernel_ms(copy)
+
+    units = B * H * L
+    tokens = B * L
+    bwd_gbps = units * BWD_BYTES / (bwd_ms * 1e-3) / 1e9
+    fwd_gbps = units * FWD_BYTES / (fwd_ms * 1e-3) / 1e9
+    step_gbps = units * (FWD_BYTES + BWD_BYTES) / (ms_per_step * 1e-3) / 1e9
+
+    out = {
+        "metric": "BTP fwd+bwd tokens/s (B1024 L128 D512 bf16); % of HBM roofline",
+        "value": tokens / (ms_per_step * 1e-3),
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {
+            "workload": f"BTP forward+backward, B={B} H={H} L={L} head_dim=16 block_len=16 k=2, bf16 coeff/x/y/dy/dx, fp32 dA ({args.config})",
+            "arithmetic": "fp32 recurrences on bf16 storage",
+            "buffer_sets": len(sets),
+        },
+        "roofline": {
+            "bound": "hbm",
+            "kernel": "btp_bwd_scan_kernel<Bf16, bf16 dy>",
+            "achieved": bwd_gbps,
+            "peak": HBM_PEAK_GBPS,
+            "unit": "GB/s",
+            "frac": bwd_gbps / HBM_PEAK_GBPS,
+            "traffic": None,
+            "avg_launch_ms": bwd_ms,
+            "algorithmic_bytes_per_launch": units * BWD_BYTES,
+        },
+        "forward_kernel": {"avg_launch_ms": fwd_ms, "achieved": fwd_gbps, "frac": fwd_gbps / HBM_PEAK_GBPS,
+                           "algorithmic_bytes_per_launch": units * FWD_BYTES},
+        "fwd_plus_bwd": {"achieved": step_gbps, "frac": step_gbps / HBM_PEAK_GBPS,
+                         "algorithmic_bytes_per_step": units * (FWD_BYTES + BWD_BYTES)},
+        "copy_kernel": {"avg_launch_ms": copy_ms, "achieved": 2 * nbytes / (copy_ms * 1e-3) / 1e9,
+                        "bytes_moved": 2 * nbytes},
+    }
+    if not args.no_cpu_baseline:
+        base = cpu_baseline(B, H, L, seed, x_std, gate)
+        out["cpu_baseline"] = base
+        out["speedup_vs_cpu_baseline"] = out["value"] / base["value"]
+    print(json.dumps(out))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())
