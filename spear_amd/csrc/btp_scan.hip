@@ -48,6 +48,30 @@
 #include "btp_device.h"
 #include "btp_launch.h"
 
+// Tuning knobs (compile-time). The defaults are the measured best on MI355X.
+#ifndef SPEAR_BTP_STREAM_LOADS   // 0: never, 1: always, 2: only when a row is a single span
+#define SPEAR_BTP_STREAM_LOADS 2
+#endif
+#ifndef SPEAR_BTP_STREAM_STORES  // 0: never, 1: always
+#define SPEAR_BTP_STREAM_STORES 1
+#endif
+#ifndef SPEAR_BTP_FWD_WAVES_PER_EU
+#define SPEAR_BTP_FWD_WAVES_PER_EU 0
+#endif
+#ifndef SPEAR_BTP_BWD_WAVES_PER_EU
+#define SPEAR_BTP_BWD_WAVES_PER_EU 0
+#endif
+#if SPEAR_BTP_FWD_WAVES_PER_EU > 0
+#define SPEAR_BTP_FWD_OCC __attribute__((amdgpu_waves_per_eu(SPEAR_BTP_FWD_WAVES_PER_EU)))
+#else
+#define SPEAR_BTP_FWD_OCC
+#endif
+#if SPEAR_BTP_BWD_WAVES_PER_EU > 0
+#define SPEAR_BTP_BWD_OCC __attribute__((amdgpu_waves_per_eu(SPEAR_BTP_BWD_WAVES_PER_EU)))
+#else
+#define SPEAR_BTP_BWD_OCC
+#endif
+
 namespace spear_btp {
 
 namespace {
@@ -61,6 +85,21 @@ __device__ __forceinline__ int swz(int r, int chunk) {
 }
 
 __device__ __forceinline__ uint4 zero4() { return make_uint4(0u, 0u, 0u, 0u); }
+
+// Streaming (non-temporal) 16-byte global accesses: every byte of the operands is touched exactly
+// once per launch, so the lines are marked for early eviction instead of displacing useful data
+// in L2 and the last-level cache.
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ uint4 stream_load16(const void* p) {
+  const u32x4_t v = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(p));
+  return make_uint4(v[0], v[1], v[2], v[3]);
+}
+
+__device__ __forceinline__ void stream_store16(void* p, const uint4& q) {
+  const u32x4_t v = {q.x, q.y, q.z, q.w};
+  __builtin_nontemporal_store(v, reinterpret_cast<u32x4_t*>(p));
+}
 
 // Loads the 16 coefficients of one block (32 bytes, wave-uniform address per lane group) and
 // returns them clamped, as floats.
@@ -78,6 +117,13 @@ __device__ __forceinline__ void load_block_coeffs(const uint16_t* p, float (&a)[
 // Stage a [16 x 128] slab of 16-bit elements: coalesced global reads -> swizzled LDS image.
 // Lane l of pass `it` handles channel row 4*it + l/16, chunk l%16 (8 steps).
 // ------------------------------------------------------------------------------------------
+template <bool kStream>
+__device__ __forceinline__ uint4 load16(const void* p) {
+  if constexpr (kStream) return stream_load16(p);
+  return *reinterpret_cast<const uint4*>(p);
+}
+
+template <bool kStream>
 __device__ __forceinline__ void slab16_global_to_regs(const uint16_t* slab, long L, int nvalid,
                                                       int lane, uint4 (&q)[4]) {
   const int lr = lane >> 4, lp = lane & 15;
@@ -85,7 +131,7 @@ __device__ __forceinline__ void slab16_global_to_regs(const uint16_t* slab, long
 #pragma unroll
   for (int it = 0; it < 4; ++it) {
     const int r = it * 4 + lr;
-    q[it] = ok ? *reinterpret_cast<const uint4*>(slab + (long)r * L + (lp << 3)) : zero4();
+    q[it] = ok ? load16<kStream>(slab + (long)r * L + (lp << 3)) : zero4();
   }
 }
 
@@ -98,6 +144,13 @@ __device__ __forceinline__ void slab16_regs_to_lds(unsigned char* img, int lane,
   }
 }
 
+template <bool kStream>
+__device__ __forceinline__ void store16(void* p, const uint4& q) {
+  if constexpr (kStream) stream_store16(p, q);
+  else *reinterpret_cast<uint4*>(p) = q;
+}
+
+template <bool kStream>
 __device__ __forceinline__ void slab16_lds_to_global(const unsigned char* img, uint16_t* slab, long L,
                                                      int nvalid, int lane) {
   const int lr = lane >> 4, lp = lane & 15;
@@ -106,12 +159,13 @@ __device__ __forceinline__ void slab16_lds_to_global(const unsigned char* img, u
   for (int it = 0; it < 4; ++it) {
     const int r = it * 4 + lr;
     const uint4 v = *reinterpret_cast<const uint4*>(img + swz<256>(r, lp));
-    if (ok) *reinterpret_cast<uint4*>(slab + (long)r * L + (lp << 3)) = v;
+    if (ok) store16<kStream>(slab + (long)r * L + (lp << 3), v);
   }
 }
 
 // Same for a [16 x 128] slab of fp32 (512 B per row, 32 chunks of 4 steps).
 // Lane l of pass `it` handles channel row 2*it + l/32, chunk l%32.
+template <bool kStream>
 __device__ __forceinline__ void slab32_global_to_regs(const float* slab, long L, int nvalid, int lane,
                                                       uint4 (&q)[8]) {
   const int lr = lane >> 5, lp = lane & 31;
@@ -119,7 +173,7 @@ __device__ __forceinline__ void slab32_global_to_regs(const float* slab, long L,
 #pragma unroll
   for (int it = 0; it < 8; ++it) {
     const int r = it * 2 + lr;
-    q[it] = ok ? *reinterpret_cast<const uint4*>(slab + (long)r * L + (lp << 2)) : zero4();
+    q[it] = ok ? load16<kStream>(slab + (long)r * L + (lp << 2)) : zero4();
   }
 }
 
@@ -132,6 +186,7 @@ __device__ __forceinline__ void slab32_regs_to_lds(unsigned char* img, int lane,
   }
 }
 
+template <bool kStream>
 __device__ __forceinline__ void slab32_lds_to_global(const unsigned char* img, float* slab, long L,
                                                      int nvalid, int lane) {
   const int lr = lane >> 5, lp = lane & 31;
@@ -140,7 +195,7 @@ __device__ __forceinline__ void slab32_lds_to_global(const unsigned char* img, f
   for (int it = 0; it < 8; ++it) {
     const int r = it * 2 + lr;
     const uint4 v = *reinterpret_cast<const uint4*>(img + swz<512>(r, lp));
-    if (ok) *reinterpret_cast<uint4*>(slab + (long)r * L + (lp << 2)) = v;
+    if (ok) store16<kStream>(slab + (long)r * L + (lp << 2), v);
   }
 }
 
@@ -180,7 +235,7 @@ __device__ __forceinline__ void lane_write32(unsigned char* img, int j, int d, c
 // reads back the 32 of its own two blocks (a broadcast read for the 16 lanes of a group).
 template <class E>
 __device__ __forceinline__ uint32_t coeff_global_to_reg(const uint16_t* arow, int nvalid, int lane) {
-  return ((lane << 1) < nvalid) ? *reinterpret_cast<const uint32_t*>(arow + (lane << 1)) : 0u;
+  return ((lane << 1) < nvalid) ? __builtin_nontemporal_load(reinterpret_cast<const uint32_t*>(arow + (lane << 1))) : 0u;
 }
 
 template <class E>
@@ -218,8 +273,8 @@ __device__ __forceinline__ SpanCoord span_coord(long span, int spans_per_row, in
 // ==========================================================================================
 // Forward
 // ==========================================================================================
-template <class E, class OutT, bool kCheckpoint>
-__global__ __launch_bounds__(64 * kWaves) void btp_fwd_scan_kernel(
+template <class E, class OutT, bool kCheckpoint, bool kStreamIn>
+__global__ __launch_bounds__(64 * kWaves) SPEAR_BTP_FWD_OCC void btp_fwd_scan_kernel(
     const uint16_t* __restrict__ coeff, const uint16_t* __restrict__ x, OutT* __restrict__ y,
     float* __restrict__ ckpt, int L, int spans_per_row, long total_spans, int k) {
   constexpr bool kOutF32 = std::is_same<OutT, float>::value;
@@ -238,8 +293,11 @@ __global__ __launch_bounds__(64 * kWaves) void btp_fwd_scan_kernel(
   const int j = lane >> 4, d = lane & 15;
 
   // ---- all global reads are issued before anything waits on them
+  // kStreamIn: the host sets it for rows that fit one span, which are read exactly once. Longer
+  // rows are re-read by the neighbouring spans' halo loads, so their lines should stay in L2.
+  constexpr bool kStreamOut = SPEAR_BTP_STREAM_STORES == 1;
   uint4 xin[4];
-  slab16_global_to_regs(xslab, L, sc.nvalid, lane, xin);
+  slab16_global_to_regs<kStreamIn>(xslab, L, sc.nvalid, lane, xin);
   const uint32_t ain = coeff_global_to_reg<E>(arow, sc.nvalid, lane);
 
   const bool halo = (k == 2) && (sc.sp > 0);  // wave-uniform
@@ -312,21 +370,21 @@ __global__ __launch_bounds__(64 * kWaves) void btp_fwd_scan_kernel(
   if constexpr (kOutF32) {
     lane_write32(img, j, d, yv);
     wave_lds_handover();
-    slab32_lds_to_global(img, reinterpret_cast<float*>(y) + (sc.row * kChan) * (long)L + sc.s0, L,
-                         sc.nvalid, lane);
+    float* yslab = reinterpret_cast<float*>(y) + (sc.row * kChan) * (long)L + sc.s0;
+    slab32_lds_to_global<kStreamOut>(img, yslab, L, sc.nvalid, lane);
   } else {
     lane_write16<E>(img, j, d, yv);
     wave_lds_handover();
-    slab16_lds_to_global(img, reinterpret_cast<uint16_t*>(y) + (sc.row * kChan) * (long)L + sc.s0, L,
-                         sc.nvalid, lane);
+    uint16_t* yslab = reinterpret_cast<uint16_t*>(y) + (sc.row * kChan) * (long)L + sc.s0;
+    slab16_lds_to_global<kStreamOut>(img, yslab, L, sc.nvalid, lane);
   }
 }
 
 // ==========================================================================================
 // Backward
 // ==========================================================================================
-template <class E, class GradT>
-__global__ __launch_bounds__(64 * kWaves) void btp_bwd_scan_kernel(
+template <class E, class GradT, bool kStreamIn>
+__global__ __launch_bounds__(64 * kWaves) SPEAR_BTP_BWD_OCC void btp_bwd_scan_kernel(
     const uint16_t* __restrict__ coeff, const uint16_t* __restrict__ x, const GradT* __restrict__ dy,
     uint16_t* __restrict__ dx, float* __restrict__ dA, int L, int spans_per_row, long total_spans,
     int k) {
@@ -348,13 +406,14 @@ __global__ __launch_bounds__(64 * kWaves) void btp_bwd_scan_kernel(
   const int j = lane >> 4, d = lane & 15;
 
   // ---- global reads
+  constexpr bool kStreamOut = SPEAR_BTP_STREAM_STORES == 1;  // see the forward kernel
   uint4 xin[4];
-  slab16_global_to_regs(xslab, L, sc.nvalid, lane, xin);
   uint4 gin[kGradF32 ? 8 : 4];
+  slab16_global_to_regs<kStreamIn>(xslab, L, sc.nvalid, lane, xin);
   if constexpr (kGradF32) {
-    slab32_global_to_regs(reinterpret_cast<const float*>(dy) + slab_off, L, sc.nvalid, lane, gin);
+    slab32_global_to_regs<kStreamIn>(reinterpret_cast<const float*>(dy) + slab_off, L, sc.nvalid, lane, gin);
   } else {
-    slab16_global_to_regs(reinterpret_cast<const uint16_t*>(dy) + slab_off, L, sc.nvalid, lane, gin);
+    slab16_global_to_regs<kStreamIn>(reinterpret_cast<const uint16_t*>(dy) + slab_off, L, sc.nvalid, lane, gin);
   }
   const uint32_t ain = coeff_global_to_reg<E>(arow, sc.nvalid, lane);
 
@@ -480,13 +539,13 @@ __global__ __launch_bounds__(64 * kWaves) void btp_bwd_scan_kernel(
   }
 
   float* dArow = dA + sc.row * (long)L + sc.s0 + 32 * j + d;
-  if (32 * j < sc.nvalid) dArow[0] = dA_A;
-  if (32 * j + 16 < sc.nvalid) dArow[16] = dA_B;
+  if (32 * j < sc.nvalid) __builtin_nontemporal_store(dA_A, dArow);
+  if (32 * j + 16 < sc.nvalid) __builtin_nontemporal_store(dA_B, dArow + 16);
 
   // dx goes back through the x image: every lane overwrites exactly the chunks it read
   lane_write16<E>(img_x, j, d, dxv);
   wave_lds_handover();
-  slab16_lds_to_global(img_x, dx + slab_off, L, sc.nvalid, lane);
+  slab16_lds_to_global<kStreamOut>(img_x, dx + slab_off, L, sc.nvalid, lane);
 }
 
 __global__ __launch_bounds__(256) void copy_kernel(const uint4* __restrict__ src, uint4* __restrict__ dst,
@@ -510,29 +569,44 @@ inline Grid make_grid(long rows, int L) {
   return g;
 }
 
+inline bool stream_inputs(const Grid& g) {
+  return SPEAR_BTP_STREAM_LOADS == 1 || (SPEAR_BTP_STREAM_LOADS == 2 && g.spans_per_row == 1);
+}
+
+template <class E, class OutT, bool kCheckpoint, bool kStreamIn>
+void launch_fwd_as(const FwdArgs& p, const Grid& g, hipStream_t s) {
+  hipLaunchKernelGGL((btp_fwd_scan_kernel<E, OutT, kCheckpoint, kStreamIn>), dim3(g.blocks), dim3(64 * kWaves), 0, s,
+                     static_cast<const uint16_t*>(p.coeff), static_cast<const uint16_t*>(p.x),
+                     static_cast<OutT*>(p.y), p.checkpoint, p.L, g.spans_per_row, g.total_spans, p.k);
+}
+
 template <class E, class OutT>
 hipError_t launch_fwd(const FwdArgs& p, hipStream_t s) {
   const Grid g = make_grid((long)p.B * p.H, p.L);
-  const auto* c = static_cast<const uint16_t*>(p.coeff);
-  const auto* x = static_cast<const uint16_t*>(p.x);
-  auto* y = static_cast<OutT*>(p.y);
-  if (p.checkpoint != nullptr) {
-    hipLaunchKernelGGL((btp_fwd_scan_kernel<E, OutT, true>), dim3(g.blocks), dim3(64 * kWaves), 0, s, c, x, y,
-                       p.checkpoint, p.L, g.spans_per_row, g.total_spans, p.k);
+  const bool ck = p.checkpoint != nullptr, st = stream_inputs(g);
+  if (ck) {
+    if (st) launch_fwd_as<E, OutT, true, true>(p, g, s);
+    else launch_fwd_as<E, OutT, true, false>(p, g, s);
   } else {
-    hipLaunchKernelGGL((btp_fwd_scan_kernel<E, OutT, false>), dim3(g.blocks), dim3(64 * kWaves), 0, s, c, x, y,
-                       static_cast<float*>(nullptr), p.L, g.spans_per_row, g.total_spans, p.k);
+    if (st) launch_fwd_as<E, OutT, false, true>(p, g, s);
+    else launch_fwd_as<E, OutT, false, false>(p, g, s);
   }
   return hipGetLastError();
+}
+
+template <class E, class GradT, bool kStreamIn>
+void launch_bwd_as(const BwdArgs& p, const Grid& g, hipStream_t s) {
+  hipLaunchKernelGGL((btp_bwd_scan_kernel<E, GradT, kStreamIn>), dim3(g.blocks), dim3(64 * kWaves), 0, s,
+                     static_cast<const uint16_t*>(p.coeff), static_cast<const uint16_t*>(p.x),
+                     static_cast<const GradT*>(p.dy), static_cast<uint16_t*>(p.dx), p.dA, p.L, g.spans_per_row,
+                     g.total_spans, p.k);
 }
 
 template <class E, class GradT>
 hipError_t launch_bwd(const BwdArgs& p, hipStream_t s) {
   const Grid g = make_grid((long)p.B * p.H, p.L);
-  hipLaunchKernelGGL((btp_bwd_scan_kernel<E, GradT>), dim3(g.blocks), dim3(64 * kWaves), 0, s,
-                     static_cast<const uint16_t*>(p.coeff), static_cast<const uint16_t*>(p.x),
-                     static_cast<const GradT*>(p.dy), static_cast<uint16_t*>(p.dx), p.dA, p.L, g.spans_per_row,
-                     g.total_spans, p.k);
+  if (stream_inputs(g)) launch_bwd_as<E, GradT, true>(p, g, s);
+  else launch_bwd_as<E, GradT, false>(p, g, s);
   return hipGetLastError();
 }
 

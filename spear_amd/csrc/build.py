@@ -44,8 +44,8 @@ def lib_path() -> str:
     return os.path.join(PKG, LIB_NAME)
 
 
-def build(verbose: bool = False, extra_flags: list[str] | None = None) -> str:
-    out = lib_path()
+def build(verbose: bool = False, extra_flags: list[str] | None = None, out: str | None = None) -> str:
+    out = out or lib_path()
     cmd = [hipcc_path(), *HIPCC_FLAGS, *(extra_flags or []), "-o", out, *[os.path.join(HERE, s) for s in SOURCES]]
     if verbose:
         print(" ".join(cmd), flush=True)
