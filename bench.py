@@ -98,6 +98,7 @@ def main() -> int:
     ap.add_argument("--config", choices=sorted(CONFIGS), default="c3")
     ap.add_argument("--sets", type=int, default=4, help="independent buffer sets to rotate over")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--settle-seconds", type=float, default=0.3, help="untimed run-in before the warm-up steps")
     args = ap.parse_args()
 
     if args.gpus != 1:
@@ -154,7 +155,7 @@ def main() -> int:
     # Untimed: let clocks and power state settle (about 0.3 s of steps), then the W warm-up steps.
     t_settle = time.perf_counter()
     i = 0
-    while time.perf_counter() - t_settle < 0.3:
+    while time.perf_counter() - t_settle < args.settle_seconds:
         step(i)
         i += 1
         if i % 64 == 0:
@@ -224,7 +225,7 @@ def main() -> int:
         },
         "roofline": {
             "bound": "hbm",
-            "kernel": "btp_bwd_scan_kernel<Bf16, bf16 dy>",
+            "kernel": "btp_bwd_scan_kernel<Bf16> (bf16 dy)",
             "achieved": bwd_gbps,
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",

@@ -58,8 +58,8 @@
 #ifndef SPEAR_BTP_FWD_WAVES_PER_EU
 #define SPEAR_BTP_FWD_WAVES_PER_EU 0
 #endif
-#ifndef SPEAR_BTP_BWD_WAVES_PER_EU
-#define SPEAR_BTP_BWD_WAVES_PER_EU 0
+#ifndef SPEAR_BTP_BWD_WAVES_PER_EU  // 4 waves per SIMD need <= 128 VGPRs; the backward body is ordered to fit
+#define SPEAR_BTP_BWD_WAVES_PER_EU 4
 #endif
 #if SPEAR_BTP_FWD_WAVES_PER_EU > 0
 #define SPEAR_BTP_FWD_OCC __attribute__((amdgpu_waves_per_eu(SPEAR_BTP_FWD_WAVES_PER_EU)))
@@ -384,13 +384,13 @@ __global__ __launch_bounds__(64 * kWaves) SPEAR_BTP_FWD_OCC void btp_fwd_scan_ke
 // Backward
 // ==========================================================================================
 template <class E, class GradT, bool kStreamIn>
-__global__ __launch_bounds__(64 * kWaves) SPEAR_BTP_BWD_OCC void btp_bwd_scan_kernel(
+__device__ __forceinline__ void btp_bwd_scan_body(
+    unsigned char (*lds)[4096 + (std::is_same<GradT, float>::value ? 8192 : 4096) + 512],
     const uint16_t* __restrict__ coeff, const uint16_t* __restrict__ x, const GradT* __restrict__ dy,
     uint16_t* __restrict__ dx, float* __restrict__ dA, int L, int spans_per_row, long total_spans,
     int k) {
   constexpr bool kGradF32 = std::is_same<GradT, float>::value;
   constexpr int kGradBytes = kGradF32 ? 8192 : 4096;
-  __shared__ __align__(16) unsigned char lds[kWaves][4096 + kGradBytes + 512];
 
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const long span = (long)blockIdx.x * kWaves + wave;
@@ -463,18 +463,17 @@ __global__ __launch_bounds__(64 * kWaves) SPEAR_BTP_BWD_OCC void btp_bwd_scan_ke
   coeff_reg_to_lds<E>(a_lds, lane, ain);
   wave_lds_handover();
 
-  float xf[32], gf[32], a[32];
-  lane_read16<E>(img_x, j, d, xf);
-  if constexpr (kGradF32) {
-    lane_read32(img_g, j, d, gf);
-  } else {
-    lane_read16<E>(img_g, j, d, gf);
-  }
-  coeff_lane_read(a_lds, j, a);
-
-  // local forward states of both blocks (zero start); v[r] for block A, v[16 + r] for block B
+  // Register-lean ordering: x and dy are consumed by the two local recurrences and are dead
+  // afterwards; dx is then formed in place from the local reverse state,
+  //   dx_r = A_r + q_r ,  q_r = (prod_{j=r+1..15} a_j) dC      (reverse running product)
+  //   e_r  = A_r (v_{r-1} + z_r) + q_r v_{r-1} ,  z_r = (prod_{j<r} a_j) c   (forward running product)
+  // The coefficients are re-read from LDS in every phase (a broadcast read) rather than held in
+  // 32 registers throughout; the compiler barriers keep the reads where they are written.
   float v[32];
   {
+    float a[32], xf[32];
+    coeff_lane_read(a_lds, j, a);
+    lane_read16<E>(img_x, j, d, xf);
     float h = 0.0f;
 #pragma unroll
     for (int r = 0; r < 16; ++r) { h = fmaf(a[r], h, xf[r]); v[r] = h; }
@@ -482,62 +481,75 @@ __global__ __launch_bounds__(64 * kWaves) SPEAR_BTP_BWD_OCC void btp_bwd_scan_ke
 #pragma unroll
     for (int r = 16; r < 32; ++r) { h = fmaf(a[r], h, xf[r]); v[r] = h; }
   }
-  // local reverse states (zero start at each block's end)
-  float A[32];
+  asm volatile("" ::: "memory");
+  float A[32];  // local reverse states, overwritten by dx below
+  float out_left, dcA_raw;
   {
+    float a[32], gf[32];
+    coeff_lane_read(a_lds, j, a);
+    if constexpr (kGradF32) {
+      lane_read32(img_g, j, d, gf);
+    } else {
+      lane_read16<E>(img_g, j, d, gf);
+    }
     float h = gf[15];
     A[15] = h;
 #pragma unroll
     for (int r = 14; r >= 0; --r) { h = fmaf(a[r + 1], h, gf[r]); A[r] = h; }
+    out_left = a[0] * h;
     h = gf[31];
     A[31] = h;
 #pragma unroll
     for (int r = 30; r >= 16; --r) { h = fmaf(a[r + 1], h, gf[r]); A[r] = h; }
+    dcA_raw = a[16] * h;
   }
+  asm volatile("" ::: "memory");
 
   const bool two = (k == 2);
-  // carries: forward ones flow to the right, gradient ones to the left
   const float from_left = lane_rotate(v[31], lane, -16);
-  const float from_right = lane_rotate(a[0] * A[0], lane, +16);
+  const float from_right = lane_rotate(out_left, lane, +16);
   const float cA = two ? (j == 0 ? c_halo : from_left) : 0.0f;
   const float cB = two ? v[15] : 0.0f;
-  const float dcA = two ? a[16] * A[16] : 0.0f;
+  const float dcA = two ? dcA_raw : 0.0f;
   const float dcB = two ? (j == 3 ? dc_halo : from_right) : 0.0f;
 
-  float dxv[32];
-  float e[16];
   float dA_A, dA_B;
-  {
-    // block A
-    float h = gf[15] + dcA;
-    dxv[15] = h;
 #pragma unroll
-    for (int r = 14; r >= 0; --r) { h = fmaf(a[r + 1], h, gf[r]); dxv[r] = h; }
-    float z = cA;
-    e[0] = A[0] * z;
+  for (int blk = 0; blk < 2; ++blk) {
+    const int o = 16 * blk;
+    float a[16];
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      const float4 q4 = *reinterpret_cast<const float4*>(a_lds + 32 * j + o + 4 * c);
+      a[4 * c + 0] = q4.x; a[4 * c + 1] = q4.y; a[4 * c + 2] = q4.z; a[4 * c + 3] = q4.w;
+    }
+    float e[16];
+    float z = blk ? cB : cA;
+    e[0] = A[o] * z;
 #pragma unroll
     for (int r = 1; r < 16; ++r) {
       z *= a[r - 1];
-      e[r] = fmaf(dxv[r], v[r - 1], A[r] * z);
+      e[r] = A[o + r] * (v[o + r - 1] + z);
     }
-    dA_A = row_transpose_reduce(e, d);
-  }
-  {
-    // block B
-    float h = gf[31] + dcB;
-    dxv[31] = h;
+    float q = blk ? dcB : dcA;
+    A[o + 15] += q;
+    e[15] = fmaf(q, v[o + 14], e[15]);
 #pragma unroll
-    for (int r = 30; r >= 16; --r) { h = fmaf(a[r + 1], h, gf[r]); dxv[r] = h; }
-    float z = cB;
-    e[0] = A[16] * z;
-#pragma unroll
-    for (int r = 1; r < 16; ++r) {
-      z *= a[16 + r - 1];
-      e[r] = fmaf(dxv[16 + r], v[16 + r - 1], A[16 + r] * z);
+    for (int r = 14; r >= 1; --r) {
+      q *= a[r + 1];
+      A[o + r] += q;
+      e[r] = fmaf(q, v[o + r - 1], e[r]);
     }
-    dA_B = row_transpose_reduce(e, d);
+    q *= a[1];
+    A[o] += q;
+    const float red = row_transpose_reduce(e, d);
+    if (blk) dA_B = red; else dA_A = red;
+    asm volatile("" ::: "memory");
   }
-
+  float (&dxv)[32] = A;
+  // dA leaves straight from registers: lane d of a group holds step d of its block, so every
+  // group writes two 64-byte runs. (Gathering the span's 128 values in LDS first to write 512
+  // contiguous bytes measured slower: the extra hand-over delays the last stores of the wave.)
   float* dArow = dA + sc.row * (long)L + sc.s0 + 32 * j + d;
   if (32 * j < sc.nvalid) __builtin_nontemporal_store(dA_A, dArow);
   if (32 * j + 16 < sc.nvalid) __builtin_nontemporal_store(dA_B, dArow + 16);
@@ -546,6 +558,24 @@ __global__ __launch_bounds__(64 * kWaves) SPEAR_BTP_BWD_OCC void btp_bwd_scan_ke
   lane_write16<E>(img_x, j, d, dxv);
   wave_lds_handover();
   slab16_lds_to_global<kStreamOut>(img_x, dx + slab_off, L, sc.nvalid, lane);
+}
+
+// 16-bit dy: the body fits 128 VGPRs, so four waves per SIMD are requested explicitly.
+template <class E, bool kStreamIn>
+__global__ __launch_bounds__(64 * kWaves) SPEAR_BTP_BWD_OCC void btp_bwd_scan_kernel(
+    const uint16_t* __restrict__ coeff, const uint16_t* __restrict__ x, const uint16_t* __restrict__ dy,
+    uint16_t* __restrict__ dx, float* __restrict__ dA, int L, int spans_per_row, long total_spans, int k) {
+  __shared__ __align__(16) unsigned char lds[kWaves][4096 + 4096 + 512];
+  btp_bwd_scan_body<E, uint16_t, kStreamIn>(lds, coeff, x, dy, dx, dA, L, spans_per_row, total_spans, k);
+}
+
+// fp32 dy: twice the staging registers and LDS; occupancy is left to the compiler.
+template <class E, bool kStreamIn>
+__global__ __launch_bounds__(64 * kWaves) void btp_bwd_scan_kernel_f32grad(
+    const uint16_t* __restrict__ coeff, const uint16_t* __restrict__ x, const float* __restrict__ dy,
+    uint16_t* __restrict__ dx, float* __restrict__ dA, int L, int spans_per_row, long total_spans, int k) {
+  __shared__ __align__(16) unsigned char lds[kWaves][4096 + 8192 + 512];
+  btp_bwd_scan_body<E, float, kStreamIn>(lds, coeff, x, dy, dx, dA, L, spans_per_row, total_spans, k);
 }
 
 __global__ __launch_bounds__(256) void copy_kernel(const uint4* __restrict__ src, uint4* __restrict__ dst,
@@ -596,10 +626,16 @@ hipError_t launch_fwd(const FwdArgs& p, hipStream_t s) {
 
 template <class E, class GradT, bool kStreamIn>
 void launch_bwd_as(const BwdArgs& p, const Grid& g, hipStream_t s) {
-  hipLaunchKernelGGL((btp_bwd_scan_kernel<E, GradT, kStreamIn>), dim3(g.blocks), dim3(64 * kWaves), 0, s,
-                     static_cast<const uint16_t*>(p.coeff), static_cast<const uint16_t*>(p.x),
-                     static_cast<const GradT*>(p.dy), static_cast<uint16_t*>(p.dx), p.dA, p.L, g.spans_per_row,
-                     g.total_spans, p.k);
+  const auto* c = static_cast<const uint16_t*>(p.coeff);
+  const auto* x = static_cast<const uint16_t*>(p.x);
+  auto* dx = static_cast<uint16_t*>(p.dx);
+  if constexpr (std::is_same<GradT, float>::value) {
+    hipLaunchKernelGGL((btp_bwd_scan_kernel_f32grad<E, kStreamIn>), dim3(g.blocks), dim3(64 * kWaves), 0, s, c, x,
+                       static_cast<const float*>(p.dy), dx, p.dA, p.L, g.spans_per_row, g.total_spans, p.k);
+  } else {
+    hipLaunchKernelGGL((btp_bwd_scan_kernel<E, kStreamIn>), dim3(g.blocks), dim3(64 * kWaves), 0, s, c, x,
+                       static_cast<const uint16_t*>(p.dy), dx, p.dA, p.L, g.spans_per_row, g.total_spans, p.k);
+  }
 }
 
 template <class E, class GradT>
