@@ -238,18 +238,25 @@ __device__ __forceinline__ uint32_t coeff_global_to_reg(const uint16_t* arow, in
   return ((lane << 1) < nvalid) ? __builtin_nontemporal_load(reinterpret_cast<const uint32_t*>(arow + (lane << 1))) : 0u;
 }
 
+// The second half of the span is stored 16 floats further on, so that the four lane groups, which
+// read four different 16-byte pieces in the same instruction, fall into four different sets of
+// LDS banks (without the gap groups 0/2 and 1/3 would collide, 128 floats = two bank periods).
+constexpr int kCoeffLdsBytes = (kSpan + 16) * 4;
+
+__device__ __forceinline__ int coeff_slot(int t) { return t + ((t >> 6) << 4); }
+
 template <class E>
 __device__ __forceinline__ void coeff_reg_to_lds(float* a_lds, int lane, uint32_t w) {
   float2 f;
   f.x = clamp_coeff<E>(E::lo(w));
   f.y = clamp_coeff<E>(E::hi(w));
-  *reinterpret_cast<float2*>(a_lds + (lane << 1)) = f;
+  *reinterpret_cast<float2*>(a_lds + coeff_slot(lane << 1)) = f;
 }
 
 __device__ __forceinline__ void coeff_lane_read(const float* a_lds, int j, float (&a)[32]) {
 #pragma unroll
   for (int c = 0; c < 8; ++c) {
-    const float4 q = *reinterpret_cast<const float4*>(a_lds + 32 * j + 4 * c);
+    const float4 q = *reinterpret_cast<const float4*>(a_lds + coeff_slot(32 * j) + 4 * c);
     a[4 * c + 0] = q.x; a[4 * c + 1] = q.y; a[4 * c + 2] = q.z; a[4 * c + 3] = q.w;
   }
 }
@@ -279,7 +286,7 @@ __global__ __launch_bounds__(64 * kWaves) SPEAR_BTP_FWD_OCC void btp_fwd_scan_ke
     float* __restrict__ ckpt, int L, int spans_per_row, long total_spans, int k) {
   constexpr bool kOutF32 = std::is_same<OutT, float>::value;
   constexpr int kImgBytes = kOutF32 ? 8192 : 4096;
-  __shared__ __align__(16) unsigned char lds[kWaves][kImgBytes + 512];
+  __shared__ __align__(16) unsigned char lds[kWaves][kImgBytes + kCoeffLdsBytes];
 
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const long span = (long)blockIdx.x * kWaves + wave;
@@ -385,7 +392,7 @@ __global__ __launch_bounds__(64 * kWaves) SPEAR_BTP_FWD_OCC void btp_fwd_scan_ke
 // ==========================================================================================
 template <class E, class GradT, bool kStreamIn>
 __device__ __forceinline__ void btp_bwd_scan_body(
-    unsigned char (*lds)[4096 + (std::is_same<GradT, float>::value ? 8192 : 4096) + 512],
+    unsigned char (*lds)[4096 + (std::is_same<GradT, float>::value ? 8192 : 4096) + kCoeffLdsBytes],
     const uint16_t* __restrict__ coeff, const uint16_t* __restrict__ x, const GradT* __restrict__ dy,
     uint16_t* __restrict__ dx, float* __restrict__ dA, int L, int spans_per_row, long total_spans,
     int k) {
@@ -520,7 +527,7 @@ __device__ __forceinline__ void btp_bwd_scan_body(
     float a[16];
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
-      const float4 q4 = *reinterpret_cast<const float4*>(a_lds + 32 * j + o + 4 * c);
+      const float4 q4 = *reinterpret_cast<const float4*>(a_lds + coeff_slot(32 * j) + o + 4 * c);
       a[4 * c + 0] = q4.x; a[4 * c + 1] = q4.y; a[4 * c + 2] = q4.z; a[4 * c + 3] = q4.w;
     }
     float e[16];
@@ -565,7 +572,7 @@ template <class E, bool kStreamIn>
 __global__ __launch_bounds__(64 * kWaves) SPEAR_BTP_BWD_OCC void btp_bwd_scan_kernel(
     const uint16_t* __restrict__ coeff, const uint16_t* __restrict__ x, const uint16_t* __restrict__ dy,
     uint16_t* __restrict__ dx, float* __restrict__ dA, int L, int spans_per_row, long total_spans, int k) {
-  __shared__ __align__(16) unsigned char lds[kWaves][4096 + 4096 + 512];
+  __shared__ __align__(16) unsigned char lds[kWaves][4096 + 4096 + kCoeffLdsBytes];
   btp_bwd_scan_body<E, uint16_t, kStreamIn>(lds, coeff, x, dy, dx, dA, L, spans_per_row, total_spans, k);
 }
 
@@ -574,7 +581,7 @@ template <class E, bool kStreamIn>
 __global__ __launch_bounds__(64 * kWaves) void btp_bwd_scan_kernel_f32grad(
     const uint16_t* __restrict__ coeff, const uint16_t* __restrict__ x, const float* __restrict__ dy,
     uint16_t* __restrict__ dx, float* __restrict__ dA, int L, int spans_per_row, long total_spans, int k) {
-  __shared__ __align__(16) unsigned char lds[kWaves][4096 + 8192 + 512];
+  __shared__ __align__(16) unsigned char lds[kWaves][4096 + 8192 + kCoeffLdsBytes];
   btp_bwd_scan_body<E, float, kStreamIn>(lds, coeff, x, dy, dx, dA, L, spans_per_row, total_spans, k);
 }
 

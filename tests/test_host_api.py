@@ -1,0 +1,178 @@
+"""Host-side behaviour that needs no GPU: the op's argument checks and messages (mirroring
+csrc/btp/_bindings.cu:19-60 and spear/ops/btp/interface.py:137-139 of the reference), the
+registered custom ops, the package surface, and the Phalanx layer's construction rules."""
+
+import pytest
+import torch
+
+import spear_amd
+from spear_amd import _btp
+from spear_amd.nn.phalanx import KVRepeat, Phalanx, SigmoidA
+from spear_amd.ops.btp import interface
+
+
+def _cpu_args(B=1, H=2, L=32, dtype=torch.bfloat16):
+    coeff = torch.rand(B, H, L).to(dtype)
+    x = torch.randn(B, H, 16, L).to(dtype)
+    y = torch.empty(B, H, 16, L, dtype=torch.float32)
+    ck = torch.empty(B, H, L // 16, 16, dtype=torch.float32)
+    return coeff, x, y, ck
+
+
+def test_package_surface():
+    assert spear_amd.__version__ == "0.1.0"
+    assert spear_amd.btp is interface.btp
+    assert spear_amd.Phalanx is Phalanx and spear_amd.SigmoidA is SigmoidA
+    assert (interface.DH, interface.BLK) == (16, 16)
+    assert interface.SUPPORTED_WPB == [4, 8, 16, 32]
+    assert (interface.WPB_K1_DEFAULT, interface.WPB_K2_DEFAULT) == (8, 32)
+
+
+def test_custom_ops_are_registered_with_the_reference_schemas():
+    fwd = torch.ops.spear_btp.forward.default._schema
+    bwd = torch.ops.spear_btp.backward.default._schema
+    assert [a.name for a in fwd.arguments] == ["coeff", "x", "y", "checkpoint", "k", "wpb"]
+    assert [a.name for a in bwd.arguments] == ["coeff", "x", "dy", "checkpoint", "dx", "dA", "k", "wpb"]
+    assert [a.name for a in fwd.arguments if a.alias_info and a.alias_info.is_write] == ["y", "checkpoint"]
+    assert [a.name for a in bwd.arguments if a.alias_info and a.alias_info.is_write] == ["dx", "dA"]
+
+
+def test_non_gpu_tensors_are_rejected_like_the_reference():
+    coeff, x, y, ck = _cpu_args()
+    with pytest.raises(RuntimeError, match="All tensors must be CUDA"):
+        _btp.forward(coeff, x, y, ck, 2, 32)
+    with pytest.raises(RuntimeError, match="coeff, x, dy, checkpoint must be CUDA"):
+        _btp.backward(coeff, x, y, ck, torch.empty_like(x), torch.empty(1, 2, 32), 2, 32)
+
+
+def test_there_is_no_cpu_fallback_for_the_op():
+    coeff, x, _, _ = _cpu_args()
+    with pytest.raises((RuntimeError, NotImplementedError)):
+        interface.btp(coeff, x)
+
+
+def test_missing_library_is_a_loud_error(monkeypatch, tmp_path):
+    monkeypatch.setattr(_btp, "_lib", None)
+    monkeypatch.setenv("SPEAR_BTP_LIBRARY", str(tmp_path / "nope.so"))
+    with pytest.raises(RuntimeError, match="could not be loaded"):
+        _btp.load_library()
+
+
+@pytest.mark.parametrize(
+    "mutate,msg",
+    [
+        (lambda a: a.__setitem__("x", a["x"][0]), r"x must be \[B, H, 16, L\]"),
+        (lambda a: a.__setitem__("x", torch.empty(1, 2, 8, 32, dtype=torch.bfloat16)), "Channel dim"),
+        (lambda a: a.__setitem__("k", 3), "k must be 1 or 2"),
+        (lambda a: a.__setitem__("wpb", 5), "Unsupported WPB value: 5"),
+        (lambda a: a.__setitem__("coeff", a["coeff"].float()), "coeff must be float16 or bfloat16"),
+        (lambda a: a.__setitem__("x", a["x"].half()), "x dtype must match coeff"),
+        (lambda a: a.__setitem__("y", a["y"].half()), "y must be float32 or match x dtype"),
+        (lambda a: a.__setitem__("ck", a["ck"].half()), "checkpoint must be float32"),
+    ],
+)
+def test_forward_checks_fire_in_the_reference_order(monkeypatch, mutate, msg):
+    # pretend the tensors live on the GPU so that the later checks are reached
+    monkeypatch.setattr(torch.Tensor, "is_cuda", property(lambda self: True))
+    coeff, x, y, ck = _cpu_args()
+    a = dict(coeff=coeff, x=x, y=y, ck=ck, k=2, wpb=32)
+    mutate(a)
+    with pytest.raises(RuntimeError, match=msg):
+        _btp.forward(a["coeff"], a["x"], a["y"], a["ck"], a["k"], a["wpb"])
+
+
+def test_shape_mismatches_raise_instead_of_reading_out_of_bounds(monkeypatch):
+    monkeypatch.setattr(torch.Tensor, "is_cuda", property(lambda self: True))
+    coeff, x, y, ck = _cpu_args()
+    with pytest.raises(RuntimeError, match="coeff must have shape"):
+        _btp.forward(coeff[:, :1], x, y, ck, 2, 32)
+    with pytest.raises(RuntimeError, match="x must be contiguous"):
+        strided = torch.randn(1, 2, 16, 64).bfloat16()[..., ::2]
+        _btp.forward(coeff, strided, y, ck, 2, 32)
+    with pytest.raises(RuntimeError, match="multiple of 16"):
+        c2 = torch.rand(1, 2, 24).bfloat16()
+        x2 = torch.randn(1, 2, 16, 24).bfloat16()
+        _btp.forward(c2, x2, torch.empty(1, 2, 16, 24), torch.empty(1, 2, 1, 16), 2, 32)
+
+
+def test_python_level_asserts():
+    coeff = torch.rand(1, 2, 24).bfloat16()
+    with pytest.raises(AssertionError, match="multiple of 16"):
+        interface.btp(coeff, torch.randn(1, 2, 16, 24).bfloat16())
+    with pytest.raises(AssertionError, match="Channel dimension"):
+        interface.btp(torch.rand(1, 2, 32).bfloat16(), torch.randn(1, 2, 8, 32).bfloat16())
+    with pytest.raises(AssertionError, match="WPB"):
+        interface.btp(torch.rand(1, 2, 32).bfloat16(), torch.randn(1, 2, 16, 32).bfloat16(), wpb=7)
+
+
+# ---- Phalanx layer ------------------------------------------------------------------------------
+
+def test_phalanx_validation_errors():
+    with pytest.raises(ValueError, match="divisible by 16"):
+        Phalanx(dim=100)
+    with pytest.raises(ValueError, match="head_dim must be 16"):
+        Phalanx(dim=256, heads=8)
+    with pytest.raises(ValueError, match="divisible by heads"):
+        Phalanx(dim=256, heads=7)
+    with pytest.raises(ValueError, match="method must be one of"):
+        Phalanx(dim=256, method="cuda")
+    with pytest.raises(ValueError, match="divisible by kv_heads"):
+        Phalanx(dim=256, kv_heads=5)
+    with pytest.raises(ValueError):
+        KVRepeat(3, 16)
+
+
+def test_phalanx_attributes_and_state_dict_keys():
+    layer = Phalanx(dim=256, length=100, method="default", dtype=torch.bfloat16)  # needs no GPU to build
+    assert (layer.heads, layer.head_dim, layer.length, layer.k, layer.wpb) == (16, 16, 112, 2, 32)
+    assert layer.output_dtype == torch.bfloat16 and layer.kv_heads == 16
+    assert set(layer.state_dict()) == {
+        "param.proj_a.weight", "param.proj_a.bias", "param.proj_b.weight", "param.proj_b.bias",
+        "param.proj_c.weight", "param.proj_c.bias", "param.proj_v.weight", "proj_out.weight",
+    }
+    assert layer.param.proj_a.weight.shape == (16, 256)
+    assert layer.param.proj_v.weight.shape == (256, 256) and layer.param.proj_v.bias is None
+
+
+def test_phalanx_default_init_is_reproducible_across_methods():
+    torch.manual_seed(7)
+    a = Phalanx(dim=128, method="pytorch", dtype=torch.bfloat16)
+    torch.manual_seed(7)
+    b = Phalanx(dim=128, method="default", dtype=torch.bfloat16)
+    for (ka, va), (kb, vb) in zip(a.state_dict().items(), b.state_dict().items()):
+        assert ka == kb and torch.equal(va, vb)
+
+
+@pytest.mark.parametrize("method", ["pytorch", "pytorch_linspace"])
+@pytest.mark.parametrize("kv_heads", [None, 2])
+def test_phalanx_pytorch_methods_run_on_cpu(method, kv_heads):
+    torch.manual_seed(0)
+    layer = Phalanx(dim=128, length=64, method=method, dtype=torch.bfloat16, kv_heads=kv_heads)
+    x = torch.randn(2, 64, 128).bfloat16()
+    y = layer(x)
+    assert y.shape == (2, 64, 128) and y.dtype == torch.bfloat16 and torch.isfinite(y.float()).all()
+    y.float().sum().backward()
+    assert all(p.grad is not None for p in layer.parameters())
+    if kv_heads:
+        assert layer.param.proj_b.weight.shape == (kv_heads * 16, 128)
+        assert not any("kv_indices" in k for k in layer.state_dict())
+
+
+def test_log_and_linear_space_layers_agree():
+    torch.manual_seed(1)
+    a = Phalanx(dim=128, length=64, method="pytorch", dtype=torch.bfloat16)
+    b = Phalanx(dim=128, length=64, method="pytorch_linspace", dtype=torch.bfloat16)
+    b.load_state_dict(a.state_dict())
+    x = torch.randn(2, 64, 128).bfloat16()
+    assert (a(x).float() - b(x).float()).abs().max() <= 1e-1  # layer forward limit of the reference tests
+
+
+def test_fused_gates_packing_order():
+    torch.manual_seed(2)
+    p = SigmoidA(64, 4, 16, dtype=torch.bfloat16, kv_heads=2)
+    x = torch.randn(1, 32, 64).bfloat16()
+    packed = p.forward_fused_gates(x)
+    assert packed.shape == (1, 3 * 4 * 16 + 4, 32)
+    a_logits, b_kv, c_kv, v = p._compute_base_projections(x)
+    assert torch.equal(packed[:, 64:128], v) and torch.equal(packed[:, -4:], a_logits)
+    assert torch.equal(packed[:, :16], b_kv[:, :16]) and torch.equal(packed[:, 16:32], b_kv[:, :16])  # heads 0,1 share kv head 0
