@@ -192,6 +192,13 @@ def main() -> int:
 
     fwd_ms, bwd_ms = kernel_ms(fwd), kernel_ms(bwd)
 
+    def fwd_mfma(s):  # same op through the bf16-MFMA tile kernel, for comparison
+        rc = lib.spear_btp_forward(s["coeff"].data_ptr(), s["x"].data_ptr(), s["y"].data_ptr(), None,
+                                   B, H, L, 2, 0, 0, 2, sp)
+        assert rc == 0, lib.spear_btp_last_error()
+
+    fwd_mfma_ms = kernel_ms(fwd_mfma)
+
     # copy kernel of the same footprint as a practical ceiling (reads n, writes n)
     nbytes = sets[0]["x"].numel() * 2
     def copy(s):
@@ -236,6 +243,9 @@ def main() -> int:
         },
         "forward_kernel": {"avg_launch_ms": fwd_ms, "achieved": fwd_gbps, "frac": fwd_gbps / HBM_PEAK_GBPS,
                            "algorithmic_bytes_per_launch": units * FWD_BYTES},
+        "forward_kernel_mfma_path": {"avg_launch_ms": fwd_mfma_ms,
+                                     "achieved": units * FWD_BYTES / (fwd_mfma_ms * 1e-3) / 1e9,
+                                     "frac": units * FWD_BYTES / (fwd_mfma_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS},
         "fwd_plus_bwd": {"achieved": step_gbps, "frac": step_gbps / HBM_PEAK_GBPS,
                          "algorithmic_bytes_per_step": units * (FWD_BYTES + BWD_BYTES)},
         "copy_kernel": {"avg_launch_ms": copy_ms, "achieved": 2 * nbytes / (copy_ms * 1e-3) / 1e9,

@@ -58,11 +58,15 @@ int spear_btp_forward(const void* coeff, const void* x, void* y, float* checkpoi
     return fail(SPEAR_BTP_ENULL, "spear_btp_forward: NULL tensor pointer");
   if (!aligned16(coeff) || !aligned16(x) || !aligned16(y) || (want_ckpt && !aligned16(checkpoint)))
     return fail(SPEAR_BTP_EINVAL, "spear_btp_forward: tensor pointers must be 16-byte aligned");
-  if (flags & SPEAR_BTP_PATH_MFMA)
-    return fail(SPEAR_BTP_EINVAL, "spear_btp_forward: the MFMA path is not built into this library");
+  const bool mfma = (flags & SPEAR_BTP_PATH_MFMA) != 0;
+  if (mfma && in_dtype != SPEAR_BTP_BF16)
+    return fail(SPEAR_BTP_EINVAL, "spear_btp_forward: the MFMA path takes bfloat16 inputs only");
+  if (mfma && want_ckpt)
+    return fail(SPEAR_BTP_EINVAL, "spear_btp_forward: the MFMA path does not store the carry checkpoint");
 
   spear_btp::FwdArgs a{coeff, x, y, want_ckpt ? checkpoint : nullptr, B, H, L, k, in_dtype, out_dtype};
-  const hipError_t err = spear_btp::scan_forward(a, static_cast<hipStream_t>(stream));
+  const hipStream_t hs = static_cast<hipStream_t>(stream);
+  const hipError_t err = mfma ? spear_btp::mfma_forward(a, hs) : spear_btp::scan_forward(a, hs);
   if (err != hipSuccess) return fail(SPEAR_BTP_ELAUNCH, "spear_btp_forward: launch failed: %s", hipGetErrorString(err));
   return 0;
 }
@@ -78,7 +82,7 @@ int spear_btp_backward(const void* coeff, const void* x, const void* dy, const f
   if (!aligned16(coeff) || !aligned16(x) || !aligned16(dy) || !aligned16(dx) || !aligned16(dA))
     return fail(SPEAR_BTP_EINVAL, "spear_btp_backward: tensor pointers must be 16-byte aligned");
   if (flags & SPEAR_BTP_PATH_MFMA)
-    return fail(SPEAR_BTP_EINVAL, "spear_btp_backward: the MFMA path is not built into this library");
+    return fail(SPEAR_BTP_EINVAL, "spear_btp_backward: there is no MFMA variant of the backward kernel");
 
   spear_btp::BwdArgs a{coeff, x, dy, dx, dA, B, H, L, k, in_dtype, dy_dtype};
   const hipError_t err = spear_btp::scan_backward(a, static_cast<hipStream_t>(stream));

@@ -33,6 +33,9 @@ struct BwdArgs {
 hipError_t scan_forward(const FwdArgs& p, hipStream_t s);
 hipError_t scan_backward(const BwdArgs& p, hipStream_t s);
 
+// bf16-MFMA tile kernels (btp_mfma.hip). bf16 inputs only; the forward one stores no checkpoint.
+hipError_t mfma_forward(const FwdArgs& p, hipStream_t s);
+
 // Plain copy kernel used for bandwidth / counter calibration (btp_scan.hip).
 hipError_t device_copy(const void* src, void* dst, unsigned long long bytes, hipStream_t s);
 

@@ -16,14 +16,15 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 
 
-def run_forward(coeff, x, k=2, out_dtype=torch.bfloat16, checkpoint=False):
+def run_forward(coeff, x, k=2, out_dtype=torch.bfloat16, checkpoint=False, mfma=False):
     from spear_amd import _btp
 
     c, xx = coeff.to(DEV), x.to(DEV)
     B, H, _, L = x.shape
     y = torch.full((B, H, 16, L), float("nan"), device=DEV, dtype=out_dtype)
     ck = torch.full((B, H, L // 16, 16), float("nan"), device=DEV, dtype=torch.float32)
-    _btp.forward(c, xx, y, ck, k, 32, flags=_btp.FLAG_WRITE_CHECKPOINT if checkpoint else 0)
+    flags = (_btp.FLAG_WRITE_CHECKPOINT if checkpoint else 0) | (_btp.FLAG_PATH_MFMA if mfma else 0)
+    _btp.forward(c, xx, y, ck, k, 32, flags=flags)
     torch.cuda.synchronize()
     return (y.cpu(), ck.cpu()) if checkpoint else y.cpu()
 
@@ -60,6 +61,41 @@ def test_forward_fp32_out_matches_oracle_to_1e4(B, H, L, k):
     print(f"fwd f32 B={B} H={H} L={L} k={k}", flush=True)
     y = run_forward(coeff, x, k=k, out_dtype=torch.float32)
     assert_close(f64(y), orc.forward(f64(coeff), f64(x), k=k), F32_ATOL, F32_RTOL, "y")
+
+
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32], ids=["bf16", "f32"])
+@pytest.mark.parametrize("k", [2, 1])
+@pytest.mark.parametrize("B,H,L", SHAPES)
+def test_forward_mfma_path_matches_oracle(B, H, L, k, out_dtype):
+    # the MFMA path rounds the decay matrix to bf16 (as the reference kernel does), so also its
+    # fp32 output is held to the bf16 tolerance
+    coeff, x, _ = make_inputs(B, H, L, seed=700 + L + k)
+    print(f"fwd mfma B={B} H={H} L={L} k={k} {out_dtype}", flush=True)
+    y = run_forward(coeff, x, k=k, out_dtype=out_dtype, mfma=True)
+    assert_close(f64(y), orc.forward(f64(coeff), f64(x), k=k), BF16_ATOL, BF16_RTOL, "y")
+
+
+def test_forward_mfma_path_stress_and_zero_coefficients():
+    coeff, x, _ = make_inputs(2, 8, 2048, seed=1236, gate="mixed")
+    y = run_forward(coeff, x, mfma=True)
+    assert_close(f64(y), orc.forward(f64(coeff), f64(x)), BF16_ATOL, BF16_RTOL, "y mixed gates")
+    coeff, x, _ = make_inputs(1, 2, 160, seed=7)
+    coeff[0, 0, [0, 5, 16, 33, 127, 128]] = 0.0
+    y = run_forward(coeff, x, out_dtype=torch.float32, mfma=True)
+    assert_close(f64(y), orc.forward(f64(coeff), f64(x)), BF16_ATOL, BF16_RTOL, "y zero coefficients")
+
+
+def test_mfma_path_rejects_what_it_does_not_do():
+    from spear_amd import _btp
+
+    coeff, x, dy = make_inputs(1, 2, 32, seed=1, dtype=torch.float16)
+    c, xx = coeff.to(DEV), x.to(DEV)
+    y = torch.empty_like(xx)
+    ck = torch.empty(1, 2, 2, 16, device=DEV)
+    with pytest.raises(RuntimeError, match="bfloat16 inputs only"):
+        _btp.forward(c, xx, y, ck, 2, 32, flags=_btp.FLAG_PATH_MFMA)
+    with pytest.raises(RuntimeError, match="no MFMA variant"):
+        _btp.backward(c, xx, dy.to(DEV), ck, torch.empty_like(xx), torch.empty(1, 2, 32, device=DEV), 2, 32, flags=_btp.FLAG_PATH_MFMA)
 
 
 @pytest.mark.parametrize("k", [2, 1])
