@@ -68,6 +68,21 @@ int spear_btp_backward(const void* coeff, const void* x, const void* dy, const f
                        void* dx, float* dA, int B, int H, int L, int k, int in_dtype, int dy_dtype,
                        unsigned flags, void* stream);
 
+/* Log-space gate variants. They have no counterpart function in the reference, whose op takes
+ * the decay already exponentiated and rounded to 16 bits (spear/ops/btp/interface.py:164-188);
+ * they serve callers that hold the gate in log space -- the Phalanx layer's -softplus(.) of a
+ * logit (spear/nn/phalanx/swr.py:216), or the fp32 log-decay gates of the benchmark
+ * configurations -- and want a_t = exp(g_t) formed in fp32 inside the kernel (a 16-bit a_t cannot
+ * represent 1 - 1e-4). Same tensors and rules as above except:
+ *     gate   [B, H, L] fp32   log-space decay g_t <= 0 (a_t = exp(g_t); exp(g_t) <= 1e-9 counts as 0)
+ *     dgate  [B, H, L] fp32   gradient w.r.t. g_t (= a_t * dL/da_t), every element written
+ * SPEAR_BTP_PATH_MFMA is not available for these. */
+int spear_btp_forward_loggate(const float* gate, const void* x, void* y, float* checkpoint, int B, int H,
+                              int L, int k, int x_dtype, int out_dtype, unsigned flags, void* stream);
+int spear_btp_backward_loggate(const float* gate, const void* x, const void* dy, void* dx, float* dgate,
+                               int B, int H, int L, int k, int x_dtype, int dy_dtype, unsigned flags,
+                               void* stream);
+
 /* Message for the last failing call on this thread ("" if none).  The reference prints launch
  * failures and carries on (csrc/btp/btp-forward.cu:501-520); here they are reported. */
 const char* spear_btp_last_error(void);

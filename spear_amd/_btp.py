@@ -18,12 +18,12 @@ import threading
 
 import torch
 
-__all__ = ["forward", "backward", "library_path", "load_library", "FLAG_WRITE_CHECKPOINT", "FLAG_PATH_MFMA"]
+__all__ = ["forward", "backward", "forward_log", "backward_log", "library_path", "load_library", "FLAG_WRITE_CHECKPOINT", "FLAG_PATH_MFMA"]
 
 _BF16, _F16, _F32 = 0, 1, 2
 FLAG_WRITE_CHECKPOINT = 0x1
 FLAG_PATH_MFMA = 0x2
-_ABI_VERSION = 1
+_ABI_VERSION = 2
 _SUPPORTED_WPB = (4, 8, 16, 32)
 
 _lock = threading.Lock()
@@ -44,6 +44,10 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.spear_btp_forward.restype = ci
     lib.spear_btp_backward.argtypes = [vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, cu, vp]
     lib.spear_btp_backward.restype = ci
+    lib.spear_btp_forward_loggate.argtypes = [vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, cu, vp]
+    lib.spear_btp_forward_loggate.restype = ci
+    lib.spear_btp_backward_loggate.argtypes = [vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, cu, vp]
+    lib.spear_btp_backward_loggate.restype = ci
     lib.spear_btp_last_error.argtypes = []
     lib.spear_btp_last_error.restype = ctypes.c_char_p
     lib.spear_btp_abi_version.argtypes = []
@@ -193,6 +197,61 @@ def backward(
         rc = lib.spear_btp_backward(
             coeff.data_ptr(), x.data_ptr(), dy.data_ptr(), checkpoint.data_ptr(), dx.data_ptr(), dA.data_ptr(),
             B, H, L, int(k), _tag(x.dtype), _tag(dy.dtype), int(flags), _stream_ptr(x.device),
+        )
+    if rc != 0:
+        _raise_native(lib, rc)
+
+
+def _check_log_common(gate: torch.Tensor, x: torch.Tensor, k: int) -> tuple[int, int, int]:
+    _check(gate.is_cuda and x.is_cuda, "All tensors must be CUDA.")
+    _check(x.dim() == 4, "x must be [B, H, 16, L].")
+    _check(x.size(2) == 16, "Channel dim (DH) must be 16.")
+    _check(k in (1, 2), "k must be 1 or 2.")
+    _check(gate.dtype == torch.float32, "gate must be float32.")
+    _check(x.dtype in (torch.float16, torch.bfloat16), "x must be float16 or bfloat16.")
+    B, H, _, L = x.shape
+    _check(L % 16 == 0, "Length L must be multiple of 16")
+    _check_layout("gate", gate, (B, H, L))
+    _check_layout("x", x, (B, H, 16, L))
+    return B, H, L
+
+
+def forward_log(gate: torch.Tensor, x: torch.Tensor, y: torch.Tensor, k: int) -> None:
+    """``y <- btp(exp(gate), x)`` with the exponential taken in fp32 inside the kernel. ``gate`` is
+    the fp32 log-space decay ``[B, H, L]``. No counterpart in the reference's extension module."""
+    B, H, L = _check_log_common(gate, x, k)
+    _check(y.is_cuda, "All tensors must be CUDA.")
+    _check(y.dtype == torch.float32 or y.dtype == x.dtype, "y must be float32 or match x dtype.")
+    _check_layout("y", y, (B, H, 16, L))
+    _check(gate.device == x.device == y.device, "All tensors must be on the same device.")
+    lib = load_library()
+    with torch.cuda.device(x.device):
+        rc = lib.spear_btp_forward_loggate(
+            gate.data_ptr(), x.data_ptr(), y.data_ptr(), None, B, H, L, int(k), _tag(x.dtype), _tag(y.dtype), 0,
+            _stream_ptr(x.device),
+        )
+    if rc != 0:
+        _raise_native(lib, rc)
+
+
+def backward_log(
+    gate: torch.Tensor, x: torch.Tensor, dy: torch.Tensor, dx: torch.Tensor, dgate: torch.Tensor, k: int
+) -> None:
+    """``dx, dgate <- vjp of btp(exp(gate), x)``; ``dgate`` is the gradient w.r.t. the log-space gate."""
+    B, H, L = _check_log_common(gate, x, k)
+    _check(dy.is_cuda and dx.is_cuda and dgate.is_cuda, "All tensors must be CUDA.")
+    _check(dx.dtype == x.dtype, "dx dtype must match x.")
+    _check(dgate.dtype == torch.float32, "dgate must be float32.")
+    _check(dy.dtype == torch.float32 or dy.dtype == x.dtype, "dy must be float32 or match x dtype.")
+    _check_layout("dy", dy, (B, H, 16, L))
+    _check_layout("dx", dx, (B, H, 16, L))
+    _check_layout("dgate", dgate, (B, H, L))
+    _check(gate.device == x.device == dy.device == dx.device == dgate.device, "All tensors must be on the same device.")
+    lib = load_library()
+    with torch.cuda.device(x.device):
+        rc = lib.spear_btp_backward_loggate(
+            gate.data_ptr(), x.data_ptr(), dy.data_ptr(), dx.data_ptr(), dgate.data_ptr(), B, H, L, int(k),
+            _tag(x.dtype), _tag(dy.dtype), 0, _stream_ptr(x.device),
         )
     if rc != 0:
         _raise_native(lib, rc)

@@ -42,7 +42,7 @@ int check_common(const char* who, int B, int H, int L, int k, int in_dtype, int 
 
 extern "C" {
 
-int spear_btp_abi_version(void) { return 1; }
+int spear_btp_abi_version(void) { return 2; }
 
 const char* spear_btp_last_error(void) { return g_error; }
 
@@ -87,6 +87,41 @@ int spear_btp_backward(const void* coeff, const void* x, const void* dy, const f
   spear_btp::BwdArgs a{coeff, x, dy, dx, dA, B, H, L, k, in_dtype, dy_dtype};
   const hipError_t err = spear_btp::scan_backward(a, static_cast<hipStream_t>(stream));
   if (err != hipSuccess) return fail(SPEAR_BTP_ELAUNCH, "spear_btp_backward: launch failed: %s", hipGetErrorString(err));
+  return 0;
+}
+
+int spear_btp_forward_loggate(const float* gate, const void* x, void* y, float* checkpoint, int B, int H, int L, int k,
+                              int x_dtype, int out_dtype, unsigned flags, void* stream) {
+  g_error[0] = '\0';
+  if (int rc = check_common("spear_btp_forward_loggate", B, H, L, k, x_dtype, out_dtype, "y", flags,
+                            SPEAR_BTP_WRITE_CHECKPOINT))
+    return rc;
+  if ((long long)B * H == 0 || L == 0) return 0;
+  const bool want_ckpt = (flags & SPEAR_BTP_WRITE_CHECKPOINT) != 0;
+  if (!gate || !x || !y || (want_ckpt && !checkpoint))
+    return fail(SPEAR_BTP_ENULL, "spear_btp_forward_loggate: NULL tensor pointer");
+  if (!aligned16(gate) || !aligned16(x) || !aligned16(y) || (want_ckpt && !aligned16(checkpoint)))
+    return fail(SPEAR_BTP_EINVAL, "spear_btp_forward_loggate: tensor pointers must be 16-byte aligned");
+  spear_btp::FwdArgs a{gate, x, y, want_ckpt ? checkpoint : nullptr, B, H, L, k, x_dtype, out_dtype, true};
+  const hipError_t err = spear_btp::scan_forward(a, static_cast<hipStream_t>(stream));
+  if (err != hipSuccess)
+    return fail(SPEAR_BTP_ELAUNCH, "spear_btp_forward_loggate: launch failed: %s", hipGetErrorString(err));
+  return 0;
+}
+
+int spear_btp_backward_loggate(const float* gate, const void* x, const void* dy, void* dx, float* dgate, int B, int H,
+                               int L, int k, int x_dtype, int dy_dtype, unsigned flags, void* stream) {
+  g_error[0] = '\0';
+  if (int rc = check_common("spear_btp_backward_loggate", B, H, L, k, x_dtype, dy_dtype, "dy", flags, 0u)) return rc;
+  if ((long long)B * H == 0 || L == 0) return 0;
+  if (!gate || !x || !dy || !dx || !dgate)
+    return fail(SPEAR_BTP_ENULL, "spear_btp_backward_loggate: NULL tensor pointer");
+  if (!aligned16(gate) || !aligned16(x) || !aligned16(dy) || !aligned16(dx) || !aligned16(dgate))
+    return fail(SPEAR_BTP_EINVAL, "spear_btp_backward_loggate: tensor pointers must be 16-byte aligned");
+  spear_btp::BwdArgs a{gate, x, dy, dx, dgate, B, H, L, k, x_dtype, dy_dtype, true};
+  const hipError_t err = spear_btp::scan_backward(a, static_cast<hipStream_t>(stream));
+  if (err != hipSuccess)
+    return fail(SPEAR_BTP_ELAUNCH, "spear_btp_backward_loggate: launch failed: %s", hipGetErrorString(err));
   return 0;
 }
 

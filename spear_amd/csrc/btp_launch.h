@@ -11,12 +11,13 @@ namespace spear_btp {
 enum Dtype : int { kBf16 = 0, kF16 = 1, kF32 = 2 };
 
 struct FwdArgs {
-  const void* coeff;
+  const void* coeff;  // 16-bit linear-space decay, or fp32 log-space gate when log_gate is set
   const void* x;
   void* y;
   float* checkpoint;  // nullptr: do not store the carry checkpoint
   int B, H, L, k;
   int in_dtype, out_dtype;
+  bool log_gate = false;
 };
 
 struct BwdArgs {
@@ -24,9 +25,10 @@ struct BwdArgs {
   const void* x;
   const void* dy;
   void* dx;
-  float* dA;
+  float* dA;  // d/d coeff, or d/d gate when log_gate is set
   int B, H, L, k;
   int in_dtype, dy_dtype;
+  bool log_gate = false;
 };
 
 // Exact-fp32 recurrence kernels (btp_scan.hip).

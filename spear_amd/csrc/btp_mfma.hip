@@ -97,7 +97,7 @@ __global__ __launch_bounds__(64 * kWaves) void btp_fwd_mfma_kernel(const uint16_
   // ---- global -> LDS
   uint4 xin[4];
   slab16_global_to_regs<kStreamIn>(xslab, L, sc.nvalid, lane, xin);
-  const uint32_t ain = coeff_global_to_reg<Bf16>(arow, sc.nvalid, lane);
+  const uint32_t ain = coeff_global_to_reg<LinCoeff<Bf16>>(arow, sc.nvalid, lane);
   const bool halo = (k == 2) && (sc.sp > 0);  // wave-uniform
   uint4 hx = zero4();
   uint32_t ha = 0u;

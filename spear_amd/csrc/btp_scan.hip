@@ -74,9 +74,9 @@ namespace {
 // ==========================================================================================
 // Forward
 // ==========================================================================================
-template <class E, class OutT, bool kCheckpoint, bool kStreamIn>
+template <class E, class C, class OutT, bool kCheckpoint, bool kStreamIn>
 __global__ __launch_bounds__(64 * kWaves) SPEAR_BTP_FWD_OCC void btp_fwd_scan_kernel(
-    const uint16_t* __restrict__ coeff, const uint16_t* __restrict__ x, OutT* __restrict__ y,
+    const typename C::elem* __restrict__ coeff, const uint16_t* __restrict__ x, OutT* __restrict__ y,
     float* __restrict__ ckpt, int L, int spans_per_row, long total_spans, int k) {
   constexpr bool kOutF32 = std::is_same<OutT, float>::value;
   constexpr int kImgBytes = kOutF32 ? 8192 : 4096;
@@ -90,7 +90,7 @@ __global__ __launch_bounds__(64 * kWaves) SPEAR_BTP_FWD_OCC void btp_fwd_scan_ke
   unsigned char* img = lds[wave];
   float* a_lds = reinterpret_cast<float*>(img + kImgBytes);
   const uint16_t* xslab = x + (sc.row * kChan) * (long)L + sc.s0;
-  const uint16_t* arow = coeff + sc.row * (long)L + sc.s0;
+  const typename C::elem* arow = coeff + sc.row * (long)L + sc.s0;
   const int j = lane >> 4, d = lane & 15;
 
   // ---- all global reads are issued before anything waits on them
@@ -99,14 +99,14 @@ __global__ __launch_bounds__(64 * kWaves) SPEAR_BTP_FWD_OCC void btp_fwd_scan_ke
   constexpr bool kStreamOut = SPEAR_BTP_STREAM_STORES == 1;
   uint4 xin[4];
   slab16_global_to_regs<kStreamIn>(xslab, L, sc.nvalid, lane, xin);
-  const uint32_t ain = coeff_global_to_reg<E>(arow, sc.nvalid, lane);
+  const typename C::pair_t ain = coeff_global_to_reg<C>(arow, sc.nvalid, lane);
 
   const bool halo = (k == 2) && (sc.sp > 0);  // wave-uniform
   float c_halo = 0.0f;
   if (halo && j == 0) {
     // local terminal state of the block just left of the span, channel d
     float ah[16], xh[16];
-    load_block_coeffs<E>(arow - kTile, ah);
+    C::load_block(arow - kTile, ah);
     const uint16_t* xp = xslab + (long)d * L - kTile;
     unpack8<E>(*reinterpret_cast<const uint4*>(xp), xh);
     unpack8<E>(*reinterpret_cast<const uint4*>(xp + 8), xh + 8);
@@ -117,7 +117,7 @@ __global__ __launch_bounds__(64 * kWaves) SPEAR_BTP_FWD_OCC void btp_fwd_scan_ke
   }
 
   slab16_regs_to_lds(img, lane, xin);
-  coeff_reg_to_lds<E>(a_lds, lane, ain);
+  coeff_reg_to_lds<C>(a_lds, lane, ain);
   wave_lds_handover();
 
   float xf[32], a[32];
@@ -184,10 +184,10 @@ __global__ __launch_bounds__(64 * kWaves) SPEAR_BTP_FWD_OCC void btp_fwd_scan_ke
 // ==========================================================================================
 // Backward
 // ==========================================================================================
-template <class E, class GradT, bool kStreamIn>
+template <class E, class C, class GradT, bool kStreamIn>
 __device__ __forceinline__ void btp_bwd_scan_body(
     unsigned char (*lds)[4096 + (std::is_same<GradT, float>::value ? 8192 : 4096) + kCoeffLdsBytes],
-    const uint16_t* __restrict__ coeff, const uint16_t* __restrict__ x, const GradT* __restrict__ dy,
+    const typename C::elem* __restrict__ coeff, const uint16_t* __restrict__ x, const GradT* __restrict__ dy,
     uint16_t* __restrict__ dx, float* __restrict__ dA, int L, int spans_per_row, long total_spans,
     int k) {
   constexpr bool kGradF32 = std::is_same<GradT, float>::value;
@@ -203,7 +203,7 @@ __device__ __forceinline__ void btp_bwd_scan_body(
   float* a_lds = reinterpret_cast<float*>(img_g + kGradBytes);
   const long slab_off = (sc.row * kChan) * (long)L + sc.s0;
   const uint16_t* xslab = x + slab_off;
-  const uint16_t* arow = coeff + sc.row * (long)L + sc.s0;
+  const typename C::elem* arow = coeff + sc.row * (long)L + sc.s0;
   const int j = lane >> 4, d = lane & 15;
 
   // ---- global reads
@@ -216,14 +216,14 @@ __device__ __forceinline__ void btp_bwd_scan_body(
   } else {
     slab16_global_to_regs<kStreamIn>(reinterpret_cast<const uint16_t*>(dy) + slab_off, L, sc.nvalid, lane, gin);
   }
-  const uint32_t ain = coeff_global_to_reg<E>(arow, sc.nvalid, lane);
+  const typename C::pair_t ain = coeff_global_to_reg<C>(arow, sc.nvalid, lane);
 
   const bool halo_left = (k == 2) && (sc.sp > 0);              // wave-uniform
   const bool halo_right = (k == 2) && (sc.s0 + kSpan < L);     // wave-uniform
   float c_halo = 0.0f, dc_halo = 0.0f;
   if (halo_left && j == 0) {
     float ah[16], xh[16];
-    load_block_coeffs<E>(arow - kTile, ah);
+    C::load_block(arow - kTile, ah);
     const uint16_t* xp = xslab + (long)d * L - kTile;
     unpack8<E>(*reinterpret_cast<const uint4*>(xp), xh);
     unpack8<E>(*reinterpret_cast<const uint4*>(xp + 8), xh + 8);
@@ -235,7 +235,7 @@ __device__ __forceinline__ void btp_bwd_scan_body(
   if (halo_right && j == 3) {
     // gradient carry sent by the block just right of the span: a_0 * A_0 of that block
     float ah[16], gh[16];
-    load_block_coeffs<E>(arow + kSpan, ah);
+    C::load_block(arow + kSpan, ah);
     if constexpr (kGradF32) {
       const float* gp = reinterpret_cast<const float*>(dy) + slab_off + (long)d * L + kSpan;
 #pragma unroll
@@ -261,7 +261,7 @@ __device__ __forceinline__ void btp_bwd_scan_body(
     uint4 g4[4] = {gin[0], gin[1], gin[2], gin[3]};
     slab16_regs_to_lds(img_g, lane, g4);
   }
-  coeff_reg_to_lds<E>(a_lds, lane, ain);
+  coeff_reg_to_lds<C>(a_lds, lane, ain);
   wave_lds_handover();
 
   // Register-lean ordering: x and dy are consumed by the two local recurrences and are dead
@@ -351,6 +351,11 @@ __device__ __forceinline__ void btp_bwd_scan_body(
   // dA leaves straight from registers: lane d of a group holds step d of its block, so every
   // group writes two 64-byte runs. (Gathering the span's 128 values in LDS first to write 512
   // contiguous bytes measured slower: the extra hand-over delays the last stores of the wave.)
+  if constexpr (C::kLog) {
+    // gradient w.r.t. the log-space gate: dg_t = a_t * dA_t (no division anywhere)
+    dA_A *= a_lds[coeff_slot(32 * j) + d];
+    dA_B *= a_lds[coeff_slot(32 * j) + 16 + d];
+  }
   float* dArow = dA + sc.row * (long)L + sc.s0 + 32 * j + d;
   if (32 * j < sc.nvalid) __builtin_nontemporal_store(dA_A, dArow);
   if (32 * j + 16 < sc.nvalid) __builtin_nontemporal_store(dA_B, dArow + 16);
@@ -362,21 +367,21 @@ __device__ __forceinline__ void btp_bwd_scan_body(
 }
 
 // 16-bit dy: the body fits 128 VGPRs, so four waves per SIMD are requested explicitly.
-template <class E, bool kStreamIn>
+template <class E, class C, bool kStreamIn>
 __global__ __launch_bounds__(64 * kWaves) SPEAR_BTP_BWD_OCC void btp_bwd_scan_kernel(
-    const uint16_t* __restrict__ coeff, const uint16_t* __restrict__ x, const uint16_t* __restrict__ dy,
+    const typename C::elem* __restrict__ coeff, const uint16_t* __restrict__ x, const uint16_t* __restrict__ dy,
     uint16_t* __restrict__ dx, float* __restrict__ dA, int L, int spans_per_row, long total_spans, int k) {
   __shared__ __align__(16) unsigned char lds[kWaves][4096 + 4096 + kCoeffLdsBytes];
-  btp_bwd_scan_body<E, uint16_t, kStreamIn>(lds, coeff, x, dy, dx, dA, L, spans_per_row, total_spans, k);
+  btp_bwd_scan_body<E, C, uint16_t, kStreamIn>(lds, coeff, x, dy, dx, dA, L, spans_per_row, total_spans, k);
 }
 
 // fp32 dy: twice the staging registers and LDS; occupancy is left to the compiler.
-template <class E, bool kStreamIn>
+template <class E, class C, bool kStreamIn>
 __global__ __launch_bounds__(64 * kWaves) void btp_bwd_scan_kernel_f32grad(
-    const uint16_t* __restrict__ coeff, const uint16_t* __restrict__ x, const float* __restrict__ dy,
+    const typename C::elem* __restrict__ coeff, const uint16_t* __restrict__ x, const float* __restrict__ dy,
     uint16_t* __restrict__ dx, float* __restrict__ dA, int L, int spans_per_row, long total_spans, int k) {
   __shared__ __align__(16) unsigned char lds[kWaves][4096 + 8192 + kCoeffLdsBytes];
-  btp_bwd_scan_body<E, float, kStreamIn>(lds, coeff, x, dy, dx, dA, L, spans_per_row, total_spans, k);
+  btp_bwd_scan_body<E, C, float, kStreamIn>(lds, coeff, x, dy, dx, dA, L, spans_per_row, total_spans, k);
 }
 
 __global__ __launch_bounds__(256) void copy_kernel(const uint4* __restrict__ src, uint4* __restrict__ dst,
@@ -386,61 +391,71 @@ __global__ __launch_bounds__(256) void copy_kernel(const uint4* __restrict__ src
     dst[i] = src[i];
 }
 
-template <class E, class OutT, bool kCheckpoint, bool kStreamIn>
+template <class E, class C, class OutT, bool kCheckpoint, bool kStreamIn>
 void launch_fwd_as(const FwdArgs& p, const Grid& g, hipStream_t s) {
-  hipLaunchKernelGGL((btp_fwd_scan_kernel<E, OutT, kCheckpoint, kStreamIn>), dim3(g.blocks), dim3(64 * kWaves), 0, s,
-                     static_cast<const uint16_t*>(p.coeff), static_cast<const uint16_t*>(p.x),
+  hipLaunchKernelGGL((btp_fwd_scan_kernel<E, C, OutT, kCheckpoint, kStreamIn>), dim3(g.blocks), dim3(64 * kWaves), 0,
+                     s, static_cast<const typename C::elem*>(p.coeff), static_cast<const uint16_t*>(p.x),
                      static_cast<OutT*>(p.y), p.checkpoint, p.L, g.spans_per_row, g.total_spans, p.k);
 }
 
-template <class E, class OutT>
+template <class E, class C, class OutT>
 hipError_t launch_fwd(const FwdArgs& p, hipStream_t s) {
   const Grid g = make_grid((long)p.B * p.H, p.L);
   const bool ck = p.checkpoint != nullptr, st = stream_inputs(g);
   if (ck) {
-    if (st) launch_fwd_as<E, OutT, true, true>(p, g, s);
-    else launch_fwd_as<E, OutT, true, false>(p, g, s);
+    if (st) launch_fwd_as<E, C, OutT, true, true>(p, g, s);
+    else launch_fwd_as<E, C, OutT, true, false>(p, g, s);
   } else {
-    if (st) launch_fwd_as<E, OutT, false, true>(p, g, s);
-    else launch_fwd_as<E, OutT, false, false>(p, g, s);
+    if (st) launch_fwd_as<E, C, OutT, false, true>(p, g, s);
+    else launch_fwd_as<E, C, OutT, false, false>(p, g, s);
   }
   return hipGetLastError();
 }
 
-template <class E, class GradT, bool kStreamIn>
+template <class E, class C, class GradT, bool kStreamIn>
 void launch_bwd_as(const BwdArgs& p, const Grid& g, hipStream_t s) {
-  const auto* c = static_cast<const uint16_t*>(p.coeff);
+  const auto* c = static_cast<const typename C::elem*>(p.coeff);
   const auto* x = static_cast<const uint16_t*>(p.x);
   auto* dx = static_cast<uint16_t*>(p.dx);
   if constexpr (std::is_same<GradT, float>::value) {
-    hipLaunchKernelGGL((btp_bwd_scan_kernel_f32grad<E, kStreamIn>), dim3(g.blocks), dim3(64 * kWaves), 0, s, c, x,
+    hipLaunchKernelGGL((btp_bwd_scan_kernel_f32grad<E, C, kStreamIn>), dim3(g.blocks), dim3(64 * kWaves), 0, s, c, x,
                        static_cast<const float*>(p.dy), dx, p.dA, p.L, g.spans_per_row, g.total_spans, p.k);
   } else {
-    hipLaunchKernelGGL((btp_bwd_scan_kernel<E, kStreamIn>), dim3(g.blocks), dim3(64 * kWaves), 0, s, c, x,
+    hipLaunchKernelGGL((btp_bwd_scan_kernel<E, C, kStreamIn>), dim3(g.blocks), dim3(64 * kWaves), 0, s, c, x,
                        static_cast<const uint16_t*>(p.dy), dx, p.dA, p.L, g.spans_per_row, g.total_spans, p.k);
   }
 }
 
-template <class E, class GradT>
+template <class E, class C, class GradT>
 hipError_t launch_bwd(const BwdArgs& p, hipStream_t s) {
   const Grid g = make_grid((long)p.B * p.H, p.L);
-  if (stream_inputs(g)) launch_bwd_as<E, GradT, true>(p, g, s);
-  else launch_bwd_as<E, GradT, false>(p, g, s);
+  if (stream_inputs(g)) launch_bwd_as<E, C, GradT, true>(p, g, s);
+  else launch_bwd_as<E, C, GradT, false>(p, g, s);
   return hipGetLastError();
+}
+
+template <class E, class C>
+hipError_t forward_by_out(const FwdArgs& p, hipStream_t s) {
+  return p.out_dtype == kF32 ? launch_fwd<E, C, float>(p, s) : launch_fwd<E, C, uint16_t>(p, s);
+}
+
+template <class E, class C>
+hipError_t backward_by_grad(const BwdArgs& p, hipStream_t s) {
+  return p.dy_dtype == kF32 ? launch_bwd<E, C, float>(p, s) : launch_bwd<E, C, uint16_t>(p, s);
 }
 
 }  // namespace
 
 hipError_t scan_forward(const FwdArgs& p, hipStream_t s) {
-  const bool bf = p.in_dtype == kBf16, f32 = p.out_dtype == kF32;
-  if (bf) return f32 ? launch_fwd<Bf16, float>(p, s) : launch_fwd<Bf16, uint16_t>(p, s);
-  return f32 ? launch_fwd<Fp16, float>(p, s) : launch_fwd<Fp16, uint16_t>(p, s);
+  if (p.in_dtype == kBf16)
+    return p.log_gate ? forward_by_out<Bf16, LogCoeff>(p, s) : forward_by_out<Bf16, LinCoeff<Bf16>>(p, s);
+  return p.log_gate ? forward_by_out<Fp16, LogCoeff>(p, s) : forward_by_out<Fp16, LinCoeff<Fp16>>(p, s);
 }
 
 hipError_t scan_backward(const BwdArgs& p, hipStream_t s) {
-  const bool bf = p.in_dtype == kBf16, f32 = p.dy_dtype == kF32;
-  if (bf) return f32 ? launch_bwd<Bf16, float>(p, s) : launch_bwd<Bf16, uint16_t>(p, s);
-  return f32 ? launch_bwd<Fp16, float>(p, s) : launch_bwd<Fp16, uint16_t>(p, s);
+  if (p.in_dtype == kBf16)
+    return p.log_gate ? backward_by_grad<Bf16, LogCoeff>(p, s) : backward_by_grad<Bf16, LinCoeff<Bf16>>(p, s);
+  return p.log_gate ? backward_by_grad<Fp16, LogCoeff>(p, s) : backward_by_grad<Fp16, LinCoeff<Fp16>>(p, s);
 }
 
 hipError_t device_copy(const void* src, void* dst, unsigned long long bytes, hipStream_t s) {

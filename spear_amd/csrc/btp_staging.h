@@ -47,17 +47,55 @@ __device__ __forceinline__ void stream_store16(void* p, const uint4& q) {
   __builtin_nontemporal_store(v, reinterpret_cast<u32x4_t*>(p));
 }
 
-// Loads the 16 coefficients of one block (32 bytes, wave-uniform address per lane group) and
-// returns them clamped, as floats.
+// ---- coefficient sources --------------------------------------------------------------------
+// LinCoeff<E>: the reference's operand, linear-space decay a_t stored as a 16-bit float of the
+//              same type as x (spear/ops/btp/interface.py:164-188, csrc/btp/_bindings.cu:29-31).
+// LogCoeff:    fp32 log-space gate g_t with a_t = exp(g_t); lets callers keep gates such as
+//              -softplus(.) at full precision (a bf16 a_t cannot represent 1 - 1e-4).
+// Both deliver clamped fp32 a_t to the kernels; nothing downstream differs.
 template <class E>
-__device__ __forceinline__ void load_block_coeffs(const uint16_t* p, float (&a)[16]) {
-  const uint4 q0 = *reinterpret_cast<const uint4*>(p);
-  const uint4 q1 = *reinterpret_cast<const uint4*>(p + 8);
-  unpack8<E>(q0, a);
-  unpack8<E>(q1, a + 8);
+struct LinCoeff {
+  typedef uint16_t elem;
+  typedef uint32_t pair_t;  // two consecutive coefficients
+  static constexpr bool kLog = false;
+  static __device__ __forceinline__ pair_t load_pair(const elem* p) {
+    return __builtin_nontemporal_load(reinterpret_cast<const uint32_t*>(p));
+  }
+  static __device__ __forceinline__ pair_t zero_pair() { return 0u; }
+  static __device__ __forceinline__ float2 to_float(pair_t w) {
+    return make_float2(clamp_coeff<E>(E::lo(w)), clamp_coeff<E>(E::hi(w)));
+  }
+  // the 16 coefficients of one block (wave-uniform address per lane group)
+  static __device__ __forceinline__ void load_block(const elem* p, float (&a)[16]) {
+    unpack8<E>(*reinterpret_cast<const uint4*>(p), a);
+    unpack8<E>(*reinterpret_cast<const uint4*>(p + 8), a + 8);
 #pragma unroll
-  for (int i = 0; i < 16; ++i) a[i] = clamp_coeff<E>(a[i]);
-}
+    for (int i = 0; i < 16; ++i) a[i] = clamp_coeff<E>(a[i]);
+  }
+};
+
+struct LogCoeff {
+  typedef float elem;
+  typedef float2 pair_t;
+  static constexpr bool kLog = true;
+  static __device__ __forceinline__ pair_t load_pair(const elem* p) {
+    const floatx2_t v = __builtin_nontemporal_load(reinterpret_cast<const floatx2_t*>(p));
+    return make_float2(v[0], v[1]);
+  }
+  static __device__ __forceinline__ pair_t zero_pair() { return make_float2(-INFINITY, -INFINITY); }
+  static __device__ __forceinline__ float decay(float g) {
+    const float a = expf(g);
+    return a > kCoeffFloor ? a : 0.0f;
+  }
+  static __device__ __forceinline__ float2 to_float(pair_t g) { return make_float2(decay(g.x), decay(g.y)); }
+  static __device__ __forceinline__ void load_block(const elem* p, float (&a)[16]) {
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      const float4 q = *reinterpret_cast<const float4*>(p + 4 * c);
+      a[4 * c + 0] = decay(q.x); a[4 * c + 1] = decay(q.y); a[4 * c + 2] = decay(q.z); a[4 * c + 3] = decay(q.w);
+    }
+  }
+};
 
 // ------------------------------------------------------------------------------------------
 // Stage a [16 x 128] slab of 16-bit elements: coalesced global reads -> swizzled LDS image.
@@ -179,9 +217,9 @@ __device__ __forceinline__ void lane_write32(unsigned char* img, int j, int d, c
 
 // Coefficients of the span: 2 per lane from global, clamped, as fp32 into LDS; every lane then
 // reads back the 32 of its own two blocks (a broadcast read for the 16 lanes of a group).
-template <class E>
-__device__ __forceinline__ uint32_t coeff_global_to_reg(const uint16_t* arow, int nvalid, int lane) {
-  return ((lane << 1) < nvalid) ? __builtin_nontemporal_load(reinterpret_cast<const uint32_t*>(arow + (lane << 1))) : 0u;
+template <class C>
+__device__ __forceinline__ typename C::pair_t coeff_global_to_reg(const typename C::elem* arow, int nvalid, int lane) {
+  return ((lane << 1) < nvalid) ? C::load_pair(arow + (lane << 1)) : C::zero_pair();
 }
 
 // The second half of the span is stored 16 floats further on, so that the four lane groups, which
@@ -191,12 +229,9 @@ constexpr int kCoeffLdsBytes = (kSpan + 16) * 4;
 
 __device__ __forceinline__ int coeff_slot(int t) { return t + ((t >> 6) << 4); }
 
-template <class E>
-__device__ __forceinline__ void coeff_reg_to_lds(float* a_lds, int lane, uint32_t w) {
-  float2 f;
-  f.x = clamp_coeff<E>(E::lo(w));
-  f.y = clamp_coeff<E>(E::hi(w));
-  *reinterpret_cast<float2*>(a_lds + coeff_slot(lane << 1)) = f;
+template <class C>
+__device__ __forceinline__ void coeff_reg_to_lds(float* a_lds, int lane, typename C::pair_t w) {
+  *reinterpret_cast<float2*>(a_lds + coeff_slot(lane << 1)) = C::to_float(w);
 }
 
 __device__ __forceinline__ void coeff_lane_read(const float* a_lds, int j, float (&a)[32]) {

@@ -1,3 +1,3 @@
-from .btp import btp
+from .btp import btp, btp_log
 
-__all__ = ["btp"]
+__all__ = ["btp", "btp_log"]

@@ -25,7 +25,7 @@ import torch.library
 
 from spear_amd import _btp
 
-__all__ = ["btp"]
+__all__ = ["btp", "btp_log"]
 
 # Fixed by the kernels (interface.py:23-27).
 DH = 16
@@ -96,9 +96,31 @@ def register_traceable_op(
     lib._register_fake(op_name, op_fake_impl)
 
 
+def _forward_log_impl(gate: torch.Tensor, x: torch.Tensor, y: torch.Tensor, k: int) -> None:
+    _btp.forward_log(gate, x, y, k)
+
+
+def _forward_log_fake(gate: torch.Tensor, x: torch.Tensor, y: torch.Tensor, k: int) -> None:
+    return None
+
+
+def _backward_log_impl(
+    gate: torch.Tensor, x: torch.Tensor, dy: torch.Tensor, dx: torch.Tensor, dgate: torch.Tensor, k: int
+) -> None:
+    _btp.backward_log(gate, x, dy, dx, dgate, k)
+
+
+def _backward_log_fake(
+    gate: torch.Tensor, x: torch.Tensor, dy: torch.Tensor, dx: torch.Tensor, dgate: torch.Tensor, k: int
+) -> None:
+    return None
+
+
 lib = torch.library.Library("spear_btp", "DEF")
 register_traceable_op(lib, "forward", _forward_impl, _forward_fake, mutates_args=["y", "checkpoint"])
 register_traceable_op(lib, "backward", _backward_impl, _backward_fake, mutates_args=["dx", "dA"])
+register_traceable_op(lib, "forward_log", _forward_log_impl, _forward_log_fake, mutates_args=["y"])
+register_traceable_op(lib, "backward_log", _backward_log_impl, _backward_log_fake, mutates_args=["dx", "dgate"])
 
 
 class _BTPFunction(torch.autograd.Function):
@@ -149,3 +171,41 @@ def btp(
     out_dtype = output_dtype or torch.float32
     wpb_val = wpb if wpb is not None else (WPB_K2_DEFAULT if k == 2 else WPB_K1_DEFAULT)
     return _BTPFunction.apply(coeff.contiguous(), x.contiguous(), k, out_dtype, wpb_val)
+
+
+class _BTPLogFunction(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, gate: torch.Tensor, x: torch.Tensor, k: int, output_dtype: torch.dtype):
+        B, H, dh_in, L = x.shape
+        assert dh_in == DH, f"Channel dimension must be {DH}"
+        assert L % BLK == 0, f"Length L must be multiple of {BLK}"
+        y = torch.empty_like(x, dtype=output_dtype)
+        torch.ops.spear_btp.forward_log(gate, x, y, int(k))
+        ctx.save_for_backward(gate, x)
+        ctx.k = int(k)
+        return y
+
+    @staticmethod
+    def backward(ctx, dy: torch.Tensor):
+        gate, x = ctx.saved_tensors
+        dx = torch.empty_like(x)
+        dgate = torch.empty_like(gate)
+        torch.ops.spear_btp.backward_log(gate, x, dy.contiguous(), dx, dgate, ctx.k)
+        return dgate, dx, None, None
+
+
+def btp_log(
+    gate: torch.Tensor,
+    x: torch.Tensor,
+    k: int = 2,
+    output_dtype: torch.dtype | None = None,
+) -> torch.Tensor:
+    """:func:`btp` for callers that hold the decay in log space: ``btp(exp(gate), x)`` with the
+    exponential taken in fp32 inside the kernel, and a gradient w.r.t. ``gate`` itself.
+
+    An addition to the reference's API (its op takes the decay already exponentiated and rounded
+    to 16 bits). ``gate``: ``[B, H, L]`` float32, ``g_t <= 0`` (e.g. ``-softplus(logit)``);
+    ``x``: ``[B, H, 16, L]`` bf16/fp16. Returns ``[B, H, 16, L]`` in ``output_dtype`` (default fp32);
+    backward yields ``dgate`` in fp32 and ``dx`` in ``x.dtype``.
+    """
+    return _BTPLogFunction.apply(gate.contiguous(), x.contiguous(), k, output_dtype or torch.float32)

@@ -20,8 +20,10 @@ def test_header_declares_the_expected_entry_points():
     assert declared_functions() == [
         "spear_btp_abi_version",
         "spear_btp_backward",
+        "spear_btp_backward_loggate",
         "spear_btp_copy",
         "spear_btp_forward",
+        "spear_btp_forward_loggate",
         "spear_btp_last_error",
     ]
 
@@ -54,7 +56,7 @@ def test_host_side_validation_needs_no_gpu():
     from spear_amd import _btp
 
     lib = _btp.load_library()
-    assert lib.spear_btp_abi_version() == 1
+    assert lib.spear_btp_abi_version() == 2
     buf = ctypes.create_string_buffer(4096)
     p = ctypes.addressof(buf)
     p -= p % 16
