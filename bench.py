@@ -98,6 +98,7 @@ def main() -> int:
     ap.add_argument("--config", choices=sorted(CONFIGS), default="c3")
     ap.add_argument("--sets", type=int, default=4, help="independent buffer sets to rotate over")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-fused", action="store_true", help="skip the fused layer-layout forward leg")
     ap.add_argument("--settle-seconds", type=float, default=0.3, help="untimed run-in before the warm-up steps")
     args = ap.parse_args()
 
@@ -205,6 +206,75 @@ def main() -> int:
         lib.spear_btp_copy(s["x"].data_ptr(), s["dx"].data_ptr(), ctypes.c_ulonglong(nbytes), sp)
     copy_ms = kernel_ms(copy)
 
+    # log-space gate entry points on the same shape (fp32 gate in, fp32 dgate out: 68 + 108 B per unit)
+    for s_ in sets:
+        s_["gate"] = torch.log(s_["coeff"].float()).contiguous()
+
+    def fwd_log(s):
+        rc = lib.spear_btp_forward_loggate(s["gate"].data_ptr(), s["x"].data_ptr(), s["y"].data_ptr(), None,
+                                           B, H, L, 2, 0, 0, 0, sp)
+        assert rc == 0, lib.spear_btp_last_error()
+
+    def bwd_log(s):
+        rc = lib.spear_btp_backward_loggate(s["gate"].data_ptr(), s["x"].data_ptr(), s["dy"].data_ptr(),
+                                            s["dx"].data_ptr(), s["dA"].data_ptr(), B, H, L, 2, 0, 0, 0, sp)
+        assert rc == 0, lib.spear_btp_last_error()
+
+    fwd_log_ms, bwd_log_ms = kernel_ms(fwd_log), kernel_ms(bwd_log)
+
+    # fused layer-layout forward (gates + recurrence + y*C+V on [B, L, features] tensors) against the
+    # same stage built from PyTorch ops around the stand-alone kernel
+    fused = None
+    if H % 4 == 0 and not args.no_fused:
+        from spear_amd.ops.btp import btp as btp_op
+
+        F = H * 16
+        g = torch.Generator(device="cpu").manual_seed(seed + 7)
+        msets = []
+        for _ in range(min(len(sets), 3)):
+            msets.append({
+                "a": torch.randn(B, L, H, generator=g).to(torch.bfloat16).to(dev),
+                "b": torch.randn(B, L, F, generator=g).to(torch.bfloat16).to(dev),
+                "c": torch.randn(B, L, F, generator=g).to(torch.bfloat16).to(dev),
+                "v": torch.randn(B, L, F, generator=g).to(torch.bfloat16).to(dev),
+                "out": torch.empty(B, L, F, device=dev, dtype=torch.bfloat16),
+            })
+
+        def mix(s):
+            rc = lib.spear_phalanx_mix_forward(s["a"].data_ptr(), s["b"].data_ptr(), s["c"].data_ptr(),
+                                               s["v"].data_ptr(), s["out"].data_ptr(), B, L, H, H, 0, 0, sp)
+            assert rc == 0, lib.spear_btp_last_error()
+
+        def mix_unfused(s):
+            with torch.no_grad():
+                A = torch.sigmoid(s["a"]).transpose(1, 2)
+                V = s["v"].transpose(1, 2).view(B, H, 16, L)
+                X = torch.sigmoid(s["b"]).transpose(1, 2).view(B, H, 16, L) * V
+                y = btp_op(A, X, 2, 32, torch.bfloat16) * s["c"].transpose(1, 2).view(B, H, 16, L) + V
+                s["out"].copy_(y.permute(0, 3, 1, 2).reshape(B, L, F))
+
+        def kernel_ms_over(fn, pool):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            for i in range(5):
+                fn(pool[i % len(pool)])
+            torch.cuda.synchronize()
+            n = max(20, args.steps // 4)
+            e0.record(stream)
+            for i in range(n):
+                fn(pool[i % len(pool)])
+            e1.record(stream)
+            torch.cuda.synchronize()
+            return e0.elapsed_time(e1) / n
+
+        mix_ms, unfused_ms = kernel_ms_over(mix, msets), kernel_ms_over(mix_unfused, msets)
+        mix_bytes = B * L * H * (2 + 3 * 32 + 32)
+        fused = {
+            "avg_launch_ms": mix_ms, "algorithmic_bytes_per_launch": mix_bytes,
+            "achieved": mix_bytes / (mix_ms * 1e-3) / 1e9, "frac": mix_bytes / (mix_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+            "same_stage_from_pytorch_ops_plus_btp_kernel_ms": unfused_ms, "speedup": unfused_ms / mix_ms,
+        }
+        del msets
+
     units = B * H * L
     tokens = B * L
     bwd_gbps = units * BWD_BYTES / (bwd_ms * 1e-3) / 1e9
@@ -246,6 +316,10 @@ def main() -> int:
         "forward_kernel_mfma_path": {"avg_launch_ms": fwd_mfma_ms,
                                      "achieved": units * FWD_BYTES / (fwd_mfma_ms * 1e-3) / 1e9,
                                      "frac": units * FWD_BYTES / (fwd_mfma_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS},
+        "log_gate_entry_points": {"forward_ms": fwd_log_ms, "backward_ms": bwd_log_ms,
+                                  "achieved": units * (68 + 108) / ((fwd_log_ms + bwd_log_ms) * 1e-3) / 1e9,
+                                  "algorithmic_bytes_per_unit": {"forward": 68, "backward": 108}},
+        "fused_layer_forward": fused,
         "fwd_plus_bwd": {"achieved": step_gbps, "frac": step_gbps / HBM_PEAK_GBPS,
                          "algorithmic_bytes_per_step": units * (FWD_BYTES + BWD_BYTES)},
         "copy_kernel": {"avg_launch_ms": copy_ms, "achieved": 2 * nbytes / (copy_ms * 1e-3) / 1e9,

@@ -83,6 +83,18 @@ int spear_btp_backward_loggate(const float* gate, const void* x, const void* dy,
                                int B, int H, int L, int k, int x_dtype, int dy_dtype, unsigned flags,
                                void* stream);
 
+/* Fused forward of the Phalanx mixing stage in the layer's own layout. No single counterpart in the
+ * reference: it stands for the chain  sigmoid / gate product (spear/nn/phalanx/swr.py:216-219),
+ * the transposing .contiguous() copies (spear/ops/btp/interface.py:186-187), the BTP forward, and
+ * `y * C + V` with the permute back (swr.py:320-323), for callers that have the projection outputs
+ * in [B, L, features] layout (time strided, features contiguous), all in `dtype` (bf16 / fp16):
+ *     a_logit [B, L, H]            b_logit, c [B, L, kv_heads * 16]        v, out [B, L, H * 16]
+ *     out = btp(sigmoid(a_logit), sigmoid(b_logit) * v) * c + v      (k = 2, fp32 arithmetic)
+ * Head h reads b / c of kv head h / (H / kv_heads). Requirements: L % 16 == 0, H % 4 == 0,
+ * H % kv_heads == 0, 16-byte aligned pointers. */
+int spear_phalanx_mix_forward(const void* a_logit, const void* b_logit, const void* c, const void* v, void* out,
+                              int B, int L, int H, int kv_heads, int dtype, unsigned flags, void* stream);
+
 /* Message for the last failing call on this thread ("" if none).  The reference prints launch
  * failures and carries on (csrc/btp/btp-forward.cu:501-520); here they are reported. */
 const char* spear_btp_last_error(void);

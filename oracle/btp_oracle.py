@@ -119,3 +119,22 @@ def windowed_bruteforce(a, x, k: int = 2) -> np.ndarray:
             decay = np.prod(a64[:, :, s + 1 : t + 1], axis=-1)  # empty product = 1
             y[:, :, :, t] += decay[:, :, None] * x64[:, :, :, s]
     return y
+
+
+def phalanx_mix_forward(a_logit, b_logit, c, v, heads: int, kv_heads: int | None = None) -> np.ndarray:
+    """float64 statement of the Phalanx mixing stage on [B, L, features] arrays
+    (spear/nn/phalanx/swr.py:196-221 for the gates, :311-323 for the recurrence, ``* C + V`` and the
+    layout): out = btp(sigmoid(a), sigmoid(b) * v) * c + v, head h using b/c of kv head
+    h // (heads // kv_heads). No intermediate rounding."""
+    kv = heads if kv_heads is None else kv_heads
+    g = heads // kv
+    a64, b64, c64, v64 = (_as_f64(t) for t in (a_logit, b_logit, c, v))
+    B, L, _ = v64.shape
+    sig = lambda z: 1.0 / (1.0 + np.exp(-z))
+    to_heads = lambda t, h: t.reshape(B, L, h, DH).transpose(0, 2, 3, 1)  # [B, h, 16, L]
+    A = sig(a64).transpose(0, 2, 1)                                        # [B, H, L]
+    G = np.repeat(sig(to_heads(b64, kv)), g, axis=1)
+    C = np.repeat(to_heads(c64, kv), g, axis=1)
+    V = to_heads(v64, heads)
+    h = forward(A, G * V, k=2)
+    return (h * C + V).transpose(0, 3, 1, 2).reshape(B, L, heads * DH)

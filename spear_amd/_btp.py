@@ -18,12 +18,12 @@ import threading
 
 import torch
 
-__all__ = ["forward", "backward", "forward_log", "backward_log", "library_path", "load_library", "FLAG_WRITE_CHECKPOINT", "FLAG_PATH_MFMA"]
+__all__ = ["forward", "backward", "forward_log", "backward_log", "mix_forward", "library_path", "load_library", "FLAG_WRITE_CHECKPOINT", "FLAG_PATH_MFMA"]
 
 _BF16, _F16, _F32 = 0, 1, 2
 FLAG_WRITE_CHECKPOINT = 0x1
 FLAG_PATH_MFMA = 0x2
-_ABI_VERSION = 2
+_ABI_VERSION = 3
 _SUPPORTED_WPB = (4, 8, 16, 32)
 
 _lock = threading.Lock()
@@ -48,6 +48,8 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.spear_btp_forward_loggate.restype = ci
     lib.spear_btp_backward_loggate.argtypes = [vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, ci, cu, vp]
     lib.spear_btp_backward_loggate.restype = ci
+    lib.spear_phalanx_mix_forward.argtypes = [vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, cu, vp]
+    lib.spear_phalanx_mix_forward.restype = ci
     lib.spear_btp_last_error.argtypes = []
     lib.spear_btp_last_error.restype = ctypes.c_char_p
     lib.spear_btp_abi_version.argtypes = []
@@ -252,6 +254,42 @@ def backward_log(
         rc = lib.spear_btp_backward_loggate(
             gate.data_ptr(), x.data_ptr(), dy.data_ptr(), dx.data_ptr(), dgate.data_ptr(), B, H, L, int(k),
             _tag(x.dtype), _tag(dy.dtype), 0, _stream_ptr(x.device),
+        )
+    if rc != 0:
+        _raise_native(lib, rc)
+
+
+def mix_forward(
+    a_logit: torch.Tensor,
+    b_logit: torch.Tensor,
+    c: torch.Tensor,
+    v: torch.Tensor,
+    out: torch.Tensor,
+    heads: int,
+    kv_heads: int,
+) -> None:
+    """``out <- btp(sigmoid(a_logit), sigmoid(b_logit) * v) * c + v`` with every operand in the
+    layer's ``[B, L, features]`` layout (see ``spear_phalanx_mix_forward`` in the C header)."""
+    _check(all(t.is_cuda for t in (a_logit, b_logit, c, v, out)), "All tensors must be CUDA.")
+    _check(v.dim() == 3, "v must be [B, L, heads * 16].")
+    B, L, F = v.shape
+    _check(F == heads * 16, "v must be [B, L, heads * 16].")
+    _check(heads % 4 == 0, "heads must be a multiple of 4.")
+    _check(kv_heads > 0 and heads % kv_heads == 0, "heads must be divisible by kv_heads.")
+    _check(v.dtype in (torch.float16, torch.bfloat16), "tensors must be float16 or bfloat16.")
+    _check(a_logit.dtype == b_logit.dtype == c.dtype == out.dtype == v.dtype, "all tensors must share one dtype.")
+    _check(L % 16 == 0, "Length L must be multiple of 16")
+    _check_layout("a_logit", a_logit, (B, L, heads))
+    _check_layout("b_logit", b_logit, (B, L, kv_heads * 16))
+    _check_layout("c", c, (B, L, kv_heads * 16))
+    _check_layout("v", v, (B, L, F))
+    _check_layout("out", out, (B, L, F))
+    _check(len({t.device for t in (a_logit, b_logit, c, v, out)}) == 1, "All tensors must be on the same device.")
+    lib = load_library()
+    with torch.cuda.device(v.device):
+        rc = lib.spear_phalanx_mix_forward(
+            a_logit.data_ptr(), b_logit.data_ptr(), c.data_ptr(), v.data_ptr(), out.data_ptr(),
+            B, L, heads, kv_heads, _tag(v.dtype), 0, _stream_ptr(v.device),
         )
     if rc != 0:
         _raise_native(lib, rc)

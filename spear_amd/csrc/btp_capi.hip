@@ -42,7 +42,7 @@ int check_common(const char* who, int B, int H, int L, int k, int in_dtype, int 
 
 extern "C" {
 
-int spear_btp_abi_version(void) { return 2; }
+int spear_btp_abi_version(void) { return 3; }
 
 const char* spear_btp_last_error(void) { return g_error; }
 
@@ -122,6 +122,29 @@ int spear_btp_backward_loggate(const float* gate, const void* x, const void* dy,
   const hipError_t err = spear_btp::scan_backward(a, static_cast<hipStream_t>(stream));
   if (err != hipSuccess)
     return fail(SPEAR_BTP_ELAUNCH, "spear_btp_backward_loggate: launch failed: %s", hipGetErrorString(err));
+  return 0;
+}
+
+int spear_phalanx_mix_forward(const void* a_logit, const void* b_logit, const void* c, const void* v, void* out, int B,
+                              int L, int H, int kv_heads, int dtype, unsigned flags, void* stream) {
+  g_error[0] = '\0';
+  const char* who = "spear_phalanx_mix_forward";
+  if (B < 0 || L < 0 || H < 0) return fail(SPEAR_BTP_EINVAL, "%s: negative dimension (B=%d L=%d H=%d)", who, B, L, H);
+  if (L % 16 != 0) return fail(SPEAR_BTP_EINVAL, "%s: Length L must be multiple of 16 (got %d)", who, L);
+  if (H % 4 != 0) return fail(SPEAR_BTP_EINVAL, "%s: heads must be a multiple of 4 (got %d)", who, H);
+  if (kv_heads <= 0 || H % kv_heads != 0)
+    return fail(SPEAR_BTP_EINVAL, "%s: heads (%d) must be divisible by kv_heads (%d)", who, H, kv_heads);
+  if (dtype != SPEAR_BTP_BF16 && dtype != SPEAR_BTP_F16)
+    return fail(SPEAR_BTP_EINVAL, "%s: tensors must be float16 or bfloat16.", who);
+  if (flags != 0) return fail(SPEAR_BTP_EINVAL, "%s: unknown flag bits 0x%x", who, flags);
+  if ((long long)B * L * H * 16ll >= (1ll << 40)) return fail(SPEAR_BTP_EINVAL, "%s: tensor too large", who);
+  if ((long long)B * H == 0 || L == 0) return 0;
+  if (!a_logit || !b_logit || !c || !v || !out) return fail(SPEAR_BTP_ENULL, "%s: NULL tensor pointer", who);
+  if (!aligned16(a_logit) || !aligned16(b_logit) || !aligned16(c) || !aligned16(v) || !aligned16(out))
+    return fail(SPEAR_BTP_EINVAL, "%s: tensor pointers must be 16-byte aligned", who);
+  spear_btp::MixArgs a{a_logit, b_logit, c, v, out, B, L, H, H / kv_heads, dtype};
+  const hipError_t err = spear_btp::fused_mix_forward(a, static_cast<hipStream_t>(stream));
+  if (err != hipSuccess) return fail(SPEAR_BTP_ELAUNCH, "%s: launch failed: %s", who, hipGetErrorString(err));
   return 0;
 }
 

@@ -38,6 +38,18 @@ hipError_t scan_backward(const BwdArgs& p, hipStream_t s);
 // bf16-MFMA tile kernels (btp_mfma.hip). bf16 inputs only; the forward one stores no checkpoint.
 hipError_t mfma_forward(const FwdArgs& p, hipStream_t s);
 
+// Fused layer-layout forward (btp_fused.hip): all operands [B, L, features], 16-bit.
+struct MixArgs {
+  const void* a_logit;  // [B, L, H]
+  const void* b_logit;  // [B, L, (H / kv_groups) * 16]
+  const void* c;        // [B, L, (H / kv_groups) * 16]
+  const void* v;        // [B, L, H * 16]
+  void* out;            // [B, L, H * 16]
+  int B, L, H, kv_groups;
+  int dtype;
+};
+hipError_t fused_mix_forward(const MixArgs& p, hipStream_t s);
+
 // Plain copy kernel used for bandwidth / counter calibration (btp_scan.hip).
 hipError_t device_copy(const void* src, void* dst, unsigned long long bytes, hipStream_t s);
 

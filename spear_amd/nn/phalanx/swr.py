@@ -14,7 +14,9 @@ initialises identical weights).
   ``"default"``           the HIP kernels through :func:`spear_amd.ops.btp.btp`
   ``"pytorch"``           the log-space PyTorch statement of the two-pass algorithm
   ``"pytorch_linspace"``  the linear-space PyTorch statement
-The choice is explicit; ``"default"`` never degrades to a PyTorch path.
+  ``"fused"``             (addition) one HIP kernel for gates + recurrence + ``* C + V`` working
+                          directly on the projection outputs; needs ``heads % 4 == 0``, ``k == 2``
+The choice is explicit; ``"default"`` and ``"fused"`` never degrade to a PyTorch path.
 """
 
 from __future__ import annotations
@@ -23,7 +25,7 @@ import torch
 import torch.nn as nn
 
 _HEAD_DIM = 16
-_METHODS = ("default", "pytorch", "pytorch_linspace")
+_METHODS = ("default", "pytorch", "pytorch_linspace", "fused")
 
 
 class KVRepeat(nn.Module):
@@ -144,6 +146,8 @@ class Phalanx(nn.Module):
                 raise ValueError(f"head_dim must be 16, got {dim // heads}. Use heads=dim//16 or leave heads=None")
         if method not in _METHODS:
             raise ValueError(f"method must be one of 'default', 'pytorch', 'pytorch_linspace', got {method}")
+        if method == "fused" and (heads % 4 != 0 or k != 2):
+            raise ValueError("method 'fused' needs heads divisible by 4 and k == 2")
 
         self.dim = dim
         self.heads = heads
@@ -166,6 +170,11 @@ class Phalanx(nn.Module):
 
             self.btp_module = btp
             self._forward_fn = self._forward_default
+        elif method == "fused":
+            from spear_amd.ops.btp import phalanx_mix
+
+            self.mix_module = phalanx_mix
+            self._forward_fn = self._forward_fused
         else:
             from spear_amd.ops.btp import reference
 
@@ -186,6 +195,12 @@ class Phalanx(nn.Module):
     def _forward_default(self, x: torch.Tensor) -> torch.Tensor:
         A, X, C, V = self.param.forward_axcv(x)
         return self._mix_and_project(self.btp_module(A, X, self.k, self.wpb, self.output_dtype), C, V)
+
+    def _forward_fused(self, x: torch.Tensor) -> torch.Tensor:
+        p = self.param
+        xc = x.to(p.compute_dtype)
+        mixed = self.mix_module(p.proj_a(xc), p.proj_b(xc), p.proj_c(xc), p.proj_v(xc), self.heads, self.kv_heads)
+        return self.proj_out(mixed)
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         return self._forward_fn(x)

@@ -1,3 +1,3 @@
-from .btp import btp, btp_log
+from .btp import btp, btp_log, phalanx_mix
 
-__all__ = ["btp", "btp_log"]
+__all__ = ["btp", "btp_log", "phalanx_mix"]

@@ -13,7 +13,7 @@ HEADER = os.path.join(ROOT, "include", "spear_btp.h")
 def declared_functions():
     text = open(HEADER).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"\b(spear_btp_\w+)\s*\(", text)))
+    return sorted(set(re.findall(r"\b(spear_(?:btp|phalanx)_\w+)\s*\(", text)))
 
 
 def test_header_declares_the_expected_entry_points():
@@ -25,6 +25,7 @@ def test_header_declares_the_expected_entry_points():
         "spear_btp_forward",
         "spear_btp_forward_loggate",
         "spear_btp_last_error",
+        "spear_phalanx_mix_forward",
     ]
 
 
@@ -56,7 +57,7 @@ def test_host_side_validation_needs_no_gpu():
     from spear_amd import _btp
 
     lib = _btp.load_library()
-    assert lib.spear_btp_abi_version() == 2
+    assert lib.spear_btp_abi_version() == 3
     buf = ctypes.create_string_buffer(4096)
     p = ctypes.addressof(buf)
     p -= p % 16
