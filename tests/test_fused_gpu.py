@@ -33,7 +33,7 @@ def run_mix(a, b, c, v, H, Hkv):
 
 @pytest.mark.parametrize("B,L,H,Hkv", [
     (1, 16, 4, 4), (2, 32, 4, 4), (2, 48, 8, 8), (1, 80, 4, 2), (3, 128, 8, 2), (2, 144, 16, 4),
-    (1, 512, 32, 32), (2, 272, 12, 3), (1, 1040, 4, 1),
+    (1, 512, 32, 32), (2, 272, 12, 3), (1, 1040, 4, 1), (1, 4096, 8, 8), (2, 2064, 16, 2),
 ])
 def test_fused_forward_matches_oracle(B, L, H, Hkv):
     a, b, c, v = make_mix_inputs(B, L, H, Hkv, seed=1000 + L + H)
