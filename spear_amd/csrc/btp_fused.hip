@@ -104,8 +104,7 @@ __global__ __launch_bounds__(64 * kWaves) void phalanx_mix_fwd_kernel(
 
   // Two register sets of one block each (16 steps x {b, c, v} words per lane): while one block is
   // being processed the next one is already in flight, so a wait only ever concerns loads that
-  // were issued a whole block earlier and never the younger stores. After the last block the
-  // look-ahead re-reads the last block (in bounds, unused).
+  // were issued a whole block earlier and never the younger stores.
   struct Words {
     uint32_t b[16], c[16], v[16];
   };
@@ -161,19 +160,23 @@ __global__ __launch_bounds__(64 * kWaves) void phalanx_mix_fwd_kernel(
 
   Words w0, w1;
   issue(w0, t_first);
-  uint32_t g0 = issue_gate(t_first), g1;
-  const int t_last = L - kTile;
+  uint32_t g0 = issue_gate(t_first), g1 = 0u;
   for (int t0 = t_first; t0 < t_end; t0 += 2 * kTile) {
     // the scheduling barriers keep the look-ahead loads in front of the arithmetic (left alone,
     // the scheduler sinks them next to their uses to save registers, which serialises the two)
-    issue(w1, min(t0 + kTile, t_last));
-    g1 = issue_gate(min(t0 + kTile, t_last));
+    const bool more1 = t0 + kTile < t_end, more2 = t0 + 2 * kTile < t_end;  // wave-uniform
+    if (more1) {
+      issue(w1, t0 + kTile);
+      g1 = issue_gate(t0 + kTile);
+    }
     __builtin_amdgcn_sched_barrier(0);
     process(w0, g0, t0);
-    if (t0 + kTile < t_end) {
+    if (more1) {
       __builtin_amdgcn_sched_barrier(0);
-      issue(w0, min(t0 + 2 * kTile, t_last));
-      g0 = issue_gate(min(t0 + 2 * kTile, t_last));
+      if (more2) {
+        issue(w0, t0 + 2 * kTile);
+        g0 = issue_gate(t0 + 2 * kTile);
+      }
       __builtin_amdgcn_sched_barrier(0);
       process(w1, g1, t0 + kTile);
     }
