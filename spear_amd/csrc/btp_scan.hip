@@ -366,7 +366,8 @@ __device__ __forceinline__ void btp_bwd_scan_body(
   slab16_lds_to_global<kStreamOut>(img_x, dx + slab_off, L, sc.nvalid, lane);
 }
 
-// 16-bit dy: the body fits 128 VGPRs, so four waves per SIMD are requested explicitly.
+// 16-bit dy and 16-bit coefficients (the reference's operands): the body fits 128 VGPRs, so four
+// waves per SIMD are requested explicitly.
 template <class E, class C, bool kStreamIn>
 __global__ __launch_bounds__(64 * kWaves) SPEAR_BTP_BWD_OCC void btp_bwd_scan_kernel(
     const typename C::elem* __restrict__ coeff, const uint16_t* __restrict__ x, const uint16_t* __restrict__ dy,
@@ -375,13 +376,15 @@ __global__ __launch_bounds__(64 * kWaves) SPEAR_BTP_BWD_OCC void btp_bwd_scan_ke
   btp_bwd_scan_body<E, C, uint16_t, kStreamIn>(lds, coeff, x, dy, dx, dA, L, spans_per_row, total_spans, k);
 }
 
-// fp32 dy: twice the staging registers and LDS; occupancy is left to the compiler.
-template <class E, class C, bool kStreamIn>
-__global__ __launch_bounds__(64 * kWaves) void btp_bwd_scan_kernel_f32grad(
-    const typename C::elem* __restrict__ coeff, const uint16_t* __restrict__ x, const float* __restrict__ dy,
+// fp32 dy (twice the staging registers and LDS) and log-space gates (an exponential per
+// coefficient): occupancy is left to the compiler.
+template <class E, class C, class GradT, bool kStreamIn>
+__global__ __launch_bounds__(64 * kWaves) void btp_bwd_scan_kernel_relaxed(
+    const typename C::elem* __restrict__ coeff, const uint16_t* __restrict__ x, const GradT* __restrict__ dy,
     uint16_t* __restrict__ dx, float* __restrict__ dA, int L, int spans_per_row, long total_spans, int k) {
-  __shared__ __align__(16) unsigned char lds[kWaves][4096 + 8192 + kCoeffLdsBytes];
-  btp_bwd_scan_body<E, C, float, kStreamIn>(lds, coeff, x, dy, dx, dA, L, spans_per_row, total_spans, k);
+  constexpr int kGradBytes = std::is_same<GradT, float>::value ? 8192 : 4096;
+  __shared__ __align__(16) unsigned char lds[kWaves][4096 + kGradBytes + kCoeffLdsBytes];
+  btp_bwd_scan_body<E, C, GradT, kStreamIn>(lds, coeff, x, dy, dx, dA, L, spans_per_row, total_spans, k);
 }
 
 __global__ __launch_bounds__(256) void copy_kernel(const uint4* __restrict__ src, uint4* __restrict__ dst,
@@ -417,9 +420,9 @@ void launch_bwd_as(const BwdArgs& p, const Grid& g, hipStream_t s) {
   const auto* c = static_cast<const typename C::elem*>(p.coeff);
   const auto* x = static_cast<const uint16_t*>(p.x);
   auto* dx = static_cast<uint16_t*>(p.dx);
-  if constexpr (std::is_same<GradT, float>::value) {
-    hipLaunchKernelGGL((btp_bwd_scan_kernel_f32grad<E, C, kStreamIn>), dim3(g.blocks), dim3(64 * kWaves), 0, s, c, x,
-                       static_cast<const float*>(p.dy), dx, p.dA, p.L, g.spans_per_row, g.total_spans, p.k);
+  if constexpr (std::is_same<GradT, float>::value || C::kLog) {
+    hipLaunchKernelGGL((btp_bwd_scan_kernel_relaxed<E, C, GradT, kStreamIn>), dim3(g.blocks), dim3(64 * kWaves), 0, s,
+                       c, x, static_cast<const GradT*>(p.dy), dx, p.dA, p.L, g.spans_per_row, g.total_spans, p.k);
   } else {
     hipLaunchKernelGGL((btp_bwd_scan_kernel<E, C, kStreamIn>), dim3(g.blocks), dim3(64 * kWaves), 0, s, c, x,
                        static_cast<const uint16_t*>(p.dy), dx, p.dA, p.L, g.spans_per_row, g.total_spans, p.k);

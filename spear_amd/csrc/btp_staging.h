@@ -84,7 +84,9 @@ struct LogCoeff {
   }
   static __device__ __forceinline__ pair_t zero_pair() { return make_float2(-INFINITY, -INFINITY); }
   static __device__ __forceinline__ float decay(float g) {
-    const float a = expf(g);
+    // exp2(g * log2 e) on the transcendental unit: relative error ~1e-6 for |g| <= 20, far inside
+    // the 1e-4 bound of the fp32 path, and cheap enough to be evaluated again in the halo code
+    const float a = __expf(g);
     return a > kCoeffFloor ? a : 0.0f;
   }
   static __device__ __forceinline__ float2 to_float(pair_t g) { return make_float2(decay(g.x), decay(g.y)); }
