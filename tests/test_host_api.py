@@ -176,3 +176,81 @@ def test_fused_gates_packing_order():
     a_logits, b_kv, c_kv, v = p._compute_base_projections(x)
     assert torch.equal(packed[:, 64:128], v) and torch.equal(packed[:, -4:], a_logits)
     assert torch.equal(packed[:, :16], b_kv[:, :16]) and torch.equal(packed[:, 16:32], b_kv[:, :16])  # heads 0,1 share kv head 0
+
+
+# ---- entry points added next to the reference API ------------------------------------------------
+
+def test_added_ops_are_registered():
+    names = {"forward_log": ["gate", "x", "y", "k"], "backward_log": ["gate", "x", "dy", "dx", "dgate", "k"],
+             "mix_forward": ["a_logits", "b_logits", "c", "v", "out", "heads", "kv_heads"]}
+    for op, args in names.items():
+        schema = getattr(torch.ops.spear_btp, op).default._schema
+        assert [a.name for a in schema.arguments] == args
+
+
+def test_log_gate_host_checks(monkeypatch):
+    from spear_amd import btp_log
+
+    gate = -torch.rand(1, 2, 32)
+    x = torch.randn(1, 2, 16, 32).bfloat16()
+    with pytest.raises(RuntimeError, match="All tensors must be CUDA"):
+        _btp.forward_log(gate, x, torch.empty(1, 2, 16, 32), 2)
+    with pytest.raises((RuntimeError, NotImplementedError)):
+        btp_log(gate, x)  # no CPU fallback
+    monkeypatch.setattr(torch.Tensor, "is_cuda", property(lambda self: True))
+    with pytest.raises(RuntimeError, match="gate must be float32"):
+        _btp.forward_log(gate.bfloat16(), x, torch.empty(1, 2, 16, 32), 2)
+    with pytest.raises(RuntimeError, match="x must be float16 or bfloat16"):
+        _btp.forward_log(gate, x.float(), torch.empty(1, 2, 16, 32), 2)
+    with pytest.raises(RuntimeError, match="gate must have shape"):
+        _btp.forward_log(gate[:, :1], x, torch.empty(1, 2, 16, 32), 2)
+    with pytest.raises(RuntimeError, match="dgate must be float32"):
+        _btp.backward_log(gate, x, x, torch.empty_like(x), torch.empty(1, 2, 32).bfloat16(), 2)
+
+
+def test_fused_mix_host_checks(monkeypatch):
+    a, b, c, v = torch.randn(1, 32, 4).bfloat16(), torch.randn(1, 32, 64).bfloat16(), torch.randn(1, 32, 64).bfloat16(), torch.randn(1, 32, 64).bfloat16()
+    out = torch.empty_like(v)
+    with pytest.raises(RuntimeError, match="All tensors must be CUDA"):
+        _btp.mix_forward(a, b, c, v, out, 4, 4)
+    monkeypatch.setattr(torch.Tensor, "is_cuda", property(lambda self: True))
+    with pytest.raises(RuntimeError, match="heads must be a multiple of 4"):
+        _btp.mix_forward(a[..., :2], b[..., :32], c[..., :32], v[..., :32], out[..., :32], 2, 2)
+    with pytest.raises(RuntimeError, match="divisible by kv_heads"):
+        _btp.mix_forward(a, b, c, v, out, 4, 3)
+    with pytest.raises(RuntimeError, match="b_logit must have shape"):
+        _btp.mix_forward(a, b, c, v, out, 4, 2)
+    with pytest.raises(RuntimeError, match="share one dtype"):
+        _btp.mix_forward(a, b.half(), c, v, out, 4, 4)
+    with pytest.raises(RuntimeError, match="multiple of 16"):
+        _btp.mix_forward(a[:, :24].contiguous(), b[:, :24].contiguous(), c[:, :24].contiguous(), v[:, :24].contiguous(), out[:, :24].contiguous(), 4, 4)
+
+
+def test_fused_method_construction_rules():
+    with pytest.raises(ValueError, match="divisible by 4"):
+        Phalanx(dim=32, method="fused", dtype=torch.bfloat16)
+    with pytest.raises(ValueError, match="k == 2"):
+        Phalanx(dim=128, method="fused", k=1, dtype=torch.bfloat16)
+    layer = Phalanx(dim=128, method="fused", dtype=torch.bfloat16, kv_heads=2)  # builds without a GPU
+    assert layer.kv_heads == 2 and layer.heads == 8
+
+
+def test_oracle_fused_composition_matches_torch_composition():
+    """The float64 composition used to check the fused kernel, against the same function written
+    with torch ops and the float64 reference recurrence."""
+    import numpy as np
+
+    from oracle import btp_oracle as orc
+    from spear_amd.ops.btp.reference import block_two_pass_ref
+
+    B, L, H, Hkv = 2, 48, 8, 2
+    g = torch.Generator().manual_seed(9)
+    a, b, c, v = (torch.randn(B, L, n, generator=g, dtype=torch.float64) for n in (H, Hkv * 16, Hkv * 16, H * 16))
+    heads = lambda t, h: t.view(B, L, h, 16).permute(0, 2, 3, 1)
+    A = torch.sigmoid(a).transpose(1, 2).contiguous()
+    G = torch.sigmoid(heads(b, Hkv)).repeat_interleave(H // Hkv, 1)
+    C = heads(c, Hkv).repeat_interleave(H // Hkv, 1)
+    V = heads(v, H)
+    want = (block_two_pass_ref(A, (G * V).contiguous()) * C + V).permute(0, 3, 1, 2).reshape(B, L, H * 16)
+    got = orc.phalanx_mix_forward(a.numpy(), b.numpy(), c.numpy(), v.numpy(), H, Hkv)
+    np.testing.assert_allclose(got, want.numpy(), rtol=1e-11, atol=1e-12)

@@ -112,6 +112,57 @@ def test_torch_compile(opts):
         _within(m, BACKWARD_LIMITS, f"compiled grad_{name}")
 
 
+def test_torch_compile_of_the_added_ops():
+    from spear_amd import btp_log, phalanx_mix
+
+    g = torch.Generator().manual_seed(3)
+    gate = (-torch.nn.functional.softplus(torch.randn(2, 4, 64, generator=g))).to(DEV)
+    x = torch.randn(2, 4, 16, 64, generator=g).bfloat16().to(DEV)
+    y_c = torch.compile(btp_log, fullgraph=True)(gate, x)
+    assert torch.equal(y_c, btp_log(gate, x))
+    a, b, c, v = (torch.randn(2, 64, n, generator=g).bfloat16().to(DEV) for n in (4, 64, 64, 64))
+    o_c = torch.compile(phalanx_mix, fullgraph=True)(a, b, c, v, 4)
+    assert torch.equal(o_c, phalanx_mix(a, b, c, v, 4))
+
+
+def test_entry_points_can_be_captured_in_a_hip_graph():
+    """The C-ABI calls allocate nothing and launch on the given stream, so they can be recorded into
+    a graph and replayed. Every replay is checked against the eager result, with eager work and
+    synchronisation between replays."""
+    from spear_amd import _btp
+
+    coeff, x, dy = make_inputs(4, 8, 256, seed=77)
+    c, xx, g = coeff.to(DEV), x.to(DEV), dy.to(DEV)
+    y = torch.empty(4, 8, 16, 256, device=DEV, dtype=torch.bfloat16)
+    dx = torch.empty_like(xx)
+    dA = torch.empty(4, 8, 256, device=DEV)
+    ck = torch.empty(4, 8, 16, 16, device=DEV)
+
+    def launch():
+        _btp.forward(c, xx, y, ck, 2, 32, flags=0)
+        _btp.backward(c, xx, g, ck, dx, dA, 2, 32)
+
+    launch()
+    torch.cuda.synchronize()
+    want = (y.clone(), dx.clone(), dA.clone())
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        launch()  # warm-up on the capture stream
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        launch()
+    for i in range(4):
+        for t in (y, dx, dA):
+            t.fill_(float("nan"))  # eager work between replays (fill kernels, not memsets in the graph)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y, want[0]) and torch.equal(dx, want[1]) and torch.equal(dA, want[2]), f"replay {i}"
+
+
 # ---- Phalanx ------------------------------------------------------------------------------------
 
 def test_config1_layer_forward_hip_vs_cpu_pytorch_path():
