@@ -138,3 +138,31 @@ def phalanx_mix_forward(a_logit, b_logit, c, v, heads: int, kv_heads: int | None
     V = to_heads(v64, heads)
     h = forward(A, G * V, k=2)
     return (h * C + V).transpose(0, 3, 1, 2).reshape(B, L, heads * DH)
+
+
+def phalanx_mix_backward(a_logit, b_logit, c, v, dout, heads: int, kv_heads: int | None = None):
+    """Reverse mode of :func:`phalanx_mix_forward` by the chain rule around the pinned BTP
+    backward: returns (da_logit, db_logit, dc, dv) in the [B, L, features] layouts of the inputs."""
+    kv = heads if kv_heads is None else kv_heads
+    g = heads // kv
+    a64, b64, c64, v64, d64 = (_as_f64(t) for t in (a_logit, b_logit, c, v, dout))
+    B, L, _ = v64.shape
+    sig = lambda z: 1.0 / (1.0 + np.exp(-z))
+    to_heads = lambda t, h: t.reshape(B, L, h, DH).transpose(0, 2, 3, 1)
+    from_heads = lambda t: t.transpose(0, 3, 1, 2).reshape(B, L, -1)
+    A = sig(a64).transpose(0, 2, 1)
+    G = np.repeat(sig(to_heads(b64, kv)), g, axis=1)
+    C = np.repeat(to_heads(c64, kv), g, axis=1)
+    V = to_heads(v64, heads)
+    dO = to_heads(d64, heads)
+    X = G * V
+    h = forward(A, X, k=2)
+    dX, dA = backward(A, X, dO * C, k=2)
+    dC = dO * h
+    dV = dO + dX * G
+    dB = dX * V * G * (1.0 - G)
+    da = (dA * A * (1.0 - A)).transpose(0, 2, 1)
+    if g > 1:
+        dC = dC.reshape(B, kv, g, DH, L).sum(2)
+        dB = dB.reshape(B, kv, g, DH, L).sum(2)
+    return da, from_heads(dB), from_heads(dC), from_heads(dV)

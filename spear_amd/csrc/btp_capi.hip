@@ -42,7 +42,7 @@ int check_common(const char* who, int B, int H, int L, int k, int in_dtype, int 
 
 extern "C" {
 
-int spear_btp_abi_version(void) { return 3; }
+int spear_btp_abi_version(void) { return 4; }
 
 const char* spear_btp_last_error(void) { return g_error; }
 
@@ -144,6 +144,30 @@ int spear_phalanx_mix_forward(const void* a_logit, const void* b_logit, const vo
     return fail(SPEAR_BTP_EINVAL, "%s: tensor pointers must be 16-byte aligned", who);
   spear_btp::MixArgs a{a_logit, b_logit, c, v, out, B, L, H, H / kv_heads, dtype};
   const hipError_t err = spear_btp::fused_mix_forward(a, static_cast<hipStream_t>(stream));
+  if (err != hipSuccess) return fail(SPEAR_BTP_ELAUNCH, "%s: launch failed: %s", who, hipGetErrorString(err));
+  return 0;
+}
+
+int spear_phalanx_mix_backward(const void* a_logit, const void* b_logit, const void* c, const void* v, const void* dout,
+                               void* da_logit, void* db_logit, void* dc, void* dv, int B, int L, int H, int dtype,
+                               unsigned flags, void* stream) {
+  g_error[0] = '\0';
+  const char* who = "spear_phalanx_mix_backward";
+  if (B < 0 || L < 0 || H < 0) return fail(SPEAR_BTP_EINVAL, "%s: negative dimension (B=%d L=%d H=%d)", who, B, L, H);
+  if (L % 16 != 0) return fail(SPEAR_BTP_EINVAL, "%s: Length L must be multiple of 16 (got %d)", who, L);
+  if (H % 4 != 0) return fail(SPEAR_BTP_EINVAL, "%s: heads must be a multiple of 4 (got %d)", who, H);
+  if (dtype != SPEAR_BTP_BF16 && dtype != SPEAR_BTP_F16)
+    return fail(SPEAR_BTP_EINVAL, "%s: tensors must be float16 or bfloat16.", who);
+  if (flags != 0) return fail(SPEAR_BTP_EINVAL, "%s: unknown flag bits 0x%x", who, flags);
+  if ((long long)B * L * H * 16ll >= (1ll << 40)) return fail(SPEAR_BTP_EINVAL, "%s: tensor too large", who);
+  if ((long long)B * H == 0 || L == 0) return 0;
+  const void* ptrs[] = {a_logit, b_logit, c, v, dout, da_logit, db_logit, dc, dv};
+  for (const void* q : ptrs) {
+    if (!q) return fail(SPEAR_BTP_ENULL, "%s: NULL tensor pointer", who);
+    if (!aligned16(q)) return fail(SPEAR_BTP_EINVAL, "%s: tensor pointers must be 16-byte aligned", who);
+  }
+  spear_btp::MixBwdArgs a{a_logit, b_logit, c, v, dout, da_logit, db_logit, dc, dv, B, L, H, dtype};
+  const hipError_t err = spear_btp::fused_mix_backward(a, static_cast<hipStream_t>(stream));
   if (err != hipSuccess) return fail(SPEAR_BTP_ELAUNCH, "%s: launch failed: %s", who, hipGetErrorString(err));
   return 0;
 }

@@ -184,6 +184,236 @@ __global__ __launch_bounds__(64 * kWaves) void phalanx_mix_fwd_kernel(
   }
 }
 
+
+// ==========================================================================================
+// Backward of the fused mixing stage, same layout and work split as the forward kernel (one
+// wavefront = 128 features of one batch row, lane = feature pair, kv_heads == heads), walking
+// through time in REVERSE block order. Inputs a_logit, b_logit, c, v, dout; outputs da_logit,
+// db_logit, dc, dv -- each big tensor is read or written exactly once.
+//
+// With A = sigmoid(a), G = sigmoid(b), x = G v, g = dout * c (the recurrence's upstream gradient),
+// per block i (local index r, fwd carry c_in = local terminal state of block i-1, gradient carry
+// dC = a_0 R_0 of block i+1):
+//   pass R (r = 15..0):  R_r = g_r + a_{r+1} R_{r+1} ;  q_r = (prod_{j=r+1..15} a_j) dC ;  dX_r = R_r + q_r
+//   pass F (r = 0..15):  vloc_r = a_r vloc_{r-1} + x_r ;  z_r = (prod_{j<r} a_j) c_in ;  h_r = vloc_r + a_r z_r
+//                        dc_r = dout_r h_r ;  dv_r = dout_r + dX_r G_r ;  db_r = dX_r v_r G_r (1 - G_r)
+//                        dA_r = sum over the head's 16 channels of  dX_r vloc_{r-1} + R_r z_r
+//                        da_r = dA_r A_r (1 - A_r)
+// R and dX run against time while vloc and z run with it, so pass R parks its 16 x 4 values per
+// lane in LDS (lane-private slots, 16 KiB per wavefront) and pass F picks them up.
+// c_in needs the block before the current one: its b, v and a are loaded one iteration early (they
+// are the next iteration's operands anyway) and a short look-ahead pass runs its zero-started
+// recurrence. A time chunk that does not end the row first runs pass R alone on the block after it
+// (one block of run-in gives the exact gradient carry, the dependency being one hop).
+// ==========================================================================================
+struct MixSet {
+  uint32_t b[16], c[16], v[16], g[16];  // g: dout words
+  uint32_t araw;
+};
+
+template <class E>
+__global__ __launch_bounds__(64 * kWaves) void phalanx_mix_bwd_kernel(
+    const uint16_t* __restrict__ a_logit, const uint16_t* __restrict__ b_logit, const uint16_t* __restrict__ c_in,
+    const uint16_t* __restrict__ v_in, const uint16_t* __restrict__ dout, uint16_t* __restrict__ da_logit,
+    uint16_t* __restrict__ db_logit, uint16_t* __restrict__ dc, uint16_t* __restrict__ dv, int L, int H,
+    int chunk_steps, int chunks, long total_waves) {
+  __shared__ __align__(16) float gate_tiles[kWaves][2][kHeadsPerWave * kGateRow];  // decay of two blocks
+  __shared__ __align__(16) float4 park[kWaves][kTile][64];                        // (R0, R1, dX0, dX1) per step, lane
+
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+  const long w = (long)blockIdx.x * kWaves + wave;
+  if (w >= total_waves) return;
+  const int octs = (H + kHeadsPerWave - 1) / kHeadsPerWave;
+  const long bc = w / octs;
+  const int ho = (int)(w - bc * octs) * kHeadsPerWave;
+  const long brow = bc / chunks;
+  const int t_begin = (int)(bc - brow * chunks) * chunk_steps;
+  const int t_end = min(L, t_begin + chunk_steps);
+
+  const int head_local = lane >> 3;
+  const bool real = ho + head_local < H;
+  const int head = real ? ho + head_local : H - 1;
+  const int d0 = (lane & 7) << 1;
+  const int F = H * kChan;
+  const int stride = 2 * F;               // bytes per time step of the [B, L, F] tensors
+  constexpr int kRsrcFlags = 0x00020000;  // raw 32-bit buffer, gfx9 encoding
+  const long big = brow * L * F, small = brow * L * H;
+  auto rsrc = [&](const uint16_t* p, long off, int bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(p + off), 0, bytes, kRsrcFlags);
+  };
+  const __amdgpu_buffer_rsrc_t rb = rsrc(b_logit, big, L * stride), rc = rsrc(c_in, big, L * stride),
+                               rv = rsrc(v_in, big, L * stride), rg = rsrc(dout, big, L * stride),
+                               rdb = rsrc(db_logit, big, L * stride), rdc = rsrc(dc, big, L * stride),
+                               rdv = rsrc(dv, big, L * stride), ra = rsrc(a_logit, small, L * H * 2),
+                               rda = rsrc(da_logit, small, L * H * 2);
+  const int f_lane = 2 * (head * kChan + d0);
+  const int o_lane = real ? f_lane : 0x7ffffff0;  // lanes without a head store nowhere
+  const int gt = lane & 15, ghead = min(ho + 2 * (lane >> 4), H - 2);
+  const int a_lane = 2 * (gt * H + ghead);
+  // da_logit: lane k of a head (k = lane % 8) ends up with steps 2k and 2k+1 of that head
+  const int da_lane = real ? 2 * ((2 * (lane & 7)) * H + head) : 0x7ffffff0;
+  constexpr int kNt = 2;
+
+  auto issue = [&](MixSet& m, int t) {
+    // b, v and the gate logits first: the look-ahead pass needs them before pass R of the next
+    // iteration needs dout and c
+    m.araw = __builtin_amdgcn_raw_buffer_load_b32(ra, a_lane, t * H * 2, 0);
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      m.b[r] = __builtin_amdgcn_raw_buffer_load_b32(rb, f_lane, (t + r) * stride, kNt);
+      m.v[r] = __builtin_amdgcn_raw_buffer_load_b32(rv, f_lane, (t + r) * stride, kNt);
+    }
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      m.g[r] = __builtin_amdgcn_raw_buffer_load_b32(rg, f_lane, (t + r) * stride, kNt);
+      m.c[r] = __builtin_amdgcn_raw_buffer_load_b32(rc, f_lane, (t + r) * stride, kNt);
+    }
+  };
+  auto write_gate_tile = [&](float* tile, uint32_t araw) {
+    tile[(2 * (lane >> 4)) * kGateRow + gt] = clamp_coeff<E>(fast_sigmoid(E::lo(araw)));
+    tile[(2 * (lane >> 4) + 1) * kGateRow + gt] = clamp_coeff<E>(fast_sigmoid(E::hi(araw)));
+  };
+  auto read_gates = [&](const float* tile, float (&a)[16]) {
+#pragma unroll
+    for (int c4 = 0; c4 < 4; ++c4) {
+      const float4 q = *reinterpret_cast<const float4*>(tile + head_local * kGateRow + 4 * c4);
+      a[4 * c4 + 0] = q.x; a[4 * c4 + 1] = q.y; a[4 * c4 + 2] = q.z; a[4 * c4 + 3] = q.w;
+    }
+  };
+
+  float dC0 = 0.0f, dC1 = 0.0f;  // gradient carry arriving from the block after the current one
+  float4* my_park = &park[wave][0][lane];
+
+  // One iteration: `cur` holds block t0 (its decay is in tile `tc`), `nxt` receives block t0 - 16.
+  auto iterate = [&](MixSet& cur, MixSet& nxt, float* tc, float* tn, int t0) {
+    const bool has_prev = t0 > 0;        // wave-uniform
+    const bool full = t0 < t_end;        // false: run-in block after the chunk, pass R only
+    if (has_prev) issue(nxt, t0 - kTile);
+    __builtin_amdgcn_sched_barrier(0);
+
+    float a[16];
+    read_gates(tc, a);
+
+    // ---- pass R
+    float R0 = 0.0f, R1 = 0.0f, q0 = dC0, q1 = dC1;
+#pragma unroll
+    for (int r = 15; r >= 0; --r) {
+      const float g0 = E::lo(cur.g[r]) * E::lo(cur.c[r]);
+      const float g1 = E::hi(cur.g[r]) * E::hi(cur.c[r]);
+      if (r < 15) {
+        R0 = fmaf(a[r + 1], R0, g0);
+        R1 = fmaf(a[r + 1], R1, g1);
+        q0 *= a[r + 1];
+        q1 *= a[r + 1];
+      } else {
+        R0 = g0;
+        R1 = g1;
+      }
+      if (full) my_park[r * 64] = make_float4(R0, R1, R0 + q0, R1 + q1);
+    }
+    dC0 = a[0] * R0;
+    dC1 = a[0] * R1;
+    if (!full) {
+      // the tile of the block before the run-in block is still needed by the next iteration
+      if (has_prev) write_gate_tile(tn, nxt.araw);
+      wave_lds_handover();
+      return;
+    }
+
+    // ---- look-ahead: terminal zero-started state of block t0 - 16 = carry into the current block
+    float cin0 = 0.0f, cin1 = 0.0f;
+    if (has_prev) {
+      write_gate_tile(tn, nxt.araw);
+      wave_lds_handover();
+      float ap[16];
+      read_gates(tn, ap);
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        cin0 = fmaf(ap[r], cin0, fast_sigmoid(E::lo(nxt.b[r])) * E::lo(nxt.v[r]));
+        cin1 = fmaf(ap[r], cin1, fast_sigmoid(E::hi(nxt.b[r])) * E::hi(nxt.v[r]));
+      }
+    } else {
+      wave_lds_handover();
+    }
+
+    // ---- pass F
+    const int o_off = (t0 >= t_begin) ? o_lane : 0x7ffffff0;
+    float e[16];
+    float vp0 = 0.0f, vp1 = 0.0f, z0 = cin0, z1 = cin1;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const float4 pk = my_park[r * 64];  // R0, R1, dX0, dX1
+      const float G0 = fast_sigmoid(E::lo(cur.b[r])), G1 = fast_sigmoid(E::hi(cur.b[r]));
+      const float v0 = E::lo(cur.v[r]), v1 = E::hi(cur.v[r]);
+      const float go0 = E::lo(cur.g[r]), go1 = E::hi(cur.g[r]);
+      e[r] = fmaf(pk.z, vp0, pk.x * z0) + fmaf(pk.w, vp1, pk.y * z1);
+      const float az0 = a[r] * z0, az1 = a[r] * z1;
+      vp0 = fmaf(a[r], vp0, G0 * v0);
+      vp1 = fmaf(a[r], vp1, G1 * v1);
+      const uint32_t wdc = E::pack2(go0 * (vp0 + az0), go1 * (vp1 + az1));
+      const uint32_t wdv = E::pack2(fmaf(pk.z, G0, go0), fmaf(pk.w, G1, go1));
+      const uint32_t wdb = E::pack2(pk.z * v0 * G0 * (1.0f - G0), pk.w * v1 * G1 * (1.0f - G1));
+      z0 = az0;
+      z1 = az1;
+      __builtin_amdgcn_raw_buffer_store_b32(wdc, rdc, o_off, (t0 + r) * stride, kNt);
+      __builtin_amdgcn_raw_buffer_store_b32(wdv, rdv, o_off, (t0 + r) * stride, kNt);
+      __builtin_amdgcn_raw_buffer_store_b32(wdb, rdb, o_off, (t0 + r) * stride, kNt);
+    }
+
+    // ---- dA: sum over the 8 lanes (16 channels) of the head, transposing: lane k keeps steps 2k, 2k+1
+    const int kk = lane & 7;
+    float f8[8], f4[4];
+    {
+      const bool hi = kk & 4;
+#pragma unroll
+      for (int t = 0; t < 8; ++t) {
+        const float keep = hi ? e[t + 8] : e[t], send = hi ? e[t] : e[t + 8];
+        f8[t] = keep + row_xor<4>(send);
+      }
+    }
+    {
+      const bool hi = kk & 2;
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        const float keep = hi ? f8[t + 4] : f8[t], send = hi ? f8[t] : f8[t + 4];
+        f4[t] = keep + row_xor<2>(send);
+      }
+    }
+    float s0, s1;
+    {
+      const bool hi = kk & 1;
+      const float k0 = hi ? f4[2] : f4[0], n0 = hi ? f4[0] : f4[2];
+      const float k1 = hi ? f4[3] : f4[1], n1 = hi ? f4[1] : f4[3];
+      s0 = k0 + row_xor<1>(n0);
+      s1 = k1 + row_xor<1>(n1);
+    }
+    const float2 aa = *reinterpret_cast<const float2*>(tc + head_local * kGateRow + 2 * kk);
+    const float da0 = s0 * aa.x * (1.0f - aa.x), da1 = s1 * aa.y * (1.0f - aa.y);
+    const int da_off = (t0 >= t_begin) ? da_lane : 0x7ffffff0;
+    const uint32_t dap = E::pack2(da0, da1);
+    __builtin_amdgcn_raw_buffer_store_b16((unsigned short)(dap & 0xffffu), rda, da_off, t0 * H * 2, 0);
+    __builtin_amdgcn_raw_buffer_store_b16((unsigned short)(dap >> 16), rda, da_off + 2 * H, t0 * H * 2, 0);
+    wave_lds_handover();  // tile `tc` and the parking slots are free for the iteration after next
+  };
+
+  // Reverse walk: start at the block after the chunk (run-in) if there is one, else at its last block.
+  const int t_start = (t_end < L) ? t_end : t_end - kTile;
+  MixSet s0, s1;
+  issue(s0, t_start);
+  float* tile0 = gate_tiles[wave][0];
+  float* tile1 = gate_tiles[wave][1];
+  __builtin_amdgcn_sched_barrier(0);
+  write_gate_tile(tile0, s0.araw);
+  wave_lds_handover();
+  // the look-ahead block before the chunk is only read, never stored: walk down to t_begin
+  for (int t0 = t_start; t0 >= t_begin; t0 -= 2 * kTile) {
+    iterate(s0, s1, tile0, tile1, t0);
+    __builtin_amdgcn_sched_barrier(0);
+    if (t0 - kTile >= t_begin) iterate(s1, s0, tile1, tile0, t0 - kTile);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+}
+
 }  // namespace
 
 hipError_t fused_mix_forward(const MixArgs& p, hipStream_t s) {
@@ -211,6 +441,32 @@ hipError_t fused_mix_forward(const MixArgs& p, hipStream_t s) {
                        static_cast<const uint16_t*>(p.a_logit), static_cast<const uint16_t*>(p.b_logit),
                        static_cast<const uint16_t*>(p.c), static_cast<const uint16_t*>(p.v),
                        static_cast<uint16_t*>(p.out), p.L, p.H, p.kv_groups, chunk_steps, (int)chunks, total);
+  }
+  return hipGetLastError();
+}
+
+hipError_t fused_mix_backward(const MixBwdArgs& p, hipStream_t s) {
+  const long per_row = (p.H + 7) / 8;
+  const int nb = p.L / kTile;
+  const char* env = getenv("SPEAR_BTP_FUSED_WAVES");
+  const long want_waves = env ? atol(env) : 1024;
+  long chunks = (want_waves + p.B * per_row - 1) / (p.B * per_row);
+  chunks = chunks < 1 ? 1 : chunks;
+  if (chunks > nb / 8) chunks = nb / 8 > 0 ? nb / 8 : 1;
+  const int chunk_blocks = (int)((nb + chunks - 1) / chunks);
+  chunks = (nb + chunk_blocks - 1) / chunk_blocks;
+  const long total = (long)p.B * chunks * per_row;
+  const unsigned blocks = (unsigned)((total + kWaves - 1) / kWaves);
+  auto u = [](const void* q) { return static_cast<const uint16_t*>(q); };
+  auto m = [](void* q) { return static_cast<uint16_t*>(q); };
+  if (p.dtype == kBf16) {
+    hipLaunchKernelGGL((phalanx_mix_bwd_kernel<Bf16>), dim3(blocks), dim3(64 * kWaves), 0, s, u(p.a_logit), u(p.b_logit),
+                       u(p.c), u(p.v), u(p.dout), m(p.da_logit), m(p.db_logit), m(p.dc), m(p.dv), p.L, p.H,
+                       chunk_blocks * kTile, (int)chunks, total);
+  } else {
+    hipLaunchKernelGGL((phalanx_mix_bwd_kernel<Fp16>), dim3(blocks), dim3(64 * kWaves), 0, s, u(p.a_logit), u(p.b_logit),
+                       u(p.c), u(p.v), u(p.dout), m(p.da_logit), m(p.db_logit), m(p.dc), m(p.dv), p.L, p.H,
+                       chunk_blocks * kTile, (int)chunks, total);
   }
   return hipGetLastError();
 }

@@ -50,6 +50,15 @@ struct MixArgs {
 };
 hipError_t fused_mix_forward(const MixArgs& p, hipStream_t s);
 
+// Fused layer-layout backward (btp_fused.hip); kv_heads == heads only.
+struct MixBwdArgs {
+  const void *a_logit, *b_logit, *c, *v, *dout;  // [B,L,H], [B,L,H*16] x 4
+  void *da_logit, *db_logit, *dc, *dv;           // same shapes as the inputs they belong to
+  int B, L, H;
+  int dtype;
+};
+hipError_t fused_mix_backward(const MixBwdArgs& p, hipStream_t s);
+
 // Plain copy kernel used for bandwidth / counter calibration (btp_scan.hip).
 hipError_t device_copy(const void* src, void* dst, unsigned long long bytes, hipStream_t s);
 

@@ -7,8 +7,10 @@ result once (no transposing copies, no intermediate tensors). It fuses what the 
 separate PyTorch ops around its BTP kernel (spear/nn/phalanx/swr.py:166-221, 311-327 and the
 ``.contiguous()`` calls of spear/ops/btp/interface.py:186-187).
 
-Backward is not fused yet: it recomputes the gates with PyTorch ops in the ``[B, H, 16, L]`` layout
-and calls the stand-alone BTP kernels, i.e. it costs what the unfused layer's backward costs.
+Backward is a second fused kernel (reverse walk through time, every operand read once, every
+gradient written once) when ``kv_heads == heads``. With shared kv heads the gradients of ``b`` and
+``c`` are sums over the heads of a group; that case recomputes the gates with PyTorch ops in the
+``[B, H, 16, L]`` layout and calls the stand-alone BTP kernels.
 """
 
 from __future__ import annotations
@@ -37,7 +39,24 @@ def _mix_forward_fake(
     return None
 
 
+def _mix_backward_impl(
+    a_logits: torch.Tensor, b_logits: torch.Tensor, c: torch.Tensor, v: torch.Tensor, dout: torch.Tensor,
+    da: torch.Tensor, db: torch.Tensor, dc: torch.Tensor, dv: torch.Tensor, heads: int,
+) -> None:
+    _btp.mix_backward(a_logits, b_logits, c, v, dout, da, db, dc, dv, heads)
+
+
+def _mix_backward_fake(
+    a_logits: torch.Tensor, b_logits: torch.Tensor, c: torch.Tensor, v: torch.Tensor, dout: torch.Tensor,
+    da: torch.Tensor, db: torch.Tensor, dc: torch.Tensor, dv: torch.Tensor, heads: int,
+) -> None:
+    return None
+
+
 register_traceable_op(lib, "mix_forward", _mix_forward_impl, _mix_forward_fake, mutates_args=["out"])
+register_traceable_op(
+    lib, "mix_backward", _mix_backward_impl, _mix_backward_fake, mutates_args=["da", "db", "dc", "dv"]
+)
 
 
 def _to_heads(t: torch.Tensor, heads: int) -> torch.Tensor:
@@ -66,6 +85,11 @@ class _PhalanxMix(torch.autograd.Function):
         a_logits, b_logits, c, v = ctx.saved_tensors
         H, Hkv = ctx.heads, ctx.kv_heads
         groups = H // Hkv
+        if groups == 1:
+            da, db, dc, dv = (torch.empty_like(t) for t in (a_logits, b_logits, c, v))
+            torch.ops.spear_btp.mix_backward(a_logits, b_logits, c, v, dout.contiguous(), da, db, dc, dv, H)
+            return da, db, dc, dv, None, None
+
         B, L, _ = v.shape
         dt = v.dtype
 

@@ -25,6 +25,7 @@ def test_header_declares_the_expected_entry_points():
         "spear_btp_forward",
         "spear_btp_forward_loggate",
         "spear_btp_last_error",
+        "spear_phalanx_mix_backward",
         "spear_phalanx_mix_forward",
     ]
 
@@ -57,7 +58,7 @@ def test_host_side_validation_needs_no_gpu():
     from spear_amd import _btp
 
     lib = _btp.load_library()
-    assert lib.spear_btp_abi_version() == 3
+    assert lib.spear_btp_abi_version() == 4
     buf = ctypes.create_string_buffer(4096)
     p = ctypes.addressof(buf)
     p -= p % 16

@@ -52,6 +52,29 @@ def test_fused_forward_fp16_and_steep_gates():
     assert_close(f64(out), ref, 4e-3, 4e-3, "out fp16")
 
 
+def run_mix_backward(a, b, c, v, dout, H):
+    from spear_amd import _btp
+
+    dev = [t.to(DEV) for t in (a, b, c, v, dout)]
+    outs = [torch.full(t.shape, float("nan"), device=DEV, dtype=t.dtype) for t in (a, b, c, v)]
+    _btp.mix_backward(*dev, *outs, H)
+    torch.cuda.synchronize()
+    return [t.cpu() for t in outs]
+
+
+@pytest.mark.parametrize("B,L,H", [(1, 16, 4), (2, 32, 4), (2, 48, 8), (1, 80, 12), (3, 128, 8), (2, 144, 16), (1, 512, 32), (1, 1040, 4), (1, 4096, 8), (2, 2064, 16)])
+def test_fused_backward_matches_oracle(B, L, H):
+    a, b, c, v = make_mix_inputs(B, L, H, H, seed=2000 + L + H)
+    dout = torch.randn(B, L, H * 16, generator=torch.Generator().manual_seed(L)).bfloat16()
+    print(f"fused bwd B={B} L={L} H={H}", flush=True)
+    da, db, dc, dv = run_mix_backward(a, b, c, v, dout, H)
+    rda, rdb, rdc, rdv = orc.phalanx_mix_backward(f64(a), f64(b), f64(c), f64(v), f64(dout), H, H)
+    assert_close(f64(dv), rdv, BF16_ATOL, BF16_RTOL, "dv")
+    assert_close(f64(dc), rdc, BF16_ATOL, BF16_RTOL, "dc")
+    assert_close(f64(db), rdb, BF16_ATOL, BF16_RTOL, "db")
+    assert_close(f64(da), rda, BF16_ATOL, BF16_RTOL, "da")
+
+
 def test_fused_op_autograd_matches_unfused_composition():
     """Gradients of phalanx_mix against autograd through the same composition built from torch ops
     and the float64 reference recurrence."""

@@ -182,7 +182,8 @@ def test_fused_gates_packing_order():
 
 def test_added_ops_are_registered():
     names = {"forward_log": ["gate", "x", "y", "k"], "backward_log": ["gate", "x", "dy", "dx", "dgate", "k"],
-             "mix_forward": ["a_logits", "b_logits", "c", "v", "out", "heads", "kv_heads"]}
+             "mix_forward": ["a_logits", "b_logits", "c", "v", "out", "heads", "kv_heads"],
+             "mix_backward": ["a_logits", "b_logits", "c", "v", "dout", "da", "db", "dc", "dv", "heads"]}
     for op, args in names.items():
         schema = getattr(torch.ops.spear_btp, op).default._schema
         assert [a.name for a in schema.arguments] == args
@@ -254,3 +255,24 @@ def test_oracle_fused_composition_matches_torch_composition():
     want = (block_two_pass_ref(A, (G * V).contiguous()) * C + V).permute(0, 3, 1, 2).reshape(B, L, H * 16)
     got = orc.phalanx_mix_forward(a.numpy(), b.numpy(), c.numpy(), v.numpy(), H, Hkv)
     np.testing.assert_allclose(got, want.numpy(), rtol=1e-11, atol=1e-12)
+
+
+def test_oracle_fused_backward_matches_torch_autograd():
+    import numpy as np
+
+    from oracle import btp_oracle as orc
+    from spear_amd.ops.btp.reference import block_two_pass_ref
+
+    B, L, H, Hkv = 2, 48, 8, 2
+    g = torch.Generator().manual_seed(9)
+    a, b, c, v = (torch.randn(B, L, n, generator=g, dtype=torch.float64, requires_grad=True) for n in (H, Hkv * 16, Hkv * 16, H * 16))
+    dout = torch.randn(B, L, H * 16, generator=g, dtype=torch.float64)
+    heads = lambda t, h: t.view(B, L, h, 16).permute(0, 2, 3, 1)
+    A = torch.sigmoid(a).transpose(1, 2).contiguous()
+    G = torch.sigmoid(heads(b, Hkv)).repeat_interleave(H // Hkv, 1)
+    C = heads(c, Hkv).repeat_interleave(H // Hkv, 1)
+    out = (block_two_pass_ref(A, (G * heads(v, H)).contiguous()) * C + heads(v, H)).permute(0, 3, 1, 2).reshape(B, L, H * 16)
+    out.backward(dout)
+    got = orc.phalanx_mix_backward(*(t.detach().numpy() for t in (a, b, c, v)), dout.numpy(), H, Hkv)
+    for name, gg, t in zip("abcv", got, (a, b, c, v)):
+        np.testing.assert_allclose(gg, t.grad.numpy(), rtol=1e-10, atol=1e-12, err_msg=f"d{name}")
