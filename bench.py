@@ -244,6 +244,11 @@ def main() -> int:
                 "c": torch.randn(B, L, F, generator=g).to(torch.bfloat16).to(dev),
                 "v": torch.randn(B, L, F, generator=g).to(torch.bfloat16).to(dev),
                 "out": torch.empty(B, L, F, device=dev, dtype=torch.bfloat16),
+                "dout": torch.randn(B, L, F, generator=g).to(torch.bfloat16).to(dev),
+                "da": torch.empty(B, L, H, device=dev, dtype=torch.bfloat16),
+                "db": torch.empty(B, L, F, device=dev, dtype=torch.bfloat16),
+                "dc": torch.empty(B, L, F, device=dev, dtype=torch.bfloat16),
+                "dv": torch.empty(B, L, F, device=dev, dtype=torch.bfloat16),
             })
 
         def mix(s):
@@ -251,13 +256,27 @@ def main() -> int:
                                                s["v"].data_ptr(), s["out"].data_ptr(), B, L, H, H, 0, 0, sp)
             assert rc == 0, lib.spear_btp_last_error()
 
+        def mix_bwd(s):
+            rc = lib.spear_phalanx_mix_backward(s["a"].data_ptr(), s["b"].data_ptr(), s["c"].data_ptr(),
+                                                s["v"].data_ptr(), s["dout"].data_ptr(), s["da"].data_ptr(),
+                                                s["db"].data_ptr(), s["dc"].data_ptr(), s["dv"].data_ptr(),
+                                                B, L, H, 0, 0, sp)
+            assert rc == 0, lib.spear_btp_last_error()
+
+        def unfused_stage(a, b, c, v):  # what the layer does around the stand-alone kernel (swr.py)
+            A = torch.sigmoid(a).transpose(1, 2)
+            V = v.transpose(1, 2).view(B, H, 16, L)
+            X = torch.sigmoid(b).transpose(1, 2).view(B, H, 16, L) * V
+            y = btp_op(A, X, 2, 32, torch.bfloat16) * c.transpose(1, 2).view(B, H, 16, L) + V
+            return y.permute(0, 3, 1, 2).reshape(B, L, F)
+
         def mix_unfused(s):
             with torch.no_grad():
-                A = torch.sigmoid(s["a"]).transpose(1, 2)
-                V = s["v"].transpose(1, 2).view(B, H, 16, L)
-                X = torch.sigmoid(s["b"]).transpose(1, 2).view(B, H, 16, L) * V
-                y = btp_op(A, X, 2, 32, torch.bfloat16) * s["c"].transpose(1, 2).view(B, H, 16, L) + V
-                s["out"].copy_(y.permute(0, 3, 1, 2).reshape(B, L, F))
+                s["out"].copy_(unfused_stage(s["a"], s["b"], s["c"], s["v"]))
+
+        def mix_unfused_train(s):  # forward + backward through autograd
+            leaves = [s[k].detach().requires_grad_(True) for k in ("a", "b", "c", "v")]
+            unfused_stage(*leaves).backward(s["dout"])
 
         def kernel_ms_over(fn, pool):
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -273,11 +292,21 @@ def main() -> int:
             return e0.elapsed_time(e1) / n
 
         mix_ms, unfused_ms = kernel_ms_over(mix, msets), kernel_ms_over(mix_unfused, msets)
-        mix_bytes = B * L * H * (2 + 3 * 32 + 32)
+        mix_bwd_ms, unfused_train_ms = kernel_ms_over(mix_bwd, msets), kernel_ms_over(mix_unfused_train, msets)
+        mix_bytes = B * L * H * (2 + 3 * 32 + 32)          # a, b, c, v read; out written
+        mix_bwd_bytes = B * L * H * (2 + 4 * 32 + 2 + 3 * 32)  # a, b, c, v, dout read; da, db, dc, dv written
         fused = {
             "avg_launch_ms": mix_ms, "algorithmic_bytes_per_launch": mix_bytes,
             "achieved": mix_bytes / (mix_ms * 1e-3) / 1e9, "frac": mix_bytes / (mix_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
             "same_stage_from_pytorch_ops_plus_btp_kernel_ms": unfused_ms, "speedup": unfused_ms / mix_ms,
+            "backward": {
+                "avg_launch_ms": mix_bwd_ms, "algorithmic_bytes_per_launch": mix_bwd_bytes,
+                "achieved": mix_bwd_bytes / (mix_bwd_ms * 1e-3) / 1e9,
+                "frac": mix_bwd_bytes / (mix_bwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+            },
+            "fwd_plus_bwd_ms": mix_ms + mix_bwd_ms,
+            "same_stage_fwd_plus_bwd_from_pytorch_ops_plus_btp_kernels_ms": unfused_train_ms,
+            "train_speedup": unfused_train_ms / (mix_ms + mix_bwd_ms),
         }
         del msets
 
@@ -325,7 +354,7 @@ def main() -> int:
         "log_gate_entry_points": {"forward_ms": fwd_log_ms, "backward_ms": bwd_log_ms,
                                   "achieved": units * (68 + 108) / ((fwd_log_ms + bwd_log_ms) * 1e-3) / 1e9,
                                   "algorithmic_bytes_per_unit": {"forward": 68, "backward": 108}},
-        "fused_layer_forward": fused,
+        "fused_layer_stage": fused,
         "fwd_plus_bwd": {"achieved": step_gbps, "frac": step_gbps / HBM_PEAK_GBPS,
                          "algorithmic_bytes_per_step": units * (FWD_BYTES + BWD_BYTES)},
         "copy_kernel": {"avg_launch_ms": copy_ms, "achieved": 2 * nbytes / (copy_ms * 1e-3) / 1e9,
