@@ -111,7 +111,7 @@ def main() -> int:
     if args.gpus != 1:
         print(
             "bench.py: this build measures one GPU only (the op shards over batch and heads with no "
-            "communication; see DESIGN.md). Run with --gpus 1.",
+            "communication, so N GPUs run N independent copies of the same kernel). Run with --gpus 1.",
             file=sys.stderr,
         )
         return 2
