@@ -17,7 +17,10 @@ namespace spear_btp {
 constexpr int kTile = 16;   // time steps per block (reference: BL / BLK)
 constexpr int kChan = 16;   // channels per head   (reference: DH)
 constexpr int kSpan = 128;  // time steps one wavefront owns per pass: 8 blocks, 256 B per bf16 row
-constexpr int kWaves = 4;   // wavefronts per workgroup; each works on its own span, no barriers
+#ifndef SPEAR_BTP_WAVES_PER_WG
+#define SPEAR_BTP_WAVES_PER_WG 4
+#endif
+constexpr int kWaves = SPEAR_BTP_WAVES_PER_WG;  // wavefronts per workgroup; each works on its own span, no barriers
 
 // Coefficients at or below this are treated as exactly zero, as in the reference kernels
 // (csrc/btp/btp-forward.cu:179, csrc/btp/btp-backwards.cu:280-286); this also maps negative

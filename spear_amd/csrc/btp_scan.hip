@@ -83,7 +83,7 @@ __global__ __launch_bounds__(64 * kWaves) SPEAR_BTP_FWD_OCC void btp_fwd_scan_ke
   __shared__ __align__(16) unsigned char lds[kWaves][kImgBytes + kCoeffLdsBytes];
 
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const long span = (long)blockIdx.x * kWaves + wave;
+  const long span = first_span_of_workgroup() + wave;
   if (span >= total_spans) return;  // wave-uniform; no workgroup barrier is used anywhere
   const SpanCoord sc = span_coord(span, spans_per_row, L);
 
@@ -194,7 +194,7 @@ __device__ __forceinline__ void btp_bwd_scan_body(
   constexpr int kGradBytes = kGradF32 ? 8192 : 4096;
 
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const long span = (long)blockIdx.x * kWaves + wave;
+  const long span = first_span_of_workgroup() + wave;
   if (span >= total_spans) return;
   const SpanCoord sc = span_coord(span, spans_per_row, L);
 

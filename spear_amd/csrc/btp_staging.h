@@ -260,6 +260,22 @@ __device__ __forceinline__ SpanCoord span_coord(long span, int spans_per_row, in
   return c;
 }
 
+// Workgroup index -> first span. Workgroups are dealt round-robin to the 8 XCDs; with
+// SPEAR_BTP_XCD_REMAP each XCD instead walks one contiguous eighth of the tensor.
+#ifndef SPEAR_BTP_XCD_REMAP
+#define SPEAR_BTP_XCD_REMAP 0
+#endif
+__device__ __forceinline__ long first_span_of_workgroup() {
+#if SPEAR_BTP_XCD_REMAP
+  const unsigned n = gridDim.x, b = blockIdx.x;
+  const unsigned per = n >> 3;
+  const unsigned mapped = (b < (per << 3)) ? (b & 7u) * per + (b >> 3) : b;
+  return (long)mapped * kWaves;
+#else
+  return (long)blockIdx.x * kWaves;
+#endif
+}
+
 struct Grid {
   int spans_per_row;
   long total_spans;
