@@ -260,7 +260,7 @@ def main() -> int:
             rc = lib.spear_phalanx_mix_backward(s["a"].data_ptr(), s["b"].data_ptr(), s["c"].data_ptr(),
                                                 s["v"].data_ptr(), s["dout"].data_ptr(), s["da"].data_ptr(),
                                                 s["db"].data_ptr(), s["dc"].data_ptr(), s["dv"].data_ptr(),
-                                                B, L, H, 0, 0, sp)
+                                                B, L, H, H, 0, 0, sp)
             assert rc == 0, lib.spear_btp_last_error()
 
         def unfused_stage(a, b, c, v):  # what the layer does around the stand-alone kernel (swr.py)

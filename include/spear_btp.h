@@ -95,13 +95,15 @@ int spear_btp_backward_loggate(const float* gate, const void* x, const void* dy,
 int spear_phalanx_mix_forward(const void* a_logit, const void* b_logit, const void* c, const void* v, void* out,
                               int B, int L, int H, int kv_heads, int dtype, unsigned flags, void* stream);
 
-/* Backward of spear_phalanx_mix_forward for kv_heads == H: reads a_logit, b_logit, c, v and the
- * upstream gradient dout [B, L, H * 16]; writes da_logit [B, L, H] and db_logit, dc, dv
- * [B, L, H * 16] (every element, no accumulation), all in `dtype`. It stands for the autograd
- * chain through the ops listed at spear_phalanx_mix_forward; no single counterpart in the reference. */
+/* Backward of spear_phalanx_mix_forward: reads a_logit, b_logit, c, v and the upstream gradient
+ * dout [B, L, H * 16]; writes da_logit [B, L, H], db_logit and dc [B, L, kv_heads * 16] (summed over
+ * the heads sharing a kv head) and dv [B, L, H * 16] -- every element, no accumulation, all in
+ * `dtype`. H / kv_heads must be 1, 2, 4 or 8 (a head group has to sit inside one wavefront's 8
+ * heads). It stands for the autograd chain through the ops listed at spear_phalanx_mix_forward; no
+ * single counterpart in the reference. */
 int spear_phalanx_mix_backward(const void* a_logit, const void* b_logit, const void* c, const void* v,
                                const void* dout, void* da_logit, void* db_logit, void* dc, void* dv, int B, int L,
-                               int H, int dtype, unsigned flags, void* stream);
+                               int H, int kv_heads, int dtype, unsigned flags, void* stream);
 
 /* Message for the last failing call on this thread ("" if none).  The reference prints launch
  * failures and carries on (csrc/btp/btp-forward.cu:501-520); here they are reported. */

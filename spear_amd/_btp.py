@@ -23,7 +23,7 @@ __all__ = ["forward", "backward", "forward_log", "backward_log", "mix_forward", 
 _BF16, _F16, _F32 = 0, 1, 2
 FLAG_WRITE_CHECKPOINT = 0x1
 FLAG_PATH_MFMA = 0x2
-_ABI_VERSION = 4
+_ABI_VERSION = 5
 _SUPPORTED_WPB = (4, 8, 16, 32)
 
 _lock = threading.Lock()
@@ -50,7 +50,7 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.spear_btp_backward_loggate.restype = ci
     lib.spear_phalanx_mix_forward.argtypes = [vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, cu, vp]
     lib.spear_phalanx_mix_forward.restype = ci
-    lib.spear_phalanx_mix_backward.argtypes = [vp] * 9 + [ci, ci, ci, ci, cu, vp]
+    lib.spear_phalanx_mix_backward.argtypes = [vp] * 9 + [ci, ci, ci, ci, ci, cu, vp]
     lib.spear_phalanx_mix_backward.restype = ci
     lib.spear_btp_last_error.argtypes = []
     lib.spear_btp_last_error.restype = ctypes.c_char_p
@@ -308,8 +308,9 @@ def mix_backward(
     dc: torch.Tensor,
     dv: torch.Tensor,
     heads: int,
+    kv_heads: int,
 ) -> None:
-    """Gradients of :func:`mix_forward` for ``kv_heads == heads``, written in place
+    """Gradients of :func:`mix_forward`, written in place; ``heads // kv_heads`` must be 1, 2, 4 or 8
     (see ``spear_phalanx_mix_backward`` in the C header)."""
     tensors = (a_logit, b_logit, c, v, dout, da_logit, db_logit, dc, dv)
     _check(all(t.is_cuda for t in tensors), "All tensors must be CUDA.")
@@ -317,13 +318,16 @@ def mix_backward(
     B, L, F = v.shape
     _check(F == heads * 16, "v must be [B, L, heads * 16].")
     _check(heads % 4 == 0, "heads must be a multiple of 4.")
+    _check(kv_heads > 0 and heads % kv_heads == 0, "heads must be divisible by kv_heads.")
+    _check(heads // kv_heads in (1, 2, 4, 8), "heads / kv_heads must be 1, 2, 4 or 8.")
     _check(v.dtype in (torch.float16, torch.bfloat16), "tensors must be float16 or bfloat16.")
     _check(all(t.dtype == v.dtype for t in tensors), "all tensors must share one dtype.")
     _check(L % 16 == 0, "Length L must be multiple of 16")
+    Fkv = kv_heads * 16
     for name, t, shape in (
         ("a_logit", a_logit, (B, L, heads)), ("da_logit", da_logit, (B, L, heads)),
-        ("b_logit", b_logit, (B, L, F)), ("c", c, (B, L, F)), ("v", v, (B, L, F)), ("dout", dout, (B, L, F)),
-        ("db_logit", db_logit, (B, L, F)), ("dc", dc, (B, L, F)), ("dv", dv, (B, L, F)),
+        ("b_logit", b_logit, (B, L, Fkv)), ("c", c, (B, L, Fkv)), ("v", v, (B, L, F)), ("dout", dout, (B, L, F)),
+        ("db_logit", db_logit, (B, L, Fkv)), ("dc", dc, (B, L, Fkv)), ("dv", dv, (B, L, F)),
     ):
         _check_layout(name, t, shape)
     _check(len({t.device for t in tensors}) == 1, "All tensors must be on the same device.")
@@ -332,7 +336,7 @@ def mix_backward(
         rc = lib.spear_phalanx_mix_backward(
             a_logit.data_ptr(), b_logit.data_ptr(), c.data_ptr(), v.data_ptr(), dout.data_ptr(),
             da_logit.data_ptr(), db_logit.data_ptr(), dc.data_ptr(), dv.data_ptr(),
-            B, L, heads, _tag(v.dtype), 0, _stream_ptr(v.device),
+            B, L, heads, kv_heads, _tag(v.dtype), 0, _stream_ptr(v.device),
         )
     if rc != 0:
         _raise_native(lib, rc)

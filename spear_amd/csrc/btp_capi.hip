@@ -42,7 +42,7 @@ int check_common(const char* who, int B, int H, int L, int k, int in_dtype, int 
 
 extern "C" {
 
-int spear_btp_abi_version(void) { return 4; }
+int spear_btp_abi_version(void) { return 5; }
 
 const char* spear_btp_last_error(void) { return g_error; }
 
@@ -149,13 +149,20 @@ int spear_phalanx_mix_forward(const void* a_logit, const void* b_logit, const vo
 }
 
 int spear_phalanx_mix_backward(const void* a_logit, const void* b_logit, const void* c, const void* v, const void* dout,
-                               void* da_logit, void* db_logit, void* dc, void* dv, int B, int L, int H, int dtype,
-                               unsigned flags, void* stream) {
+                               void* da_logit, void* db_logit, void* dc, void* dv, int B, int L, int H, int kv_heads,
+                               int dtype, unsigned flags, void* stream) {
   g_error[0] = '\0';
   const char* who = "spear_phalanx_mix_backward";
   if (B < 0 || L < 0 || H < 0) return fail(SPEAR_BTP_EINVAL, "%s: negative dimension (B=%d L=%d H=%d)", who, B, L, H);
   if (L % 16 != 0) return fail(SPEAR_BTP_EINVAL, "%s: Length L must be multiple of 16 (got %d)", who, L);
   if (H % 4 != 0) return fail(SPEAR_BTP_EINVAL, "%s: heads must be a multiple of 4 (got %d)", who, H);
+  if (kv_heads <= 0 || H % kv_heads != 0)
+    return fail(SPEAR_BTP_EINVAL, "%s: heads (%d) must be divisible by kv_heads (%d)", who, H, kv_heads);
+  const int groups = H / kv_heads;
+  if (groups != 1 && groups != 2 && groups != 4 && groups != 8)
+    return fail(SPEAR_BTP_EINVAL, "%s: heads / kv_heads must be 1, 2, 4 or 8 (got %d)", who, groups);
+  if (groups == 8 && H % 8 != 0)
+    return fail(SPEAR_BTP_EINVAL, "%s: groups of 8 heads need heads divisible by 8 (got %d)", who, H);
   if (dtype != SPEAR_BTP_BF16 && dtype != SPEAR_BTP_F16)
     return fail(SPEAR_BTP_EINVAL, "%s: tensors must be float16 or bfloat16.", who);
   if (flags != 0) return fail(SPEAR_BTP_EINVAL, "%s: unknown flag bits 0x%x", who, flags);
@@ -166,7 +173,7 @@ int spear_phalanx_mix_backward(const void* a_logit, const void* b_logit, const v
     if (!q) return fail(SPEAR_BTP_ENULL, "%s: NULL tensor pointer", who);
     if (!aligned16(q)) return fail(SPEAR_BTP_EINVAL, "%s: tensor pointers must be 16-byte aligned", who);
   }
-  spear_btp::MixBwdArgs a{a_logit, b_logit, c, v, dout, da_logit, db_logit, dc, dv, B, L, H, dtype};
+  spear_btp::MixBwdArgs a{a_logit, b_logit, c, v, dout, da_logit, db_logit, dc, dv, B, L, H, groups, dtype};
   const hipError_t err = spear_btp::fused_mix_backward(a, static_cast<hipStream_t>(stream));
   if (err != hipSuccess) return fail(SPEAR_BTP_ELAUNCH, "%s: launch failed: %s", who, hipGetErrorString(err));
   return 0;

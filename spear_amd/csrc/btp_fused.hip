@@ -38,6 +38,11 @@ namespace spear_btp {
 
 namespace {
 
+// Value of `v` held by lane ^ mask (any mask; goes through the LDS crossbar, no memory access).
+__device__ __forceinline__ float lane_xor(float v, int lane, int mask) {
+  return __int_as_float(__builtin_amdgcn_ds_bpermute((lane ^ mask) << 2, __float_as_int(v)));
+}
+
 __device__ __forceinline__ float fast_sigmoid(float z) {
   return __builtin_amdgcn_rcpf(1.0f + __expf(-z));
 }
@@ -187,7 +192,8 @@ __global__ __launch_bounds__(64 * kWaves) void phalanx_mix_fwd_kernel(
 
 // ==========================================================================================
 // Backward of the fused mixing stage, same layout and work split as the forward kernel (one
-// wavefront = 128 features of one batch row, lane = feature pair, kv_heads == heads), walking
+// wavefront = 128 features of one batch row, lane = feature pair; kv head groups of 1, 2, 4 or 8
+// heads), walking
 // through time in REVERSE block order. Inputs a_logit, b_logit, c, v, dout; outputs da_logit,
 // db_logit, dc, dv -- each big tensor is read or written exactly once.
 //
@@ -216,7 +222,7 @@ __global__ __launch_bounds__(64 * kWaves) void phalanx_mix_bwd_kernel(
     const uint16_t* __restrict__ a_logit, const uint16_t* __restrict__ b_logit, const uint16_t* __restrict__ c_in,
     const uint16_t* __restrict__ v_in, const uint16_t* __restrict__ dout, uint16_t* __restrict__ da_logit,
     uint16_t* __restrict__ db_logit, uint16_t* __restrict__ dc, uint16_t* __restrict__ dv, int L, int H,
-    int chunk_steps, int chunks, long total_waves) {
+    int kv_groups, int chunk_steps, int chunks, long total_waves) {
   __shared__ __align__(16) float gate_tiles[kWaves][2][kHeadsPerWave * kGateRow];  // decay of two blocks
   __shared__ __align__(16) float4 park[kWaves][kTile][64];                        // (R0, R1, dX0, dX1) per step, lane
 
@@ -234,20 +240,24 @@ __global__ __launch_bounds__(64 * kWaves) void phalanx_mix_bwd_kernel(
   const bool real = ho + head_local < H;
   const int head = real ? ho + head_local : H - 1;
   const int d0 = (lane & 7) << 1;
-  const int F = H * kChan;
-  const int stride = 2 * F;               // bytes per time step of the [B, L, F] tensors
-  constexpr int kRsrcFlags = 0x00020000;  // raw 32-bit buffer, gfx9 encoding
-  const long big = brow * L * F, small = brow * L * H;
+  const int F = H * kChan, Fkv = (H / kv_groups) * kChan;
+  const int stride = 2 * F, kv_stride = 2 * Fkv;  // bytes per time step of the [B, L, F] / [B, L, Fkv] tensors
+  constexpr int kRsrcFlags = 0x00020000;          // raw 32-bit buffer, gfx9 encoding
+  const long big = brow * L * F, kvbig = brow * L * Fkv, small = brow * L * H;
   auto rsrc = [&](const uint16_t* p, long off, int bytes) {
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(p + off), 0, bytes, kRsrcFlags);
   };
-  const __amdgpu_buffer_rsrc_t rb = rsrc(b_logit, big, L * stride), rc = rsrc(c_in, big, L * stride),
+  const __amdgpu_buffer_rsrc_t rb = rsrc(b_logit, kvbig, L * kv_stride), rc = rsrc(c_in, kvbig, L * kv_stride),
                                rv = rsrc(v_in, big, L * stride), rg = rsrc(dout, big, L * stride),
-                               rdb = rsrc(db_logit, big, L * stride), rdc = rsrc(dc, big, L * stride),
+                               rdb = rsrc(db_logit, kvbig, L * kv_stride), rdc = rsrc(dc, kvbig, L * kv_stride),
                                rdv = rsrc(dv, big, L * stride), ra = rsrc(a_logit, small, L * H * 2),
                                rda = rsrc(da_logit, small, L * H * 2);
   const int f_lane = 2 * (head * kChan + d0);
+  const int kv_lane = 2 * ((head / kv_groups) * kChan + d0);
   const int o_lane = real ? f_lane : 0x7ffffff0;  // lanes without a head store nowhere
+  // With shared kv heads (kv_groups = 2, 4 or 8 consecutive heads, all inside this wavefront) the
+  // gradients of b and c are summed over the group's lanes and stored by its first head only.
+  const int okv_lane = (real && (head % kv_groups) == 0) ? kv_lane : 0x7ffffff0;
   const int gt = lane & 15, ghead = min(ho + 2 * (lane >> 4), H - 2);
   const int a_lane = 2 * (gt * H + ghead);
   // da_logit: lane k of a head (k = lane % 8) ends up with steps 2k and 2k+1 of that head
@@ -260,13 +270,13 @@ __global__ __launch_bounds__(64 * kWaves) void phalanx_mix_bwd_kernel(
     m.araw = __builtin_amdgcn_raw_buffer_load_b32(ra, a_lane, t * H * 2, 0);
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
-      m.b[r] = __builtin_amdgcn_raw_buffer_load_b32(rb, f_lane, (t + r) * stride, kNt);
+      m.b[r] = __builtin_amdgcn_raw_buffer_load_b32(rb, kv_lane, (t + r) * kv_stride, kNt);
       m.v[r] = __builtin_amdgcn_raw_buffer_load_b32(rv, f_lane, (t + r) * stride, kNt);
     }
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
       m.g[r] = __builtin_amdgcn_raw_buffer_load_b32(rg, f_lane, (t + r) * stride, kNt);
-      m.c[r] = __builtin_amdgcn_raw_buffer_load_b32(rc, f_lane, (t + r) * stride, kNt);
+      m.c[r] = __builtin_amdgcn_raw_buffer_load_b32(rc, kv_lane, (t + r) * kv_stride, kNt);
     }
   };
   auto write_gate_tile = [&](float* tile, uint32_t araw) {
@@ -338,6 +348,7 @@ __global__ __launch_bounds__(64 * kWaves) void phalanx_mix_bwd_kernel(
 
     // ---- pass F
     const int o_off = (t0 >= t_begin) ? o_lane : 0x7ffffff0;
+    const int okv_off = (t0 >= t_begin) ? okv_lane : 0x7ffffff0;
     float e[16];
     float vp0 = 0.0f, vp1 = 0.0f, z0 = cin0, z1 = cin1;
 #pragma unroll
@@ -350,14 +361,27 @@ __global__ __launch_bounds__(64 * kWaves) void phalanx_mix_bwd_kernel(
       const float az0 = a[r] * z0, az1 = a[r] * z1;
       vp0 = fmaf(a[r], vp0, G0 * v0);
       vp1 = fmaf(a[r], vp1, G1 * v1);
-      const uint32_t wdc = E::pack2(go0 * (vp0 + az0), go1 * (vp1 + az1));
+      float dc0 = go0 * (vp0 + az0), dc1 = go1 * (vp1 + az1);
+      float db0 = pk.z * v0 * G0 * (1.0f - G0), db1 = pk.w * v1 * G1 * (1.0f - G1);
+      if (kv_groups > 1) {  // wave-uniform: sum over the heads that share this kv head
+        dc0 += row_xor<8>(dc0); dc1 += row_xor<8>(dc1); db0 += row_xor<8>(db0); db1 += row_xor<8>(db1);
+        if (kv_groups > 2) {
+          dc0 += lane_xor(dc0, lane, 16); dc1 += lane_xor(dc1, lane, 16);
+          db0 += lane_xor(db0, lane, 16); db1 += lane_xor(db1, lane, 16);
+        }
+        if (kv_groups > 4) {
+          dc0 += lane_xor(dc0, lane, 32); dc1 += lane_xor(dc1, lane, 32);
+          db0 += lane_xor(db0, lane, 32); db1 += lane_xor(db1, lane, 32);
+        }
+      }
+      const uint32_t wdc = E::pack2(dc0, dc1);
       const uint32_t wdv = E::pack2(fmaf(pk.z, G0, go0), fmaf(pk.w, G1, go1));
-      const uint32_t wdb = E::pack2(pk.z * v0 * G0 * (1.0f - G0), pk.w * v1 * G1 * (1.0f - G1));
+      const uint32_t wdb = E::pack2(db0, db1);
       z0 = az0;
       z1 = az1;
-      __builtin_amdgcn_raw_buffer_store_b32(wdc, rdc, o_off, (t0 + r) * stride, kNt);
+      __builtin_amdgcn_raw_buffer_store_b32(wdc, rdc, okv_off, (t0 + r) * kv_stride, kNt);
       __builtin_amdgcn_raw_buffer_store_b32(wdv, rdv, o_off, (t0 + r) * stride, kNt);
-      __builtin_amdgcn_raw_buffer_store_b32(wdb, rdb, o_off, (t0 + r) * stride, kNt);
+      __builtin_amdgcn_raw_buffer_store_b32(wdb, rdb, okv_off, (t0 + r) * kv_stride, kNt);
     }
 
     // ---- dA: sum over the 8 lanes (16 channels) of the head, transposing: lane k keeps steps 2k, 2k+1
@@ -462,11 +486,11 @@ hipError_t fused_mix_backward(const MixBwdArgs& p, hipStream_t s) {
   if (p.dtype == kBf16) {
     hipLaunchKernelGGL((phalanx_mix_bwd_kernel<Bf16>), dim3(blocks), dim3(64 * kWaves), 0, s, u(p.a_logit), u(p.b_logit),
                        u(p.c), u(p.v), u(p.dout), m(p.da_logit), m(p.db_logit), m(p.dc), m(p.dv), p.L, p.H,
-                       chunk_blocks * kTile, (int)chunks, total);
+                       p.kv_groups, chunk_blocks * kTile, (int)chunks, total);
   } else {
     hipLaunchKernelGGL((phalanx_mix_bwd_kernel<Fp16>), dim3(blocks), dim3(64 * kWaves), 0, s, u(p.a_logit), u(p.b_logit),
                        u(p.c), u(p.v), u(p.dout), m(p.da_logit), m(p.db_logit), m(p.dc), m(p.dv), p.L, p.H,
-                       chunk_blocks * kTile, (int)chunks, total);
+                       p.kv_groups, chunk_blocks * kTile, (int)chunks, total);
   }
   return hipGetLastError();
 }

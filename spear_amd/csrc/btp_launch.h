@@ -50,11 +50,11 @@ struct MixArgs {
 };
 hipError_t fused_mix_forward(const MixArgs& p, hipStream_t s);
 
-// Fused layer-layout backward (btp_fused.hip); kv_heads == heads only.
+// Fused layer-layout backward (btp_fused.hip); kv_groups = H / kv_heads must be 1, 2, 4 or 8.
 struct MixBwdArgs {
-  const void *a_logit, *b_logit, *c, *v, *dout;  // [B,L,H], [B,L,H*16] x 4
+  const void *a_logit, *b_logit, *c, *v, *dout;  // [B,L,H], [B,L,Hkv*16] x 2, [B,L,H*16] x 2
   void *da_logit, *db_logit, *dc, *dv;           // same shapes as the inputs they belong to
-  int B, L, H;
+  int B, L, H, kv_groups;
   int dtype;
 };
 hipError_t fused_mix_backward(const MixBwdArgs& p, hipStream_t s);

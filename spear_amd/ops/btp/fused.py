@@ -8,9 +8,10 @@ separate PyTorch ops around its BTP kernel (spear/nn/phalanx/swr.py:166-221, 311
 ``.contiguous()`` calls of spear/ops/btp/interface.py:186-187).
 
 Backward is a second fused kernel (reverse walk through time, every operand read once, every
-gradient written once) when ``kv_heads == heads``. With shared kv heads the gradients of ``b`` and
-``c`` are sums over the heads of a group; that case recomputes the gates with PyTorch ops in the
-``[B, H, 16, L]`` layout and calls the stand-alone BTP kernels.
+gradient written once), including the sum of the ``b`` / ``c`` gradients over the heads that share
+a kv head when a group has 2, 4 or 8 heads. Larger groups span several wavefronts; that case
+recomputes the gates with PyTorch ops in the ``[B, H, 16, L]`` layout and calls the stand-alone
+BTP kernels.
 """
 
 from __future__ import annotations
@@ -41,14 +42,14 @@ def _mix_forward_fake(
 
 def _mix_backward_impl(
     a_logits: torch.Tensor, b_logits: torch.Tensor, c: torch.Tensor, v: torch.Tensor, dout: torch.Tensor,
-    da: torch.Tensor, db: torch.Tensor, dc: torch.Tensor, dv: torch.Tensor, heads: int,
+    da: torch.Tensor, db: torch.Tensor, dc: torch.Tensor, dv: torch.Tensor, heads: int, kv_heads: int,
 ) -> None:
-    _btp.mix_backward(a_logits, b_logits, c, v, dout, da, db, dc, dv, heads)
+    _btp.mix_backward(a_logits, b_logits, c, v, dout, da, db, dc, dv, heads, kv_heads)
 
 
 def _mix_backward_fake(
     a_logits: torch.Tensor, b_logits: torch.Tensor, c: torch.Tensor, v: torch.Tensor, dout: torch.Tensor,
-    da: torch.Tensor, db: torch.Tensor, dc: torch.Tensor, dv: torch.Tensor, heads: int,
+    da: torch.Tensor, db: torch.Tensor, dc: torch.Tensor, dv: torch.Tensor, heads: int, kv_heads: int,
 ) -> None:
     return None
 
@@ -85,9 +86,9 @@ class _PhalanxMix(torch.autograd.Function):
         a_logits, b_logits, c, v = ctx.saved_tensors
         H, Hkv = ctx.heads, ctx.kv_heads
         groups = H // Hkv
-        if groups == 1:
+        if groups in (1, 2, 4, 8) and (groups < 8 or H % 8 == 0):
             da, db, dc, dv = (torch.empty_like(t) for t in (a_logits, b_logits, c, v))
-            torch.ops.spear_btp.mix_backward(a_logits, b_logits, c, v, dout.contiguous(), da, db, dc, dv, H)
+            torch.ops.spear_btp.mix_backward(a_logits, b_logits, c, v, dout.contiguous(), da, db, dc, dv, H, Hkv)
             return da, db, dc, dv, None, None
 
         B, L, _ = v.shape

@@ -58,7 +58,7 @@ def test_host_side_validation_needs_no_gpu():
     from spear_amd import _btp
 
     lib = _btp.load_library()
-    assert lib.spear_btp_abi_version() == 4
+    assert lib.spear_btp_abi_version() == 5
     buf = ctypes.create_string_buffer(4096)
     p = ctypes.addressof(buf)
     p -= p % 16

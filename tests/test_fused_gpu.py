@@ -52,12 +52,12 @@ def test_fused_forward_fp16_and_steep_gates():
     assert_close(f64(out), ref, 4e-3, 4e-3, "out fp16")
 
 
-def run_mix_backward(a, b, c, v, dout, H):
+def run_mix_backward(a, b, c, v, dout, H, Hkv=None):
     from spear_amd import _btp
 
     dev = [t.to(DEV) for t in (a, b, c, v, dout)]
     outs = [torch.full(t.shape, float("nan"), device=DEV, dtype=t.dtype) for t in (a, b, c, v)]
-    _btp.mix_backward(*dev, *outs, H)
+    _btp.mix_backward(*dev, *outs, H, H if Hkv is None else Hkv)
     torch.cuda.synchronize()
     return [t.cpu() for t in outs]
 
@@ -75,13 +75,38 @@ def test_fused_backward_matches_oracle(B, L, H):
     assert_close(f64(da), rda, BF16_ATOL, BF16_RTOL, "da")
 
 
-def test_fused_op_autograd_matches_unfused_composition():
+@pytest.mark.parametrize("B,L,H,Hkv", [(2, 48, 8, 4), (1, 80, 12, 3), (2, 144, 16, 2), (1, 272, 32, 8), (2, 64, 4, 2), (1, 2064, 8, 1)])
+def test_fused_backward_with_shared_kv_heads(B, L, H, Hkv):
+    a, b, c, v = make_mix_inputs(B, L, H, Hkv, seed=3000 + L + H)
+    dout = torch.randn(B, L, H * 16, generator=torch.Generator().manual_seed(L + 1)).bfloat16()
+    print(f"fused bwd kv B={B} L={L} H={H} Hkv={Hkv}", flush=True)
+    da, db, dc, dv = run_mix_backward(a, b, c, v, dout, H, Hkv)
+    rda, rdb, rdc, rdv = orc.phalanx_mix_backward(f64(a), f64(b), f64(c), f64(v), f64(dout), H, Hkv)
+    assert_close(f64(dv), rdv, BF16_ATOL, BF16_RTOL, "dv")
+    # sums over up to 8 heads: magnitudes grow, the relative term carries the tolerance
+    assert_close(f64(dc), rdc, 3e-2, BF16_RTOL, "dc")
+    assert_close(f64(db), rdb, 3e-2, BF16_RTOL, "db")
+    assert_close(f64(da), rda, BF16_ATOL, BF16_RTOL, "da")
+
+
+def test_fused_backward_rejects_groups_it_cannot_reduce():
+    from spear_amd import _btp
+
+    a, b, c, v = make_mix_inputs(1, 32, 16, 1, seed=1)
+    dev = [t.to(DEV) for t in (a, b, c, v, v)]
+    outs = [torch.empty_like(t, device=DEV) for t in (a, b, c, v)]
+    with pytest.raises(RuntimeError, match="1, 2, 4 or 8"):
+        _btp.mix_backward(*dev, *outs, 16, 1)
+
+
+@pytest.mark.parametrize("H,Hkv", [(8, 4), (16, 1)])  # fused backward; group of 16 -> stand-alone kernels
+def test_fused_op_autograd_matches_unfused_composition(H, Hkv):
     """Gradients of phalanx_mix against autograd through the same composition built from torch ops
     and the float64 reference recurrence."""
     from spear_amd import phalanx_mix
     from spear_amd.ops.btp.reference import block_two_pass_ref
 
-    B, L, H, Hkv = 2, 64, 8, 4
+    B, L = 2, 64
     a, b, c, v = make_mix_inputs(B, L, H, Hkv, seed=21)
     dout = torch.randn(B, L, H * 16, generator=torch.Generator().manual_seed(22)).bfloat16()
 
@@ -104,7 +129,7 @@ def test_fused_op_autograd_matches_unfused_composition():
     assert_close(f64(out), ref_out.detach().numpy(), BF16_ATOL, BF16_RTOL, "out")
     for name, got, want in zip("abcv", leaves, ref_leaves):
         # gradients land in bf16 leaves; sums over 16 channels / kv groups reach magnitudes ~10
-        assert_close(f64(got.grad), want.grad.numpy(), 5e-2, 3e-2, f"d{name}")
+        assert_close(f64(got.grad), want.grad.numpy(), 5e-2 * max(1, H // Hkv // 4), 3e-2, f"d{name}")
 
 
 def test_phalanx_fused_method_matches_default_and_pytorch():

@@ -183,7 +183,7 @@ def test_fused_gates_packing_order():
 def test_added_ops_are_registered():
     names = {"forward_log": ["gate", "x", "y", "k"], "backward_log": ["gate", "x", "dy", "dx", "dgate", "k"],
              "mix_forward": ["a_logits", "b_logits", "c", "v", "out", "heads", "kv_heads"],
-             "mix_backward": ["a_logits", "b_logits", "c", "v", "dout", "da", "db", "dc", "dv", "heads"]}
+             "mix_backward": ["a_logits", "b_logits", "c", "v", "dout", "da", "db", "dc", "dv", "heads", "kv_heads"]}
     for op, args in names.items():
         schema = getattr(torch.ops.spear_btp, op).default._schema
         assert [a.name for a in schema.arguments] == args
