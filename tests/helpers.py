@@ -51,3 +51,16 @@ def assert_close(got, ref, atol, rtol, what=""):
         f"{what}: max |err|={err.max():.3e}; worst excess at flat index {worst}: "
         f"got {got.flat[worst]:.6g} ref {ref.flat[worst]:.6g} bound {bound.flat[worst]:.3e}"
     )
+
+
+def golden_vectors():
+    """The committed closed-form vectors (tests/golden/make_vectors.py): {case: {name: array}} with the
+    inputs as [1, H, ...] bfloat16-exact float32 arrays and y / dx / dA per k in float64."""
+    import pathlib
+
+    blob = np.load(pathlib.Path(__file__).with_name("golden") / "btp_window_vectors.npz")
+    out: dict = {}
+    for key in blob.files:
+        case, rest = key.split(".", 1)
+        out.setdefault(case, {})[rest] = blob[key][None]  # add the batch axis
+    return out

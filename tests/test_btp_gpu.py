@@ -204,3 +204,22 @@ def test_empty_batch_is_a_noop():
     ck = torch.empty(0, 4, 4, 16, device=DEV, dtype=torch.float32)
     _btp.forward(coeff, x, y, ck, 2, 32)
     torch.cuda.synchronize()
+
+
+# ---- committed closed-form vectors (tests/golden) ------------------------------------------------
+@pytest.mark.parametrize("k", [2, 1])
+@pytest.mark.parametrize("case", ["smooth", "edges", "one_block"])
+def test_kernels_match_committed_closed_form_vectors(case, k):
+    from helpers import golden_vectors
+
+    v = golden_vectors()[case]
+    coeff, x, dy = (torch.from_numpy(v[n]).bfloat16() for n in ("coeff", "x", "dy"))
+    for n, t in (("coeff", coeff), ("x", x), ("dy", dy)):
+        assert np.array_equal(f64(t), v[n].astype(np.float64)), f"{n} is not bfloat16-exact"
+    print(f"golden {case} k={k}", flush=True)
+    assert_close(f64(run_forward(coeff, x, k=k)), v[f"k{k}.y"], BF16_ATOL, BF16_RTOL, "y bf16")
+    assert_close(f64(run_forward(coeff, x, k=k, out_dtype=torch.float32)), v[f"k{k}.y"], F32_ATOL, F32_RTOL, "y fp32")
+    dx, dA = run_backward(coeff, x, dy, k=k)
+    assert_close(f64(dx), v[f"k{k}.dx"], BF16_ATOL, BF16_RTOL, "dx")
+    assert_close(f64(dA), v[f"k{k}.dA"], BF16_ATOL, BF16_RTOL, "dA")
+    assert_close(f64(run_forward(coeff, x, k=k, mfma=True)), v[f"k{k}.y"], BF16_ATOL, BF16_RTOL, "y mfma")

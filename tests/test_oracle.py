@@ -175,3 +175,19 @@ def test_rejects_bad_arguments():
     a, x = rand_case(1, 1, 32)
     with pytest.raises(ValueError):
         orc.forward(a, x, k=3)
+
+
+# ---- committed closed-form vectors -------------------------------------------------------------
+@pytest.mark.parametrize("k", [1, 2])
+@pytest.mark.parametrize("case", ["smooth", "edges", "one_block"])
+def test_oracle_reproduces_committed_closed_form_vectors(case, k):
+    from helpers import golden_vectors
+
+    v = golden_vectors()[case]
+    a, x, dy = (v[n].astype(np.float64) for n in ("coeff", "x", "dy"))
+    for mode in (orc.L_PRODUCT, orc.L_LOGSUM, orc.L_CUMPROD):
+        np.testing.assert_allclose(orc.forward(a, x, k=k, l_mode=mode), v[f"k{k}.y"], rtol=1e-11, atol=1e-12)
+    np.testing.assert_allclose(orc.forward_sequential(a, x, k=k), v[f"k{k}.y"], rtol=1e-11, atol=1e-12)
+    dx, dA = orc.backward(a, x, dy, k=k)
+    np.testing.assert_allclose(dx, v[f"k{k}.dx"], rtol=1e-11, atol=1e-12)
+    np.testing.assert_allclose(dA, v[f"k{k}.dA"], rtol=1e-10, atol=1e-11)

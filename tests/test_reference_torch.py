@@ -77,3 +77,19 @@ def test_bf16_cpu_path_stays_within_the_reference_forward_limits():
     want = torch.from_numpy(orc.forward(a.double().numpy(), x.double().numpy()))
     m = compute_error_metrics(got, want)
     assert m["max_abs"] <= 6e-2 and m["rmse"] <= 1.2e-2 and m["mean_abs"] <= 4e-3
+
+
+@pytest.mark.parametrize("fn", [ref.block_two_pass_ref, ref.block_two_pass_linspace, ref.block_two_pass_log])
+@pytest.mark.parametrize("case", ["smooth", "one_block"])
+def test_torch_port_matches_committed_closed_form_vectors(fn, case):
+    from helpers import golden_vectors
+
+    v = golden_vectors()[case]
+    a, x, dy = (torch.from_numpy(v[n].astype(np.float64)) for n in ("coeff", "x", "dy"))
+    a.requires_grad_(True)
+    x.requires_grad_(True)
+    y = fn(a, x, 16)
+    y.backward(dy)
+    np.testing.assert_allclose(y.detach().numpy(), v["k2.y"], rtol=1e-10, atol=1e-11)
+    np.testing.assert_allclose(x.grad.numpy(), v["k2.dx"], rtol=1e-10, atol=1e-11)
+    np.testing.assert_allclose(a.grad.numpy(), v["k2.dA"], rtol=1e-8, atol=1e-9)
