@@ -105,6 +105,44 @@ int spear_phalanx_mix_backward(const void* a_logit, const void* b_logit, const v
                                const void* dout, void* da_logit, void* db_logit, void* dc, void* dv, int B, int L,
                                int H, int kv_heads, int dtype, unsigned flags, void* stream);
 
+/* ---- streaming form: prompt prefill with state hand-over, and the one-token decode step --------
+ * They replace the PyTorch loops of spear/nn/phalanx/inference.py. Tensors are dense, row-major:
+ *     a         [B, H, L]      a_dtype (x_dtype or fp32)   a_t, or log(a_t) with SPEAR_JAGGED_LOG_A
+ *     x, c, v   [B, H, D, L]   x_dtype (bf16 / fp16 / fp32)
+ *     y         [B, H, D, L]   x_dtype
+ *     h, c_prev [B, H, D]      state_dtype (x_dtype or fp32)
+ *     r         [B, H]         r_dtype (any of the three)
+ * Arithmetic is fp32 whatever the storage types. */
+#define SPEAR_JAGGED_LOG_A 0x4u /* a / a_t hold log(a_t)                                         */
+#define SPEAR_JAGGED_LOG_R 0x8u /* step: the r buffers hold log(r)                               */
+
+/* Replaces parallel_jagged (spear/nn/phalanx/inference.py:281-360) and, with c = v = NULL and no state
+ * pointers, jagged_band_infer_sequential (inference.py:36-92; `carry_init`, [B, H, D] in state_dtype or
+ * NULL, is the carry into the first block):
+ *     y_t = (h_loc_t + r_t * c_prev) * c_t + v_t      h_loc, r: block-local scan and gate product
+ * and writes the state after step L-1 as the reference assembles it (inference.py:327-357): h_tail the
+ * block-local state, r_tail the in-block gate product (1 when L ends a block), c_prev_tail the terminal
+ * local state of the last completed block. The three state pointers are given together or all NULL.
+ * Any L >= 0, D > 0, block_len > 0. 16-bit tensors with D = 16, block_len = 16, L % 8 == 0, 16-byte
+ * aligned pointers and either a in x_dtype (linear) or fp32 log(a_t) run the tiled kernel (HBM-bound);
+ * everything else runs an element-granular kernel. */
+int spear_jagged_prefill(const void* a, const void* x, const void* c, const void* v, const void* carry_init, void* y,
+                         void* h_tail, void* r_tail, void* c_prev_tail, int B, int H, int D, int L, int block_len,
+                         int a_dtype, int x_dtype, int state_dtype, int r_dtype, unsigned flags, void* stream);
+
+/* Replaces step_jagged (spear/nn/phalanx/inference.py:178-278) and, with c_t = v_t = NULL,
+ * JaggedBandState.step (inference.py:121-140). One token for every (batch, head):
+ *     h = a_t * h_in + x_t;   r = a_t * r_in   (or exp(r_in + log max(a_t, tiny)) with SPEAR_JAGGED_LOG_R)
+ *     y_t = (h + r * c_prev_in) * c_t + v_t
+ * `boundary` != 0 says this token completes a block: then c_prev_out = h, h_out = 0, r_out = 1 (log: 0);
+ * otherwise h_out = h, r_out = r (log: log r) and c_prev_out is not written (may be NULL). a_t [B, H] in
+ * a_dtype; x_t, c_t, v_t, y_t [B, H, D] in x_dtype. Each output state buffer may be the same memory as
+ * its input (in-place update); calls on one state must not overlap. */
+int spear_jagged_step(const void* a_t, const void* x_t, const void* c_t, const void* v_t, void* y_t, const void* h_in,
+                      const void* r_in, const void* c_prev_in, void* h_out, void* r_out, void* c_prev_out, int B, int H,
+                      int D, int boundary, int a_dtype, int x_dtype, int state_dtype, int r_dtype, unsigned flags,
+                      float tiny, void* stream);
+
 /* Message for the last failing call on this thread ("" if none).  The reference prints launch
  * failures and carries on (csrc/btp/btp-forward.cu:501-520); here they are reported. */
 const char* spear_btp_last_error(void);

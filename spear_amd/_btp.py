@@ -18,12 +18,14 @@ import threading
 
 import torch
 
-__all__ = ["forward", "backward", "forward_log", "backward_log", "mix_forward", "mix_backward", "library_path", "load_library", "FLAG_WRITE_CHECKPOINT", "FLAG_PATH_MFMA"]
+__all__ = ["forward", "backward", "forward_log", "backward_log", "mix_forward", "mix_backward", "jagged_prefill", "jagged_step", "library_path", "load_library", "FLAG_WRITE_CHECKPOINT", "FLAG_PATH_MFMA", "FLAG_JAGGED_LOG_A", "FLAG_JAGGED_LOG_R"]
 
 _BF16, _F16, _F32 = 0, 1, 2
 FLAG_WRITE_CHECKPOINT = 0x1
 FLAG_PATH_MFMA = 0x2
-_ABI_VERSION = 5
+FLAG_JAGGED_LOG_A = 0x4
+FLAG_JAGGED_LOG_R = 0x8
+_ABI_VERSION = 6
 _SUPPORTED_WPB = (4, 8, 16, 32)
 
 _lock = threading.Lock()
@@ -52,6 +54,10 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.spear_phalanx_mix_forward.restype = ci
     lib.spear_phalanx_mix_backward.argtypes = [vp] * 9 + [ci, ci, ci, ci, ci, cu, vp]
     lib.spear_phalanx_mix_backward.restype = ci
+    lib.spear_jagged_prefill.argtypes = [vp] * 9 + [ci] * 9 + [cu, vp]
+    lib.spear_jagged_prefill.restype = ci
+    lib.spear_jagged_step.argtypes = [vp] * 11 + [ci] * 8 + [cu, ctypes.c_float, vp]
+    lib.spear_jagged_step.restype = ci
     lib.spear_btp_last_error.argtypes = []
     lib.spear_btp_last_error.restype = ctypes.c_char_p
     lib.spear_btp_abi_version.argtypes = []
@@ -337,6 +343,124 @@ def mix_backward(
             a_logit.data_ptr(), b_logit.data_ptr(), c.data_ptr(), v.data_ptr(), dout.data_ptr(),
             da_logit.data_ptr(), db_logit.data_ptr(), dc.data_ptr(), dv.data_ptr(),
             B, L, heads, kv_heads, _tag(v.dtype), 0, _stream_ptr(v.device),
+        )
+    if rc != 0:
+        _raise_native(lib, rc)
+
+
+def _ptr(t: torch.Tensor | None):
+    return None if t is None else t.data_ptr()
+
+
+def jagged_prefill(
+    a: torch.Tensor,
+    x: torch.Tensor,
+    c: torch.Tensor | None,
+    v: torch.Tensor | None,
+    carry_init: torch.Tensor | None,
+    y: torch.Tensor,
+    h_tail: torch.Tensor | None,
+    r_tail: torch.Tensor | None,
+    c_prev_tail: torch.Tensor | None,
+    block_len: int,
+    log_a: bool,
+) -> None:
+    """``y <- (block-local scan of (a, x) + one-hop carry) * c + v`` on ``[B, H, D, L]`` tensors and, if
+    the three state tensors are given, the state after the last step (see ``spear_jagged_prefill`` in
+    the C header). Everything is written in place; nothing is allocated."""
+    given = [t for t in (a, x, c, v, carry_init, y, h_tail, r_tail, c_prev_tail) if t is not None]
+    _check(all(t.is_cuda for t in given), "All tensors must be CUDA.")
+    _check(len({t.device for t in given}) == 1, "All tensors must be on the same device.")
+    _check(x.dim() == 4, "x must be [B, H, D, L].")
+    B, H, D, L = x.shape
+    _check(_tag(x.dtype) >= 0, "x must be float32, float16 or bfloat16.")
+    _check(a.dtype == x.dtype or a.dtype == torch.float32, "a must be float32 or match x dtype.")
+    _check((c is None) == (v is None), "c and v must be given together.")
+    _check(block_len > 0, "block_len must be positive.")
+    _check_layout("a", a, (B, H, L))
+    _check_layout("x", x, (B, H, D, L))
+    _check_layout("y", y, (B, H, D, L))
+    _check(y.dtype == x.dtype, "y dtype must match x.")
+    for name, t in (("c", c), ("v", v)):
+        if t is not None:
+            _check_layout(name, t, (B, H, D, L))
+            _check(t.dtype == x.dtype, f"{name} dtype must match x.")
+    state = (h_tail, r_tail, c_prev_tail)
+    _check(all(t is None for t in state) or all(t is not None for t in state), "state tensors must be given together.")
+    state_dtype = x.dtype
+    if h_tail is not None:
+        _check_layout("h_tail", h_tail, (B, H, D))
+        _check_layout("c_prev_tail", c_prev_tail, (B, H, D))
+        _check_layout("r_tail", r_tail, (B, H))
+        _check(h_tail.dtype == c_prev_tail.dtype, "h_tail and c_prev_tail must share a dtype.")
+        _check(h_tail.dtype in (x.dtype, torch.float32), "the state must be float32 or match x dtype.")
+        _check(_tag(r_tail.dtype) >= 0, "r_tail must be float32, float16 or bfloat16.")
+        state_dtype = h_tail.dtype
+    if carry_init is not None:
+        _check_layout("carry_init", carry_init, (B, H, D))
+        _check(h_tail is None or carry_init.dtype == state_dtype, "carry_init must have the state's dtype.")
+        _check(carry_init.dtype in (x.dtype, torch.float32), "carry_init must be float32 or match x dtype.")
+        state_dtype = carry_init.dtype
+    lib = load_library()
+    with torch.cuda.device(x.device):
+        rc = lib.spear_jagged_prefill(
+            a.data_ptr(), x.data_ptr(), _ptr(c), _ptr(v), _ptr(carry_init), y.data_ptr(),
+            _ptr(h_tail), _ptr(r_tail), _ptr(c_prev_tail), B, H, D, L, int(block_len),
+            _tag(a.dtype), _tag(x.dtype), _tag(state_dtype), _tag(r_tail.dtype) if r_tail is not None else _F32,
+            FLAG_JAGGED_LOG_A if log_a else 0, _stream_ptr(x.device),
+        )
+    if rc != 0:
+        _raise_native(lib, rc)
+
+
+def jagged_step(
+    a_t: torch.Tensor,
+    x_t: torch.Tensor,
+    c_t: torch.Tensor | None,
+    v_t: torch.Tensor | None,
+    y_t: torch.Tensor,
+    h_in: torch.Tensor,
+    r_in: torch.Tensor,
+    c_prev_in: torch.Tensor,
+    h_out: torch.Tensor,
+    r_out: torch.Tensor,
+    c_prev_out: torch.Tensor | None,
+    boundary: bool,
+    log_a: bool,
+    log_r: bool,
+    tiny: float,
+) -> None:
+    """One decode token for every (batch, head) (see ``spear_jagged_step`` in the C header). Outputs
+    are written in place; each ``*_out`` may be the same tensor as its ``*_in``."""
+    given = [t for t in (a_t, x_t, c_t, v_t, y_t, h_in, r_in, c_prev_in, h_out, r_out, c_prev_out) if t is not None]
+    _check(all(t.is_cuda for t in given), "All tensors must be CUDA.")
+    _check(len({t.device for t in given}) == 1, "All tensors must be on the same device.")
+    _check(x_t.dim() == 3, "x_t must be [B, H, D].")
+    B, H, D = x_t.shape
+    _check(_tag(x_t.dtype) >= 0 and _tag(a_t.dtype) >= 0, "tensors must be float32, float16 or bfloat16.")
+    _check((c_t is None) == (v_t is None), "c_t and v_t must be given together.")
+    _check(not boundary or c_prev_out is not None, "c_prev_out is required at a block boundary.")
+    _check_layout("a_t", a_t, (B, H))
+    for name, t in (("x_t", x_t), ("c_t", c_t), ("v_t", v_t), ("y_t", y_t)):
+        if t is not None:
+            _check_layout(name, t, (B, H, D))
+            _check(t.dtype == x_t.dtype, f"{name} dtype must match x_t.")
+    for name, t in (("h_in", h_in), ("c_prev_in", c_prev_in), ("h_out", h_out), ("c_prev_out", c_prev_out)):
+        if t is not None:
+            _check_layout(name, t, (B, H, D))
+            _check(t.dtype == h_in.dtype, "state tensors must share a dtype.")
+    _check(h_in.dtype in (x_t.dtype, torch.float32), "the state must be float32 or match x_t dtype.")
+    _check_layout("r_in", r_in, (B, H))
+    _check_layout("r_out", r_out, (B, H))
+    _check(r_in.dtype == r_out.dtype and _tag(r_in.dtype) >= 0, "r_in and r_out must share a float dtype.")
+    flags = (FLAG_JAGGED_LOG_A if log_a else 0) | (FLAG_JAGGED_LOG_R if log_r else 0)
+    lib = load_library()
+    with torch.cuda.device(x_t.device):
+        rc = lib.spear_jagged_step(
+            a_t.data_ptr(), x_t.data_ptr(), _ptr(c_t), _ptr(v_t), y_t.data_ptr(), h_in.data_ptr(), r_in.data_ptr(),
+            c_prev_in.data_ptr(), h_out.data_ptr(), r_out.data_ptr(), _ptr(c_prev_out), B, H, D, int(bool(boundary)),
+            _tag(a_t.dtype), _tag(x_t.dtype), _tag(h_in.dtype), _tag(r_in.dtype), flags, float(tiny),
+            _stream_ptr(x_t.device),
         )
     if rc != 0:
         _raise_native(lib, rc)

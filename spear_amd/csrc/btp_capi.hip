@@ -24,6 +24,8 @@ int fail(int code, const char* fmt, ...) {
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
+bool dtype_ok(int d) { return d == SPEAR_BTP_BF16 || d == SPEAR_BTP_F16 || d == SPEAR_BTP_F32; }
+
 int check_common(const char* who, int B, int H, int L, int k, int in_dtype, int io_dtype, const char* io_name,
                  unsigned flags, unsigned allowed_flags) {
   if (B < 0 || H < 0 || L < 0) return fail(SPEAR_BTP_EINVAL, "%s: negative dimension (B=%d H=%d L=%d)", who, B, H, L);
@@ -42,7 +44,7 @@ int check_common(const char* who, int B, int H, int L, int k, int in_dtype, int 
 
 extern "C" {
 
-int spear_btp_abi_version(void) { return 5; }
+int spear_btp_abi_version(void) { return 6; }
 
 const char* spear_btp_last_error(void) { return g_error; }
 
@@ -175,6 +177,65 @@ int spear_phalanx_mix_backward(const void* a_logit, const void* b_logit, const v
   }
   spear_btp::MixBwdArgs a{a_logit, b_logit, c, v, dout, da_logit, db_logit, dc, dv, B, L, H, groups, dtype};
   const hipError_t err = spear_btp::fused_mix_backward(a, static_cast<hipStream_t>(stream));
+  if (err != hipSuccess) return fail(SPEAR_BTP_ELAUNCH, "%s: launch failed: %s", who, hipGetErrorString(err));
+  return 0;
+}
+
+int spear_jagged_prefill(const void* a, const void* x, const void* c, const void* v, const void* carry_init, void* y,
+                         void* h_tail, void* r_tail, void* c_prev_tail, int B, int H, int D, int L, int block_len,
+                         int a_dtype, int x_dtype, int state_dtype, int r_dtype, unsigned flags, void* stream) {
+  g_error[0] = '\0';
+  const char* who = "spear_jagged_prefill";
+  if (B < 0 || H < 0 || L < 0) return fail(SPEAR_BTP_EINVAL, "%s: negative dimension (B=%d H=%d L=%d)", who, B, H, L);
+  if (D <= 0 || block_len <= 0)
+    return fail(SPEAR_BTP_EINVAL, "%s: D and block_len must be positive (D=%d block_len=%d)", who, D, block_len);
+  if (!dtype_ok(a_dtype) || !dtype_ok(x_dtype) || !dtype_ok(state_dtype) || !dtype_ok(r_dtype))
+    return fail(SPEAR_BTP_EINVAL, "%s: unknown dtype tag", who);
+  if (a_dtype != x_dtype && a_dtype != SPEAR_BTP_F32)
+    return fail(SPEAR_BTP_EINVAL, "%s: a must be float32 or match x dtype.", who);
+  if (state_dtype != x_dtype && state_dtype != SPEAR_BTP_F32)
+    return fail(SPEAR_BTP_EINVAL, "%s: the state must be float32 or match x dtype.", who);
+  if (flags & ~SPEAR_JAGGED_LOG_A) return fail(SPEAR_BTP_EINVAL, "%s: unknown flag bits 0x%x", who, flags & ~SPEAR_JAGGED_LOG_A);
+  if ((long long)B * H * (long long)D * L >= (1ll << 40)) return fail(SPEAR_BTP_EINVAL, "%s: tensor too large", who);
+  if ((c == nullptr) != (v == nullptr)) return fail(SPEAR_BTP_EINVAL, "%s: c and v must be given together", who);
+  const int n_state = (h_tail != nullptr) + (r_tail != nullptr) + (c_prev_tail != nullptr);
+  if (n_state != 0 && n_state != 3)
+    return fail(SPEAR_BTP_EINVAL, "%s: h_tail, r_tail and c_prev_tail must be given together", who);
+  if ((long long)B * H == 0 || L == 0) return 0;
+  if (!a || !x || !y) return fail(SPEAR_BTP_ENULL, "%s: NULL tensor pointer", who);
+  const bool al = aligned16(a) && aligned16(x) && aligned16(y) && aligned16(c) && aligned16(v);
+  spear_btp::JagPrefillArgs p{a, x, c, v, carry_init, y, h_tail, r_tail, c_prev_tail, B, H, D, L, block_len,
+                              a_dtype, x_dtype, state_dtype, r_dtype, (flags & SPEAR_JAGGED_LOG_A) != 0, al};
+  const hipError_t err = spear_btp::jagged_prefill(p, static_cast<hipStream_t>(stream));
+  if (err != hipSuccess) return fail(SPEAR_BTP_ELAUNCH, "%s: launch failed: %s", who, hipGetErrorString(err));
+  return 0;
+}
+
+int spear_jagged_step(const void* a_t, const void* x_t, const void* c_t, const void* v_t, void* y_t, const void* h_in,
+                      const void* r_in, const void* c_prev_in, void* h_out, void* r_out, void* c_prev_out, int B, int H,
+                      int D, int boundary, int a_dtype, int x_dtype, int state_dtype, int r_dtype, unsigned flags,
+                      float tiny, void* stream) {
+  g_error[0] = '\0';
+  const char* who = "spear_jagged_step";
+  if (B < 0 || H < 0) return fail(SPEAR_BTP_EINVAL, "%s: negative dimension (B=%d H=%d)", who, B, H);
+  if (D <= 0) return fail(SPEAR_BTP_EINVAL, "%s: D must be positive (got %d)", who, D);
+  if (!dtype_ok(a_dtype) || !dtype_ok(x_dtype) || !dtype_ok(state_dtype) || !dtype_ok(r_dtype))
+    return fail(SPEAR_BTP_EINVAL, "%s: unknown dtype tag", who);
+  if (state_dtype != x_dtype && state_dtype != SPEAR_BTP_F32)
+    return fail(SPEAR_BTP_EINVAL, "%s: the state must be float32 or match x dtype.", who);
+  const unsigned known = SPEAR_JAGGED_LOG_A | SPEAR_JAGGED_LOG_R;
+  if (flags & ~known) return fail(SPEAR_BTP_EINVAL, "%s: unknown flag bits 0x%x", who, flags & ~known);
+  if ((long long)B * H * (long long)D >= (1ll << 40)) return fail(SPEAR_BTP_EINVAL, "%s: tensor too large", who);
+  if ((c_t == nullptr) != (v_t == nullptr)) return fail(SPEAR_BTP_EINVAL, "%s: c_t and v_t must be given together", who);
+  if ((long long)B * H == 0) return 0;
+  if (!a_t || !x_t || !y_t || !h_in || !r_in || !c_prev_in || !h_out || !r_out || (boundary && !c_prev_out))
+    return fail(SPEAR_BTP_ENULL, "%s: NULL tensor pointer", who);
+  const bool al = aligned16(x_t) && aligned16(c_t) && aligned16(v_t) && aligned16(y_t) && aligned16(h_in) &&
+                  aligned16(c_prev_in) && aligned16(h_out) && aligned16(c_prev_out);
+  spear_btp::JagStepArgs p{a_t, x_t, c_t, v_t, y_t, h_in, r_in, c_prev_in, h_out, r_out, c_prev_out, B, H, D,
+                           boundary ? 1 : 0, a_dtype, x_dtype, state_dtype, r_dtype,
+                           (flags & SPEAR_JAGGED_LOG_A) ? 1 : 0, (flags & SPEAR_JAGGED_LOG_R) ? 1 : 0, tiny, al};
+  const hipError_t err = spear_btp::jagged_step(p, static_cast<hipStream_t>(stream));
   if (err != hipSuccess) return fail(SPEAR_BTP_ELAUNCH, "%s: launch failed: %s", who, hipGetErrorString(err));
   return 0;
 }

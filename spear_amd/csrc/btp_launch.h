@@ -59,6 +59,34 @@ struct MixBwdArgs {
 };
 hipError_t fused_mix_backward(const MixBwdArgs& p, hipStream_t s);
 
+// Streaming form (btp_jagged.hip). Tensors [B, H, D, L] / [B, H, L]; state vectors [B, H, D] / [B, H].
+struct JagPrefillArgs {
+  const void *a, *x, *c, *v;  // c and v both null: no "* C + V" epilogue
+  const void* carry_init;     // null, or the carry into the first block, [B, H, D] in state_dtype
+  void* y;
+  void *h_tail, *r_tail, *c_prev_tail;  // all null: no state wanted
+  int B, H, D, L, block_len;
+  int a_dtype, x_dtype, state_dtype, r_dtype;
+  bool log_a;    // a holds log(a_t)
+  bool aligned;  // every tensor pointer is 16-byte aligned (the tiled kernel needs it)
+};
+bool jagged_prefill_is_tiled(const JagPrefillArgs& p);
+hipError_t jagged_prefill(const JagPrefillArgs& p, hipStream_t s);
+
+struct JagStepArgs {
+  const void *a_t, *x_t, *c_t, *v_t;  // c_t and v_t both null: y_t without "* C + V"
+  void* y_t;
+  const void *h_in, *r_in, *c_prev_in;
+  void *h_out, *r_out, *c_prev_out;  // may alias the inputs; c_prev_out is written only at a block boundary
+  int B, H, D;
+  int boundary;  // this token completes a block: snapshot the carry, reset the local state
+  int a_dtype, x_dtype, state_dtype, r_dtype;
+  int log_a, log_r;  // a_t holds log(a_t); the r buffers hold log(r)
+  float tiny;        // lower clamp of a_t before the logarithm (log_r only)
+  bool aligned;      // every tensor pointer is 16-byte aligned (the 8-channel kernel needs it)
+};
+hipError_t jagged_step(const JagStepArgs& p, hipStream_t s);
+
 // Plain copy kernel used for bandwidth / counter calibration (btp_scan.hip).
 hipError_t device_copy(const void* src, void* dst, unsigned long long bytes, hipStream_t s);
 

@@ -13,7 +13,7 @@ HEADER = os.path.join(ROOT, "include", "spear_btp.h")
 def declared_functions():
     text = open(HEADER).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"\b(spear_(?:btp|phalanx)_\w+)\s*\(", text)))
+    return sorted(set(re.findall(r"\b(spear_(?:btp|phalanx|jagged)_\w+)\s*\(", text)))
 
 
 def test_header_declares_the_expected_entry_points():
@@ -25,6 +25,8 @@ def test_header_declares_the_expected_entry_points():
         "spear_btp_forward",
         "spear_btp_forward_loggate",
         "spear_btp_last_error",
+        "spear_jagged_prefill",
+        "spear_jagged_step",
         "spear_phalanx_mix_backward",
         "spear_phalanx_mix_forward",
     ]
@@ -51,6 +53,9 @@ def test_constants_match_the_header():
     assert int(defs["SPEAR_BTP_F32"]) == _btp._F32
     assert int(defs["SPEAR_BTP_WRITE_CHECKPOINT"], 16) == _btp.FLAG_WRITE_CHECKPOINT
     assert int(defs["SPEAR_BTP_PATH_MFMA"], 16) == _btp.FLAG_PATH_MFMA
+    jag = dict(re.findall(r"#define\s+(SPEAR_JAGGED_\w+)\s+(0x[0-9a-fA-F]+)u", text))
+    assert int(jag["SPEAR_JAGGED_LOG_A"], 16) == _btp.FLAG_JAGGED_LOG_A
+    assert int(jag["SPEAR_JAGGED_LOG_R"], 16) == _btp.FLAG_JAGGED_LOG_R
 
 
 def test_host_side_validation_needs_no_gpu():
@@ -58,7 +63,7 @@ def test_host_side_validation_needs_no_gpu():
     from spear_amd import _btp
 
     lib = _btp.load_library()
-    assert lib.spear_btp_abi_version() == 5
+    assert lib.spear_btp_abi_version() == 6
     buf = ctypes.create_string_buffer(4096)
     p = ctypes.addressof(buf)
     p -= p % 16
@@ -88,3 +93,37 @@ def test_host_side_validation_needs_no_gpu():
     assert lib.spear_btp_forward(p, p, p, None, 0, 4, 32, 2, 0, 0, 0, None) == 0
     assert lib.spear_btp_last_error() == b""
     assert lib.spear_btp_copy(p, p, 24, None) == -1
+
+
+def test_streaming_entry_points_validate_on_the_host():
+    from spear_amd import _btp
+
+    lib = _btp.load_library()
+    buf = ctypes.create_string_buffer(4096)
+    p = ctypes.addressof(buf)
+    p += 16 - p % 16
+    pre = lambda *a: lib.spear_jagged_prefill(*a)
+    # a, x, c, v, carry, y, h, r, cprev, B, H, D, L, block_len, a_dt, x_dt, state_dt, r_dt, flags, stream
+    assert pre(p, p, p, None, None, p, None, None, None, 1, 1, 16, 32, 16, 0, 0, 0, 0, 0, None) == -1
+    assert b"c and v must be given together" in lib.spear_btp_last_error()
+    assert pre(p, p, None, None, None, p, p, None, None, 1, 1, 16, 32, 16, 0, 0, 0, 0, 0, None) == -1
+    assert b"given together" in lib.spear_btp_last_error()
+    assert pre(p, p, None, None, None, p, None, None, None, 1, 1, 16, 32, 0, 0, 0, 0, 0, 0, None) == -1
+    assert b"block_len must be positive" in lib.spear_btp_last_error()
+    assert pre(p, p, None, None, None, p, None, None, None, 1, 1, 16, 32, 16, 1, 0, 0, 0, 0, None) == -1
+    assert b"a must be float32 or match x dtype" in lib.spear_btp_last_error()
+    assert pre(p, p, None, None, None, p, None, None, None, 1, 1, 16, 32, 16, 0, 0, 1, 0, 0, None) == -1
+    assert b"state must be float32 or match x dtype" in lib.spear_btp_last_error()
+    assert pre(p, p, None, None, None, p, None, None, None, 1, 1, 16, 32, 16, 0, 0, 0, 0, 0x8, None) == -1
+    assert pre(None, p, None, None, None, p, None, None, None, 1, 1, 16, 32, 16, 0, 0, 0, 0, 0, None) == -2
+    assert pre(p, p, None, None, None, p, None, None, None, 1, 0, 16, 32, 16, 0, 0, 0, 0, 0, None) == 0
+    step = lambda *a: lib.spear_jagged_step(*a)
+    # a_t, x_t, c_t, v_t, y_t, h_in, r_in, cp_in, h_out, r_out, cp_out, B, H, D, boundary, dtypes x4, flags, tiny, stream
+    assert step(p, p, None, None, p, p, p, p, p, p, None, 1, 1, 16, 1, 0, 0, 0, 0, 0, 0.0, None) == -2  # boundary needs c_prev_out
+    assert step(p, p, p, None, p, p, p, p, p, p, p, 1, 1, 16, 0, 0, 0, 0, 0, 0, 0.0, None) == -1
+    assert b"c_t and v_t must be given together" in lib.spear_btp_last_error()
+    assert step(p, p, None, None, p, p, p, p, p, p, p, 1, 1, 0, 0, 0, 0, 0, 0, 0, 0.0, None) == -1
+    assert b"D must be positive" in lib.spear_btp_last_error()
+    assert step(p, p, None, None, p, p, p, p, p, p, p, 1, 1, 16, 0, 0, 0, 7, 0, 0, 0.0, None) == -1
+    assert step(p, p, None, None, p, p, p, p, p, p, p, 0, 1, 16, 0, 0, 0, 0, 0, 0, 0.0, None) == 0
+    assert lib.spear_btp_last_error() == b""

@@ -276,3 +276,21 @@ def test_oracle_fused_backward_matches_torch_autograd():
     got = orc.phalanx_mix_backward(*(t.detach().numpy() for t in (a, b, c, v)), dout.numpy(), H, Hkv)
     for name, gg, t in zip("abcv", got, (a, b, c, v)):
         np.testing.assert_allclose(gg, t.grad.numpy(), rtol=1e-10, atol=1e-12, err_msg=f"d{name}")
+
+
+def test_streaming_module_surface_and_state_dataclass():
+    from spear_amd.nn.phalanx import inference as inf
+
+    assert inf.__all__ == ["jagged_band_infer_sequential", "JaggedBandState", "JagState", "step_jagged", "parallel_jagged"]
+    st = inf.JagState(torch.zeros(1, 2, 3), torch.ones(1, 2), torch.zeros(1, 2, 3), 5, 16)
+    assert (st.use_log_r, st.log_r_pref) == (False, None)
+    cl = st.clone_detached()
+    cl.h_loc += 1
+    assert float(st.h_loc.abs().max()) == 0.0 and cl.i == 5 and cl.block_len == 16
+    # no CPU path: host tensors are refused before anything is computed
+    with pytest.raises(RuntimeError, match="must be on a GPU"):
+        inf.step_jagged(torch.ones(1, 2), torch.zeros(1, 2, 3), torch.ones(1, 2, 3), torch.zeros(1, 2, 3), st)
+    with pytest.raises(RuntimeError, match="must be on a GPU"):
+        inf.parallel_jagged(torch.ones(1, 2, 8), *(torch.zeros(1, 2, 3, 8) for _ in range(3)), block_len=4)
+    with pytest.raises(AssertionError):
+        inf.jagged_band_infer_sequential(torch.zeros(1, 2, 3, 8), torch.ones(1, 2, 7), 4)
