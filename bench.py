@@ -109,6 +109,7 @@ def main() -> int:
     ap.add_argument("--sets", type=int, default=4, help="independent buffer sets to rotate over")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-fused", action="store_true", help="skip the fused layer-layout forward leg")
+    ap.add_argument("--no-streaming", action="store_true", help="skip the prefill / decode-step leg")
     ap.add_argument("--settle-seconds", type=float, default=0.3, help="untimed run-in before the warm-up steps")
     args = ap.parse_args()
 
@@ -330,6 +331,83 @@ def main() -> int:
         }
         del msets
 
+    # streaming form: prompt prefill (recurrence + y*C+V + state hand-over) on the same tensors, and
+    # the one-token decode step on [B, H, 16] operands with fp32 state
+    streaming = None
+    if not args.no_streaming:
+        st_h = torch.zeros(B, H, 16, device=dev)
+        st_c = torch.zeros(B, H, 16, device=dev)
+        st_r = torch.ones(B, H, device=dev)
+
+        def prefill(s):
+            rc = lib.spear_jagged_prefill(s["coeff"].data_ptr(), s["x"].data_ptr(), s["dy"].data_ptr(),
+                                          s["dx"].data_ptr(), None, s["y"].data_ptr(), st_h.data_ptr(),
+                                          st_r.data_ptr(), st_c.data_ptr(), B, H, 16, L, 16, 0, 0, 2, 2, 0, sp)
+            assert rc == 0, lib.spear_btp_last_error()
+
+        prefill_ms = kernel_ms(prefill)
+        prefill_bytes = B * H * L * (2 + 3 * 32 + 32) + B * H * (2 * 64 + 4)
+
+        g = torch.Generator(device="cpu").manual_seed(seed + 11)
+        tok = [{
+            "a": torch.sigmoid(torch.randn(B, H, generator=g)).to(torch.bfloat16).to(dev),
+            "x": torch.randn(B, H, 16, generator=g).to(torch.bfloat16).to(dev),
+            "c": torch.randn(B, H, 16, generator=g).to(torch.bfloat16).to(dev),
+            "v": torch.randn(B, H, 16, generator=g).to(torch.bfloat16).to(dev),
+            "y": torch.empty(B, H, 16, device=dev, dtype=torch.bfloat16),
+        } for _ in range(16)]
+        counter = [0]
+
+        def decode(s):
+            i = counter[0]
+            counter[0] = (i + 1) % 16
+            rc = lib.spear_jagged_step(s["a"].data_ptr(), s["x"].data_ptr(), s["c"].data_ptr(), s["v"].data_ptr(),
+                                       s["y"].data_ptr(), st_h.data_ptr(), st_r.data_ptr(), st_c.data_ptr(),
+                                       st_h.data_ptr(), st_r.data_ptr(), st_c.data_ptr(), B, H, 16, int(i == 15),
+                                       0, 0, 2, 2, 0, 0.0, sp)
+            assert rc == 0, lib.spear_btp_last_error()
+
+        def decode_torch(s):  # the same update as a chain of PyTorch ops (spear/nn/phalanx/inference.py:200-262)
+            i = counter[0]
+            counter[0] = (i + 1) % 16
+            a = s["a"].unsqueeze(-1)
+            h = a * st_h + s["x"]
+            r = s["a"] * st_r
+            s["y"].copy_((h + r.unsqueeze(-1) * st_c) * s["c"] + s["v"])
+            if i == 15:
+                st_c.copy_(h)
+                st_h.zero_()
+                st_r.fill_(1.0)
+            else:
+                st_h.copy_(h)
+                st_r.copy_(r)
+
+        def tokens_ms(fn):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            for i in range(16):
+                fn(tok[i])
+            torch.cuda.synchronize()
+            n = 16 * max(4, args.steps // 16)
+            e0.record(stream)
+            for i in range(n):
+                fn(tok[i % 16])
+            e1.record(stream)
+            torch.cuda.synchronize()
+            return e0.elapsed_time(e1) / n
+
+        step_ms, step_torch_ms = tokens_ms(decode), tokens_ms(decode_torch)
+        step_bytes = B * H * (2 + 8 + 3 * 32 + 32 + 2 * 64 + 64)  # a, r in/out, x c v, y, h in/out, c_prev
+        streaming = {
+            "prefill": {"avg_launch_ms": prefill_ms, "algorithmic_bytes_per_launch": prefill_bytes,
+                        "achieved": prefill_bytes / (prefill_ms * 1e-3) / 1e9,
+                        "frac": prefill_bytes / (prefill_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS},
+            "decode_step": {"avg_launch_ms": step_ms, "algorithmic_bytes_per_launch": step_bytes,
+                            "achieved": step_bytes / (step_ms * 1e-3) / 1e9,
+                            "frac": step_bytes / (step_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+                            "tokens_per_s": B / (step_ms * 1e-3),
+                            "same_step_from_pytorch_ops_ms": step_torch_ms, "speedup": step_torch_ms / step_ms},
+        }
+
     units = B * H * L
     tokens = B * L
     bwd_gbps = units * BWD_BYTES / (bwd_ms * 1e-3) / 1e9
@@ -375,6 +453,7 @@ def main() -> int:
                                   "achieved": units * (68 + 108) / ((fwd_log_ms + bwd_log_ms) * 1e-3) / 1e9,
                                   "algorithmic_bytes_per_unit": {"forward": 68, "backward": 108}},
         "fused_layer_stage": fused,
+        "streaming": streaming,
         "fwd_plus_bwd": {"achieved": step_gbps, "frac": step_gbps / HBM_PEAK_GBPS,
                          "algorithmic_bytes_per_step": units * (FWD_BYTES + BWD_BYTES)},
         "step_spread": spread,
