@@ -100,7 +100,9 @@ def test_layer_parametrised_backward_case_that_the_reference_documents_as_failin
         _within(m, BACKWARD_LIMITS, f"exact_layer_grad_{name}")
 
 
-@pytest.mark.parametrize("opts", [{}, {"fullgraph": True}], ids=["default", "fullgraph"])
+# the three compile configurations of the reference's tests (tests/btp/test_numerics.py:51-53)
+@pytest.mark.parametrize("opts", [{}, {"fullgraph": True}, {"fullgraph": True, "mode": "max-autotune"}],
+                         ids=["default", "fullgraph", "max-autotune"])
 def test_torch_compile(opts):
     from spear_amd.ops.btp.runners import compare_backward_gradients, run_kernel_forward, run_reference, sample_inputs
     from spear_amd.testing.numerics import compute_error_metrics
