@@ -357,6 +357,7 @@ def main() -> int:
             "y": torch.empty(B, H, 16, device=dev, dtype=torch.bfloat16),
         } for _ in range(16)]
         counter = [0]
+        step_stream = [sp]  # the stream the step kernel is launched on (the capture stream while recording)
 
         def decode(s):
             i = counter[0]
@@ -364,7 +365,7 @@ def main() -> int:
             rc = lib.spear_jagged_step(s["a"].data_ptr(), s["x"].data_ptr(), s["c"].data_ptr(), s["v"].data_ptr(),
                                        s["y"].data_ptr(), st_h.data_ptr(), st_r.data_ptr(), st_c.data_ptr(),
                                        st_h.data_ptr(), st_r.data_ptr(), st_c.data_ptr(), B, H, 16, int(i == 15),
-                                       0, 0, 2, 2, 0, 0.0, sp)
+                                       0, 0, 2, 2, 0, 0.0, step_stream[0])
             assert rc == 0, lib.spear_btp_last_error()
 
         def decode_torch(s):  # the same update as a chain of PyTorch ops (spear/nn/phalanx/inference.py:200-262)
@@ -396,6 +397,36 @@ def main() -> int:
             return e0.elapsed_time(e1) / n
 
         step_ms, step_torch_ms = tokens_ms(decode), tokens_ms(decode_torch)
+
+        # the same 16 launches of one block period as a HIP graph (no memset nodes: the step kernel
+        # resets the state itself at the boundary)
+        def period():
+            for i in range(16):
+                decode(tok[i])
+
+        counter[0] = 0
+        side = torch.cuda.Stream()
+        side.wait_stream(stream)
+        step_stream[0] = ctypes.c_void_p(side.cuda_stream)
+        with torch.cuda.stream(side):
+            period()  # warm-up on the capture stream
+        stream.wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            period()
+        step_stream[0] = sp
+        torch.cuda.synchronize()
+        for _ in range(3):
+            graph.replay()
+        torch.cuda.synchronize()
+        n_rep = max(4, args.steps // 16)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(stream)
+        for _ in range(n_rep):
+            graph.replay()
+        e1.record(stream)
+        torch.cuda.synchronize()
+        step_graph_ms = e0.elapsed_time(e1) / (16 * n_rep)
         step_bytes = B * H * (2 + 8 + 3 * 32 + 32 + 2 * 64 + 64)  # a, r in/out, x c v, y, h in/out, c_prev
         streaming = {
             "prefill": {"avg_launch_ms": prefill_ms, "algorithmic_bytes_per_launch": prefill_bytes,
@@ -405,7 +436,8 @@ def main() -> int:
                             "achieved": step_bytes / (step_ms * 1e-3) / 1e9,
                             "frac": step_bytes / (step_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
                             "tokens_per_s": B / (step_ms * 1e-3),
-                            "same_step_from_pytorch_ops_ms": step_torch_ms, "speedup": step_torch_ms / step_ms},
+                            "same_step_from_pytorch_ops_ms": step_torch_ms, "speedup": step_torch_ms / step_ms,
+                            "avg_launch_ms_in_hip_graph": step_graph_ms},
         }
 
     units = B * H * L

@@ -248,3 +248,52 @@ def test_streaming_functions_reject_cpu_tensors_and_bad_arguments():
         _btp.jagged_prefill(Ad[..., :16].contiguous(), Xd, None, None, None, torch.empty_like(Xd), None, None, None, 16, False)
     with pytest.raises(RuntimeError, match="float32 or match"):
         _btp.jagged_prefill(Ad.half(), Xd, None, None, None, torch.empty_like(Xd), None, None, None, 16, False)
+
+
+def test_one_block_period_of_decode_steps_replays_as_a_hip_graph():
+    """The step entry point allocates nothing and takes the block boundary as an argument, so the 16
+    steps of one block period, updating the state in place, form a graph that can be replayed for
+    every following period. Each replay (with eager work and synchronisation in between) is checked
+    against the oracle continuing from the same state."""
+    from spear_amd import _btp
+
+    B, H, D, bl = 3, 4, 16, 16
+    A, X, C, V = make(B, H, D, 4 * bl, seed=31, a_dtype=torch.float32)
+    rY, _ = jag.prefill(f64(A), f64(X), f64(C), f64(V), block_len=bl)
+    # static input buffers, [token][...] so that every captured launch reads a fixed address
+    a_buf = torch.empty(bl, B, H, device=DEV)
+    x_buf, c_buf, v_buf, y_buf = (torch.empty(bl, B, H, D, device=DEV, dtype=torch.bfloat16) for _ in range(4))
+    h = torch.zeros(B, H, D, device=DEV)
+    cp = torch.zeros(B, H, D, device=DEV)
+    r = torch.ones(B, H, device=DEV)
+
+    def period():
+        for i in range(bl):
+            _btp.jagged_step(a_buf[i], x_buf[i], c_buf[i], v_buf[i], y_buf[i], h, r, cp, h, r, cp,
+                             i == bl - 1, False, False, 0.0)
+
+    def load(p):  # eager copies between replays
+        sl = slice(p * bl, (p + 1) * bl)
+        a_buf.copy_(A[..., sl].permute(2, 0, 1))
+        for buf, src in ((x_buf, X), (c_buf, C), (v_buf, V)):
+            buf.copy_(src[..., sl].permute(3, 0, 1, 2))
+
+    load(0)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        period()  # warm-up on a side stream; its state update is undone below
+    torch.cuda.current_stream().wait_stream(side)
+    h.zero_(); cp.zero_(); r.fill_(1.0)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        period()
+    h.zero_(); cp.zero_(); r.fill_(1.0)  # capture does not run the kernels, but be explicit
+    for p in range(4):
+        load(p)
+        y_buf.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        got = f64(y_buf).transpose(1, 2, 3, 0)  # [B, H, D, token]
+        assert_close(got, rY[..., p * bl:(p + 1) * bl], BF16_ATOL, BF16_RTOL, f"period {p}")
