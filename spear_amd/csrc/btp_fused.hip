@@ -360,15 +360,17 @@ __global__ __launch_bounds__(64 * kWaves) void phalanx_mix_bwd_kernel(
     // ---- pass F
     const int o_off = (t0 >= t_begin) ? o_lane : 0x7ffffff0;
     const int okv_off = (t0 >= t_begin) ? okv_lane : 0x7ffffff0;
-    float e[16];
     float vp0 = 0.0f, vp1 = 0.0f, z0 = cin0, z1 = cin1;
+    // the per-step partial sums of dA go back into the parking slot they were computed from (its
+    // first word is free once read), so that they do not occupy 16 registers during this pass
+    float* my_e = reinterpret_cast<float*>(my_park);
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
       const float4 pk = my_park[r * 64];  // R0, R1, dX0, dX1
       const float G0 = fast_sigmoid(E::lo(cur.b[r])), G1 = fast_sigmoid(E::hi(cur.b[r]));
       const float v0 = E::lo(cur.v[r]), v1 = E::hi(cur.v[r]);
       const float go0 = E::lo(cur.g[r]), go1 = E::hi(cur.g[r]);
-      e[r] = fmaf(pk.z, vp0, pk.x * z0) + fmaf(pk.w, vp1, pk.y * z1);
+      my_e[r * 256] = fmaf(pk.z, vp0, pk.x * z0) + fmaf(pk.w, vp1, pk.y * z1);
       const float az0 = a[r] * z0, az1 = a[r] * z1;
       vp0 = fmaf(a[r], vp0, G0 * v0);
       vp1 = fmaf(a[r], vp1, G1 * v1);
@@ -397,7 +399,9 @@ __global__ __launch_bounds__(64 * kWaves) void phalanx_mix_bwd_kernel(
 
     // ---- dA: sum over the 8 lanes (16 channels) of the head, transposing: lane k keeps steps 2k, 2k+1
     const int kk = lane & 7;
-    float f8[8], f4[4];
+    float e[16], f8[8], f4[4];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) e[r] = my_e[r * 256];
     {
       const bool hi = kk & 4;
 #pragma unroll
