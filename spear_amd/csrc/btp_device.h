@@ -20,7 +20,13 @@ constexpr int kSpan = 128;  // time steps one wavefront owns per pass: 8 blocks,
 #ifndef SPEAR_BTP_WAVES_PER_WG
 #define SPEAR_BTP_WAVES_PER_WG 4
 #endif
-constexpr int kWaves = SPEAR_BTP_WAVES_PER_WG;  // wavefronts per workgroup; each works on its own span, no barriers
+constexpr int kWaves = SPEAR_BTP_WAVES_PER_WG;  // wavefronts per workgroup; each works on its own span
+#ifndef SPEAR_BTP_WAVES_PER_WG_LONG
+#define SPEAR_BTP_WAVES_PER_WG_LONG 8
+#endif
+// Rows of several spans, backward recurrence kernel: neighbouring spans of a workgroup hand their
+// carries over through LDS, so a larger workgroup means fewer halo reads (measured: -3 %).
+constexpr int kWavesLong = SPEAR_BTP_WAVES_PER_WG_LONG;
 
 // Coefficients at or below this are treated as exactly zero, as in the reference kernels
 // (csrc/btp/btp-forward.cu:179, csrc/btp/btp-backwards.cu:280-286); this also maps negative

@@ -69,9 +69,17 @@ __global__ __launch_bounds__(64 * kWaves) void jagged_prefill_kernel(
   constexpr int kImages = kEpilogue ? 3 : 1;
   __shared__ __align__(16) unsigned char lds[kWaves][kImages * 4096 + kCoeffLdsBytes];
 
+  // rows of several spans: the carry into a span's first block comes from the neighbouring
+  // wavefront through LDS (one workgroup barrier), as in the forward kernel
+  constexpr bool kHandOver = !kStreamIn && kWaves > 1;
+  __shared__ float left_state[kHandOver ? kWaves : 1][kChan];
+
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const long span = first_span_of_workgroup() + wave;
-  if (span >= total_spans) return;  // wave-uniform; no workgroup barrier is used anywhere
+  if (span >= total_spans) {  // wave-uniform
+    if constexpr (kHandOver) __syncthreads();  // keep the barrier count equal for every wavefront
+    return;
+  }
   const SpanCoord sc = span_coord(span, spans_per_row, L);
 
   unsigned char* img = lds[wave];
@@ -81,7 +89,7 @@ __global__ __launch_bounds__(64 * kWaves) void jagged_prefill_kernel(
   const int j = lane >> 4, d = lane & 15;
 
   uint4 xin[4], cin[4], vin[4];
-  slab16_global_to_regs<kStreamIn>(x + slab_off, L, sc.nvalid, lane, xin);
+  slab16_global_to_regs<nt_loads(kStreamIn)>(x + slab_off, L, sc.nvalid, lane, xin);
   const typename C::pair_t ain = coeff_global_to_reg<C>(arow, sc.nvalid, lane);
   if constexpr (kEpilogue) {
     slab16_global_to_regs<true>(cmul + slab_off, L, sc.nvalid, lane, cin);  // read once, by this span only
@@ -90,7 +98,7 @@ __global__ __launch_bounds__(64 * kWaves) void jagged_prefill_kernel(
 
   float c_halo = 0.0f;
   if (j == 0) {
-    if (sc.sp > 0) {  // local terminal state of the block just left of the span, channel d
+    if (sc.sp > 0 && !(kHandOver && wave > 0)) {  // local terminal state of the block left of the span, channel d
       float ah[16], xh[16];
       C::load_block(arow - kTile, ah);
       const uint16_t* xp = x + slab_off + (long)d * L - kTile;
@@ -100,7 +108,7 @@ __global__ __launch_bounds__(64 * kWaves) void jagged_prefill_kernel(
 #pragma unroll
       for (int r = 0; r < 16; ++r) h = fmaf(ah[r], h, xh[r]);
       c_halo = h;
-    } else if (carry_init != nullptr) {
+    } else if (sc.sp == 0 && carry_init != nullptr) {
       c_halo = load_scalar(carry_init, sc.row * kChan + d, state_dtype);
     }
   }
@@ -132,6 +140,11 @@ __global__ __launch_bounds__(64 * kWaves) void jagged_prefill_kernel(
 #pragma unroll
   for (int r = 16; r < 32; ++r) vB_last = fmaf(a[r], vB_last, xf[r]);
   const float from_left = lane_rotate(vB_last, lane, -16);
+  if constexpr (kHandOver) {
+    if (j == 3) left_state[wave][d] = vB_last;
+    __syncthreads();
+    if (sc.sp > 0 && wave > 0 && j == 0) c_halo = left_state[wave - 1][d];
+  }
   const float cA = j == 0 ? c_halo : from_left;
   h = cA;
 #pragma unroll

@@ -56,6 +56,9 @@
 #ifndef SPEAR_BTP_BWD_WAVES_PER_EU  // 4 waves per SIMD need <= 128 VGPRs; the backward body is ordered to fit
 #define SPEAR_BTP_BWD_WAVES_PER_EU 4
 #endif
+#ifndef SPEAR_BTP_HANDOVER  // 1: carries between the spans of a workgroup go through LDS; 0: every span reads its halo
+#define SPEAR_BTP_HANDOVER 1
+#endif
 #if SPEAR_BTP_FWD_WAVES_PER_EU > 0
 #define SPEAR_BTP_FWD_OCC __attribute__((amdgpu_waves_per_eu(SPEAR_BTP_FWD_WAVES_PER_EU)))
 #else
@@ -80,11 +83,22 @@ __global__ __launch_bounds__(64 * kWaves) SPEAR_BTP_FWD_OCC void btp_fwd_scan_ke
     float* __restrict__ ckpt, int L, int spans_per_row, long total_spans, int k) {
   constexpr bool kOutF32 = std::is_same<OutT, float>::value;
   constexpr int kImgBytes = kOutF32 ? 8192 : 4096;
-  __shared__ __align__(16) unsigned char lds[kWaves][kImgBytes + kCoeffLdsBytes];
+  constexpr int kW = kWaves;  // wavefronts in this workgroup (8 measured 1-3 % slower here, unlike backward)
+  __shared__ __align__(16) unsigned char lds[kW][kImgBytes + kCoeffLdsBytes];
+  // Rows longer than one span (kStreamIn == false): a span's first block needs the terminal local
+  // state of the block before it. Inside a workgroup the neighbouring wavefront has just computed
+  // it, so it is handed over through LDS with the kernel's only workgroup barrier; only the first
+  // wavefront of a workgroup recomputes it from a halo read (measured: the halo reads of every span
+  // added 12 % to the bytes fetched).
+  constexpr bool kHandOver = SPEAR_BTP_HANDOVER && !kStreamIn && kW > 1;
+  __shared__ float left_state[kHandOver ? kW : 1][kChan];
 
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const long span = first_span_of_workgroup() + wave;
-  if (span >= total_spans) return;  // wave-uniform; no workgroup barrier is used anywhere
+  const long span = first_span_of_workgroup(kW) + wave;
+  if (span >= total_spans) {  // wave-uniform
+    if constexpr (kHandOver) __syncthreads();  // keep the barrier count equal for every wavefront
+    return;
+  }
   const SpanCoord sc = span_coord(span, spans_per_row, L);
 
   unsigned char* img = lds[wave];
@@ -94,14 +108,15 @@ __global__ __launch_bounds__(64 * kWaves) SPEAR_BTP_FWD_OCC void btp_fwd_scan_ke
   const int j = lane >> 4, d = lane & 15;
 
   // ---- all global reads are issued before anything waits on them
-  // kStreamIn: the host sets it for rows that fit one span, which are read exactly once. Longer
-  // rows are re-read by the neighbouring spans' halo loads, so their lines should stay in L2.
+  // kStreamIn: the host sets it for rows that fit one span. Longer rows hand carries over between
+  // the wavefronts of a workgroup (below); only a workgroup's first span re-reads 16 steps.
   constexpr bool kStreamOut = SPEAR_BTP_STREAM_STORES == 1;
   uint4 xin[4];
-  slab16_global_to_regs<kStreamIn>(xslab, L, sc.nvalid, lane, xin);
+  slab16_global_to_regs<nt_loads(kStreamIn)>(xslab, L, sc.nvalid, lane, xin);
   const typename C::pair_t ain = coeff_global_to_reg<C>(arow, sc.nvalid, lane);
 
-  const bool halo = (k == 2) && (sc.sp > 0);  // wave-uniform
+  const bool needs_left = (k == 2) && (sc.sp > 0);            // wave-uniform
+  const bool halo = needs_left && !(kHandOver && wave > 0);     // recompute from a halo read
   float c_halo = 0.0f;
   if (halo && j == 0) {
     // local terminal state of the block just left of the span, channel d
@@ -147,6 +162,11 @@ __global__ __launch_bounds__(64 * kWaves) SPEAR_BTP_FWD_OCC void btp_fwd_scan_ke
     vB_last = h3;
   }
   const float from_left = lane_rotate(vB_last, lane, -16);
+  if constexpr (kHandOver) {
+    if (j == 3) left_state[wave][d] = vB_last;  // terminal state of the span's last block
+    __syncthreads();
+    if (needs_left && wave > 0 && j == 0) c_halo = left_state[wave - 1][d];
+  }
   const float cA = (k == 2) ? (j == 0 ? c_halo : from_left) : 0.0f;
   // chain 3: block A started from its carry
   h = cA;
@@ -184,7 +204,15 @@ __global__ __launch_bounds__(64 * kWaves) SPEAR_BTP_FWD_OCC void btp_fwd_scan_ke
 // ==========================================================================================
 // Backward
 // ==========================================================================================
-template <class E, class C, class GradT, bool kStreamIn>
+// Wavefronts per workgroup of the backward kernels: the larger workgroup for rows of several spans
+// where 4 waves per SIMD fit (16-bit dy, 16-bit coefficients). The other variants need more than
+// 128 registers, and two 8-wave workgroups would then no longer fit a CU (measured: -33 %).
+template <bool kLean, bool kStreamIn>
+constexpr int bwd_waves() {
+  return (kStreamIn || !kLean) ? kWaves : kWavesLong;
+}
+
+template <class E, class C, class GradT, bool kStreamIn, int kW>
 __device__ __forceinline__ void btp_bwd_scan_body(
     unsigned char (*lds)[4096 + (std::is_same<GradT, float>::value ? 8192 : 4096) + kCoeffLdsBytes],
     const typename C::elem* __restrict__ coeff, const uint16_t* __restrict__ x, const GradT* __restrict__ dy,
@@ -193,9 +221,18 @@ __device__ __forceinline__ void btp_bwd_scan_body(
   constexpr bool kGradF32 = std::is_same<GradT, float>::value;
   constexpr int kGradBytes = kGradF32 ? 8192 : 4096;
 
+  // Rows longer than one span: the carries that cross a span boundary inside the workgroup (the
+  // forward state from the left neighbour, the gradient carry from the right one) are handed over
+  // through LDS with one workgroup barrier; only the workgroup's outer edges read a halo.
+  constexpr bool kHandOver = SPEAR_BTP_HANDOVER && !kStreamIn && kW > 1;
+  __shared__ float edge_state[kHandOver ? kW : 1][2][kChan];
+
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const long span = first_span_of_workgroup() + wave;
-  if (span >= total_spans) return;
+  const long span = first_span_of_workgroup(kW) + wave;
+  if (span >= total_spans) {  // wave-uniform
+    if constexpr (kHandOver) __syncthreads();  // keep the barrier count equal for every wavefront
+    return;
+  }
   const SpanCoord sc = span_coord(span, spans_per_row, L);
 
   unsigned char* img_x = lds[wave];
@@ -210,16 +247,20 @@ __device__ __forceinline__ void btp_bwd_scan_body(
   constexpr bool kStreamOut = SPEAR_BTP_STREAM_STORES == 1;  // see the forward kernel
   uint4 xin[4];
   uint4 gin[kGradF32 ? 8 : 4];
-  slab16_global_to_regs<kStreamIn>(xslab, L, sc.nvalid, lane, xin);
+  slab16_global_to_regs<nt_loads(kStreamIn)>(xslab, L, sc.nvalid, lane, xin);
   if constexpr (kGradF32) {
-    slab32_global_to_regs<kStreamIn>(reinterpret_cast<const float*>(dy) + slab_off, L, sc.nvalid, lane, gin);
+    slab32_global_to_regs<nt_loads(kStreamIn)>(reinterpret_cast<const float*>(dy) + slab_off, L, sc.nvalid, lane, gin);
   } else {
-    slab16_global_to_regs<kStreamIn>(reinterpret_cast<const uint16_t*>(dy) + slab_off, L, sc.nvalid, lane, gin);
+    slab16_global_to_regs<nt_loads(kStreamIn)>(reinterpret_cast<const uint16_t*>(dy) + slab_off, L, sc.nvalid, lane, gin);
   }
   const typename C::pair_t ain = coeff_global_to_reg<C>(arow, sc.nvalid, lane);
 
-  const bool halo_left = (k == 2) && (sc.sp > 0);              // wave-uniform
-  const bool halo_right = (k == 2) && (sc.s0 + kSpan < L);     // wave-uniform
+  const bool needs_left = (k == 2) && (sc.sp > 0);             // wave-uniform
+  const bool needs_right = (k == 2) && (sc.s0 + kSpan < L);    // wave-uniform
+  // the right neighbour is in this workgroup unless this is its last wavefront or the last span overall
+  const bool right_here = kHandOver && wave + 1 < kW && span + 1 < total_spans;
+  const bool halo_left = needs_left && !(kHandOver && wave > 0);
+  const bool halo_right = needs_right && !right_here;
   float c_halo = 0.0f, dc_halo = 0.0f;
   if (halo_left && j == 0) {
     float ah[16], xh[16];
@@ -309,6 +350,13 @@ __device__ __forceinline__ void btp_bwd_scan_body(
   const bool two = (k == 2);
   const float from_left = lane_rotate(v[31], lane, -16);
   const float from_right = lane_rotate(out_left, lane, +16);
+  if constexpr (kHandOver) {
+    if (j == 3) edge_state[wave][0][d] = v[31];     // forward state leaving the span on the right
+    if (j == 0) edge_state[wave][1][d] = out_left;  // gradient carry leaving the span on the left
+    __syncthreads();
+    if (needs_left && wave > 0 && j == 0) c_halo = edge_state[wave - 1][0][d];
+    if (needs_right && right_here && j == 3) dc_halo = edge_state[wave + 1][1][d];
+  }
   const float cA = two ? (j == 0 ? c_halo : from_left) : 0.0f;
   const float cB = two ? v[15] : 0.0f;
   const float dcA = two ? dcA_raw : 0.0f;
@@ -369,22 +417,24 @@ __device__ __forceinline__ void btp_bwd_scan_body(
 // 16-bit dy and 16-bit coefficients (the reference's operands): the body fits 128 VGPRs, so four
 // waves per SIMD are requested explicitly.
 template <class E, class C, bool kStreamIn>
-__global__ __launch_bounds__(64 * kWaves) SPEAR_BTP_BWD_OCC void btp_bwd_scan_kernel(
+__global__ __launch_bounds__((64 * bwd_waves<true, kStreamIn>())) SPEAR_BTP_BWD_OCC void btp_bwd_scan_kernel(
     const typename C::elem* __restrict__ coeff, const uint16_t* __restrict__ x, const uint16_t* __restrict__ dy,
     uint16_t* __restrict__ dx, float* __restrict__ dA, int L, int spans_per_row, long total_spans, int k) {
-  __shared__ __align__(16) unsigned char lds[kWaves][4096 + 4096 + kCoeffLdsBytes];
-  btp_bwd_scan_body<E, C, uint16_t, kStreamIn>(lds, coeff, x, dy, dx, dA, L, spans_per_row, total_spans, k);
+  constexpr int kW = bwd_waves<true, kStreamIn>();
+  __shared__ __align__(16) unsigned char lds[kW][4096 + 4096 + kCoeffLdsBytes];
+  btp_bwd_scan_body<E, C, uint16_t, kStreamIn, kW>(lds, coeff, x, dy, dx, dA, L, spans_per_row, total_spans, k);
 }
 
 // fp32 dy (twice the staging registers and LDS) and log-space gates (an exponential per
 // coefficient): occupancy is left to the compiler.
 template <class E, class C, class GradT, bool kStreamIn>
-__global__ __launch_bounds__(64 * kWaves) void btp_bwd_scan_kernel_relaxed(
+__global__ __launch_bounds__((64 * bwd_waves<false, kStreamIn>())) void btp_bwd_scan_kernel_relaxed(
     const typename C::elem* __restrict__ coeff, const uint16_t* __restrict__ x, const GradT* __restrict__ dy,
     uint16_t* __restrict__ dx, float* __restrict__ dA, int L, int spans_per_row, long total_spans, int k) {
   constexpr int kGradBytes = std::is_same<GradT, float>::value ? 8192 : 4096;
-  __shared__ __align__(16) unsigned char lds[kWaves][4096 + kGradBytes + kCoeffLdsBytes];
-  btp_bwd_scan_body<E, C, GradT, kStreamIn>(lds, coeff, x, dy, dx, dA, L, spans_per_row, total_spans, k);
+  constexpr int kW = bwd_waves<false, kStreamIn>();
+  __shared__ __align__(16) unsigned char lds[kW][4096 + kGradBytes + kCoeffLdsBytes];
+  btp_bwd_scan_body<E, C, GradT, kStreamIn, kW>(lds, coeff, x, dy, dx, dA, L, spans_per_row, total_spans, k);
 }
 
 __global__ __launch_bounds__(256) void copy_kernel(const uint4* __restrict__ src, uint4* __restrict__ dst,
@@ -396,7 +446,7 @@ __global__ __launch_bounds__(256) void copy_kernel(const uint4* __restrict__ src
 
 template <class E, class C, class OutT, bool kCheckpoint, bool kStreamIn>
 void launch_fwd_as(const FwdArgs& p, const Grid& g, hipStream_t s) {
-  hipLaunchKernelGGL((btp_fwd_scan_kernel<E, C, OutT, kCheckpoint, kStreamIn>), dim3(g.blocks), dim3(64 * kWaves), 0,
+  hipLaunchKernelGGL((btp_fwd_scan_kernel<E, C, OutT, kCheckpoint, kStreamIn>), dim3(g.blocks), dim3(64 * g.waves), 0,
                      s, static_cast<const typename C::elem*>(p.coeff), static_cast<const uint16_t*>(p.x),
                      static_cast<OutT*>(p.y), p.checkpoint, p.L, g.spans_per_row, g.total_spans, p.k);
 }
@@ -421,17 +471,18 @@ void launch_bwd_as(const BwdArgs& p, const Grid& g, hipStream_t s) {
   const auto* x = static_cast<const uint16_t*>(p.x);
   auto* dx = static_cast<uint16_t*>(p.dx);
   if constexpr (std::is_same<GradT, float>::value || C::kLog) {
-    hipLaunchKernelGGL((btp_bwd_scan_kernel_relaxed<E, C, GradT, kStreamIn>), dim3(g.blocks), dim3(64 * kWaves), 0, s,
+    hipLaunchKernelGGL((btp_bwd_scan_kernel_relaxed<E, C, GradT, kStreamIn>), dim3(g.blocks), dim3(64 * g.waves), 0, s,
                        c, x, static_cast<const GradT*>(p.dy), dx, p.dA, p.L, g.spans_per_row, g.total_spans, p.k);
   } else {
-    hipLaunchKernelGGL((btp_bwd_scan_kernel<E, C, kStreamIn>), dim3(g.blocks), dim3(64 * kWaves), 0, s, c, x,
+    hipLaunchKernelGGL((btp_bwd_scan_kernel<E, C, kStreamIn>), dim3(g.blocks), dim3(64 * g.waves), 0, s, c, x,
                        static_cast<const uint16_t*>(p.dy), dx, p.dA, p.L, g.spans_per_row, g.total_spans, p.k);
   }
 }
 
 template <class E, class C, class GradT>
 hipError_t launch_bwd(const BwdArgs& p, hipStream_t s) {
-  const Grid g = make_grid((long)p.B * p.H, p.L);
+  constexpr bool kLean = !(std::is_same<GradT, float>::value || C::kLog);  // the kernel launch_bwd_as picks
+  const Grid g = make_grid((long)p.B * p.H, p.L, bwd_waves<kLean, false>());
   if (stream_inputs(g)) launch_bwd_as<E, C, GradT, true>(p, g, s);
   else launch_bwd_as<E, C, GradT, false>(p, g, s);
   return hipGetLastError();

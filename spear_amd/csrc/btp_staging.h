@@ -13,8 +13,12 @@
 #include "btp_device.h"
 
 // Tuning knobs (compile-time). The defaults are the measured best on MI355X.
+// Non-temporal slab loads. With the carries of neighbouring spans handed over through LDS almost
+// nothing is read twice, and plain loads measured 1-2.5 % slower on long rows and fetched 6-12 % more
+// than they used (one extra line per contiguous run of a workgroup). The MFMA kernel, whose spans all
+// read their halo, keeps plain loads for rows of several spans.
 #ifndef SPEAR_BTP_STREAM_LOADS   // 0: never, 1: always, 2: only when a row is a single span
-#define SPEAR_BTP_STREAM_LOADS 2
+#define SPEAR_BTP_STREAM_LOADS 1
 #endif
 #ifndef SPEAR_BTP_STREAM_STORES  // 0: never, 1: always
 #define SPEAR_BTP_STREAM_STORES 1
@@ -265,35 +269,44 @@ __device__ __forceinline__ SpanCoord span_coord(long span, int spans_per_row, in
 #ifndef SPEAR_BTP_XCD_REMAP
 #define SPEAR_BTP_XCD_REMAP 0
 #endif
-__device__ __forceinline__ long first_span_of_workgroup() {
+__device__ __forceinline__ long first_span_of_workgroup(int waves = kWaves) {
 #if SPEAR_BTP_XCD_REMAP
   const unsigned n = gridDim.x, b = blockIdx.x;
   const unsigned per = n >> 3;
   const unsigned mapped = (b < (per << 3)) ? (b & 7u) * per + (b >> 3) : b;
-  return (long)mapped * kWaves;
+  return (long)mapped * waves;
 #else
-  return (long)blockIdx.x * kWaves;
+  return (long)blockIdx.x * waves;
 #endif
 }
 
 struct Grid {
   int spans_per_row;
   long total_spans;
+  bool stream;     // kStreamIn of the kernels
+  int waves;       // wavefronts per workgroup
   unsigned blocks;
 };
 
-inline Grid make_grid(long rows, int L) {
+// Rows that fit one span are read exactly once and can be streamed; longer rows are re-read by
+// neighbouring spans' halo loads, so their lines should stay in L2. `waves_long` is the workgroup
+// size (in wavefronts) the calling kernel family uses for those longer rows.
+inline Grid make_grid(long rows, int L, int waves_long = kWaves) {
   Grid g;
   g.spans_per_row = (L + kSpan - 1) / kSpan;
   g.total_spans = rows * g.spans_per_row;
-  g.blocks = (unsigned)((g.total_spans + kWaves - 1) / kWaves);
+  g.stream = g.spans_per_row == 1;  // template argument kStreamIn of the kernels: rows of a single span
+  g.waves = g.stream ? kWaves : waves_long;
+  g.blocks = (unsigned)((g.total_spans + g.waves - 1) / g.waves);
   return g;
 }
 
-// Rows that fit one span are read exactly once and can be streamed; longer rows are re-read by
-// the neighbouring spans' halo loads, so their lines should stay in L2.
-inline bool stream_inputs(const Grid& g) {
-  return SPEAR_BTP_STREAM_LOADS == 1 || (SPEAR_BTP_STREAM_LOADS == 2 && g.spans_per_row == 1);
+inline bool stream_inputs(const Grid& g) { return g.stream; }
+
+// Whether a kernel instance reads its slabs with non-temporal loads, from the knob above and from
+// whether its rows are single spans (the kernels' template argument).
+constexpr bool nt_loads(bool single_span) {
+  return SPEAR_BTP_STREAM_LOADS == 1 || (SPEAR_BTP_STREAM_LOADS == 2 && single_span);
 }
 
 }  // namespace spear_btp
