@@ -31,9 +31,9 @@ FWD_BYTES, BWD_BYTES = 66, 102  # per (token, head), bf16 y / dy
 
 # HBM bytes per launch of the dominant (backward) kernel, measured with rocprofv3 --pmc FETCH_SIZE /
 # WRITE_SIZE and scaled by what the same counters read for the copy kernel (x1.9997 / x1.0000);
-# figures and commands are in profiles/btp_kernels_c3_B1024_H32_L128.txt. Counters cannot be read
+# figures and commands are in profiles/btp_kernels_c3_B1024_H32_L128.txt (and the c4 / c5 files beside it). Counters cannot be read
 # from inside this script, so the value is recorded here; it is null for shapes never profiled.
-MEASURED_BWD_TRAFFIC_BYTES = {"c3": 429.29e6}
+MEASURED_BWD_TRAFFIC_BYTES = {"c3": 429.29e6, "c4": 891.20e6, "c5": 1756.40e6}
 
 CONFIGS = {
     # name: (B, H, L, seed, x_std, gate)
