@@ -25,10 +25,12 @@
 //     cancellation; results agree with a float64 evaluation to fp32 rounding.
 //   * The previous block's terminal state travels between lane groups with one ds_bpermute
 //     (the reference uses shared memory plus a DSMEM bulk copy and cluster barriers,
-//     btp-forward.cu:287-374). At the left edge of a span it is recomputed from the 16 steps
-//     before the span (a halo read that normally hits L2), so spans are fully independent:
-//     no flags, no look-back, no second kernel, and the carry is never dropped at a launch-shape
-//     boundary (the reference drops it at cluster boundaries, btp-forward.cu:359-366).
+//     btp-forward.cu:287-374). At the left edge of a span it comes from the neighbouring
+//     wavefront of the workgroup through LDS (one workgroup barrier, rows of several spans only),
+//     and at the left edge of a workgroup it is recomputed from the 16 steps before the span (a
+//     halo read), so workgroups are fully independent: no flags, no look-back, no second kernel,
+//     and the carry is never dropped at a launch-shape boundary (the reference drops it at
+//     cluster boundaries, btp-forward.cu:359-366).
 //
 // Backward uses, per block i with local index r (g = dy, c = carry into the block,
 // dC = carry of the gradient coming back from block i+1):
