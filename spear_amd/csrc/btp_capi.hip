@@ -140,6 +140,8 @@ int spear_phalanx_mix_forward(const void* a_logit, const void* b_logit, const vo
     return fail(SPEAR_BTP_EINVAL, "%s: tensors must be float16 or bfloat16.", who);
   if (flags != 0) return fail(SPEAR_BTP_EINVAL, "%s: unknown flag bits 0x%x", who, flags);
   if ((long long)B * L * H * 16ll >= (1ll << 40)) return fail(SPEAR_BTP_EINVAL, "%s: tensor too large", who);
+  if ((long long)L * H * 32ll >= (1ll << 31))  // a batch row is addressed through one 32-bit buffer resource
+    return fail(SPEAR_BTP_EINVAL, "%s: one batch row (L * H * 16 elements) must stay below 2 GiB", who);
   if ((long long)B * H == 0 || L == 0) return 0;
   if (!a_logit || !b_logit || !c || !v || !out) return fail(SPEAR_BTP_ENULL, "%s: NULL tensor pointer", who);
   if (!aligned16(a_logit) || !aligned16(b_logit) || !aligned16(c) || !aligned16(v) || !aligned16(out))
@@ -169,6 +171,8 @@ int spear_phalanx_mix_backward(const void* a_logit, const void* b_logit, const v
     return fail(SPEAR_BTP_EINVAL, "%s: tensors must be float16 or bfloat16.", who);
   if (flags != 0) return fail(SPEAR_BTP_EINVAL, "%s: unknown flag bits 0x%x", who, flags);
   if ((long long)B * L * H * 16ll >= (1ll << 40)) return fail(SPEAR_BTP_EINVAL, "%s: tensor too large", who);
+  if ((long long)L * H * 32ll >= (1ll << 31))  // a batch row is addressed through one 32-bit buffer resource
+    return fail(SPEAR_BTP_EINVAL, "%s: one batch row (L * H * 16 elements) must stay below 2 GiB", who);
   if ((long long)B * H == 0 || L == 0) return 0;
   const void* ptrs[] = {a_logit, b_logit, c, v, dout, da_logit, db_logit, dc, dv};
   for (const void* q : ptrs) {

@@ -93,6 +93,9 @@ def test_host_side_validation_needs_no_gpu():
     assert lib.spear_btp_forward(p, p, p, None, 0, 4, 32, 2, 0, 0, 0, None) == 0
     assert lib.spear_btp_last_error() == b""
     assert lib.spear_btp_copy(p, p, 24, None) == -1
+    # fused layer kernels: a batch row must fit one 32-bit buffer resource
+    assert lib.spear_phalanx_mix_forward(p, p, p, p, p, 1, 1 << 20, 128, 128, 0, 0, None) == -1
+    assert b"below 2 GiB" in lib.spear_btp_last_error()
 
 
 def test_streaming_entry_points_validate_on_the_host():
