@@ -89,6 +89,18 @@ def test_fused_backward_with_shared_kv_heads(B, L, H, Hkv):
     assert_close(f64(da), rda, BF16_ATOL, BF16_RTOL, "da")
 
 
+def test_fused_backward_fp16_and_steep_gates():
+    a, b, c, v = make_mix_inputs(2, 96, 8, 4, seed=6, dtype=torch.float16, scale=3.0)
+    a[0, :10, :] = -30.0  # decay ~ 1e-13: counts as zero
+    a[1, 20:40, 3] = 30.0  # decay -> 1
+    dout = torch.randn(2, 96, 128, generator=torch.Generator().manual_seed(7)).half()
+    da, db, dc, dv = run_mix_backward(a, b, c, v, dout, 8, 4)
+    rda, rdb, rdc, rdv = orc.phalanx_mix_backward(f64(a), f64(b), f64(c), f64(v), f64(dout), 8, 4)
+    # fp16 storage: 11 significant bits; sums over two heads and up to 32 steps of undamped states
+    for name, got, want in (("dv", dv, rdv), ("dc", dc, rdc), ("db", db, rdb), ("da", da, rda)):
+        assert_close(f64(got), want, 2e-2, 4e-3, name + " fp16")
+
+
 def test_fused_backward_rejects_groups_it_cannot_reduce():
     from spear_amd import _btp
 
