@@ -223,3 +223,40 @@ def test_kernels_match_committed_closed_form_vectors(case, k):
     assert_close(f64(dx), v[f"k{k}.dx"], BF16_ATOL, BF16_RTOL, "dx")
     assert_close(f64(dA), v[f"k{k}.dA"], BF16_ATOL, BF16_RTOL, "dA")
     assert_close(f64(run_forward(coeff, x, k=k, mfma=True)), v[f"k{k}.y"], BF16_ATOL, BF16_RTOL, "y mfma")
+
+
+# ---- seeded sweep over odd launch shapes ---------------------------------------------------------
+def _sweep_cases(n=36, seed=2024):
+    rng = np.random.RandomState(seed)
+    cases = []
+    for i in range(n):
+        B, H = int(rng.randint(1, 6)), int(rng.randint(1, 8))
+        # lengths around span (128) and workgroup (4 or 8 spans) boundaries, plus ragged last spans
+        L = 16 * int(rng.choice([1, 2, 7, 8, 9, 15, 16, 17, 24, 31, 32, 33, 40, 63, 64, 65, 72, 129]))
+        if B * H * L > 60000:
+            H = max(1, 60000 // (B * L))
+        cases.append((B, H, L, int(rng.choice([1, 2, 2, 2])), bool(rng.randint(2)), 4000 + i))
+    return cases
+
+
+@pytest.mark.parametrize("B,H,L,k,f32,seed", _sweep_cases())
+def test_forward_and_backward_on_odd_launch_shapes(B, H, L, k, f32, seed):
+    """Rows that end inside a span, rows of 1..17 spans, span counts that do not fill the last workgroup:
+    every hand-over / halo / early-exit combination of the launch geometry, against the oracle."""
+    coeff, x, dy = make_inputs(B, H, L, seed=seed, stress=1.5)
+    print(f"sweep B={B} H={H} L={L} k={k} f32={f32} seed={seed}", flush=True)
+    out_dtype = torch.float32 if f32 else torch.bfloat16
+    y = run_forward(coeff, x, k=k, out_dtype=out_dtype)
+    atol, rtol = (F32_ATOL, F32_RTOL) if f32 else (BF16_ATOL, BF16_RTOL)
+    assert_close(f64(y), orc.forward(f64(coeff), f64(x), k=k), atol, rtol, "y")
+    if f32:
+        dy = dy.float()
+    c, xx, g = coeff.to(DEV), x.to(DEV), dy.to(DEV)
+    from spear_amd import _btp
+
+    dx = torch.full((B, H, 16, L), float("nan"), device=DEV, dtype=x.dtype)
+    dA = torch.full((B, H, L), float("nan"), device=DEV, dtype=torch.float32)
+    _btp.backward(c, xx, g, torch.empty((B, H, L // 16, 16), device=DEV), dx, dA, k, 32)
+    rdx, rdA = orc.backward(f64(coeff), f64(x), f64(dy), k=k)
+    assert_close(f64(dx), rdx, BF16_ATOL, BF16_RTOL, "dx")
+    assert_close(f64(dA), rdA, F32_ATOL * 10, F32_RTOL * 10, "dA")
