@@ -9,9 +9,10 @@
 // halo recompute as btp_scan.hip) with three additions: the epilogue y * C + V applied in
 // registers before the coalesced store, an optional carry into the first block, and the state a
 // decoder continues from (block-local state, in-block gate product, previous block's terminal
-// state) written by the 16 lanes that own the row's last step. A second, element-granular kernel
-// covers what the tiled one does not (fp32 tensors, row lengths that break 16-byte alignment,
-// other block lengths and head sizes).
+// state) written by the 16 lanes that own the row's last step. Prompts have any length, so rows
+// that are not 16-byte aligned are handled too, by realigning 32-bit words in registers. A second,
+// element-granular kernel covers what the tiled one does not (fp32 tensors, other block lengths and
+// head sizes).
 //
 // The step kernel is element-wise over [B, H, D]: a thread owns 8 consecutive channels of one head
 // (one 16-byte access per 16-bit operand), the per-head scalars are read by every thread of the
@@ -58,14 +59,18 @@ __device__ __forceinline__ void local_state_at(const float (&a)[32], const float
 }
 
 // ==========================================================================================
-// Prefill, tiled: 16-bit tensors, 16 channels, block length 16, L a multiple of 8
+// Prefill, tiled: 16-bit tensors, 16 channels, block length 16
 // ==========================================================================================
-template <class E, class C, bool kEpilogue, bool kStreamIn>
+// kAlign: what every channel row's start is aligned to, in bytes. 16: L is a multiple of 8 and every
+// pointer 16-byte aligned (16-byte accesses); 4 or 2: rows of any length (see
+// slab16_global_to_regs_ragged), starting on words when L is even and the tensors are word-aligned.
+template <class E, class C, bool kEpilogue, bool kStreamIn, int kAlign>
 __global__ __launch_bounds__(64 * kWaves) void jagged_prefill_kernel(
     const typename C::elem* __restrict__ coeff, const uint16_t* __restrict__ x, const uint16_t* __restrict__ cmul,
     const uint16_t* __restrict__ vadd, const void* __restrict__ carry_init, uint16_t* __restrict__ y,
     void* __restrict__ h_tail, void* __restrict__ r_tail, void* __restrict__ c_prev_tail, int state_dtype,
     int r_dtype, int L, int spans_per_row, long total_spans) {
+  constexpr bool kRagged = kAlign < 16;
   constexpr int kImages = kEpilogue ? 3 : 1;
   __shared__ __align__(16) unsigned char lds[kWaves][kImages * 4096 + kCoeffLdsBytes];
 
@@ -89,21 +94,39 @@ __global__ __launch_bounds__(64 * kWaves) void jagged_prefill_kernel(
   const int j = lane >> 4, d = lane & 15;
 
   uint4 xin[4], cin[4], vin[4];
-  slab16_global_to_regs<nt_loads(kStreamIn)>(x + slab_off, L, sc.nvalid, lane, xin);
-  const typename C::pair_t ain = coeff_global_to_reg<C>(arow, sc.nvalid, lane);
-  if constexpr (kEpilogue) {
-    slab16_global_to_regs<true>(cmul + slab_off, L, sc.nvalid, lane, cin);  // read once, by this span only
-    slab16_global_to_regs<true>(vadd + slab_off, L, sc.nvalid, lane, vin);
+  uint32_t xw[kRagged ? 16 : 1], cw[kRagged ? 16 : 1], vw[kRagged ? 16 : 1];  // the ragged path's words
+  uint32_t xe = 0u, ce = 0u, ve = 0u;
+  typename C::pair_t ain;
+  if constexpr (kRagged) {
+    slab16_global_to_regs_ragged<kAlign == 4>(x + slab_off, L, sc.nvalid, lane, xw, xe);
+    ain = coeff_global_to_reg_ragged<C>(arow, sc.nvalid, lane);
+    if constexpr (kEpilogue) {
+      slab16_global_to_regs_ragged<kAlign == 4>(cmul + slab_off, L, sc.nvalid, lane, cw, ce);
+      slab16_global_to_regs_ragged<kAlign == 4>(vadd + slab_off, L, sc.nvalid, lane, vw, ve);
+    }
+  } else {
+    slab16_global_to_regs<nt_loads(kStreamIn)>(x + slab_off, L, sc.nvalid, lane, xin);
+    ain = coeff_global_to_reg<C>(arow, sc.nvalid, lane);
+    if constexpr (kEpilogue) {
+      slab16_global_to_regs<true>(cmul + slab_off, L, sc.nvalid, lane, cin);  // read once, by this span only
+      slab16_global_to_regs<true>(vadd + slab_off, L, sc.nvalid, lane, vin);
+    }
   }
 
   float c_halo = 0.0f;
   if (j == 0) {
     if (sc.sp > 0 && !(kHandOver && wave > 0)) {  // local terminal state of the block left of the span, channel d
       float ah[16], xh[16];
-      C::load_block(arow - kTile, ah);
       const uint16_t* xp = x + slab_off + (long)d * L - kTile;
-      unpack8<E>(*reinterpret_cast<const uint4*>(xp), xh);
-      unpack8<E>(*reinterpret_cast<const uint4*>(xp + 8), xh + 8);
+      if constexpr (kRagged) {
+        C::load_block_ragged(arow - kTile, ah);
+        unpack8<E>(load16_plain_unaligned(xp), xh);
+        unpack8<E>(load16_plain_unaligned(xp + 8), xh + 8);
+      } else {
+        C::load_block(arow - kTile, ah);
+        unpack8<E>(*reinterpret_cast<const uint4*>(xp), xh);
+        unpack8<E>(*reinterpret_cast<const uint4*>(xp + 8), xh + 8);
+      }
       float h = 0.0f;
 #pragma unroll
       for (int r = 0; r < 16; ++r) h = fmaf(ah[r], h, xh[r]);
@@ -113,11 +136,22 @@ __global__ __launch_bounds__(64 * kWaves) void jagged_prefill_kernel(
     }
   }
 
-  slab16_regs_to_lds(img, lane, xin);
   coeff_reg_to_lds<C>(a_lds, lane, ain);
-  if constexpr (kEpilogue) {
-    slab16_regs_to_lds(img + 4096, lane, cin);
-    slab16_regs_to_lds(img + 8192, lane, vin);
+  if constexpr (kRagged) {
+    slab16_regs_realign<kAlign == 4>(x + slab_off, L, sc.nvalid, lane, xw, xe);
+    slab16_regs_to_lds_ragged(img, lane, xw);
+    if constexpr (kEpilogue) {
+      slab16_regs_realign<kAlign == 4>(cmul + slab_off, L, sc.nvalid, lane, cw, ce);
+      slab16_regs_to_lds_ragged(img + 4096, lane, cw);
+      slab16_regs_realign<kAlign == 4>(vadd + slab_off, L, sc.nvalid, lane, vw, ve);
+      slab16_regs_to_lds_ragged(img + 8192, lane, vw);
+    }
+  } else {
+    slab16_regs_to_lds(img, lane, xin);
+    if constexpr (kEpilogue) {
+      slab16_regs_to_lds(img + 4096, lane, cin);
+      slab16_regs_to_lds(img + 8192, lane, vin);
+    }
   }
   wave_lds_handover();
 
@@ -185,7 +219,8 @@ __global__ __launch_bounds__(64 * kWaves) void jagged_prefill_kernel(
   wave_lds_handover();
   lane_write16<E>(img, j, d, yv);
   wave_lds_handover();
-  slab16_lds_to_global<true>(img, y + slab_off, L, sc.nvalid, lane);
+  if constexpr (kRagged) slab16_lds_to_global_ragged<kAlign == 4>(img, y + slab_off, L, sc.nvalid, lane);
+  else slab16_lds_to_global<true>(img, y + slab_off, L, sc.nvalid, lane);
 }
 
 // ==========================================================================================
@@ -403,17 +438,29 @@ void launch_prefill_tiled(const JagPrefillArgs& p, hipStream_t s) {
   const auto* v = static_cast<const uint16_t*>(p.v);
   auto* y = static_cast<uint16_t*>(p.y);
   const bool st = stream_inputs(g);
-#define SPEAR_JAG_LAUNCH(EPI, ST)                                                                                  \
-  hipLaunchKernelGGL((jagged_prefill_kernel<E, C, EPI, ST>), dim3(g.blocks), dim3(64 * kWaves), 0, s, a, x, c, v, \
-                     p.carry_init, y, p.h_tail, p.r_tail, p.c_prev_tail, p.state_dtype, p.r_dtype, p.L,           \
+  auto word_aligned = [](const void* q) { return (reinterpret_cast<uintptr_t>(q) & 3u) == 0; };
+  const int align = (p.L % 8 == 0 && p.aligned) ? 16
+                    : (p.L % 2 == 0 && word_aligned(p.x) && word_aligned(p.c) && word_aligned(p.v) && word_aligned(p.y)) ? 4
+                                                                                                                        : 2;
+#define SPEAR_JAG_LAUNCH(EPI, ST, AL)                                                                         \
+  hipLaunchKernelGGL((jagged_prefill_kernel<E, C, EPI, ST, AL>), dim3(g.blocks), dim3(64 * kWaves), 0, s, a, x, \
+                     c, v, p.carry_init, y, p.h_tail, p.r_tail, p.c_prev_tail, p.state_dtype, p.r_dtype, p.L,   \
                      g.spans_per_row, g.total_spans)
-  if (p.c != nullptr) {
-    if (st) SPEAR_JAG_LAUNCH(true, true);
-    else SPEAR_JAG_LAUNCH(true, false);
-  } else {
-    if (st) SPEAR_JAG_LAUNCH(false, true);
-    else SPEAR_JAG_LAUNCH(false, false);
-  }
+#define SPEAR_JAG_BY_SPAN(EPI, AL) \
+  do {                             \
+    if (st) SPEAR_JAG_LAUNCH(EPI, true, AL); \
+    else SPEAR_JAG_LAUNCH(EPI, false, AL);   \
+  } while (0)
+#define SPEAR_JAG_BY_ALIGN(EPI)                       \
+  do {                                                \
+    if (align == 16) SPEAR_JAG_BY_SPAN(EPI, 16);      \
+    else if (align == 4) SPEAR_JAG_BY_SPAN(EPI, 4);   \
+    else SPEAR_JAG_BY_SPAN(EPI, 2);                   \
+  } while (0)
+  if (p.c != nullptr) SPEAR_JAG_BY_ALIGN(true);
+  else SPEAR_JAG_BY_ALIGN(false);
+#undef SPEAR_JAG_BY_ALIGN
+#undef SPEAR_JAG_BY_SPAN
 #undef SPEAR_JAG_LAUNCH
 }
 
@@ -434,7 +481,7 @@ void launch_prefill_any(const JagPrefillArgs& p, hipStream_t s) {
 bool jagged_prefill_is_tiled(const JagPrefillArgs& p) {
   const bool lin16 = !p.log_a && p.a_dtype == p.x_dtype;  // the reference's operand: a_t in the tensors' 16-bit type
   const bool log32 = p.log_a && p.a_dtype == kF32;        // fp32 log-space gate
-  return p.aligned && p.x_dtype != kF32 && p.D == kChan && p.block_len == kTile && p.L % 8 == 0 && (lin16 || log32);
+  return p.x_dtype != kF32 && p.D == kChan && p.block_len == kTile && (lin16 || log32);
 }
 
 hipError_t jagged_prefill(const JagPrefillArgs& p, hipStream_t s) {

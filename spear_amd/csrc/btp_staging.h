@@ -51,6 +51,13 @@ __device__ __forceinline__ void stream_store16(void* p, const uint4& q) {
   __builtin_nontemporal_store(v, reinterpret_cast<u32x4_t*>(p));
 }
 
+// 16 bytes from an address that is only 2-byte aligned (used by the row-of-any-length paths).
+typedef uint32_t u32x4_a2_t __attribute__((ext_vector_type(4), aligned(2)));
+__device__ __forceinline__ uint4 load16_plain_unaligned_fwd(const uint16_t* p) {
+  const u32x4_a2_t v = *reinterpret_cast<const u32x4_a2_t*>(p);
+  return make_uint4(v[0], v[1], v[2], v[3]);
+}
+
 // ---- coefficient sources --------------------------------------------------------------------
 // LinCoeff<E>: the reference's operand, linear-space decay a_t stored as a 16-bit float of the
 //              same type as x (spear/ops/btp/interface.py:164-188, csrc/btp/_bindings.cu:29-31).
@@ -73,6 +80,16 @@ struct LinCoeff {
   static __device__ __forceinline__ void load_block(const elem* p, float (&a)[16]) {
     unpack8<E>(*reinterpret_cast<const uint4*>(p), a);
     unpack8<E>(*reinterpret_cast<const uint4*>(p + 8), a + 8);
+#pragma unroll
+    for (int i = 0; i < 16; ++i) a[i] = clamp_coeff<E>(a[i]);
+  }
+  // element-aligned rows: a pair of which `n` (1 or 2) coefficients exist, and a whole block
+  static __device__ __forceinline__ pair_t load_pair_ragged(const elem* p, int n) {
+    return (uint32_t)p[0] | (n > 1 ? (uint32_t)p[1] << 16 : 0u);
+  }
+  static __device__ __forceinline__ void load_block_ragged(const elem* p, float (&a)[16]) {
+    unpack8<E>(load16_plain_unaligned_fwd(p), a);
+    unpack8<E>(load16_plain_unaligned_fwd(p + 8), a + 8);
 #pragma unroll
     for (int i = 0; i < 16; ++i) a[i] = clamp_coeff<E>(a[i]);
   }
@@ -100,6 +117,13 @@ struct LogCoeff {
       const float4 q = *reinterpret_cast<const float4*>(p + 4 * c);
       a[4 * c + 0] = decay(q.x); a[4 * c + 1] = decay(q.y); a[4 * c + 2] = decay(q.z); a[4 * c + 3] = decay(q.w);
     }
+  }
+  static __device__ __forceinline__ pair_t load_pair_ragged(const elem* p, int n) {
+    return make_float2(p[0], n > 1 ? p[1] : -INFINITY);
+  }
+  static __device__ __forceinline__ void load_block_ragged(const elem* p, float (&a)[16]) {
+#pragma unroll
+    for (int i = 0; i < 16; ++i) a[i] = decay(p[i]);
   }
 };
 
@@ -150,6 +174,110 @@ __device__ __forceinline__ void slab16_lds_to_global(const unsigned char* img, u
     const int r = it * 4 + lr;
     const uint4 v = *reinterpret_cast<const uint4*>(img + swz<256>(r, lp));
     if (ok) store16<kStream>(slab + (long)r * L + (lp << 3), v);
+  }
+}
+
+// ---- rows of any length and alignment (prompt prefill) --------------------------------------
+// The same slab movement for rows whose start is only element-aligned (L not a multiple of 8) and
+// whose last elements may stop anywhere. Under-aligned 16-byte accesses are served by the hardware
+// but measured 4x slower than aligned ones, so this path moves aligned 32-bit words instead: one
+// wave instruction covers one channel row of the span (64 lanes x 4 bytes = 128 steps). A row that
+// starts on an odd element is read as the aligned words around it and shifted by 16 bits in
+// registers; every word that is read contains at least one element of the row, so nothing outside
+// the row's own 4-byte blocks is touched, and stores never write an element that is not the row's.
+__device__ __forceinline__ uint4 load16_plain_unaligned(const uint16_t* p) { return load16_plain_unaligned_fwd(p); }
+
+// Step 1, all loads, no dependent work between them (so that a slab's 16 loads -- and those of the
+// other slabs -- are in flight together): q[r] = the aligned word `lane` of channel row r, i.e.
+// elements (2*lane, 2*lane+1) of the span if the row starts on a word and (2*lane-1, 2*lane) if it
+// starts on an odd element. `edge` (lanes 0..15, lane = row) is word 64 of the row, which only rows on
+// an odd element need. kWordRows: every row starts on a word (L even, word-aligned tensors).
+template <bool kWordRows>
+__device__ __forceinline__ void slab16_global_to_regs_ragged(const uint16_t* slab, long L, int nvalid, int lane,
+                                                             uint32_t (&q)[16], uint32_t& edge) {
+  // (pointer arithmetic, not an integer round trip: the compiler must keep seeing global memory)
+  auto words_of = [&](int r, int& last) {
+    const uint16_t* row = slab + (long)r * L;
+    const int odd = (int)((reinterpret_cast<uintptr_t>(row) >> 1) & 1);
+    last = odd ? (nvalid >> 1) : ((nvalid - 1) >> 1);  // last word that holds an element of the row
+    return reinterpret_cast<const uint32_t*>(row - odd);
+  };
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    int last;
+    const uint32_t* words = words_of(r, last);
+    q[r] = __builtin_nontemporal_load(words + min(lane, last));
+  }
+  edge = 0u;
+  if constexpr (!kWordRows) {
+    int last;
+    const uint32_t* words = words_of(lane & 15, last);
+    edge = words[min(64, last)];
+  }
+}
+
+// Step 2, in registers: shift the rows that start on an odd element by 16 bits (the upper neighbour
+// word comes from the next lane, for lane 63 from `edge`), and zero what lies beyond the row's end.
+template <bool kWordRows>
+__device__ __forceinline__ void slab16_regs_realign(const uint16_t* slab, long L, int nvalid, int lane,
+                                                    uint32_t (&q)[16], uint32_t edge) {
+  const int e = lane << 1;
+  const uint32_t keep = e + 1 < nvalid ? 0xffffffffu : (e < nvalid ? 0x0000ffffu : 0u);
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    uint32_t w = q[r];
+    if constexpr (!kWordRows) {
+      const bool odd = (reinterpret_cast<uintptr_t>(slab + (long)r * L) >> 1) & 1;  // wave-uniform
+      // the word held by lane + 1: a whole-wavefront DPP shift (wave_shl:1), no LDS traffic
+      const uint32_t up = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)w, 0x130, 0xF, 0xF, false);
+      const uint32_t w64 = (uint32_t)__builtin_amdgcn_readlane((int)edge, r);
+      const uint32_t w1 = lane == 63 ? w64 : up;
+      w = odd ? (w >> 16) | (w1 << 16) : w;
+    }
+    q[r] = w & keep;
+  }
+}
+
+__device__ __forceinline__ void slab16_regs_to_lds_ragged(unsigned char* img, int lane, const uint32_t (&q)[16]) {
+#pragma unroll
+  for (int r = 0; r < 16; ++r)
+    *reinterpret_cast<uint32_t*>(img + swz<256>(r, lane >> 2) + ((lane & 3) << 2)) = q[r];
+}
+
+// Image -> global. Whole aligned words first (for a row on an odd element, memory word i holds the
+// high half of lane i-1's image word and the low half of lane i's); the one or two elements per row
+// that no whole word covers are then written by lanes 0..31 acting as per-row workers.
+template <bool kWordRows>
+__device__ __forceinline__ void slab16_lds_to_global_ragged(const unsigned char* img, uint16_t* slab, long L,
+                                                            int nvalid, int lane) {
+  const int e = lane << 1;
+  auto image_word = [&](int r, int i) {
+    return *reinterpret_cast<const uint32_t*>(img + swz<256>(r, i >> 2) + ((i & 3) << 2));
+  };
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    uint16_t* row = slab + (long)r * L;
+    const bool odd = !kWordRows && ((reinterpret_cast<uintptr_t>(row) >> 1) & 1);  // wave-uniform
+    const uint32_t w = image_word(r, lane);
+    const uint32_t below = image_word(r, (lane + 63) & 63);
+    const uint32_t mw = odd ? (below >> 16) | (w << 16) : w;
+    // row on a word: lane covers (e, e+1); on an odd element: (e-1, e), lane 0 has no whole word
+    const bool whole = odd ? (lane > 0 && e < nvalid) : (e + 1 < nvalid);
+    if (whole) __builtin_nontemporal_store(mw, reinterpret_cast<uint32_t*>(row + e - (odd ? 1 : 0)));
+  }
+  if (lane < 32) {
+    const int r = lane & 15;
+    uint16_t* row = slab + (long)r * L;
+    const bool odd = !kWordRows && ((reinterpret_cast<uintptr_t>(row) >> 1) & 1);
+    // lanes 0..15: first element of a row on an odd element; lanes 16..31: the last element when no
+    // whole word reaches it (even count on an odd start, odd count on a word start)
+    const bool first = lane < 16;
+    const int t = first ? 0 : nvalid - 1;
+    const bool need = first ? (odd && nvalid > 0) : (nvalid > 0 && ((nvalid & 1) != (odd ? 1 : 0)) && !(odd && nvalid == 1));
+    if (need) {
+      const uint32_t w = image_word(r, t >> 1);
+      row[t] = (uint16_t)(t & 1 ? w >> 16 : w);
+    }
   }
 }
 
@@ -226,6 +354,14 @@ __device__ __forceinline__ void lane_write32(unsigned char* img, int j, int d, c
 template <class C>
 __device__ __forceinline__ typename C::pair_t coeff_global_to_reg(const typename C::elem* arow, int nvalid, int lane) {
   return ((lane << 1) < nvalid) ? C::load_pair(arow + (lane << 1)) : C::zero_pair();
+}
+
+// rows of any length: element-aligned address, and the last pair may hold a single coefficient
+template <class C>
+__device__ __forceinline__ typename C::pair_t coeff_global_to_reg_ragged(const typename C::elem* arow, int nvalid,
+                                                                          int lane) {
+  const int n = nvalid - (lane << 1);
+  return n > 0 ? C::load_pair_ragged(arow + (lane << 1), n) : C::zero_pair();
 }
 
 // The second half of the span is stored 16 floats further on, so that the four lane groups, which

@@ -297,3 +297,36 @@ def test_one_block_period_of_decode_steps_replays_as_a_hip_graph():
         torch.cuda.synchronize()
         got = f64(y_buf).transpose(1, 2, 3, 0)  # [B, H, D, token]
         assert_close(got, rY[..., p * bl:(p + 1) * bl], BF16_ATOL, BF16_RTOL, f"period {p}")
+
+
+@pytest.mark.parametrize("offset", [0, 1, 2, 3], ids=lambda o: f"off{o}")
+@pytest.mark.parametrize("L", [1, 2, 3, 7, 9, 15, 17, 31, 33, 126, 127, 129, 130, 255, 257, 1037])
+def test_prefill_rows_of_any_length_and_alignment(L, offset):
+    """Prompt lengths that are not a multiple of 8 and tensors that start on any 2-byte boundary: the
+    tiled kernel realigns rows in registers. Output and state against the oracle, and the elements
+    around the output tensor must stay untouched."""
+    from spear_amd import _btp
+
+    B, H, D = 2, 3, 16
+    A, X, C, V = make(B, H, D, L, seed=7000 + L)
+
+    def shifted(t):  # the same values in a buffer that starts `offset` elements into an allocation
+        buf = torch.full((t.numel() + 16,), float("nan"), dtype=t.dtype, device=DEV)
+        view = buf[offset:offset + t.numel()].view(t.shape)
+        view.copy_(t)
+        return buf, view
+
+    (_, a), (_, x), (_, c), (_, v) = (shifted(t) for t in (A, X, C, V))
+    ybuf, y = shifted(torch.full(X.shape, float("nan"), dtype=X.dtype))
+    h, cp = (torch.full((B, H, D), float("nan"), device=DEV) for _ in range(2))
+    r = torch.full((B, H), float("nan"), device=DEV)
+    print(f"ragged prefill L={L} offset={offset}", flush=True)
+    _btp.jagged_prefill(a, x, c, v, None, y, h, r, cp, 16, False)
+    torch.cuda.synchronize()
+    rY, rst = jag.prefill(f64(A), f64(X), f64(C), f64(V), block_len=16)
+    assert_close(f64(y), rY, BF16_ATOL, BF16_RTOL, "Y")
+    assert_close(f64(h), rst.h_loc, F32_ATOL, F32_RTOL, "h_loc")
+    assert_close(f64(cp), rst.c_prev_loc, F32_ATOL, F32_RTOL, "c_prev_loc")
+    assert_close(f64(r), rst.r_pref, F32_ATOL, F32_RTOL, "r_pref")
+    guard = torch.cat([ybuf[:offset], ybuf[offset + X.numel():]])
+    assert bool(torch.isnan(guard).all()), "elements outside the output tensor were written"
