@@ -124,9 +124,9 @@ int spear_phalanx_mix_backward(const void* a_logit, const void* b_logit, const v
  * block-local state, r_tail the in-block gate product (1 when L ends a block), c_prev_tail the terminal
  * local state of the last completed block. The three state pointers are given together or all NULL.
  * Any L >= 0, D > 0, block_len > 0, pointers aligned to their element size. 16-bit tensors with D = 16,
- * block_len = 16 and either a in x_dtype (linear) or fp32 log(a_t) run the tiled kernel (HBM-bound; rows
+ * block_len = 16 and a in x_dtype (a_t or log a_t) or fp32 log(a_t) run the tiled kernel (HBM-bound; rows
  * whose length is not a multiple of 8 or that are not 16-byte aligned are realigned in registers, at
- * 0.5-0.65 of peak instead of 0.75); everything else (fp32 tensors, other D / block_len, 16-bit log(a_t))
+ * 0.5-0.65 of peak instead of 0.75); everything else (fp32 tensors, other D / block_len, fp32 linear a_t)
  * runs an element-granular kernel. */
 int spear_jagged_prefill(const void* a, const void* x, const void* c, const void* v, const void* carry_init, void* y,
                          void* h_tail, void* r_tail, void* c_prev_tail, int B, int H, int D, int L, int block_len,

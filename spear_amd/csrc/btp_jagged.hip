@@ -479,19 +479,21 @@ void launch_prefill_any(const JagPrefillArgs& p, hipStream_t s) {
 }  // namespace
 
 bool jagged_prefill_is_tiled(const JagPrefillArgs& p) {
-  const bool lin16 = !p.log_a && p.a_dtype == p.x_dtype;  // the reference's operand: a_t in the tensors' 16-bit type
-  const bool log32 = p.log_a && p.a_dtype == kF32;        // fp32 log-space gate
-  return p.x_dtype != kF32 && p.D == kChan && p.block_len == kTile && (lin16 || log32);
+  const bool own16 = p.a_dtype == p.x_dtype;        // a_t or log(a_t) in the tensors' 16-bit type
+  const bool log32 = p.log_a && p.a_dtype == kF32;  // fp32 log-space gate
+  return p.x_dtype != kF32 && p.D == kChan && p.block_len == kTile && (own16 || log32);
 }
 
 hipError_t jagged_prefill(const JagPrefillArgs& p, hipStream_t s) {
   if (jagged_prefill_is_tiled(p)) {
     if (p.x_dtype == kBf16) {
-      if (p.log_a) launch_prefill_tiled<Bf16, LogCoeff>(p, s);
-      else launch_prefill_tiled<Bf16, LinCoeff<Bf16>>(p, s);
+      if (!p.log_a) launch_prefill_tiled<Bf16, LinCoeff<Bf16>>(p, s);
+      else if (p.a_dtype == kF32) launch_prefill_tiled<Bf16, LogCoeff>(p, s);
+      else launch_prefill_tiled<Bf16, LogCoeff16<Bf16>>(p, s);
     } else {
-      if (p.log_a) launch_prefill_tiled<Fp16, LogCoeff>(p, s);
-      else launch_prefill_tiled<Fp16, LinCoeff<Fp16>>(p, s);
+      if (!p.log_a) launch_prefill_tiled<Fp16, LinCoeff<Fp16>>(p, s);
+      else if (p.a_dtype == kF32) launch_prefill_tiled<Fp16, LogCoeff>(p, s);
+      else launch_prefill_tiled<Fp16, LogCoeff16<Fp16>>(p, s);
     }
   } else if (p.x_dtype == kBf16) {
     launch_prefill_any<Bf16>(p, s);

@@ -127,6 +127,38 @@ struct LogCoeff {
   }
 };
 
+// Log-space gate stored in the tensors' own 16-bit type (prompt prefill with use_log_a on 16-bit
+// tensors, spear/nn/phalanx/inference.py:296): a_t = exp(g_t) formed in fp32.
+template <class E>
+struct LogCoeff16 {
+  typedef uint16_t elem;
+  typedef uint32_t pair_t;
+  static constexpr bool kLog = true;
+  static __device__ __forceinline__ uint32_t minus_inf() { return E::pack2(-INFINITY, -INFINITY); }
+  static __device__ __forceinline__ pair_t load_pair(const elem* p) {
+    return __builtin_nontemporal_load(reinterpret_cast<const uint32_t*>(p));
+  }
+  static __device__ __forceinline__ pair_t zero_pair() { return minus_inf(); }
+  static __device__ __forceinline__ float2 to_float(pair_t w) {
+    return make_float2(LogCoeff::decay(E::lo(w)), LogCoeff::decay(E::hi(w)));
+  }
+  static __device__ __forceinline__ void load_block(const elem* p, float (&a)[16]) {
+    unpack8<E>(*reinterpret_cast<const uint4*>(p), a);
+    unpack8<E>(*reinterpret_cast<const uint4*>(p + 8), a + 8);
+#pragma unroll
+    for (int i = 0; i < 16; ++i) a[i] = LogCoeff::decay(a[i]);
+  }
+  static __device__ __forceinline__ pair_t load_pair_ragged(const elem* p, int n) {
+    return (uint32_t)p[0] | (n > 1 ? (uint32_t)p[1] << 16 : minus_inf() & 0xffff0000u);
+  }
+  static __device__ __forceinline__ void load_block_ragged(const elem* p, float (&a)[16]) {
+    unpack8<E>(load16_plain_unaligned_fwd(p), a);
+    unpack8<E>(load16_plain_unaligned_fwd(p + 8), a + 8);
+#pragma unroll
+    for (int i = 0; i < 16; ++i) a[i] = LogCoeff::decay(a[i]);
+  }
+};
+
 // ------------------------------------------------------------------------------------------
 // Stage a [16 x 128] slab of 16-bit elements: coalesced global reads -> swizzled LDS image.
 // Lane l of pass `it` handles channel row 4*it + l/16, chunk l%16 (8 steps).

@@ -78,6 +78,7 @@ ANY = [  # B, H, D, L, block_len, dtype, a_dtype, log_a
     (1, 2, 16, 64, 16, torch.float32, None, False),       # fp32 tensors
     (2, 2, 16, 50, 16, torch.float32, None, True),
     (1, 2, 16, 48, 16, torch.bfloat16, None, True),       # 16-bit log gate
+    (2, 2, 16, 203, 16, torch.float16, None, True),       # 16-bit log gate, odd length, two spans
     (1, 2, 16, 48, 16, torch.bfloat16, torch.float32, False),  # fp32 linear gate with 16-bit tensors
     (2, 3, 8, 45, 4, torch.bfloat16, None, False),        # other block length and head size
     (1, 2, 3, 23, 5, torch.float32, None, False),
