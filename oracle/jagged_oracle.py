@@ -9,17 +9,18 @@ What follows what (paths relative to the reference repository):
                                                           which is the same update without ``* C + V``)
     prefill()     spear/nn/phalanx/inference.py:281-360  parallel_jagged: outputs and the hand-over state
 
-How each is pinned (tests/test_jagged_oracle.py), without importing the reference:
+How each is pinned (tests/test_jagged_oracle.py); none of the tests imports the reference:
     sequential    equals the committed closed-form vectors at block length 16 and a windowed brute-force
                   sum at other block lengths; carry_init equals cutting a longer sequence
     step          N steps from the zero state equal sequential() * C + V across block boundaries, in
                   linear and in log-r mode
     prefill       Y equals sequential() * C + V; the state is pinned by continuing: prefill(L) followed
                   by steps equals prefill(L + n) whenever L is not a multiple of the block length.
-    PARITY UNPINNED: the state prefill() returns when L IS a multiple of the block length. The
-                  reference then hands over h_loc = the last block's terminal local state instead of
-                  zero (inference.py:327-341), which no identity fixes (stepping from it counts that
-                  state twice). It is restated from the text and exercised, not proved.
+                  When L IS a multiple of the block length the reference hands over h_loc = the last
+                  block's terminal local state instead of zero (inference.py:327-341), which no
+                  identity fixes (stepping from it counts that state twice); that case, like the others,
+                  is pinned by vectors computed with the reference's own parallel_jagged / step_jagged
+                  (tests/golden/make_jagged_vectors.py -> jagged_reference_vectors.npz).
 """
 
 from __future__ import annotations

@@ -64,3 +64,16 @@ def golden_vectors():
         case, rest = key.split(".", 1)
         out.setdefault(case, {})[rest] = blob[key][None]  # add the batch axis
     return out
+
+
+def jagged_reference_vectors():
+    """Vectors written by tests/golden/make_jagged_vectors.py from the reference's own streaming
+    functions: {case: {name: array}}; ``meta`` = (prompt length, block length, decode steps, state.i)."""
+    import pathlib
+
+    blob = np.load(pathlib.Path(__file__).with_name("golden") / "jagged_reference_vectors.npz")
+    out: dict = {}
+    for key in blob.files:
+        case, rest = key.split(".", 1)
+        out.setdefault(case, {})[rest] = blob[key]
+    return out

@@ -331,3 +331,30 @@ def test_prefill_rows_of_any_length_and_alignment(L, offset):
     assert_close(f64(r), rst.r_pref, F32_ATOL, F32_RTOL, "r_pref")
     guard = torch.cat([ybuf[:offset], ybuf[offset + X.numel():]])
     assert bool(torch.isnan(guard).all()), "elements outside the output tensor were written"
+
+
+@pytest.mark.parametrize("case", ["full", "ragged", "short", "one_block", "bl4"])
+def test_kernels_match_the_reference_vectors(case):
+    """The HIP prefill and decode kernels against vectors computed by the reference's own
+    parallel_jagged / step_jagged (tests/golden/make_jagged_vectors.py), including the state handed
+    over after a full last block and the steps taken from it."""
+    from helpers import jagged_reference_vectors
+    from spear_amd.nn.phalanx.inference import parallel_jagged, step_jagged
+
+    v = jagged_reference_vectors()[case]
+    L, bl, steps, i_ref = (int(t) for t in v["meta"])
+    A, X, C, V = (torch.from_numpy(v[n]).bfloat16().to(DEV) for n in "AXCV")
+    for n, t in zip("AXCV", (A, X, C, V)):
+        assert np.array_equal(f64(t), v[n].astype(np.float64)), f"{n} is not bfloat16-exact"
+    print(f"reference vectors {case}", flush=True)
+    Y, st = parallel_jagged(A[..., :L].contiguous(), X[..., :L].contiguous(), C[..., :L].contiguous(),
+                            V[..., :L].contiguous(), block_len=bl, state_dtype=torch.float32)
+    assert_close(f64(Y), v["Y"], BF16_ATOL, BF16_RTOL, "Y")
+    assert st.i == i_ref
+    assert_close(f64(st.h_loc), v["h_loc"], F32_ATOL, F32_RTOL, "h_loc")
+    assert_close(f64(st.r_pref), v["r_pref"], F32_ATOL, F32_RTOL, "r_pref")
+    assert_close(f64(st.c_prev_loc), v["c_prev_loc"], F32_ATOL, F32_RTOL, "c_prev_loc")
+    for k in range(steps):
+        t = L + k
+        y, st = step_jagged(A[:, :, t].float(), X[..., t], C[..., t], V[..., t], st, inplace=True)
+        assert_close(f64(y), v["y_steps"][..., k], BF16_ATOL, BF16_RTOL, f"decode step {k}")

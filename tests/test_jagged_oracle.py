@@ -105,7 +105,8 @@ def test_decoding_continues_a_prefill_that_ends_inside_a_block(bl, L, n):
 
 def test_prefill_state_after_a_full_block_follows_the_reference_text():
     # inference.py:327-341: carry snapshot taken and gate product reset, but h_loc keeps the block's
-    # terminal local state; a step from that state therefore counts it twice. Restated, not derived.
+    # terminal local state; a step from that state therefore counts it twice. (The same case against
+    # the reference's own output: test_oracle_reproduces_the_reference_vectors[full].)
     bl, L = 4, 8
     a, x, c, v = _rand(1, 2, 3, L + 1, seed=3)
     _, st = jag.prefill(a[..., :L], x[..., :L], c[..., :L], v[..., :L], block_len=bl)
@@ -118,3 +119,28 @@ def test_prefill_state_after_a_full_block_follows_the_reference_text():
     np.testing.assert_allclose(st.r_pref, 1.0)
     y, _ = jag.step(a[:, :, L], x[..., L], c[..., L], v[..., L], st)
     np.testing.assert_allclose(y, (x[..., L] + 2 * a[:, :, L, None] * h_last) * c[..., L] + v[..., L], rtol=1e-12)
+
+
+# ---- vectors from the reference's own functions ------------------------------------------------------
+@pytest.mark.parametrize("case", ["full", "ragged", "short", "one_block", "bl4"])
+def test_oracle_reproduces_the_reference_vectors(case):
+    """Prefill output, hand-over state (also after a full last block, the case no identity pins) and the
+    decode steps taken from that state, against vectors computed by the reference's parallel_jagged /
+    step_jagged in float64 (tests/golden/make_jagged_vectors.py)."""
+    from helpers import jagged_reference_vectors
+
+    v = jagged_reference_vectors()[case]
+    L, bl, steps, i_ref = (int(t) for t in v["meta"])
+    A, X, C, V = (v[n].astype(np.float64) for n in "AXCV")
+    Y, st = jag.prefill(A[..., :L], X[..., :L], C[..., :L], V[..., :L], block_len=bl)
+    np.testing.assert_allclose(Y, v["Y"], rtol=1e-12, atol=1e-13)
+    assert st.i == i_ref
+    np.testing.assert_allclose(st.h_loc, v["h_loc"], rtol=1e-12, atol=1e-13)
+    np.testing.assert_allclose(st.r_pref, v["r_pref"], rtol=1e-12, atol=1e-13)
+    np.testing.assert_allclose(st.c_prev_loc, v["c_prev_loc"], rtol=1e-12, atol=1e-13)
+    for k in range(steps):
+        t = L + k
+        y, st = jag.step(A[:, :, t], X[..., t], C[..., t], V[..., t], st)
+        np.testing.assert_allclose(y, v["y_steps"][..., k], rtol=1e-11, atol=1e-12)
+    final = np.concatenate([st.h_loc.ravel(), st.r_pref.ravel(), st.c_prev_loc.ravel(), [st.i]])
+    np.testing.assert_allclose(final, v["final"], rtol=1e-11, atol=1e-12)
