@@ -93,3 +93,22 @@ def test_torch_port_matches_committed_closed_form_vectors(fn, case):
     np.testing.assert_allclose(y.detach().numpy(), v["k2.y"], rtol=1e-10, atol=1e-11)
     np.testing.assert_allclose(x.grad.numpy(), v["k2.dx"], rtol=1e-10, atol=1e-11)
     np.testing.assert_allclose(a.grad.numpy(), v["k2.dA"], rtol=1e-8, atol=1e-9)
+
+
+@pytest.mark.parametrize("name", ["log", "linspace"])
+def test_cpu_path_matches_vectors_from_the_reference_cpu_path(name):
+    """The bfloat16 and float32 CPU paths against outputs of the reference's own functions
+    (tests/golden/make_cpu_path_vectors.py). On the machine that wrote the vectors the results are
+    bit-identical; the assertion allows one unit in the last place of the dtype, because another CPU's
+    matmul kernels may sum in another order."""
+    import pathlib
+
+    v = np.load(pathlib.Path(__file__).with_name("golden") / "cpu_path_reference_vectors.npz")
+    fn = {"log": ref.block_two_pass_log, "linspace": ref.block_two_pass_linspace}[name]
+    a, x = torch.from_numpy(v["a"]).bfloat16(), torch.from_numpy(v["x"]).bfloat16()
+    y16 = fn(a, x, 16).float().numpy()
+    y32 = fn(a.float(), x.float(), 16).numpy()
+    np.testing.assert_allclose(y16, v[f"{name}.bf16"], rtol=2.0 ** -7, atol=2.0 ** -9)
+    np.testing.assert_allclose(y32, v[f"{name}.f32"], rtol=2e-6, atol=1e-6)
+    y64 = ref.block_two_pass_ref(a.double(), x.double()).numpy()
+    np.testing.assert_allclose(y64, v["ref.f64"], rtol=1e-14, atol=1e-15)
