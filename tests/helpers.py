@@ -77,3 +77,21 @@ def jagged_reference_vectors():
         case, rest = key.split(".", 1)
         out.setdefault(case, {})[rest] = blob[key]
     return out
+
+
+def layer_reference_vectors():
+    """Configuration 1 computed by the reference's own layer on its CPU path
+    (tests/golden/make_layer_vectors.py)."""
+    import pathlib
+
+    return np.load(pathlib.Path(__file__).with_name("golden") / "layer_reference_vectors.npz")
+
+
+def config1_layer_and_input(method: str, device="cpu"):
+    """The layer and input of configuration 1, drawn exactly as the vectors' generator draws them."""
+    from spear_amd import Phalanx
+
+    torch.manual_seed(0)
+    layer = Phalanx(dim=512, length=128, method=method, dtype=torch.bfloat16)
+    x = torch.randn(8, 128, 512).to(torch.bfloat16)
+    return layer.to(device), x.to(device)

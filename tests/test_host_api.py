@@ -2,6 +2,7 @@
 csrc/btp/_bindings.cu:19-60 and spear/ops/btp/interface.py:137-139 of the reference), the
 registered custom ops, the package surface, and the Phalanx layer's construction rules."""
 
+import numpy as np
 import pytest
 import torch
 
@@ -294,3 +295,23 @@ def test_streaming_module_surface_and_state_dataclass():
         inf.parallel_jagged(torch.ones(1, 2, 8), *(torch.zeros(1, 2, 3, 8) for _ in range(3)), block_len=4)
     with pytest.raises(AssertionError):
         inf.jagged_band_infer_sequential(torch.zeros(1, 2, 3, 8), torch.ones(1, 2, 7), 4)
+
+
+def test_config1_cpu_path_reproduces_the_reference_layer():
+    """Default initialisation draws the same weights in the same order as the reference's layer, and the
+    bfloat16 CPU path gives the reference's output (bit-identical on the machine that wrote the vectors;
+    one unit in the last place is allowed for another CPU's matmul kernels)."""
+    from helpers import config1_layer_and_input, layer_reference_vectors
+
+    v = layer_reference_vectors()
+    layer, x = config1_layer_and_input("pytorch")
+    assert np.array_equal(v["x.sums"], [x.double().sum().item(), x.double().square().sum().item()])
+    for name, p in layer.state_dict().items():
+        d, want = p.double(), v[f"param.{name}"]
+        got = np.concatenate([[float(n) for n in p.shape] + [0.0] * (2 - p.dim()),
+                              [d.sum().item(), d.square().sum().item()], d.flatten()[:8].numpy()])
+        assert np.array_equal(got, want), f"{name}: default initialisation differs from the reference's"
+    with torch.no_grad():
+        y = layer(x)
+    assert y.dtype == torch.bfloat16 and bool(v["y.dtype_is_bf16"][0])
+    np.testing.assert_allclose(y[:, ::8, :].float().numpy(), v["y.every8"], rtol=2.0 ** -7, atol=2.0 ** -8)

@@ -185,6 +185,24 @@ def test_config1_layer_forward_hip_vs_cpu_pytorch_path():
     assert_close(f64(y_gpu), f64(y_cpu), 2e-2, 2e-2, "layer y")
 
 
+@pytest.mark.parametrize("method", ["default", "fused"])
+def test_config1_layer_on_the_gpu_against_the_reference_cpu_output(method):
+    """Configuration 1 end to end: same seed, hence the reference's default weights and input; the HIP
+    methods on the GPU against the output of the reference's own layer on its CPU path
+    (tests/golden/make_layer_vectors.py), within the reference's layer limits and 2e-2."""
+    from helpers import config1_layer_and_input, layer_reference_vectors
+    from spear_amd.testing.numerics import compute_error_metrics
+
+    v = layer_reference_vectors()
+    layer, x = config1_layer_and_input(method, device=DEV)
+    with torch.no_grad():
+        y = layer(x)
+    got, want = y[:, ::8, :].float().cpu(), torch.from_numpy(v["y.every8"])
+    m = compute_error_metrics(got, want)
+    assert m["max_abs"] <= 1e-1 and m["mean_abs"] <= 1e-2 and m["rmse"] <= 5e-2, m  # tests/phalanx/test_phalanx_numerics.py:41-47
+    assert_close(f64(got), f64(want), 2e-2, 2e-2, f"y ({method})")
+
+
 @pytest.mark.parametrize("kv_heads", [None, 4])
 def test_layer_methods_agree_forward_and_backward(kv_heads):
     from spear_amd.nn.phalanx.runners import compare_layer_gradients, compare_layer_outputs, create_phalanx_layers, sample_layer_inputs
