@@ -191,3 +191,15 @@ def test_oracle_reproduces_committed_closed_form_vectors(case, k):
     dx, dA = orc.backward(a, x, dy, k=k)
     np.testing.assert_allclose(dx, v[f"k{k}.dx"], rtol=1e-11, atol=1e-12)
     np.testing.assert_allclose(dA, v[f"k{k}.dA"], rtol=1e-10, atol=1e-11)
+
+
+def test_oracle_matches_the_reference_float64_path_vectors():
+    """The C oracle against the output of the reference's own block_two_pass_ref in float64
+    (tests/golden/make_cpu_path_vectors.py)."""
+    import pathlib
+
+    v = np.load(pathlib.Path(__file__).with_name("golden") / "cpu_path_reference_vectors.npz")
+    a, x = v["a"].astype(np.float64), v["x"].astype(np.float64)
+    for mode in (orc.L_PRODUCT, orc.L_LOGSUM, orc.L_CUMPROD):
+        np.testing.assert_allclose(orc.forward(a, x, k=2, l_mode=mode), v["ref.f64"], rtol=1e-12, atol=1e-13)
+    np.testing.assert_allclose(orc.forward_sequential(a, x, k=2), v["ref.f64"], rtol=1e-12, atol=1e-13)
