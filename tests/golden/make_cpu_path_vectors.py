@@ -1,5 +1,6 @@
 """Writes cpu_path_reference_vectors.npz beside this file: outputs of the reference's CPU path
-(spear/ops/btp/reference.py: block_two_pass_log / _linspace / _ref) in the dtypes the layer uses.
+(spear/ops/btp/reference.py: block_two_pass_log / _linspace / _ref) in the dtypes the layer uses, and
+the float64 gradients its harness compares kernels with.
 
 What the mathematics pins about these functions is checked elsewhere against the float64 oracle; what
 it cannot pin is the exact sequence of roundings of the bfloat16 path (log -> repeat -> masked_fill ->
@@ -42,6 +43,12 @@ def main() -> None:
         blob[f"{name}.bf16"] = fn(a, x, 16).float().numpy()
         blob[f"{name}.f32"] = fn(a.float(), x.float(), 16).numpy()
     blob["ref.f64"] = ref.block_two_pass_ref(a.double(), x.double()).numpy()
+    # gradients the way the reference's harness takes them (spear/ops/btp/runners.py:152-164): autograd
+    # through the float64 path, upstream gradient rounded to bfloat16
+    dy = torch.randn(B, H, 16, L, generator=g).to(torch.bfloat16)
+    a64, x64 = a.double().requires_grad_(True), x.double().requires_grad_(True)
+    ref.block_two_pass_ref(a64, x64).backward(dy.double())
+    blob.update({"dy": dy.float().numpy(), "ref.f64.dx": x64.grad.numpy(), "ref.f64.dA": a64.grad.numpy()})
     path = pathlib.Path(__file__).with_name("cpu_path_reference_vectors.npz")
     np.savez_compressed(path, **blob)
     print(f"wrote {path} ({path.stat().st_size} bytes)")

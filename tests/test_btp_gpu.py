@@ -260,3 +260,17 @@ def test_forward_and_backward_on_odd_launch_shapes(B, H, L, k, f32, seed):
     rdx, rdA = orc.backward(f64(coeff), f64(x), f64(dy), k=k)
     assert_close(f64(dx), rdx, BF16_ATOL, BF16_RTOL, "dx")
     assert_close(f64(dA), rdA, F32_ATOL * 10, F32_RTOL * 10, "dA")
+
+
+def test_kernels_match_the_reference_float64_path_vectors():
+    """Forward and backward kernels against y, dx, dA computed by the reference's own float64 path and
+    autograd (tests/golden/make_cpu_path_vectors.py)."""
+    import pathlib
+
+    v = np.load(pathlib.Path(__file__).with_name("golden") / "cpu_path_reference_vectors.npz")
+    coeff, x, dy = (torch.from_numpy(v[n]).bfloat16() for n in ("a", "x", "dy"))
+    assert_close(f64(run_forward(coeff, x)), v["ref.f64"], BF16_ATOL, BF16_RTOL, "y bf16")
+    assert_close(f64(run_forward(coeff, x, out_dtype=torch.float32)), v["ref.f64"], F32_ATOL, F32_RTOL, "y fp32")
+    dx, dA = run_backward(coeff, x, dy)
+    assert_close(f64(dx), v["ref.f64.dx"], BF16_ATOL, BF16_RTOL, "dx")
+    assert_close(f64(dA), v["ref.f64.dA"], F32_ATOL * 10, F32_RTOL * 10, "dA")

@@ -203,3 +203,6 @@ def test_oracle_matches_the_reference_float64_path_vectors():
     for mode in (orc.L_PRODUCT, orc.L_LOGSUM, orc.L_CUMPROD):
         np.testing.assert_allclose(orc.forward(a, x, k=2, l_mode=mode), v["ref.f64"], rtol=1e-12, atol=1e-13)
     np.testing.assert_allclose(orc.forward_sequential(a, x, k=2), v["ref.f64"], rtol=1e-12, atol=1e-13)
+    dx, dA = orc.backward(a, x, v["dy"].astype(np.float64), k=2)
+    np.testing.assert_allclose(dx, v["ref.f64.dx"], rtol=1e-11, atol=1e-12)
+    np.testing.assert_allclose(dA, v["ref.f64.dA"], rtol=1e-10, atol=1e-11)
