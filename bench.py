@@ -233,6 +233,21 @@ def main() -> int:
         lib.spear_btp_copy(s["x"].data_ptr(), s["dx"].data_ptr(), ctypes.c_ulonglong(nbytes), sp)
     copy_ms = kernel_ms(copy)
 
+    # the operator's own access shape and cache policy without its arithmetic: 4 KiB per wavefront,
+    # non-temporal loads and stores; one input (copy) and two inputs (the backward kernel's mix)
+    def probe_copy(s):
+        rc = lib.spear_btp_stream_probe(s["x"].data_ptr(), None, s["dx"].data_ptr(), ctypes.c_ulonglong(nbytes), sp)
+        assert rc == 0, lib.spear_btp_last_error()
+
+    def probe_2r1w(s):
+        rc = lib.spear_btp_stream_probe(s["x"].data_ptr(), s["dy"].data_ptr(), s["dx"].data_ptr(),
+                                        ctypes.c_ulonglong(nbytes), sp)
+        assert rc == 0, lib.spear_btp_last_error()
+
+    probe_copy_ms, probe_2r1w_ms = kernel_ms(probe_copy), kernel_ms(probe_2r1w)
+    ceil_copy = 2 * nbytes / (probe_copy_ms * 1e-3) / 1e9
+    ceil_2r1w = 3 * nbytes / (probe_2r1w_ms * 1e-3) / 1e9
+
     # log-space gate entry points on the same shape (fp32 gate in, fp32 dgate out: 68 + 108 B per unit)
     for s_ in sets:
         s_["gate"] = torch.log(s_["coeff"].float()).contiguous()
@@ -491,6 +506,13 @@ def main() -> int:
         "step_spread": spread,
         "copy_kernel": {"avg_launch_ms": copy_ms, "achieved": 2 * nbytes / (copy_ms * 1e-3) / 1e9,
                         "bytes_moved": 2 * nbytes},
+        "ceilings": {
+            "what": "same 4 KiB-per-wavefront non-temporal access shape as the kernels, no arithmetic, same buffers",
+            "nt_copy_1r1w": {"avg_launch_ms": probe_copy_ms, "achieved": ceil_copy, "unit": "GB/s"},
+            "nt_2r1w": {"avg_launch_ms": probe_2r1w_ms, "achieved": ceil_2r1w, "unit": "GB/s"},
+            "forward_kernel_vs_nt_copy": fwd_gbps / ceil_copy,
+            "backward_kernel_vs_nt_2r1w": bwd_gbps / ceil_2r1w,
+        },
     }
     if not args.no_cpu_baseline:
         base = cpu_baseline(B, H, L, seed, x_std, gate)

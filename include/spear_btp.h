@@ -157,6 +157,14 @@ int spear_btp_abi_version(void);
  * counters and to measure the copy bandwidth the BTP kernels are compared with. */
 int spear_btp_copy(const void* src, void* dst, unsigned long long bytes, void* stream);
 
+/* Measurement aid as well: the operator's own access shape and cache policy without its arithmetic.
+ * Every wavefront moves one 4 KiB slab with non-temporal 16-byte loads and stores; with src_b == NULL
+ * it is a copy (reads `bytes`, writes `bytes`), otherwise dst = src_a ^ src_b (reads 2 x `bytes`, writes
+ * `bytes`: the backward kernel's read/write mix). `bytes` a multiple of 4096. What this reaches is what
+ * the memory system gives kernels of this shape, which is the practical ceiling the BTP kernels are
+ * compared with beside the 8 TB/s peak. */
+int spear_btp_stream_probe(const void* src_a, const void* src_b, void* dst, unsigned long long bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -25,7 +25,7 @@ FLAG_WRITE_CHECKPOINT = 0x1
 FLAG_PATH_MFMA = 0x2
 FLAG_JAGGED_LOG_A = 0x4
 FLAG_JAGGED_LOG_R = 0x8
-_ABI_VERSION = 6
+_ABI_VERSION = 7
 _SUPPORTED_WPB = (4, 8, 16, 32)
 
 _lock = threading.Lock()
@@ -64,6 +64,8 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.spear_btp_abi_version.restype = ci
     lib.spear_btp_copy.argtypes = [vp, vp, ctypes.c_ulonglong, vp]
     lib.spear_btp_copy.restype = ci
+    lib.spear_btp_stream_probe.argtypes = [vp, vp, vp, ctypes.c_ulonglong, vp]
+    lib.spear_btp_stream_probe.restype = ci
 
 
 def load_library() -> ctypes.CDLL:

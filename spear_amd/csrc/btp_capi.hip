@@ -44,7 +44,7 @@ int check_common(const char* who, int B, int H, int L, int k, int in_dtype, int 
 
 extern "C" {
 
-int spear_btp_abi_version(void) { return 6; }
+int spear_btp_abi_version(void) { return 7; }
 
 const char* spear_btp_last_error(void) { return g_error; }
 
@@ -251,6 +251,17 @@ int spear_btp_copy(const void* src, void* dst, unsigned long long bytes, void* s
     return fail(SPEAR_BTP_EINVAL, "spear_btp_copy: size and pointers must be multiples of 16 bytes");
   const hipError_t err = spear_btp::device_copy(src, dst, bytes, static_cast<hipStream_t>(stream));
   if (err != hipSuccess) return fail(SPEAR_BTP_ELAUNCH, "spear_btp_copy: launch failed: %s", hipGetErrorString(err));
+  return 0;
+}
+
+int spear_btp_stream_probe(const void* src_a, const void* src_b, void* dst, unsigned long long bytes, void* stream) {
+  g_error[0] = '\0';
+  if (!src_a || !dst) return fail(SPEAR_BTP_ENULL, "spear_btp_stream_probe: NULL pointer");
+  if (bytes % 4096 != 0 || !aligned16(src_a) || !aligned16(src_b) || !aligned16(dst))
+    return fail(SPEAR_BTP_EINVAL, "spear_btp_stream_probe: size must be a multiple of 4096, pointers of 16 bytes");
+  const hipError_t err = spear_btp::stream_probe(src_a, src_b, dst, bytes, static_cast<hipStream_t>(stream));
+  if (err != hipSuccess)
+    return fail(SPEAR_BTP_ELAUNCH, "spear_btp_stream_probe: launch failed: %s", hipGetErrorString(err));
   return 0;
 }
 

@@ -90,4 +90,8 @@ hipError_t jagged_step(const JagStepArgs& p, hipStream_t s);
 // Plain copy kernel used for bandwidth / counter calibration (btp_scan.hip).
 hipError_t device_copy(const void* src, void* dst, unsigned long long bytes, hipStream_t s);
 
+// Slab-shaped non-temporal copy (b == nullptr) or two-input combine, for measuring what the memory
+// system gives the operator's access pattern (btp_scan.hip).
+hipError_t stream_probe(const void* a, const void* b, void* dst, unsigned long long bytes, hipStream_t s);
+
 }  // namespace spear_btp

@@ -446,6 +446,29 @@ __global__ __launch_bounds__(256) void copy_kernel(const uint4* __restrict__ src
     dst[i] = src[i];
 }
 
+// Bandwidth probe with the operator's own access shape and cache policy and no arithmetic: every
+// wavefront moves one 4 KiB slab (four 16-byte accesses per lane) with non-temporal loads and stores.
+// kReads = 1: copy; kReads = 2: two inputs combined into one output, the backward kernel's mix.
+template <int kReads>
+__global__ __launch_bounds__(64 * kWaves) void stream_probe_kernel(const uint4* __restrict__ a,
+                                                                   const uint4* __restrict__ b,
+                                                                   uint4* __restrict__ dst, unsigned long long slabs) {
+  const unsigned long long slab = (unsigned long long)blockIdx.x * kWaves + (threadIdx.x >> 6);
+  if (slab >= slabs) return;
+  const unsigned long long base = slab * 256 + (threadIdx.x & 63);
+  uint4 q[4], r[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    q[i] = stream_load16(a + base + 64 * i);
+    if constexpr (kReads == 2) r[i] = stream_load16(b + base + 64 * i);
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    if constexpr (kReads == 2) q[i] = make_uint4(q[i].x ^ r[i].x, q[i].y ^ r[i].y, q[i].z ^ r[i].z, q[i].w ^ r[i].w);
+    stream_store16(dst + base + 64 * i, q[i]);
+  }
+}
+
 template <class E, class C, class OutT, bool kCheckpoint, bool kStreamIn>
 void launch_fwd_as(const FwdArgs& p, const Grid& g, hipStream_t s) {
   hipLaunchKernelGGL((btp_fwd_scan_kernel<E, C, OutT, kCheckpoint, kStreamIn>), dim3(g.blocks), dim3(64 * g.waves), 0,
@@ -512,6 +535,19 @@ hipError_t scan_backward(const BwdArgs& p, hipStream_t s) {
   if (p.in_dtype == kBf16)
     return p.log_gate ? backward_by_grad<Bf16, LogCoeff>(p, s) : backward_by_grad<Bf16, LinCoeff<Bf16>>(p, s);
   return p.log_gate ? backward_by_grad<Fp16, LogCoeff>(p, s) : backward_by_grad<Fp16, LinCoeff<Fp16>>(p, s);
+}
+
+hipError_t stream_probe(const void* a, const void* b, void* dst, unsigned long long bytes, hipStream_t s) {
+  const unsigned long long slabs = bytes / 4096;
+  if (slabs == 0) return hipSuccess;
+  const unsigned blocks = (unsigned)((slabs + kWaves - 1) / kWaves);
+  if (b == nullptr)
+    hipLaunchKernelGGL(stream_probe_kernel<1>, dim3(blocks), dim3(64 * kWaves), 0, s, static_cast<const uint4*>(a),
+                       static_cast<const uint4*>(nullptr), static_cast<uint4*>(dst), slabs);
+  else
+    hipLaunchKernelGGL(stream_probe_kernel<2>, dim3(blocks), dim3(64 * kWaves), 0, s, static_cast<const uint4*>(a),
+                       static_cast<const uint4*>(b), static_cast<uint4*>(dst), slabs);
+  return hipGetLastError();
 }
 
 hipError_t device_copy(const void* src, void* dst, unsigned long long bytes, hipStream_t s) {

@@ -274,3 +274,32 @@ def test_kernels_match_the_reference_float64_path_vectors():
     dx, dA = run_backward(coeff, x, dy)
     assert_close(f64(dx), v["ref.f64.dx"], BF16_ATOL, BF16_RTOL, "dx")
     assert_close(f64(dA), v["ref.f64.dA"], F32_ATOL * 10, F32_RTOL * 10, "dA")
+
+
+@pytest.mark.parametrize("slabs", [1, 3, 4, 1025])
+def test_measurement_aids_move_the_bytes_they_are_timed_for(slabs):
+    """spear_btp_copy and spear_btp_stream_probe are timed as ceilings, so they must really move every byte."""
+    import ctypes
+
+    from spear_amd import _btp
+
+    lib = _btp.load_library()
+    n = slabs * 4096
+    g = torch.Generator(device="cpu").manual_seed(slabs)
+    a = torch.randint(0, 256, (n,), dtype=torch.uint8, generator=g).to(DEV)
+    b = torch.randint(0, 256, (n,), dtype=torch.uint8, generator=g).to(DEV)
+    guard = 4096
+    out = torch.full((n + guard,), 0xA5, dtype=torch.uint8, device=DEV)
+    sp = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    for second, want in ((None, a), (b, a ^ b)):
+        out.fill_(0xA5)
+        rc = lib.spear_btp_stream_probe(a.data_ptr(), None if second is None else second.data_ptr(), out.data_ptr(),
+                                        ctypes.c_ulonglong(n), sp)
+        assert rc == 0, lib.spear_btp_last_error()
+        torch.cuda.synchronize()
+        assert torch.equal(out[:n], want)
+        assert bool((out[n:] == 0xA5).all())
+    out.fill_(0xA5)
+    assert lib.spear_btp_copy(a.data_ptr(), out.data_ptr(), ctypes.c_ulonglong(n), sp) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(out[:n], a) and bool((out[n:] == 0xA5).all())

@@ -25,6 +25,7 @@ def test_header_declares_the_expected_entry_points():
         "spear_btp_forward",
         "spear_btp_forward_loggate",
         "spear_btp_last_error",
+        "spear_btp_stream_probe",
         "spear_jagged_prefill",
         "spear_jagged_step",
         "spear_phalanx_mix_backward",
@@ -63,7 +64,7 @@ def test_host_side_validation_needs_no_gpu():
     from spear_amd import _btp
 
     lib = _btp.load_library()
-    assert lib.spear_btp_abi_version() == 6
+    assert lib.spear_btp_abi_version() == 7
     buf = ctypes.create_string_buffer(4096)
     p = ctypes.addressof(buf)
     p -= p % 16
@@ -93,6 +94,7 @@ def test_host_side_validation_needs_no_gpu():
     assert lib.spear_btp_forward(p, p, p, None, 0, 4, 32, 2, 0, 0, 0, None) == 0
     assert lib.spear_btp_last_error() == b""
     assert lib.spear_btp_copy(p, p, 24, None) == -1
+    assert lib.spear_btp_stream_probe(p, None, p, 100, None) == -1
     # fused layer kernels: a batch row must fit one 32-bit buffer resource
     assert lib.spear_phalanx_mix_forward(p, p, p, p, p, 1, 1 << 20, 128, 128, 0, 0, None) == -1
     assert b"below 2 GiB" in lib.spear_btp_last_error()
