@@ -1,0 +1,122 @@
+"""The layer's linear projections with a backward pass shaped for long token axes.
+
+The Phalanx layer (spear/nn/phalanx/swr.py:166-175, 271) is five ``nn.Linear`` calls around the
+mixing stage. With ``M = B*L`` tokens their weight gradients are ``[N, M] x [M, K]`` products whose
+output is a few hundred columns wide while the reduction runs over 10^5 tokens: as one GEMM that is a
+few dozen output tiles for 256 compute units. Here the token axis is cut into ``S`` slices that are
+multiplied as one batched GEMM with fp32 partial results and then summed (the same fp32 accumulation,
+associated differently). The four input projections also share one backward: their input gradients
+accumulate in one buffer through the GEMM's own ``beta = 1`` epilogue instead of four products and
+three additions.
+
+Short token axes gain nothing (their step is bound by launch overhead, of which this path has more), so
+the layer uses these functions from 8192 tokens on (``pays_off``).
+
+Forward results are those of ``torch.nn.functional.linear``. Parameters stay in the layer's
+``nn.Linear`` modules; these functions only take their tensors.
+"""
+
+from __future__ import annotations
+
+import torch
+import torch.nn.functional as F
+
+__all__ = ["weight_grad", "input_projections", "linear", "pays_off"]
+
+_TILE = 128           # output tile edge the slice count is sized against
+_TARGET_TILES = 1024  # about four tiles per compute unit
+_MIN_SLICE_ROWS = 1024
+_MAX_SLICES = 64
+_MIN_TOKENS = 8192    # below this a step is bound by launches, and these functions add a few
+
+
+def pays_off(x: torch.Tensor) -> bool:
+    """Whether ``x[..., K]`` has enough tokens for the sliced backward to beat plain ``nn.Linear``."""
+    return x.is_cuda and x.numel() // x.shape[-1] >= _MIN_TOKENS
+
+
+def slice_count(M: int, N: int, K: int) -> int:
+    """How many slices the token axis of an ``[N, M] x [M, K]`` product is cut into."""
+    tiles = -(-N // _TILE) * -(-K // _TILE)
+    s = 1
+    while s < _MAX_SLICES and tiles * s < _TARGET_TILES and M % (2 * s) == 0 and M // (2 * s) >= _MIN_SLICE_ROWS:
+        s *= 2
+    return s
+
+
+@torch.library.custom_op("spear_amd::weight_grad", mutates_args=())
+def weight_grad(dy: torch.Tensor, x: torch.Tensor) -> torch.Tensor:
+    """``dy[M, N]^T @ x[M, K] -> [N, K]`` in ``dy``'s dtype, accumulated in fp32."""
+    M, N = dy.shape
+    K = x.shape[1]
+    s = slice_count(M, N, K) if dy.is_cuda and dy.dtype in (torch.bfloat16, torch.float16) else 1
+    if s == 1:
+        return dy.t() @ x
+    dy3 = dy.contiguous().view(s, M // s, N)
+    x3 = x.contiguous().view(s, M // s, K)
+    return torch.bmm(dy3.transpose(1, 2), x3, out_dtype=torch.float32).sum(0).to(dy.dtype)
+
+
+@weight_grad.register_fake
+def _(dy, x):
+    return dy.new_empty((dy.shape[1], x.shape[1]))
+
+
+class _InputProjections(torch.autograd.Function):
+    """x[M, K] -> (x W_a^T + b_a, x W_b^T + b_b, x W_c^T + b_c, x W_v^T)."""
+
+    @staticmethod
+    def forward(ctx, x, w_a, b_a, w_b, b_b, w_c, b_c, w_v):
+        ctx.save_for_backward(x, w_a, w_b, w_c, w_v)
+        return F.linear(x, w_a, b_a), F.linear(x, w_b, b_b), F.linear(x, w_c, b_c), F.linear(x, w_v)
+
+    @staticmethod
+    def backward(ctx, d_a, d_b, d_c, d_v):
+        x, w_a, w_b, w_c, w_v = ctx.saved_tensors
+        need = ctx.needs_input_grad
+        pairs = [(d, w) for d, w in ((d_v, w_v), (d_b, w_b), (d_c, w_c), (d_a, w_a)) if d is not None]
+        dx = None
+        if need[0] and pairs:
+            dx = pairs[0][0] @ pairs[0][1]
+            for d, w in pairs[1:]:
+                dx.addmm_(d, w)
+
+        def wgrad(d, wanted):
+            return weight_grad(d, x) if wanted and d is not None else None
+
+        def bgrad(d, wanted):
+            return d.sum(0) if wanted and d is not None else None
+
+        return (dx, wgrad(d_a, need[1]), bgrad(d_a, need[2]), wgrad(d_b, need[3]), bgrad(d_b, need[4]),
+                wgrad(d_c, need[5]), bgrad(d_c, need[6]), wgrad(d_v, need[7]))
+
+
+class _Linear(torch.autograd.Function):
+    """x[M, K] -> x W^T (no bias)."""
+
+    @staticmethod
+    def forward(ctx, x, w):
+        ctx.save_for_backward(x, w)
+        return F.linear(x, w)
+
+    @staticmethod
+    def backward(ctx, d):
+        x, w = ctx.saved_tensors
+        return (d @ w if ctx.needs_input_grad[0] else None, weight_grad(d, x) if ctx.needs_input_grad[1] else None)
+
+
+def input_projections(x: torch.Tensor, proj_a, proj_b, proj_c, proj_v):
+    """The four input projections of ``x[..., K]`` (``nn.Linear`` modules; ``proj_v`` without bias)."""
+    lead = x.shape[:-1]
+    outs = _InputProjections.apply(
+        x.reshape(-1, x.shape[-1]), proj_a.weight, proj_a.bias, proj_b.weight, proj_b.bias,
+        proj_c.weight, proj_c.bias, proj_v.weight,
+    )
+    return tuple(o.view(*lead, o.shape[-1]) for o in outs)
+
+
+def linear(x: torch.Tensor, proj) -> torch.Tensor:
+    """``proj(x)`` for a bias-free ``nn.Linear``."""
+    lead = x.shape[:-1]
+    out = _Linear.apply(x.reshape(-1, x.shape[-1]), proj.weight)
+    return out.view(*lead, out.shape[-1])

@@ -17,12 +17,19 @@ initialises identical weights).
   ``"fused"``             (addition) one HIP kernel for gates + recurrence + ``* C + V`` working
                           directly on the projection outputs; needs ``heads % 4 == 0``, ``k == 2``
 The choice is explicit; ``"default"`` and ``"fused"`` never degrade to a PyTorch path.
+
+On a GPU, from 8192 tokens per call on, the ``"default"`` and ``"fused"`` layers run their five
+projections through :mod:`.projections` (same forward; weight gradients cut along the token axis, one
+shared input gradient). The two ``"pytorch*"`` methods keep plain ``nn.Linear`` autograd, which is what the
+other two are compared with.
 """
 
 from __future__ import annotations
 
 import torch
 import torch.nn as nn
+
+from .projections import input_projections, linear, pays_off
 
 _HEAD_DIM = 16
 _METHODS = ("default", "pytorch", "pytorch_linspace", "fused")
@@ -89,6 +96,7 @@ class SigmoidA(nn.Module):
         self.kv_repeat = KVRepeat(self.kv_heads, heads)
         self.dim_bvc = 3 * heads * head_dim
         self.dim_a = heads
+        self.token_sliced_backward = False  # set by Phalanx for the methods that run HIP kernels
 
         # creation order fixes the RNG draw order of the default initialisation
         self.proj_a = nn.Linear(dim, heads, bias=True, dtype=dtype)
@@ -96,10 +104,16 @@ class SigmoidA(nn.Module):
         self.proj_c = nn.Linear(dim, self.kv_heads * head_dim, bias=True, dtype=dtype)
         self.proj_v = nn.Linear(dim, heads * head_dim, bias=False, dtype=dtype)
 
+    def project(self, x: torch.Tensor):
+        """``(proj_a(x), proj_b(x), proj_c(x), proj_v(x))`` as [B, L, features] tensors."""
+        xc = x.to(self.compute_dtype)
+        if self.token_sliced_backward and pays_off(xc):
+            return input_projections(xc, self.proj_a, self.proj_b, self.proj_c, self.proj_v)
+        return tuple(p(xc) for p in (self.proj_a, self.proj_b, self.proj_c, self.proj_v))
+
     def _compute_base_projections(self, x: torch.Tensor):
         """Raw projections as [B, features, L] views (time last, not yet contiguous)."""
-        xc = x.to(self.compute_dtype)
-        return tuple(p(xc).transpose(1, 2) for p in (self.proj_a, self.proj_b, self.proj_c, self.proj_v))
+        return tuple(t.transpose(1, 2) for t in self.project(x))
 
     def forward_fused_gates(self, x: torch.Tensor) -> torch.Tensor:
         """Packed ``[B_gate, V, C, A]`` along the feature axis: ``[B, 3*H*16 + H, L]``."""
@@ -164,6 +178,7 @@ class Phalanx(nn.Module):
 
         self.param = SigmoidA(dim, heads, self.head_dim, dtype=dtype, kv_heads=kv_heads)
         self.proj_out = nn.Linear(dim, dim, bias=False, dtype=dtype)
+        self.param.token_sliced_backward = method in ("default", "fused")
 
         if method == "default":
             from spear_amd.ops.btp import btp
@@ -186,7 +201,12 @@ class Phalanx(nn.Module):
     def _mix_and_project(self, h: torch.Tensor, C: torch.Tensor, V: torch.Tensor) -> torch.Tensor:
         out = h * C + V  # [B, H, 16, L]
         B, H, DH, L = out.shape
-        return self.proj_out(out.permute(0, 3, 1, 2).reshape(B, L, H * DH))
+        return self._project_out(out.permute(0, 3, 1, 2).reshape(B, L, H * DH))
+
+    def _project_out(self, mixed: torch.Tensor) -> torch.Tensor:
+        if self.param.token_sliced_backward and pays_off(mixed):
+            return linear(mixed, self.proj_out)
+        return self.proj_out(mixed)
 
     def _forward_pytorch(self, x: torch.Tensor) -> torch.Tensor:
         A, X, C, V = self.param.forward_axcv(x)
@@ -197,10 +217,8 @@ class Phalanx(nn.Module):
         return self._mix_and_project(self.btp_module(A, X, self.k, self.wpb, self.output_dtype), C, V)
 
     def _forward_fused(self, x: torch.Tensor) -> torch.Tensor:
-        p = self.param
-        xc = x.to(p.compute_dtype)
-        mixed = self.mix_module(p.proj_a(xc), p.proj_b(xc), p.proj_c(xc), p.proj_v(xc), self.heads, self.kv_heads)
-        return self.proj_out(mixed)
+        a_logits, b_logits, c, v = self.param.project(x)
+        return self._project_out(self.mix_module(a_logits, b_logits, c, v, self.heads, self.kv_heads))
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         return self._forward_fn(x)

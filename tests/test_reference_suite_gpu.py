@@ -287,6 +287,15 @@ def test_layer_backward_consistency_basic(compile, opts):  # test_phalanx_numeri
     _layer_backward_case(2, 128, 256, 789, 987, 1.0, ("default", "pytorch", "fused"), compile=compile, opts=opts)
 
 
+# Not in the reference: enough tokens (80 * 128) for the layer to take its token-sliced projection backward.
+@pytest.mark.parametrize("compile,opts", [COMPILE_CASES[0], COMPILE_CASES[2]])
+def test_layer_backward_consistency_with_many_tokens(compile, opts):
+    from spear_amd.nn.phalanx.projections import slice_count
+
+    assert slice_count(80 * 128, 256, 256) > 1
+    _layer_backward_case(80, 128, 256, 789, 987, 1.0, ("default", "pytorch", "fused"), compile=compile, opts=opts)
+
+
 # The reference crosses these with all four compile configurations; the autotuning ones spend most of a
 # minute each on the layer's GEMMs, which are not what is under test, so the stress shapes run eagerly
 # and as one full graph (all four configurations are exercised by the two "basic" tests above).
