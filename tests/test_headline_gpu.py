@@ -97,3 +97,89 @@ def test_full_size_properties(name):
         rdx, rdA = orc.backward(a_, x_, g_)
         assert_close(f64(dx[b : b + 1, h : h + 1]), rdx, BF16_ATOL, BF16_RTOL, f"dx[{b},{h}]")
         assert_close(f64(dA[b : b + 1, h : h + 1]), rdA, F32_ATOL, F32_RTOL, f"dA[{b},{h}]")
+
+
+def _free_gib():
+    free, _ = torch.cuda.mem_get_info()
+    return free / 2**30
+
+
+def test_rows_past_2_31_elements_equal_the_same_rows_run_alone():
+    """64-bit addressing: tensors of more than 2^31 elements (4.6 GB each in bf16). Every (b, h) row is
+    independent, so the rows that lie beyond the 2^31-element mark must come out bit-identical to a
+    call on those rows alone (offsets near zero)."""
+    if _free_gib() < 48:
+        pytest.skip("needs about 40 GiB of device memory")
+    rows, L = 1100, 131072                      # 1100 * 16 * 131072 = 2.31e9 elements
+    assert rows * 16 * L > 2**31
+    g = torch.Generator(device=DEV).manual_seed(77)
+    print("scan kernels past 2^31: inputs", flush=True)
+    coeff = torch.sigmoid(torch.randn(1, rows, L, device=DEV, generator=g)).bfloat16()
+    x = torch.empty(1, rows, 16, L, device=DEV, dtype=torch.bfloat16).normal_(0, 0.25, generator=g)
+    dy = torch.empty(1, rows, 16, L, device=DEV, dtype=torch.bfloat16).normal_(0, 1, generator=g)
+    print("scan kernels past 2^31: forward/backward", flush=True)
+    y = _fwd(coeff, x)
+    dx, dA = _bwd(coeff, x, dy)
+    torch.cuda.synchronize()
+    for lo, hi in ((0, 2), (1023, 1026), (rows - 3, rows)):   # row 1024 starts exactly at element 2^31
+        sub = slice(lo, hi)
+        cs, xs, gs = (t[:, sub].contiguous() for t in (coeff, x, dy))
+        assert torch.equal(_fwd(cs, xs), y[:, sub]), f"y rows {lo}:{hi}"
+        dxs, dAs = _bwd(cs, xs, gs)
+        assert torch.equal(dxs, dx[:, sub]), f"dx rows {lo}:{hi}"
+        assert torch.equal(dAs, dA[:, sub]), f"dA rows {lo}:{hi}"
+    # and against the oracle on the head of the last row (a block depends on itself and its predecessor only)
+    n = 256
+    a_, x_ = f64(coeff[:, -1:, :n].cpu()), f64(x[:, -1:, :, :n].cpu())
+    assert_close(f64(y[:, -1:, :, :n].cpu()), orc.forward(a_, x_), BF16_ATOL, BF16_RTOL, "y last row")
+
+
+def test_fused_and_prefill_batches_past_2_31_elements_equal_the_same_batch_run_alone():
+    from spear_amd import _btp
+
+    if _free_gib() < 64:
+        pytest.skip("needs about 50 GiB of device memory")
+    g = torch.Generator(device=DEV).manual_seed(78)
+    B, L, H = 5, 1 << 20, 32                    # 5 * 2^20 * 512 = 2.68e9 elements; batch row 4 starts at 2^31
+    F = H * 16
+    print("fused kernels past 2^31: inputs", flush=True)
+    a = torch.empty(B, L, H, device=DEV, dtype=torch.bfloat16).normal_(0, 1, generator=g)
+    b, c, v, dout = (torch.empty(B, L, F, device=DEV, dtype=torch.bfloat16).normal_(0, 1, generator=g) for _ in range(4))
+    out = torch.empty_like(v)
+    grads = [torch.empty_like(t) for t in (a, b, c, v)]
+    print("fused kernels past 2^31: forward/backward", flush=True)
+    _btp.mix_forward(a, b, c, v, out, H, H)
+    _btp.mix_backward(a, b, c, v, dout, *grads, H, H)
+    torch.cuda.synchronize()
+    last = [t[B - 1:].contiguous() for t in (a, b, c, v, dout)]
+    out1 = torch.empty_like(last[3])
+    grads1 = [torch.empty_like(t) for t in last[:4]]
+    _btp.mix_forward(*last[:4], out1, H, H)
+    _btp.mix_backward(*last, *grads1, H, H)
+    torch.cuda.synchronize()
+    assert torch.equal(out1, out[B - 1:])
+    for name, g1, gall in zip("abcv", grads1, grads):
+        assert torch.equal(g1, gall[B - 1:]), f"d{name}"
+    del a, b, c, v, dout, out, grads, last, out1, grads1
+    torch.cuda.empty_cache()
+
+    rows, Lp = 1100, 131072
+    print("prefill past 2^31: inputs", flush=True)
+    A = torch.sigmoid(torch.randn(1, rows, Lp, device=DEV, generator=g)).bfloat16()
+    X, C, V = (torch.empty(1, rows, 16, Lp, device=DEV, dtype=torch.bfloat16).normal_(0, 0.5, generator=g) for _ in range(3))
+
+    def prefill(A_, X_, C_, V_):
+        n = A_.shape[1]
+        Y = torch.empty_like(X_)
+        h, cp = (torch.empty(1, n, 16, device=DEV) for _ in range(2))
+        r = torch.empty(1, n, device=DEV)
+        _btp.jagged_prefill(A_, X_, C_, V_, None, Y, h, r, cp, 16, False)
+        return Y, h, r, cp
+
+    print("prefill past 2^31: run", flush=True)
+    whole = prefill(A, X, C, V)
+    sub = slice(rows - 3, rows)
+    part = prefill(*(t[:, sub].contiguous() for t in (A, X, C, V)))
+    torch.cuda.synchronize()
+    for name, w, p in zip(("Y", "h", "r", "c_prev"), whole, part):
+        assert torch.equal(p, w[:, sub]), name
