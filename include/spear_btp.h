@@ -105,6 +105,22 @@ int spear_phalanx_mix_backward(const void* a_logit, const void* b_logit, const v
                                const void* dout, void* da_logit, void* db_logit, void* dc, void* dv, int B, int L,
                                int H, int kv_heads, int dtype, unsigned flags, void* stream);
 
+/* The same backward, which in addition leaves the column sums of da_logit, db_logit and dc -- the bias
+ * gradients of the projections that produced a_logit, b_logit and c (spear/nn/phalanx/swr.py:157-163 gives
+ * proj_a, proj_b and proj_c a bias) -- so that the caller does not read the three gradients again to
+ * sum them. The kernel cannot finish the sums without a second pass, so it leaves partial sums in fp32:
+ *     sum_da [sum_rows, H],  sum_db [sum_rows, kv_heads * 16],  sum_dc [sum_rows, kv_heads * 16]
+ * where row r sums the time steps of one (batch row, time chunk) and the caller adds the rows up
+ * (sum_rows is a few per batch row at most). sum_rows must equal
+ * spear_phalanx_mix_backward_sum_rows(B, L, H); every element of the three arrays is written; the sums
+ * are taken before the gradients are rounded to `dtype`. All three NULL: exactly
+ * spear_phalanx_mix_backward. */
+long long spear_phalanx_mix_backward_sum_rows(int B, int L, int H);
+int spear_phalanx_mix_backward_sums(const void* a_logit, const void* b_logit, const void* c, const void* v,
+                                    const void* dout, void* da_logit, void* db_logit, void* dc, void* dv, float* sum_da,
+                                    float* sum_db, float* sum_dc, long long sum_rows, int B, int L, int H, int kv_heads,
+                                    int dtype, unsigned flags, void* stream);
+
 /* ---- streaming form: prompt prefill with state hand-over, and the one-token decode step --------
  * They replace the PyTorch loops of spear/nn/phalanx/inference.py. Tensors are dense, row-major:
  *     a         [B, H, L]      a_dtype (x_dtype or fp32)   a_t, or log(a_t) with SPEAR_JAGGED_LOG_A

@@ -25,7 +25,7 @@ FLAG_WRITE_CHECKPOINT = 0x1
 FLAG_PATH_MFMA = 0x2
 FLAG_JAGGED_LOG_A = 0x4
 FLAG_JAGGED_LOG_R = 0x8
-_ABI_VERSION = 7
+_ABI_VERSION = 8
 _SUPPORTED_WPB = (4, 8, 16, 32)
 
 _lock = threading.Lock()
@@ -54,6 +54,10 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.spear_phalanx_mix_forward.restype = ci
     lib.spear_phalanx_mix_backward.argtypes = [vp] * 9 + [ci, ci, ci, ci, ci, cu, vp]
     lib.spear_phalanx_mix_backward.restype = ci
+    lib.spear_phalanx_mix_backward_sums.argtypes = [vp] * 12 + [ctypes.c_longlong, ci, ci, ci, ci, ci, cu, vp]
+    lib.spear_phalanx_mix_backward_sums.restype = ci
+    lib.spear_phalanx_mix_backward_sum_rows.argtypes = [ci, ci, ci]
+    lib.spear_phalanx_mix_backward_sum_rows.restype = ctypes.c_longlong
     lib.spear_jagged_prefill.argtypes = [vp] * 9 + [ci] * 9 + [cu, vp]
     lib.spear_jagged_prefill.restype = ci
     lib.spear_jagged_step.argtypes = [vp] * 11 + [ci] * 8 + [cu, ctypes.c_float, vp]
@@ -305,6 +309,11 @@ def mix_forward(
         _raise_native(lib, rc)
 
 
+def mix_backward_sum_rows(B: int, L: int, heads: int) -> int:
+    """Rows of the partial-sum arrays :func:`mix_backward` fills for this shape."""
+    return int(load_library().spear_phalanx_mix_backward_sum_rows(B, L, heads))
+
+
 def mix_backward(
     a_logit: torch.Tensor,
     b_logit: torch.Tensor,
@@ -317,9 +326,12 @@ def mix_backward(
     dv: torch.Tensor,
     heads: int,
     kv_heads: int,
+    sums: tuple[torch.Tensor, torch.Tensor, torch.Tensor] | None = None,
 ) -> None:
     """Gradients of :func:`mix_forward`, written in place; ``heads // kv_heads`` must be 1, 2, 4 or 8
-    (see ``spear_phalanx_mix_backward`` in the C header)."""
+    (see ``spear_phalanx_mix_backward`` in the C header). ``sums``: three fp32 tensors
+    ``[mix_backward_sum_rows(B, L, heads), heads | kv_heads*16 | kv_heads*16]`` that receive the per-chunk
+    column sums of ``da_logit``, ``db_logit`` and ``dc`` (``spear_phalanx_mix_backward_sums``)."""
     tensors = (a_logit, b_logit, c, v, dout, da_logit, db_logit, dc, dv)
     _check(all(t.is_cuda for t in tensors), "All tensors must be CUDA.")
     _check(v.dim() == 3, "v must be [B, L, heads * 16].")
@@ -340,10 +352,18 @@ def mix_backward(
         _check_layout(name, t, shape)
     _check(len({t.device for t in tensors}) == 1, "All tensors must be on the same device.")
     lib = load_library()
+    rows = 0
+    if sums is not None:
+        rows = int(lib.spear_phalanx_mix_backward_sum_rows(B, L, heads))
+        for name, t, width in (("sum_da", sums[0], heads), ("sum_db", sums[1], Fkv), ("sum_dc", sums[2], Fkv)):
+            _check(t.is_cuda and t.device == v.device and t.dtype == torch.float32, f"{name} must be float32 on v's device.")
+            _check_layout(name, t, (rows, width))
+    sum_ptrs = [t.data_ptr() for t in sums] if rows > 0 else [None, None, None]
     with torch.cuda.device(v.device):
-        rc = lib.spear_phalanx_mix_backward(
+        rc = lib.spear_phalanx_mix_backward_sums(
             a_logit.data_ptr(), b_logit.data_ptr(), c.data_ptr(), v.data_ptr(), dout.data_ptr(),
             da_logit.data_ptr(), db_logit.data_ptr(), dc.data_ptr(), dv.data_ptr(),
+            *sum_ptrs, rows,
             B, L, heads, kv_heads, _tag(v.dtype), 0, _stream_ptr(v.device),
         )
     if rc != 0:

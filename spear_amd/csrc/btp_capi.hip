@@ -44,7 +44,7 @@ int check_common(const char* who, int B, int H, int L, int k, int in_dtype, int 
 
 extern "C" {
 
-int spear_btp_abi_version(void) { return 7; }
+int spear_btp_abi_version(void) { return 8; }
 
 const char* spear_btp_last_error(void) { return g_error; }
 
@@ -152,9 +152,22 @@ int spear_phalanx_mix_forward(const void* a_logit, const void* b_logit, const vo
   return 0;
 }
 
+long long spear_phalanx_mix_backward_sum_rows(int B, int L, int H) {
+  if (B <= 0 || L <= 0 || H <= 0 || L % 16 != 0) return 0;
+  return spear_btp::fused_mix_backward_sum_rows(B, H, L);
+}
+
 int spear_phalanx_mix_backward(const void* a_logit, const void* b_logit, const void* c, const void* v, const void* dout,
                                void* da_logit, void* db_logit, void* dc, void* dv, int B, int L, int H, int kv_heads,
                                int dtype, unsigned flags, void* stream) {
+  return spear_phalanx_mix_backward_sums(a_logit, b_logit, c, v, dout, da_logit, db_logit, dc, dv, nullptr, nullptr,
+                                         nullptr, 0, B, L, H, kv_heads, dtype, flags, stream);
+}
+
+int spear_phalanx_mix_backward_sums(const void* a_logit, const void* b_logit, const void* c, const void* v,
+                                    const void* dout, void* da_logit, void* db_logit, void* dc, void* dv, float* sum_da,
+                                    float* sum_db, float* sum_dc, long long sum_rows, int B, int L, int H, int kv_heads,
+                                    int dtype, unsigned flags, void* stream) {
   g_error[0] = '\0';
   const char* who = "spear_phalanx_mix_backward";
   if (B < 0 || L < 0 || H < 0) return fail(SPEAR_BTP_EINVAL, "%s: negative dimension (B=%d L=%d H=%d)", who, B, L, H);
@@ -179,7 +192,17 @@ int spear_phalanx_mix_backward(const void* a_logit, const void* b_logit, const v
     if (!q) return fail(SPEAR_BTP_ENULL, "%s: NULL tensor pointer", who);
     if (!aligned16(q)) return fail(SPEAR_BTP_EINVAL, "%s: tensor pointers must be 16-byte aligned", who);
   }
-  spear_btp::MixBwdArgs a{a_logit, b_logit, c, v, dout, da_logit, db_logit, dc, dv, B, L, H, groups, dtype};
+  const bool sums = sum_da || sum_db || sum_dc;
+  if (sums) {
+    if (!sum_da || !sum_db || !sum_dc) return fail(SPEAR_BTP_ENULL, "%s: the three sum arrays must be given together", who);
+    if (!aligned16(sum_da) || !aligned16(sum_db) || !aligned16(sum_dc))
+      return fail(SPEAR_BTP_EINVAL, "%s: sum arrays must be 16-byte aligned", who);
+    const long long want = spear_btp::fused_mix_backward_sum_rows(B, H, L);
+    if (sum_rows != want)
+      return fail(SPEAR_BTP_EINVAL, "%s: sum arrays must have %lld rows for this shape (got %lld)", who, want, sum_rows);
+  }
+  spear_btp::MixBwdArgs a{a_logit, b_logit, c, v, dout, da_logit, db_logit, dc, dv, B, L, H, groups, dtype,
+                          sum_da, sum_db, sum_dc};
   const hipError_t err = spear_btp::fused_mix_backward(a, static_cast<hipStream_t>(stream));
   if (err != hipSuccess) return fail(SPEAR_BTP_ELAUNCH, "%s: launch failed: %s", who, hipGetErrorString(err));
   return 0;

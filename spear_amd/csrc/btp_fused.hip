@@ -228,12 +228,17 @@ struct MixSet {
   uint32_t araw;
 };
 
-template <class E>
+// kSums: also leave, per (batch row, time chunk), the sums over the chunk's time steps of da_logit, db_logit
+// and dc in fp32 (before their rounding to 16 bits) -- the bias gradients of the projections that produced
+// a_logit, b_logit and c, up to a sum over those few rows. A lane keeps its features for the whole walk, so
+// this is five accumulators per lane and one store at the end.
+template <class E, bool kSums>
 __global__ __launch_bounds__(64 * kWaves) void phalanx_mix_bwd_kernel(
     const uint16_t* __restrict__ a_logit, const uint16_t* __restrict__ b_logit, const uint16_t* __restrict__ c_in,
     const uint16_t* __restrict__ v_in, const uint16_t* __restrict__ dout, uint16_t* __restrict__ da_logit,
-    uint16_t* __restrict__ db_logit, uint16_t* __restrict__ dc, uint16_t* __restrict__ dv, int L, int H,
-    int kv_groups, int chunk_steps, int chunks, long total_waves) {
+    uint16_t* __restrict__ db_logit, uint16_t* __restrict__ dc, uint16_t* __restrict__ dv, float* __restrict__ sum_da,
+    float* __restrict__ sum_db, float* __restrict__ sum_dc, int L, int H, int kv_groups, int chunk_steps, int chunks,
+    long total_waves) {
   __shared__ __align__(16) float gate_tiles[kWaves][2][kHeadsPerWave * kGateRow];  // decay of two blocks
   __shared__ __align__(16) float4 park[kWaves][kTile][64];                        // (R0, R1, dX0, dX1) per step, lane
 
@@ -303,6 +308,7 @@ __global__ __launch_bounds__(64 * kWaves) void phalanx_mix_bwd_kernel(
   };
 
   float dC0 = 0.0f, dC1 = 0.0f;  // gradient carry arriving from the block after the current one
+  float acc_a = 0.0f, acc_b0 = 0.0f, acc_b1 = 0.0f, acc_c0 = 0.0f, acc_c1 = 0.0f;  // kSums only
   float4* my_park = &park[wave][0][lane];
 
   // One iteration: `cur` holds block t0 (its decay is in tile `tc`), `nxt` receives block t0 - 16.
@@ -387,6 +393,9 @@ __global__ __launch_bounds__(64 * kWaves) void phalanx_mix_bwd_kernel(
           db0 += lane_xor(db0, lane, 32); db1 += lane_xor(db1, lane, 32);
         }
       }
+      if constexpr (kSums) {
+        acc_b0 += db0; acc_b1 += db1; acc_c0 += dc0; acc_c1 += dc1;
+      }
       const uint32_t wdc = E::pack2(dc0, dc1);
       const uint32_t wdv = E::pack2(fmaf(pk.z, G0, go0), fmaf(pk.w, G1, go1));
       const uint32_t wdb = E::pack2(db0, db1);
@@ -428,6 +437,7 @@ __global__ __launch_bounds__(64 * kWaves) void phalanx_mix_bwd_kernel(
     }
     const float2 aa = *reinterpret_cast<const float2*>(tc + head_local * kGateRow + 2 * kk);
     const float da0 = s0 * aa.x * (1.0f - aa.x), da1 = s1 * aa.y * (1.0f - aa.y);
+    if constexpr (kSums) acc_a += da0 + da1;
     const int da_off = (t0 >= t_begin) ? da_lane : 0x7ffffff0;
     const uint32_t dap = E::pack2(da0, da1);
     __builtin_amdgcn_raw_buffer_store_b16((unsigned short)(dap & 0xffffu), rda, da_off, t0 * H * 2, 0);
@@ -450,6 +460,19 @@ __global__ __launch_bounds__(64 * kWaves) void phalanx_mix_bwd_kernel(
     __builtin_amdgcn_sched_barrier(0);
     if (t0 - kTile >= t_begin) iterate(s1, s0, tile1, tile0, t0 - kTile);
     __builtin_amdgcn_sched_barrier(0);
+  }
+
+  if constexpr (kSums) {
+    // row `bc` of the sum arrays belongs to this (batch row, chunk); columns as in the tensors
+    acc_a += row_xor<1>(acc_a);
+    acc_a += row_xor<2>(acc_a);
+    acc_a += row_xor<4>(acc_a);  // lane k of a head held steps 2k, 2k+1: now every lane has the head's sum
+    if (real && (lane & 7) == 0) sum_da[bc * H + head] = acc_a;
+    if (real && (head % kv_groups) == 0) {  // the group's sum is in every lane of the group
+      const long col = bc * Fkv + (head / kv_groups) * kChan + d0;
+      *reinterpret_cast<float2*>(sum_db + col) = make_float2(acc_b0, acc_b1);
+      *reinterpret_cast<float2*>(sum_dc + col) = make_float2(acc_c0, acc_c1);
+    }
   }
 }
 
@@ -532,23 +555,34 @@ MixPlan plan_mix_bwd(long B, int H, int L) {
   return m;
 }
 
-template <class E>
+template <class E, bool kSums>
 void launch_mix_bwd(const MixBwdArgs& p, const MixPlan& m, hipStream_t s) {
   const long total = (long)p.B * m.chunks * ((p.H + 7) / 8);
   const unsigned blocks = (unsigned)((total + kWaves - 1) / kWaves);
   auto u = [](const void* q) { return static_cast<const uint16_t*>(q); };
   auto w = [](void* q) { return static_cast<uint16_t*>(q); };
-  hipLaunchKernelGGL((phalanx_mix_bwd_kernel<E>), dim3(blocks), dim3(64 * kWaves), 0, s, u(p.a_logit), u(p.b_logit),
-                     u(p.c), u(p.v), u(p.dout), w(p.da_logit), w(p.db_logit), w(p.dc), w(p.dv), p.L, p.H, p.kv_groups,
-                     m.chunk_blocks * kTile, m.chunks, total);
+  hipLaunchKernelGGL((phalanx_mix_bwd_kernel<E, kSums>), dim3(blocks), dim3(64 * kWaves), 0, s, u(p.a_logit),
+                     u(p.b_logit), u(p.c), u(p.v), u(p.dout), w(p.da_logit), w(p.db_logit), w(p.dc), w(p.dv), p.sum_da,
+                     p.sum_db, p.sum_dc, p.L, p.H, p.kv_groups, m.chunk_blocks * kTile, m.chunks, total);
 }
 
 }  // namespace
 
+long fused_mix_backward_sum_rows(long B, int H, int L) {
+  if (B <= 0 || H <= 0 || L <= 0) return 0;
+  return B * plan_mix_bwd(B, H, L).chunks;
+}
+
 hipError_t fused_mix_backward(const MixBwdArgs& p, hipStream_t s) {
   const MixPlan m = plan_mix_bwd(p.B, p.H, p.L);
-  if (p.dtype == kBf16) launch_mix_bwd<Bf16>(p, m, s);
-  else launch_mix_bwd<Fp16>(p, m, s);
+  const bool sums = p.sum_da != nullptr;
+  if (p.dtype == kBf16) {
+    if (sums) launch_mix_bwd<Bf16, true>(p, m, s);
+    else launch_mix_bwd<Bf16, false>(p, m, s);
+  } else {
+    if (sums) launch_mix_bwd<Fp16, true>(p, m, s);
+    else launch_mix_bwd<Fp16, false>(p, m, s);
+  }
   return hipGetLastError();
 }
 

@@ -56,8 +56,11 @@ struct MixBwdArgs {
   void *da_logit, *db_logit, *dc, *dv;           // same shapes as the inputs they belong to
   int B, L, H, kv_groups;
   int dtype;
+  // all three null, or fp32 [fused_mix_backward_sum_rows(B, H, L), H | Hkv*16 | Hkv*16]: per-chunk sums over time
+  float *sum_da = nullptr, *sum_db = nullptr, *sum_dc = nullptr;
 };
 hipError_t fused_mix_backward(const MixBwdArgs& p, hipStream_t s);
+long fused_mix_backward_sum_rows(long B, int H, int L);
 
 // Streaming form (btp_jagged.hip). Tensors [B, H, D, L] / [B, H, L]; state vectors [B, H, D] / [B, H].
 struct JagPrefillArgs {

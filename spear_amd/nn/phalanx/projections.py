@@ -7,7 +7,9 @@ few dozen output tiles for 256 compute units. Here the token axis is cut into ``
 multiplied as one batched GEMM with fp32 partial results and then summed (the same fp32 accumulation,
 associated differently). The four input projections also share one backward: their input gradients
 accumulate in one buffer through the GEMM's own ``beta = 1`` epilogue instead of four products and
-three additions.
+three additions. ``project_and_mix`` goes one step further for the fused mixing stage: the stage's backward
+kernel leaves the column sums of the gate gradients (the three bias gradients) as it walks through time, so
+they are not read a second time to be summed.
 
 Short token axes gain nothing (their step is bound by launch overhead, of which this path has more), so
 the layer uses these functions from 8192 tokens on (``pays_off``).
@@ -21,7 +23,7 @@ from __future__ import annotations
 import torch
 import torch.nn.functional as F
 
-__all__ = ["weight_grad", "input_projections", "linear", "pays_off"]
+__all__ = ["weight_grad", "input_projections", "linear", "pays_off", "project_and_mix", "mix_kernel_sums_groups"]
 
 _TILE = 128           # output tile edge the slice count is sized against
 _TARGET_TILES = 1024  # about four tiles per compute unit
@@ -103,6 +105,77 @@ class _Linear(torch.autograd.Function):
     def backward(ctx, d):
         x, w = ctx.saved_tensors
         return (d @ w if ctx.needs_input_grad[0] else None, weight_grad(d, x) if ctx.needs_input_grad[1] else None)
+
+
+def mix_kernel_sums_groups(heads: int, kv_heads: int) -> bool:
+    """Whether the fused backward kernel handles this head grouping (a group inside one wavefront)."""
+    groups = heads // kv_heads
+    return heads % 4 == 0 and heads % kv_heads == 0 and groups in (1, 2, 4, 8) and (groups < 8 or heads % 8 == 0)
+
+
+@torch.library.custom_op("spear_amd::mix_backward_with_bias_grads", mutates_args=())
+def _mix_backward_with_bias_grads(
+    a_logits: torch.Tensor, b_logits: torch.Tensor, c: torch.Tensor, v: torch.Tensor, dout: torch.Tensor,
+    heads: int, kv_heads: int,
+) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    """Gradients of the fused mixing stage and the column sums of the first three: ``(da, db, dc, dv,
+    da.sum over tokens, db.sum over tokens, dc.sum over tokens)``."""
+    from spear_amd import _btp
+
+    B, L, _ = v.shape
+    grads = [torch.empty_like(t) for t in (a_logits, b_logits, c, v)]
+    rows = _btp.mix_backward_sum_rows(B, L, heads)
+    sums = [torch.empty((rows, t.shape[-1]), device=v.device, dtype=torch.float32) for t in (a_logits, b_logits, c)]
+    _btp.mix_backward(a_logits, b_logits, c, v, dout, *grads, heads, kv_heads, sums=tuple(sums))
+    return (*grads, *(s.sum(0).to(v.dtype) for s in sums))
+
+
+@_mix_backward_with_bias_grads.register_fake
+def _(a_logits, b_logits, c, v, dout, heads, kv_heads):
+    grads = [torch.empty_like(t) for t in (a_logits, b_logits, c, v)]
+    return (*grads, *(t.new_empty((t.shape[-1],)) for t in (a_logits, b_logits, c)))
+
+
+class _ProjectAndMix(torch.autograd.Function):
+    """x[B, L, K] -> mixing stage of its four projections, [B, L, heads*16]."""
+
+    @staticmethod
+    def forward(ctx, x, w_a, b_a, w_b, b_b, w_c, b_c, w_v, heads: int, kv_heads: int):
+        a, b, c, v = F.linear(x, w_a, b_a), F.linear(x, w_b, b_b), F.linear(x, w_c, b_c), F.linear(x, w_v)
+        out = torch.empty_like(v)
+        torch.ops.spear_btp.mix_forward(a, b, c, v, out, heads, kv_heads)
+        ctx.save_for_backward(x, w_a, w_b, w_c, w_v, a, b, c, v)
+        ctx.heads, ctx.kv_heads = heads, kv_heads
+        return out
+
+    @staticmethod
+    def backward(ctx, dout):
+        x, w_a, w_b, w_c, w_v, a, b, c, v = ctx.saved_tensors
+        need = ctx.needs_input_grad
+        d_a, d_b, d_c, d_v, s_a, s_b, s_c = _mix_backward_with_bias_grads(
+            a, b, c, v, dout.contiguous(), ctx.heads, ctx.kv_heads)
+        x2 = x.reshape(-1, x.shape[-1])
+        d_a, d_b, d_c, d_v = (t.view(-1, t.shape[-1]) for t in (d_a, d_b, d_c, d_v))
+        dx = None
+        if need[0]:
+            dx = d_v @ w_v
+            dx.addmm_(d_b, w_b).addmm_(d_c, w_c).addmm_(d_a, w_a)
+            dx = dx.view(x.shape)
+        return (dx,
+                weight_grad(d_a, x2) if need[1] else None, s_a if need[2] else None,
+                weight_grad(d_b, x2) if need[3] else None, s_b if need[4] else None,
+                weight_grad(d_c, x2) if need[5] else None, s_c if need[6] else None,
+                weight_grad(d_v, x2) if need[7] else None, None, None)
+
+
+def project_and_mix(x: torch.Tensor, proj_a, proj_b, proj_c, proj_v, heads: int, kv_heads: int) -> torch.Tensor:
+    """``phalanx_mix(proj_a(x), proj_b(x), proj_c(x), proj_v(x), heads, kv_heads)`` for ``x[B, L, K]`` with the
+    projections' backward of this module and the bias gradients taken from the mixing kernel. Needs a head
+    grouping the fused backward kernel handles (``mix_kernel_sums_groups``)."""
+    import spear_amd.ops.btp.fused  # noqa: F401  (registers torch.ops.spear_btp.mix_forward)
+
+    return _ProjectAndMix.apply(x.contiguous(), proj_a.weight, proj_a.bias, proj_b.weight, proj_b.bias,
+                                proj_c.weight, proj_c.bias, proj_v.weight, heads, kv_heads)
 
 
 def input_projections(x: torch.Tensor, proj_a, proj_b, proj_c, proj_v):

@@ -29,7 +29,7 @@ from __future__ import annotations
 import torch
 import torch.nn as nn
 
-from .projections import input_projections, linear, pays_off
+from .projections import input_projections, linear, mix_kernel_sums_groups, pays_off, project_and_mix
 
 _HEAD_DIM = 16
 _METHODS = ("default", "pytorch", "pytorch_linspace", "fused")
@@ -217,8 +217,13 @@ class Phalanx(nn.Module):
         return self._mix_and_project(self.btp_module(A, X, self.k, self.wpb, self.output_dtype), C, V)
 
     def _forward_fused(self, x: torch.Tensor) -> torch.Tensor:
-        a_logits, b_logits, c, v = self.param.project(x)
-        return self._project_out(self.mix_module(a_logits, b_logits, c, v, self.heads, self.kv_heads))
+        p = self.param
+        xc = x.to(p.compute_dtype)
+        if xc.dim() == 3 and pays_off(xc) and mix_kernel_sums_groups(self.heads, self.kv_heads):
+            mixed = project_and_mix(xc, p.proj_a, p.proj_b, p.proj_c, p.proj_v, self.heads, self.kv_heads)
+        else:
+            mixed = self.mix_module(*p.project(xc), self.heads, self.kv_heads)
+        return self._project_out(mixed)
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         return self._forward_fn(x)

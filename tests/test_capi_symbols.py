@@ -29,6 +29,8 @@ def test_header_declares_the_expected_entry_points():
         "spear_jagged_prefill",
         "spear_jagged_step",
         "spear_phalanx_mix_backward",
+        "spear_phalanx_mix_backward_sum_rows",
+        "spear_phalanx_mix_backward_sums",
         "spear_phalanx_mix_forward",
     ]
 
@@ -64,7 +66,7 @@ def test_host_side_validation_needs_no_gpu():
     from spear_amd import _btp
 
     lib = _btp.load_library()
-    assert lib.spear_btp_abi_version() == 7
+    assert lib.spear_btp_abi_version() == 8
     buf = ctypes.create_string_buffer(4096)
     p = ctypes.addressof(buf)
     p -= p % 16
@@ -98,6 +100,16 @@ def test_host_side_validation_needs_no_gpu():
     # fused layer kernels: a batch row must fit one 32-bit buffer resource
     assert lib.spear_phalanx_mix_forward(p, p, p, p, p, 1, 1 << 20, 128, 128, 0, 0, None) == -1
     assert b"below 2 GiB" in lib.spear_btp_last_error()
+    # backward with column sums: the three arrays come together and with the row count the library states
+    rows = lib.spear_phalanx_mix_backward_sum_rows(2, 64, 8)
+    assert rows >= 2 and rows % 2 == 0
+    assert lib.spear_phalanx_mix_backward_sum_rows(2, 60, 8) == 0 and lib.spear_phalanx_mix_backward_sum_rows(0, 64, 8) == 0
+    sums = lambda sa, sb, sc, n: lib.spear_phalanx_mix_backward_sums(p, p, p, p, p, p, p, p, p, sa, sb, sc, n, 2, 64, 8, 8, 0, 0, None)
+    assert sums(p, p, None, rows) == -2
+    assert b"given together" in lib.spear_btp_last_error()
+    assert sums(p, p, p, rows + 1) == -1
+    assert b"rows for this shape" in lib.spear_btp_last_error()
+    assert sums(p + 4, p, p, rows) == -1
 
 
 def test_streaming_entry_points_validate_on_the_host():

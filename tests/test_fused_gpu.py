@@ -89,6 +89,36 @@ def test_fused_backward_with_shared_kv_heads(B, L, H, Hkv):
     assert_close(f64(da), rda, BF16_ATOL, BF16_RTOL, "da")
 
 
+@pytest.mark.parametrize("B,L,H,Hkv", [(1, 16, 4, 4), (3, 128, 8, 8), (2, 144, 16, 2), (1, 80, 12, 3), (1, 272, 32, 4),
+                                       (2, 2064, 8, 1), (40, 64, 32, 32), (1, 8192, 8, 8)])
+def test_fused_backward_column_sums_match_oracle(B, L, H, Hkv):
+    """The partial sums the backward kernel leaves add up to the oracle's gradients summed over batch and
+    time (the bias gradients of proj_a, proj_b, proj_c); the gradients themselves are unchanged by asking."""
+    from spear_amd import _btp
+
+    a, b, c, v = make_mix_inputs(B, L, H, Hkv, seed=5000 + L + H)
+    dout = torch.randn(B, L, H * 16, generator=torch.Generator().manual_seed(L + 2)).bfloat16()
+    print(f"fused bwd sums B={B} L={L} H={H} Hkv={Hkv}", flush=True)
+    plain = run_mix_backward(a, b, c, v, dout, H, Hkv)
+    dev = [t.to(DEV) for t in (a, b, c, v, dout)]
+    outs = [torch.full(t.shape, float("nan"), device=DEV, dtype=t.dtype) for t in (a, b, c, v)]
+    rows = _btp.mix_backward_sum_rows(B, L, H)
+    assert rows >= B and rows % B == 0
+    sums = tuple(torch.full((rows, w), float("nan"), device=DEV) for w in (H, Hkv * 16, Hkv * 16))
+    _btp.mix_backward(*dev, *outs, H, Hkv, sums=sums)
+    torch.cuda.synchronize()
+    for got, want in zip(outs, plain):
+        assert torch.equal(got.cpu(), want)
+    rda, rdb, rdc, _ = orc.phalanx_mix_backward(f64(a), f64(b), f64(c), f64(v), f64(dout), H, Hkv)
+    for name, s, ref in (("da", sums[0], rda), ("db", sums[1], rdb), ("dc", sums[2], rdc)):
+        got = f64(s.cpu()).sum(0)
+        want, mass = ref.sum((0, 1)), np.abs(ref).sum((0, 1))
+        # fp32 arithmetic on bf16 inputs; the sums are taken before any rounding to bf16
+        assert np.all(np.abs(got - want) <= 2e-4 * mass + 1e-5), (name, np.abs(got - want).max(), mass.max())
+    with pytest.raises(RuntimeError, match="shape"):
+        _btp.mix_backward(*dev, *outs, H, Hkv, sums=tuple(torch.empty(rows + 1, w, device=DEV) for w in (H, Hkv * 16, Hkv * 16)))
+
+
 def test_fused_backward_fp16_and_steep_gates():
     a, b, c, v = make_mix_inputs(2, 96, 8, 4, seed=6, dtype=torch.float16, scale=3.0)
     a[0, :10, :] = -30.0  # decay ~ 1e-13: counts as zero
