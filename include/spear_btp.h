@@ -105,7 +105,14 @@ int spear_phalanx_mix_backward(const void* a_logit, const void* b_logit, const v
                                const void* dout, void* da_logit, void* db_logit, void* dc, void* dv, int B, int L,
                                int H, int kv_heads, int dtype, unsigned flags, void* stream);
 
-/* The same backward, which in addition leaves the column sums of da_logit, db_logit and dc -- the bias
+/* The same backward with two options.
+ * (1) Row strides for the outputs: ld_da, ld_db, ld_dc, ld_dv are the elements per time step of the four
+ * gradient tensors, 0 meaning dense (the tensor's own width). With strides the four can be column blocks of
+ * one [B, L, ld] buffer (all four ld equal, the pointers offset into its first row), which is then the
+ * gradient of the four projections' concatenated output: one GEMM each for the input and the weight gradient
+ * instead of four. A stride is an even number of elements not below the tensor's width; elements between
+ * the blocks are not touched.
+ * (2) It leaves the column sums of da_logit, db_logit and dc -- the bias
  * gradients of the projections that produced a_logit, b_logit and c (spear/nn/phalanx/swr.py:157-163 gives
  * proj_a, proj_b and proj_c a bias) -- so that the caller does not read the three gradients again to
  * sum them. The kernel cannot finish the sums without a second pass, so it leaves partial sums in fp32:
@@ -113,13 +120,14 @@ int spear_phalanx_mix_backward(const void* a_logit, const void* b_logit, const v
  * where row r sums the time steps of one (batch row, time chunk) and the caller adds the rows up
  * (sum_rows is a few per batch row at most). sum_rows must equal
  * spear_phalanx_mix_backward_sum_rows(B, L, H); every element of the three arrays is written; the sums
- * are taken before the gradients are rounded to `dtype`. All three NULL: exactly
- * spear_phalanx_mix_backward. */
+ * are taken before the gradients are rounded to `dtype`. All three NULL: no sums. With neither option it is
+ * exactly spear_phalanx_mix_backward. */
 long long spear_phalanx_mix_backward_sum_rows(int B, int L, int H);
-int spear_phalanx_mix_backward_sums(const void* a_logit, const void* b_logit, const void* c, const void* v,
-                                    const void* dout, void* da_logit, void* db_logit, void* dc, void* dv, float* sum_da,
-                                    float* sum_db, float* sum_dc, long long sum_rows, int B, int L, int H, int kv_heads,
-                                    int dtype, unsigned flags, void* stream);
+int spear_phalanx_mix_backward_ex(const void* a_logit, const void* b_logit, const void* c, const void* v,
+                                  const void* dout, void* da_logit, void* db_logit, void* dc, void* dv, int ld_da,
+                                  int ld_db, int ld_dc, int ld_dv, float* sum_da, float* sum_db, float* sum_dc,
+                                  long long sum_rows, int B, int L, int H, int kv_heads, int dtype, unsigned flags,
+                                  void* stream);
 
 /* ---- streaming form: prompt prefill with state hand-over, and the one-token decode step --------
  * They replace the PyTorch loops of spear/nn/phalanx/inference.py. Tensors are dense, row-major:

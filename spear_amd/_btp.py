@@ -54,8 +54,8 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.spear_phalanx_mix_forward.restype = ci
     lib.spear_phalanx_mix_backward.argtypes = [vp] * 9 + [ci, ci, ci, ci, ci, cu, vp]
     lib.spear_phalanx_mix_backward.restype = ci
-    lib.spear_phalanx_mix_backward_sums.argtypes = [vp] * 12 + [ctypes.c_longlong, ci, ci, ci, ci, ci, cu, vp]
-    lib.spear_phalanx_mix_backward_sums.restype = ci
+    lib.spear_phalanx_mix_backward_ex.argtypes = [vp] * 9 + [ci] * 4 + [vp] * 3 + [ctypes.c_longlong, ci, ci, ci, ci, ci, cu, vp]
+    lib.spear_phalanx_mix_backward_ex.restype = ci
     lib.spear_phalanx_mix_backward_sum_rows.argtypes = [ci, ci, ci]
     lib.spear_phalanx_mix_backward_sum_rows.restype = ctypes.c_longlong
     lib.spear_jagged_prefill.argtypes = [vp] * 9 + [ci] * 9 + [cu, vp]
@@ -127,6 +127,17 @@ def _check_layout(name: str, t: torch.Tensor, shape: tuple[int, ...]) -> None:
     # (csrc/btp/_bindings.cu:80-87); a wrong shape there is an out-of-bounds read. Here it raises.
     _check(tuple(t.shape) == shape, f"{name} must have shape {list(shape)}, got {list(t.shape)}.")
     _check(t.is_contiguous(), f"{name} must be contiguous.")
+
+
+def _row_stride(name: str, t: torch.Tensor, shape: tuple[int, int, int]) -> int:
+    """Elements per time step of a ``[B, L, width]`` tensor that is dense or a column block of a wider
+    ``[B, L, ld]`` buffer."""
+    _check(tuple(t.shape) == shape, f"{name} must have shape {list(shape)}, got {list(t.shape)}.")
+    B, L, _ = shape
+    ld = t.stride(1) if L > 1 else (t.stride(0) if B > 1 else shape[2])
+    _check(t.stride(2) == 1 and (L <= 1 or t.stride(1) == ld) and (B <= 1 or t.stride(0) == L * ld),
+           f"{name} must be dense or a column block of a dense [B, L, ld] buffer.")
+    return ld
 
 
 def _raise_native(lib: ctypes.CDLL, rc: int) -> None:
@@ -331,7 +342,8 @@ def mix_backward(
     """Gradients of :func:`mix_forward`, written in place; ``heads // kv_heads`` must be 1, 2, 4 or 8
     (see ``spear_phalanx_mix_backward`` in the C header). ``sums``: three fp32 tensors
     ``[mix_backward_sum_rows(B, L, heads), heads | kv_heads*16 | kv_heads*16]`` that receive the per-chunk
-    column sums of ``da_logit``, ``db_logit`` and ``dc`` (``spear_phalanx_mix_backward_sums``)."""
+    column sums of ``da_logit``, ``db_logit`` and ``dc``. The four gradient tensors may be column blocks of one
+    wider ``[B, L, ld]`` buffer (``spear_phalanx_mix_backward_ex``)."""
     tensors = (a_logit, b_logit, c, v, dout, da_logit, db_logit, dc, dv)
     _check(all(t.is_cuda for t in tensors), "All tensors must be CUDA.")
     _check(v.dim() == 3, "v must be [B, L, heads * 16].")
@@ -345,11 +357,12 @@ def mix_backward(
     _check(L % 16 == 0, "Length L must be multiple of 16")
     Fkv = kv_heads * 16
     for name, t, shape in (
-        ("a_logit", a_logit, (B, L, heads)), ("da_logit", da_logit, (B, L, heads)),
-        ("b_logit", b_logit, (B, L, Fkv)), ("c", c, (B, L, Fkv)), ("v", v, (B, L, F)), ("dout", dout, (B, L, F)),
-        ("db_logit", db_logit, (B, L, Fkv)), ("dc", dc, (B, L, Fkv)), ("dv", dv, (B, L, F)),
+        ("a_logit", a_logit, (B, L, heads)), ("b_logit", b_logit, (B, L, Fkv)), ("c", c, (B, L, Fkv)),
+        ("v", v, (B, L, F)), ("dout", dout, (B, L, F)),
     ):
         _check_layout(name, t, shape)
+    lds = [_row_stride(name, t, (B, L, width)) for name, t, width in
+           (("da_logit", da_logit, heads), ("db_logit", db_logit, Fkv), ("dc", dc, Fkv), ("dv", dv, F))]
     _check(len({t.device for t in tensors}) == 1, "All tensors must be on the same device.")
     lib = load_library()
     rows = 0
@@ -360,9 +373,9 @@ def mix_backward(
             _check_layout(name, t, (rows, width))
     sum_ptrs = [t.data_ptr() for t in sums] if rows > 0 else [None, None, None]
     with torch.cuda.device(v.device):
-        rc = lib.spear_phalanx_mix_backward_sums(
+        rc = lib.spear_phalanx_mix_backward_ex(
             a_logit.data_ptr(), b_logit.data_ptr(), c.data_ptr(), v.data_ptr(), dout.data_ptr(),
-            da_logit.data_ptr(), db_logit.data_ptr(), dc.data_ptr(), dv.data_ptr(),
+            da_logit.data_ptr(), db_logit.data_ptr(), dc.data_ptr(), dv.data_ptr(), *lds,
             *sum_ptrs, rows,
             B, L, heads, kv_heads, _tag(v.dtype), 0, _stream_ptr(v.device),
         )

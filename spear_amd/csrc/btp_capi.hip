@@ -160,14 +160,15 @@ long long spear_phalanx_mix_backward_sum_rows(int B, int L, int H) {
 int spear_phalanx_mix_backward(const void* a_logit, const void* b_logit, const void* c, const void* v, const void* dout,
                                void* da_logit, void* db_logit, void* dc, void* dv, int B, int L, int H, int kv_heads,
                                int dtype, unsigned flags, void* stream) {
-  return spear_phalanx_mix_backward_sums(a_logit, b_logit, c, v, dout, da_logit, db_logit, dc, dv, nullptr, nullptr,
-                                         nullptr, 0, B, L, H, kv_heads, dtype, flags, stream);
+  return spear_phalanx_mix_backward_ex(a_logit, b_logit, c, v, dout, da_logit, db_logit, dc, dv, 0, 0, 0, 0, nullptr,
+                                       nullptr, nullptr, 0, B, L, H, kv_heads, dtype, flags, stream);
 }
 
-int spear_phalanx_mix_backward_sums(const void* a_logit, const void* b_logit, const void* c, const void* v,
-                                    const void* dout, void* da_logit, void* db_logit, void* dc, void* dv, float* sum_da,
-                                    float* sum_db, float* sum_dc, long long sum_rows, int B, int L, int H, int kv_heads,
-                                    int dtype, unsigned flags, void* stream) {
+int spear_phalanx_mix_backward_ex(const void* a_logit, const void* b_logit, const void* c, const void* v,
+                                  const void* dout, void* da_logit, void* db_logit, void* dc, void* dv, int ld_da,
+                                  int ld_db, int ld_dc, int ld_dv, float* sum_da, float* sum_db, float* sum_dc,
+                                  long long sum_rows, int B, int L, int H, int kv_heads, int dtype, unsigned flags,
+                                  void* stream) {
   g_error[0] = '\0';
   const char* who = "spear_phalanx_mix_backward";
   if (B < 0 || L < 0 || H < 0) return fail(SPEAR_BTP_EINVAL, "%s: negative dimension (B=%d L=%d H=%d)", who, B, L, H);
@@ -192,6 +193,14 @@ int spear_phalanx_mix_backward_sums(const void* a_logit, const void* b_logit, co
     if (!q) return fail(SPEAR_BTP_ENULL, "%s: NULL tensor pointer", who);
     if (!aligned16(q)) return fail(SPEAR_BTP_EINVAL, "%s: tensor pointers must be 16-byte aligned", who);
   }
+  const int widths[4] = {H, kv_heads * 16, kv_heads * 16, H * 16}, lds[4] = {ld_da, ld_db, ld_dc, ld_dv};
+  for (int i = 0; i < 4; ++i) {
+    if (lds[i] == 0) continue;
+    if (lds[i] < widths[i] || lds[i] % 2 != 0)
+      return fail(SPEAR_BTP_EINVAL, "%s: a gradient's row stride must be 0 (dense) or an even number of elements not below its width (got %d for width %d)", who, lds[i], widths[i]);
+    if ((long long)L * lds[i] * 2ll >= (1ll << 31))
+      return fail(SPEAR_BTP_EINVAL, "%s: one batch row (L * row stride) must stay below 2 GiB", who);
+  }
   const bool sums = sum_da || sum_db || sum_dc;
   if (sums) {
     if (!sum_da || !sum_db || !sum_dc) return fail(SPEAR_BTP_ENULL, "%s: the three sum arrays must be given together", who);
@@ -202,7 +211,7 @@ int spear_phalanx_mix_backward_sums(const void* a_logit, const void* b_logit, co
       return fail(SPEAR_BTP_EINVAL, "%s: sum arrays must have %lld rows for this shape (got %lld)", who, want, sum_rows);
   }
   spear_btp::MixBwdArgs a{a_logit, b_logit, c, v, dout, da_logit, db_logit, dc, dv, B, L, H, groups, dtype,
-                          sum_da, sum_db, sum_dc};
+                          sum_da, sum_db, sum_dc, ld_da, ld_db, ld_dc, ld_dv};
   const hipError_t err = spear_btp::fused_mix_backward(a, static_cast<hipStream_t>(stream));
   if (err != hipSuccess) return fail(SPEAR_BTP_ELAUNCH, "%s: launch failed: %s", who, hipGetErrorString(err));
   return 0;

@@ -237,8 +237,8 @@ __global__ __launch_bounds__(64 * kWaves) void phalanx_mix_bwd_kernel(
     const uint16_t* __restrict__ a_logit, const uint16_t* __restrict__ b_logit, const uint16_t* __restrict__ c_in,
     const uint16_t* __restrict__ v_in, const uint16_t* __restrict__ dout, uint16_t* __restrict__ da_logit,
     uint16_t* __restrict__ db_logit, uint16_t* __restrict__ dc, uint16_t* __restrict__ dv, float* __restrict__ sum_da,
-    float* __restrict__ sum_db, float* __restrict__ sum_dc, int L, int H, int kv_groups, int chunk_steps, int chunks,
-    long total_waves) {
+    float* __restrict__ sum_db, float* __restrict__ sum_dc, int ld_da, int ld_db, int ld_dc, int ld_dv, int L, int H,
+    int kv_groups, int chunk_steps, int chunks, long total_waves) {
   __shared__ __align__(16) float gate_tiles[kWaves][2][kHeadsPerWave * kGateRow];  // decay of two blocks
   __shared__ __align__(16) float4 park[kWaves][kTile][64];                        // (R0, R1, dX0, dX1) per step, lane
 
@@ -265,9 +265,13 @@ __global__ __launch_bounds__(64 * kWaves) void phalanx_mix_bwd_kernel(
   };
   const __amdgpu_buffer_rsrc_t rb = rsrc(b_logit, kvbig, L * kv_stride), rc = rsrc(c_in, kvbig, L * kv_stride),
                                rv = rsrc(v_in, big, L * stride), rg = rsrc(dout, big, L * stride),
-                               rdb = rsrc(db_logit, kvbig, L * kv_stride), rdc = rsrc(dc, kvbig, L * kv_stride),
-                               rdv = rsrc(dv, big, L * stride), ra = rsrc(a_logit, small, L * H * 2),
-                               rda = rsrc(da_logit, small, L * H * 2);
+                               ra = rsrc(a_logit, small, L * H * 2),
+                               // the four gradients may sit side by side in one wider buffer: each has its
+                               // own elements-per-time-step (ld_*), equal to its width when it is dense
+                               rdb = rsrc(db_logit, brow * L * ld_db, L * ld_db * 2),
+                               rdc = rsrc(dc, brow * L * ld_dc, L * ld_dc * 2),
+                               rdv = rsrc(dv, brow * L * ld_dv, L * ld_dv * 2),
+                               rda = rsrc(da_logit, brow * L * ld_da, L * ld_da * 2);
   const int f_lane = 2 * (head * kChan + d0);
   const int kv_lane = 2 * ((head / kv_groups) * kChan + d0);
   const int o_lane = real ? f_lane : 0x7ffffff0;  // lanes without a head store nowhere
@@ -277,7 +281,7 @@ __global__ __launch_bounds__(64 * kWaves) void phalanx_mix_bwd_kernel(
   const int gt = lane & 15, ghead = min(ho + 2 * (lane >> 4), H - 2);
   const int a_lane = 2 * (gt * H + ghead);
   // da_logit: lane k of a head (k = lane % 8) ends up with steps 2k and 2k+1 of that head
-  const int da_lane = real ? 2 * ((2 * (lane & 7)) * H + head) : 0x7ffffff0;
+  const int da_lane = real ? 2 * ((2 * (lane & 7)) * ld_da + head) : 0x7ffffff0;
   constexpr int kNt = 2;
 
   auto issue = [&](MixSet& m, int t) {
@@ -401,9 +405,9 @@ __global__ __launch_bounds__(64 * kWaves) void phalanx_mix_bwd_kernel(
       const uint32_t wdb = E::pack2(db0, db1);
       z0 = az0;
       z1 = az1;
-      __builtin_amdgcn_raw_buffer_store_b32(wdc, rdc, okv_off, (t0 + r) * kv_stride, kNt);
-      __builtin_amdgcn_raw_buffer_store_b32(wdv, rdv, o_off, (t0 + r) * stride, kNt);
-      __builtin_amdgcn_raw_buffer_store_b32(wdb, rdb, okv_off, (t0 + r) * kv_stride, kNt);
+      __builtin_amdgcn_raw_buffer_store_b32(wdc, rdc, okv_off, (t0 + r) * 2 * ld_dc, kNt);
+      __builtin_amdgcn_raw_buffer_store_b32(wdv, rdv, o_off, (t0 + r) * 2 * ld_dv, kNt);
+      __builtin_amdgcn_raw_buffer_store_b32(wdb, rdb, okv_off, (t0 + r) * 2 * ld_db, kNt);
     }
 
     // ---- dA: sum over the 8 lanes (16 channels) of the head, transposing: lane k keeps steps 2k, 2k+1
@@ -440,8 +444,8 @@ __global__ __launch_bounds__(64 * kWaves) void phalanx_mix_bwd_kernel(
     if constexpr (kSums) acc_a += da0 + da1;
     const int da_off = (t0 >= t_begin) ? da_lane : 0x7ffffff0;
     const uint32_t dap = E::pack2(da0, da1);
-    __builtin_amdgcn_raw_buffer_store_b16((unsigned short)(dap & 0xffffu), rda, da_off, t0 * H * 2, 0);
-    __builtin_amdgcn_raw_buffer_store_b16((unsigned short)(dap >> 16), rda, da_off + 2 * H, t0 * H * 2, 0);
+    __builtin_amdgcn_raw_buffer_store_b16((unsigned short)(dap & 0xffffu), rda, da_off, t0 * ld_da * 2, 0);
+    __builtin_amdgcn_raw_buffer_store_b16((unsigned short)(dap >> 16), rda, da_off + 2 * ld_da, t0 * ld_da * 2, 0);
     wave_lds_handover();  // tile `tc` and the parking slots are free for the iteration after next
   };
 
@@ -561,9 +565,11 @@ void launch_mix_bwd(const MixBwdArgs& p, const MixPlan& m, hipStream_t s) {
   const unsigned blocks = (unsigned)((total + kWaves - 1) / kWaves);
   auto u = [](const void* q) { return static_cast<const uint16_t*>(q); };
   auto w = [](void* q) { return static_cast<uint16_t*>(q); };
+  const int Fkv = (p.H / p.kv_groups) * kChan;
   hipLaunchKernelGGL((phalanx_mix_bwd_kernel<E, kSums>), dim3(blocks), dim3(64 * kWaves), 0, s, u(p.a_logit),
                      u(p.b_logit), u(p.c), u(p.v), u(p.dout), w(p.da_logit), w(p.db_logit), w(p.dc), w(p.dv), p.sum_da,
-                     p.sum_db, p.sum_dc, p.L, p.H, p.kv_groups, m.chunk_blocks * kTile, m.chunks, total);
+                     p.sum_db, p.sum_dc, p.ld_da ? p.ld_da : p.H, p.ld_db ? p.ld_db : Fkv, p.ld_dc ? p.ld_dc : Fkv,
+                     p.ld_dv ? p.ld_dv : p.H * kChan, p.L, p.H, p.kv_groups, m.chunk_blocks * kTile, m.chunks, total);
 }
 
 }  // namespace

@@ -58,6 +58,8 @@ struct MixBwdArgs {
   int dtype;
   // all three null, or fp32 [fused_mix_backward_sum_rows(B, H, L), H | Hkv*16 | Hkv*16]: per-chunk sums over time
   float *sum_da = nullptr, *sum_db = nullptr, *sum_dc = nullptr;
+  // elements per time step of each gradient tensor; 0 = dense (its own width)
+  int ld_da = 0, ld_db = 0, ld_dc = 0, ld_dv = 0;
 };
 hipError_t fused_mix_backward(const MixBwdArgs& p, hipStream_t s);
 long fused_mix_backward_sum_rows(long B, int H, int L);

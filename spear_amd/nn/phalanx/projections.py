@@ -7,9 +7,11 @@ few dozen output tiles for 256 compute units. Here the token axis is cut into ``
 multiplied as one batched GEMM with fp32 partial results and then summed (the same fp32 accumulation,
 associated differently). The four input projections also share one backward: their input gradients
 accumulate in one buffer through the GEMM's own ``beta = 1`` epilogue instead of four products and
-three additions. ``project_and_mix`` goes one step further for the fused mixing stage: the stage's backward
-kernel leaves the column sums of the gate gradients (the three bias gradients) as it walks through time, so
-they are not read a second time to be summed.
+three additions. ``project_and_mix`` goes further for the fused mixing stage: its backward kernel writes the
+four gradients side by side into one ``[B, L, ld]`` buffer, which is the gradient of the concatenated
+projection, so input and weight gradients are one GEMM each against the stacked weights (the forward stays
+four GEMMs, which measured faster than one wide one); and the kernel leaves the column sums of the gate
+gradients (the three bias gradients) as it walks through time, so they are not read again to be summed.
 
 Short token axes gain nothing (their step is bound by launch overhead, of which this path has more), so
 the layer uses these functions from 8192 tokens on (``pays_off``).
@@ -23,7 +25,8 @@ from __future__ import annotations
 import torch
 import torch.nn.functional as F
 
-__all__ = ["weight_grad", "input_projections", "linear", "pays_off", "project_and_mix", "mix_kernel_sums_groups"]
+__all__ = ["weight_grad", "input_projections", "linear", "pays_off", "project_and_mix", "mix_kernel_sums_groups",
+           "packed_columns"]
 
 _TILE = 128           # output tile edge the slice count is sized against
 _TARGET_TILES = 1024  # about four tiles per compute unit
@@ -113,27 +116,44 @@ def mix_kernel_sums_groups(heads: int, kv_heads: int) -> bool:
     return heads % 4 == 0 and heads % kv_heads == 0 and groups in (1, 2, 4, 8) and (groups < 8 or heads % 8 == 0)
 
 
-@torch.library.custom_op("spear_amd::mix_backward_with_bias_grads", mutates_args=())
-def _mix_backward_with_bias_grads(
+def packed_columns(heads: int, kv_heads: int) -> tuple[dict[str, tuple[int, int]], int]:
+    """Column blocks ``name -> (first column, width)`` of the four projections' outputs laid side by side
+    as ``[b | c | v | a | padding]``, and the padded row length (a multiple of 64 elements, so that every
+    row of the packed buffer starts on a 128-byte line)."""
+    Fkv, F = kv_heads * 16, heads * 16
+    cols = {"b": (0, Fkv), "c": (Fkv, Fkv), "v": (2 * Fkv, F), "a": (2 * Fkv + F, heads)}
+    used = 2 * Fkv + F + heads
+    return cols, -(-used // 64) * 64
+
+
+@torch.library.custom_op("spear_amd::mix_backward_packed", mutates_args=())
+def _mix_backward_packed(
     a_logits: torch.Tensor, b_logits: torch.Tensor, c: torch.Tensor, v: torch.Tensor, dout: torch.Tensor,
     heads: int, kv_heads: int,
-) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
-    """Gradients of the fused mixing stage and the column sums of the first three: ``(da, db, dc, dv,
-    da.sum over tokens, db.sum over tokens, dc.sum over tokens)``."""
+) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    """Backward of the fused mixing stage with its four gradients written side by side into one
+    ``[B, L, ld]`` buffer (``packed_columns``; padding columns zero), and the sums over all tokens of the
+    ``a``, ``b`` and ``c`` blocks: ``(packed, da.sum, db.sum, dc.sum)``."""
     from spear_amd import _btp
 
     B, L, _ = v.shape
-    grads = [torch.empty_like(t) for t in (a_logits, b_logits, c, v)]
+    cols, ld = packed_columns(heads, kv_heads)
+    packed = torch.empty((B, L, ld), device=v.device, dtype=v.dtype)
+    used = cols["a"][0] + cols["a"][1]
+    if used < ld:
+        packed[..., used:].zero_()
+    da, db, dc, dv = (packed[..., cols[k][0]:cols[k][0] + cols[k][1]] for k in "abcv")
     rows = _btp.mix_backward_sum_rows(B, L, heads)
     sums = [torch.empty((rows, t.shape[-1]), device=v.device, dtype=torch.float32) for t in (a_logits, b_logits, c)]
-    _btp.mix_backward(a_logits, b_logits, c, v, dout, *grads, heads, kv_heads, sums=tuple(sums))
-    return (*grads, *(s.sum(0).to(v.dtype) for s in sums))
+    _btp.mix_backward(a_logits, b_logits, c, v, dout, da, db, dc, dv, heads, kv_heads, sums=tuple(sums))
+    return (packed, *(s.sum(0).to(v.dtype) for s in sums))
 
 
-@_mix_backward_with_bias_grads.register_fake
+@_mix_backward_packed.register_fake
 def _(a_logits, b_logits, c, v, dout, heads, kv_heads):
-    grads = [torch.empty_like(t) for t in (a_logits, b_logits, c, v)]
-    return (*grads, *(t.new_empty((t.shape[-1],)) for t in (a_logits, b_logits, c)))
+    B, L, _ = v.shape
+    packed = v.new_empty((B, L, packed_columns(heads, kv_heads)[1]))
+    return (packed, *(t.new_empty((t.shape[-1],)) for t in (a_logits, b_logits, c)))
 
 
 class _ProjectAndMix(torch.autograd.Function):
@@ -152,20 +172,24 @@ class _ProjectAndMix(torch.autograd.Function):
     def backward(ctx, dout):
         x, w_a, w_b, w_c, w_v, a, b, c, v = ctx.saved_tensors
         need = ctx.needs_input_grad
-        d_a, d_b, d_c, d_v, s_a, s_b, s_c = _mix_backward_with_bias_grads(
-            a, b, c, v, dout.contiguous(), ctx.heads, ctx.kv_heads)
-        x2 = x.reshape(-1, x.shape[-1])
-        d_a, d_b, d_c, d_v = (t.view(-1, t.shape[-1]) for t in (d_a, d_b, d_c, d_v))
+        packed, s_a, s_b, s_c = _mix_backward_packed(a, b, c, v, dout.contiguous(), ctx.heads, ctx.kv_heads)
+        cols, ld = packed_columns(ctx.heads, ctx.kv_heads)
+        x2, d2 = x.reshape(-1, x.shape[-1]), packed.view(-1, ld)
+        # one GEMM each against the weights stacked in the buffer's column order
         dx = None
         if need[0]:
-            dx = d_v @ w_v
-            dx.addmm_(d_b, w_b).addmm_(d_c, w_c).addmm_(d_a, w_a)
-            dx = dx.view(x.shape)
-        return (dx,
-                weight_grad(d_a, x2) if need[1] else None, s_a if need[2] else None,
-                weight_grad(d_b, x2) if need[3] else None, s_b if need[4] else None,
-                weight_grad(d_c, x2) if need[5] else None, s_c if need[6] else None,
-                weight_grad(d_v, x2) if need[7] else None, None, None)
+            stacked = [w_b, w_c, w_v, w_a]
+            pad = ld - (cols["a"][0] + cols["a"][1])
+            if pad:
+                stacked.append(w_a.new_zeros((pad, w_a.shape[1])))
+            dx = (d2 @ torch.cat(stacked)).view(x.shape)
+        dw = weight_grad(d2, x2) if any(need[i] for i in (1, 3, 5, 7)) else None
+
+        def rows_of(name, wanted):
+            return dw[cols[name][0]:cols[name][0] + cols[name][1]] if wanted else None
+
+        return (dx, rows_of("a", need[1]), s_a if need[2] else None, rows_of("b", need[3]), s_b if need[4] else None,
+                rows_of("c", need[5]), s_c if need[6] else None, rows_of("v", need[7]), None, None)
 
 
 def project_and_mix(x: torch.Tensor, proj_a, proj_b, proj_c, proj_v, heads: int, kv_heads: int) -> torch.Tensor:

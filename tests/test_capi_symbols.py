@@ -29,8 +29,8 @@ def test_header_declares_the_expected_entry_points():
         "spear_jagged_prefill",
         "spear_jagged_step",
         "spear_phalanx_mix_backward",
+        "spear_phalanx_mix_backward_ex",
         "spear_phalanx_mix_backward_sum_rows",
-        "spear_phalanx_mix_backward_sums",
         "spear_phalanx_mix_forward",
     ]
 
@@ -104,12 +104,19 @@ def test_host_side_validation_needs_no_gpu():
     rows = lib.spear_phalanx_mix_backward_sum_rows(2, 64, 8)
     assert rows >= 2 and rows % 2 == 0
     assert lib.spear_phalanx_mix_backward_sum_rows(2, 60, 8) == 0 and lib.spear_phalanx_mix_backward_sum_rows(0, 64, 8) == 0
-    sums = lambda sa, sb, sc, n: lib.spear_phalanx_mix_backward_sums(p, p, p, p, p, p, p, p, p, sa, sb, sc, n, 2, 64, 8, 8, 0, 0, None)
+    sums = lambda sa, sb, sc, n, ld=(0, 0, 0, 0): lib.spear_phalanx_mix_backward_ex(
+        p, p, p, p, p, p, p, p, p, *ld, sa, sb, sc, n, 2, 64, 8, 8, 0, 0, None)
     assert sums(p, p, None, rows) == -2
     assert b"given together" in lib.spear_btp_last_error()
     assert sums(p, p, p, rows + 1) == -1
     assert b"rows for this shape" in lib.spear_btp_last_error()
     assert sums(p + 4, p, p, rows) == -1
+    # output row strides: 0 or an even number of elements not below the tensor's width
+    assert sums(None, None, None, 0, (4, 0, 0, 0)) == -1
+    assert b"row stride" in lib.spear_btp_last_error()
+    assert sums(None, None, None, 0, (0, 0, 0, 131)) == -1
+    assert sums(None, None, None, 0, (0, 0, 0, 1 << 24)) == -1
+    assert b"below 2 GiB" in lib.spear_btp_last_error()
 
 
 def test_streaming_entry_points_validate_on_the_host():

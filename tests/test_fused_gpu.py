@@ -119,6 +119,36 @@ def test_fused_backward_column_sums_match_oracle(B, L, H, Hkv):
         _btp.mix_backward(*dev, *outs, H, Hkv, sums=tuple(torch.empty(rows + 1, w, device=DEV) for w in (H, Hkv * 16, Hkv * 16)))
 
 
+@pytest.mark.parametrize("B,L,H,Hkv", [(1, 16, 4, 4), (3, 128, 8, 8), (2, 144, 16, 2), (1, 80, 12, 3), (2, 2064, 8, 1), (40, 64, 32, 32)])
+def test_fused_backward_into_column_blocks_of_one_buffer(B, L, H, Hkv):
+    """The four gradients written side by side into one [B, L, ld] buffer are bit-identical to the dense
+    ones, and the columns between and after the blocks are left alone."""
+    from spear_amd import _btp
+    from spear_amd.nn.phalanx.projections import packed_columns
+
+    a, b, c, v = make_mix_inputs(B, L, H, Hkv, seed=6000 + L + H)
+    dout = torch.randn(B, L, H * 16, generator=torch.Generator().manual_seed(L + 3)).bfloat16()
+    print(f"fused bwd packed B={B} L={L} H={H} Hkv={Hkv}", flush=True)
+    plain = run_mix_backward(a, b, c, v, dout, H, Hkv)
+    cols, ld = packed_columns(H, Hkv)
+    assert ld % 64 == 0 and ld >= cols["a"][0] + cols["a"][1]
+    ld += 64                                              # more slack than needed, so there is padding to check
+    dev = [t.to(DEV) for t in (a, b, c, v, dout)]
+    marker = 12345.0
+    packed = torch.full((B, L, ld), marker, device=DEV, dtype=torch.bfloat16)
+    views = [packed[..., cols[k][0]:cols[k][0] + cols[k][1]] for k in "abcv"]
+    _btp.mix_backward(*dev, *views, H, Hkv)
+    torch.cuda.synchronize()
+    for got, want in zip(views, plain):
+        assert torch.equal(got.cpu(), want)
+    used = cols["a"][0] + cols["a"][1]
+    assert bool((packed[..., used:] == marker).all())
+    # a block that is not a column block of a dense buffer is refused
+    with pytest.raises(RuntimeError, match="column block"):
+        every_other = torch.empty(B, L, 2 * H * 16, device=DEV, dtype=torch.bfloat16)[..., ::2]
+        _btp.mix_backward(*dev, views[0], views[1], views[2], every_other, H, Hkv)
+
+
 def test_fused_backward_fp16_and_steep_gates():
     a, b, c, v = make_mix_inputs(2, 96, 8, 4, seed=6, dtype=torch.float16, scale=3.0)
     a[0, :10, :] = -30.0  # decay ~ 1e-13: counts as zero

@@ -82,3 +82,35 @@ def test_token_sliced_gradients_match_linear_autograd_on_the_gpu(B, L, dim, head
         got, ref = got.float(), ref.float()
         scale = ref.abs().max().item()
         assert (got - ref).abs().max().item() <= 2 ** -6 * scale, (got - ref).abs().max().item() / scale
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("B,L,dim,heads,kv_heads", [(2, 64, 128, 8, 8), (3, 128, 256, 16, 4), (96, 128, 256, 16, 16), (72, 128, 192, 12, 3)])
+def test_project_and_mix_matches_the_mixing_op_on_linear_autograd(B, L, dim, heads, kv_heads):
+    """``project_and_mix`` (packed gradient buffer, bias gradients from the kernel's sums) against
+    ``phalanx_mix`` applied to four ``nn.Linear`` outputs under plain autograd."""
+    from spear_amd.ops.btp import phalanx_mix
+
+    mods = _modules(dim, heads, kv_heads, torch.bfloat16, "cuda:0", 11)[:4]
+    g = torch.Generator(device="cpu").manual_seed(12)
+    x0 = torch.randn(B, L, dim, generator=g).bfloat16().to("cuda:0")
+    dout = torch.randn(B, L, heads * 16, generator=g).bfloat16().to("cuda:0")
+
+    def run(custom):
+        for m in mods:
+            m.zero_grad(set_to_none=True)
+        x = x0.clone().requires_grad_(True)
+        out = (pj.project_and_mix(x, *mods, heads, kv_heads) if custom
+               else phalanx_mix(*(m(x) for m in mods), heads, kv_heads))
+        out.backward(dout)
+        return out.detach(), [x.grad] + [p.grad for m in mods for p in m.parameters()]
+
+    (out, grads), (ref_out, ref_grads) = run(True), run(False)
+    assert torch.equal(out, ref_out)
+    names = ["x", "w_a", "b_a", "w_b", "b_b", "w_c", "b_c", "w_v"]
+    for name, got, ref in zip(names, grads, ref_grads):
+        assert got.shape == ref.shape, name
+        got, ref = got.float(), ref.float()
+        scale = ref.abs().max().item()
+        # bf16 results of fp32-accumulated sums; the bias sums are taken before the gradients' rounding
+        assert (got - ref).abs().max().item() <= 2 ** -6 * scale, (name, (got - ref).abs().max().item() / scale)
