@@ -110,6 +110,7 @@ def main() -> int:
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-fused", action="store_true", help="skip the fused layer-layout forward leg")
     ap.add_argument("--no-streaming", action="store_true", help="skip the prefill / decode-step leg")
+    ap.add_argument("--no-layer", action="store_true", help="skip the whole-layer (projections + mixing) leg")
     ap.add_argument("--settle-seconds", type=float, default=0.3, help="untimed run-in before the warm-up steps")
     args = ap.parse_args()
 
@@ -346,6 +347,52 @@ def main() -> int:
         }
         del msets
 
+    # the Phalanx layer end to end (five projections + mixing stage) on x[B, L, H*16], forward and
+    # forward+backward, for the reference's PyTorch-ops method, its kernel method and the fused method
+    layer = None
+    if H % 4 == 0 and not args.no_layer:
+        from spear_amd import Phalanx
+
+        dim = H * 16
+        gl = torch.Generator(device="cpu").manual_seed(seed + 13)
+        xl = torch.randn(B, L, dim, generator=gl).to(torch.bfloat16).to(dev).requires_grad_(True)
+        gout = torch.randn(B, L, dim, generator=gl).to(torch.bfloat16).to(dev)
+        layer = {"shape": {"B": B, "L": L, "dim": dim}, "unit": "ms", "methods": {}}
+        weights = None
+        for method in ("pytorch", "default", "fused"):
+            torch.manual_seed(seed)
+            mod = Phalanx(dim=dim, length=L, method=method, dtype=torch.bfloat16).to(dev)
+            if weights is None:
+                weights = mod.state_dict()
+            else:
+                mod.load_state_dict(weights)
+
+            def layer_fwd():
+                with torch.no_grad():
+                    mod(xl)
+
+            def layer_train():
+                mod.zero_grad(set_to_none=True)
+                xl.grad = None
+                mod(xl).backward(gout)
+
+            def layer_ms(fn, n=10):
+                for _ in range(2):
+                    fn()
+                torch.cuda.synchronize()
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record(stream)
+                for _ in range(n):
+                    fn()
+                e1.record(stream)
+                torch.cuda.synchronize()
+                return e0.elapsed_time(e1) / n
+
+            layer["methods"][method] = {"forward": layer_ms(layer_fwd), "forward_backward": layer_ms(layer_train)}
+            del mod
+        del xl, gout
+        torch.cuda.empty_cache()
+
     # streaming form: prompt prefill (recurrence + y*C+V + state hand-over) on the same tensors, and
     # the one-token decode step on [B, H, 16] operands with fp32 state
     streaming = None
@@ -501,6 +548,7 @@ def main() -> int:
                                   "algorithmic_bytes_per_unit": {"forward": 68, "backward": 108}},
         "fused_layer_stage": fused,
         "streaming": streaming,
+        "phalanx_layer": layer,
         "fwd_plus_bwd": {"achieved": step_gbps, "frac": step_gbps / HBM_PEAK_GBPS,
                          "algorithmic_bytes_per_step": units * (FWD_BYTES + BWD_BYTES)},
         "step_spread": spread,
