@@ -495,6 +495,13 @@ struct MixPlan {
   int wg_waves, chunk_blocks, chunks;
 };
 
+// Tuning overrides, read once per process (0 = not set).
+int env_override(const char* name) {
+  const char* e = getenv(name);
+  const int v = e ? atoi(e) : 0;
+  return v > 0 ? v : 0;
+}
+
 MixPlan plan_mix(long B, int H, int L) {
   const long octs = (H + 7) / 8;
   const int nb = L / kTile;
@@ -509,8 +516,10 @@ MixPlan plan_mix(long B, int H, int L) {
     if (chunks > nb / 8) chunks = nb / 8 > 0 ? nb / 8 : 1;
     m.chunk_blocks = (int)((nb + chunks - 1) / chunks);
   }
-  if (const char* e = getenv("SPEAR_BTP_FUSED_CHUNK_BLOCKS")) m.chunk_blocks = atoi(e) > 0 ? atoi(e) : m.chunk_blocks;
-  if (const char* e = getenv("SPEAR_BTP_FUSED_WG_WAVES")) m.wg_waves = atoi(e) == 8 ? 8 : 4;
+  static const int chunk_override = env_override("SPEAR_BTP_FUSED_CHUNK_BLOCKS");
+  static const int waves_override = env_override("SPEAR_BTP_FUSED_WG_WAVES");
+  if (chunk_override) m.chunk_blocks = chunk_override;
+  if (waves_override) m.wg_waves = waves_override == 8 ? 8 : 4;
   if (m.chunk_blocks > nb) m.chunk_blocks = nb;
   m.chunks = (nb + m.chunk_blocks - 1) / m.chunk_blocks;
   return m;
@@ -553,7 +562,8 @@ MixPlan plan_mix_bwd(long B, int H, int L) {
   const int min_blocks = B * octs * ((nb + 7) / 8) < 512 ? 2 : 8;  // badly underfilled: shorter chunks still pay
   if (chunks > nb / min_blocks) chunks = nb / min_blocks > 0 ? nb / min_blocks : 1;
   m.chunk_blocks = (int)((nb + chunks - 1) / chunks);
-  if (const char* e = getenv("SPEAR_BTP_FUSED_BWD_CHUNK_BLOCKS")) m.chunk_blocks = atoi(e) > 0 ? atoi(e) : m.chunk_blocks;
+  static const int chunk_override = env_override("SPEAR_BTP_FUSED_BWD_CHUNK_BLOCKS");
+  if (chunk_override) m.chunk_blocks = chunk_override;
   if (m.chunk_blocks > nb) m.chunk_blocks = nb;
   m.chunks = (nb + m.chunk_blocks - 1) / m.chunk_blocks;
   return m;
