@@ -224,3 +224,35 @@ def test_layer_is_deterministic_and_keeps_shape():
     x = torch.randn(3, 64, 128, device=DEV).bfloat16()
     y1, y2 = layer(x), layer(x)
     assert y1.shape == x.shape and torch.equal(y1, y2)
+
+
+@pytest.mark.parametrize("method", ["default", "fused"])
+def test_layer_forward_replays_as_a_hip_graph(method):
+    """Configuration-1-sized calls are bound by launches; a caller can record the layer's forward once
+    and replay it. Every replay is checked against the eager result for that replay's input, with eager
+    work and synchronisations in between."""
+    from spear_amd import Phalanx
+
+    torch.manual_seed(0)
+    layer = Phalanx(dim=512, length=128, method=method, dtype=torch.bfloat16).to(DEV)
+    g = torch.Generator(device="cpu").manual_seed(5)
+    inputs = [torch.randn(8, 128, 512, generator=g).bfloat16().to(DEV) for _ in range(4)]
+    static_x = inputs[0].clone()
+    with torch.no_grad():
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(2):
+                layer(static_x)  # warm-up on the capture stream (library handles, workspaces)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            static_y = layer(static_x)
+        for i, x in enumerate(inputs + inputs[:2]):
+            want = layer(x)               # eager work between the replays
+            torch.cuda.synchronize()
+            static_x.copy_(x)
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(static_y, want), f"replay {i}"
