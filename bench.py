@@ -328,6 +328,29 @@ def main() -> int:
             torch.cuda.synchronize()
             return e0.elapsed_time(e1) / n
 
+        # the same kernels in q/k/v/gate terms: fp32 log-decay gate, out = q * btp(exp(gate), k * v) + v,
+        # gradients dq, dk, dv and fp32 dgate; time-major [B, L, H, 16] tensors
+        for s_ in msets:
+            s_["gate"] = (-torch.nn.functional.softplus(s_["a"].float())).contiguous()
+            s_["dgate"] = torch.empty(B, L, H, device=dev, dtype=torch.float32)
+        QKV = 0x1
+
+        def qkv(s):
+            rc = lib.spear_phalanx_mix_forward(s["gate"].data_ptr(), s["b"].data_ptr(), s["c"].data_ptr(),
+                                               s["v"].data_ptr(), s["out"].data_ptr(), B, L, H, H, 0, QKV, sp)
+            assert rc == 0, lib.spear_btp_last_error()
+
+        def qkv_bwd(s):
+            rc = lib.spear_phalanx_mix_backward(s["gate"].data_ptr(), s["b"].data_ptr(), s["c"].data_ptr(),
+                                                s["v"].data_ptr(), s["dout"].data_ptr(), s["dgate"].data_ptr(),
+                                                s["db"].data_ptr(), s["dc"].data_ptr(), s["dv"].data_ptr(),
+                                                B, L, H, H, 0, QKV, sp)
+            assert rc == 0, lib.spear_btp_last_error()
+
+        qkv_ms, qkv_bwd_ms = kernel_ms_over(qkv, msets), kernel_ms_over(qkv_bwd, msets)
+        qkv_bytes = B * L * H * (4 + 3 * 32 + 32)             # gate, q, k, v read; out written
+        qkv_bwd_bytes = B * L * H * (4 + 4 * 32 + 4 + 3 * 32)  # gate, q, k, v, dout read; dgate, dq, dk, dv written
+
         mix_ms, unfused_ms = kernel_ms_over(mix, msets), kernel_ms_over(mix_unfused, msets)
         mix_bwd_ms, unfused_train_ms = kernel_ms_over(mix_bwd, msets), kernel_ms_over(mix_unfused_train, msets)
         mix_bytes = B * L * H * (2 + 3 * 32 + 32)          # a, b, c, v read; out written
@@ -344,6 +367,13 @@ def main() -> int:
             "fwd_plus_bwd_ms": mix_ms + mix_bwd_ms,
             "same_stage_fwd_plus_bwd_from_pytorch_ops_plus_btp_kernels_ms": unfused_train_ms,
             "train_speedup": unfused_train_ms / (mix_ms + mix_bwd_ms),
+            "qkv_gate_form": {
+                "what": "out = q * btp(exp(gate), k * v) + v on [B, L, H, 16] bf16 with an fp32 log-decay gate; dq, dk, dv, dgate",
+                "forward_ms": qkv_ms, "backward_ms": qkv_bwd_ms, "tokens_per_s": B * L / ((qkv_ms + qkv_bwd_ms) * 1e-3),
+                "algorithmic_bytes_per_unit": {"forward": 132, "backward": 232},
+                "achieved": (qkv_bytes + qkv_bwd_bytes) / ((qkv_ms + qkv_bwd_ms) * 1e-3) / 1e9,
+                "frac": (qkv_bytes + qkv_bwd_bytes) / ((qkv_ms + qkv_bwd_ms) * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+            },
         }
         del msets
 

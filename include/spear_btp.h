@@ -95,6 +95,17 @@ int spear_btp_backward_loggate(const float* gate, const void* x, const void* dy,
 int spear_phalanx_mix_forward(const void* a_logit, const void* b_logit, const void* c, const void* v, void* out,
                               int B, int L, int H, int kv_heads, int dtype, unsigned flags, void* stream);
 
+/* Flag for spear_phalanx_mix_forward / _backward / _backward_ex: the q/k/v/gate convention of the same
+ * kernels, for callers that hold the operands of linear attention rather than the layer's logits:
+ *     a_logit  is an fp32 log-decay gate [B, L, H]:       a = exp(gate), formed in fp32 (no 16-bit rounding
+ *              of the decay, so gates next to 0 stay distinct from 0)
+ *     b_logit  is k [B, L, kv_heads * 16], used as it is (no sigmoid);   c is q;   v is v
+ *     out = q * btp(exp(gate), k * v) + v      in the layout [B, L, H, 16]
+ * In the backward, da_logit is the fp32 gradient of the gate (dA * a), db_logit = dk, dc = dq, dv = dv.
+ * This is the composition written out at spear/nn/phalanx/swr.py:196-221, 311-327 with the two sigmoids
+ * left to the caller; the reference has no single function for it. */
+#define SPEAR_MIX_QKV_GATE 0x1u
+
 /* Backward of spear_phalanx_mix_forward: reads a_logit, b_logit, c, v and the upstream gradient
  * dout [B, L, H * 16]; writes da_logit [B, L, H], db_logit and dc [B, L, kv_heads * 16] (summed over
  * the heads sharing a kv head) and dv [B, L, H * 16] -- every element, no accumulation, all in

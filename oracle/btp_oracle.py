@@ -166,3 +166,43 @@ def phalanx_mix_backward(a_logit, b_logit, c, v, dout, heads: int, kv_heads: int
         dC = dC.reshape(B, kv, g, DH, L).sum(2)
         dB = dB.reshape(B, kv, g, DH, L).sum(2)
     return da, from_heads(dB), from_heads(dC), from_heads(dV)
+
+
+def qkv_gate_forward(q, k, v, gate, heads: int, kv_heads: int | None = None) -> np.ndarray:
+    """float64 statement of the same stage in q/k/v/gate terms, the composition written out at
+    spear/nn/phalanx/swr.py:196-221, 311-327 with the two sigmoids left to the caller:
+    out = q * btp(exp(gate), k * v) + v on [B, L, features] arrays, gate [B, L, heads] a log-decay;
+    head h uses q/k of kv head h // (heads // kv_heads)."""
+    kv = heads if kv_heads is None else kv_heads
+    g = heads // kv
+    q64, k64, v64, g64 = (_as_f64(t) for t in (q, k, v, gate))
+    B, L, _ = v64.shape
+    to_heads = lambda t, h: t.reshape(B, L, h, DH).transpose(0, 2, 3, 1)
+    A = np.exp(g64).transpose(0, 2, 1)
+    K = np.repeat(to_heads(k64, kv), g, axis=1)
+    Q = np.repeat(to_heads(q64, kv), g, axis=1)
+    V = to_heads(v64, heads)
+    return (forward(A, K * V, k=2) * Q + V).transpose(0, 3, 1, 2).reshape(B, L, heads * DH)
+
+
+def qkv_gate_backward(q, k, v, gate, dout, heads: int, kv_heads: int | None = None):
+    """Reverse mode of :func:`qkv_gate_forward` around the pinned BTP backward: returns
+    (dgate, dk, dq, dv); dgate = dA * a because gate = log a."""
+    kv = heads if kv_heads is None else kv_heads
+    g = heads // kv
+    q64, k64, v64, g64, d64 = (_as_f64(t) for t in (q, k, v, gate, dout))
+    B, L, _ = v64.shape
+    to_heads = lambda t, h: t.reshape(B, L, h, DH).transpose(0, 2, 3, 1)
+    from_heads = lambda t: t.transpose(0, 3, 1, 2).reshape(B, L, -1)
+    A = np.exp(g64).transpose(0, 2, 1)
+    K = np.repeat(to_heads(k64, kv), g, axis=1)
+    Q = np.repeat(to_heads(q64, kv), g, axis=1)
+    V = to_heads(v64, heads)
+    dO = to_heads(d64, heads)
+    h = forward(A, K * V, k=2)
+    dX, dA = backward(A, K * V, dO * Q, k=2)
+    dQ, dK, dV = dO * h, dX * V, dX * K + dO
+    if g > 1:
+        dQ = dQ.reshape(B, kv, g, DH, L).sum(2)
+        dK = dK.reshape(B, kv, g, DH, L).sum(2)
+    return (dA * A).transpose(0, 2, 1), from_heads(dK), from_heads(dQ), from_heads(dV)

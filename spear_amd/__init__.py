@@ -5,8 +5,8 @@ Mirrors the reference's top-level package (spear/__init__.py:6-9): ``Phalanx``, 
 """
 
 from spear_amd.nn.phalanx import Phalanx, SigmoidA
-from spear_amd.ops.btp import btp, btp_log, phalanx_mix
+from spear_amd.ops.btp import btp, btp_log, btp_qkv, phalanx_mix
 
 __version__ = "0.1.0"
 
-__all__ = ["Phalanx", "SigmoidA", "btp", "btp_log", "phalanx_mix", "__version__"]
+__all__ = ["Phalanx", "SigmoidA", "btp", "btp_log", "btp_qkv", "phalanx_mix", "__version__"]

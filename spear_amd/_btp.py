@@ -18,13 +18,14 @@ import threading
 
 import torch
 
-__all__ = ["forward", "backward", "forward_log", "backward_log", "mix_forward", "mix_backward", "jagged_prefill", "jagged_step", "library_path", "load_library", "FLAG_WRITE_CHECKPOINT", "FLAG_PATH_MFMA", "FLAG_JAGGED_LOG_A", "FLAG_JAGGED_LOG_R"]
+__all__ = ["forward", "backward", "forward_log", "backward_log", "mix_forward", "mix_backward", "jagged_prefill", "jagged_step", "library_path", "load_library", "FLAG_WRITE_CHECKPOINT", "FLAG_PATH_MFMA", "FLAG_JAGGED_LOG_A", "FLAG_JAGGED_LOG_R", "FLAG_MIX_QKV_GATE", "mix_backward_sum_rows"]
 
 _BF16, _F16, _F32 = 0, 1, 2
 FLAG_WRITE_CHECKPOINT = 0x1
 FLAG_PATH_MFMA = 0x2
 FLAG_JAGGED_LOG_A = 0x4
 FLAG_JAGGED_LOG_R = 0x8
+FLAG_MIX_QKV_GATE = 0x1
 _ABI_VERSION = 8
 _SUPPORTED_WPB = (4, 8, 16, 32)
 
@@ -292,9 +293,12 @@ def mix_forward(
     out: torch.Tensor,
     heads: int,
     kv_heads: int,
+    qkv_gate: bool = False,
 ) -> None:
     """``out <- btp(sigmoid(a_logit), sigmoid(b_logit) * v) * c + v`` with every operand in the
-    layer's ``[B, L, features]`` layout (see ``spear_phalanx_mix_forward`` in the C header)."""
+    layer's ``[B, L, features]`` layout (see ``spear_phalanx_mix_forward`` in the C header).
+    ``qkv_gate``: ``a_logit`` is an fp32 log-decay gate, ``b_logit`` is k, ``c`` is q:
+    ``out <- c * btp(exp(a_logit), b_logit * v) + v`` (``SPEAR_MIX_QKV_GATE``)."""
     _check(all(t.is_cuda for t in (a_logit, b_logit, c, v, out)), "All tensors must be CUDA.")
     _check(v.dim() == 3, "v must be [B, L, heads * 16].")
     B, L, F = v.shape
@@ -302,7 +306,11 @@ def mix_forward(
     _check(heads % 4 == 0, "heads must be a multiple of 4.")
     _check(kv_heads > 0 and heads % kv_heads == 0, "heads must be divisible by kv_heads.")
     _check(v.dtype in (torch.float16, torch.bfloat16), "tensors must be float16 or bfloat16.")
-    _check(a_logit.dtype == b_logit.dtype == c.dtype == out.dtype == v.dtype, "all tensors must share one dtype.")
+    _check(b_logit.dtype == c.dtype == out.dtype == v.dtype, "all tensors must share one dtype.")
+    if qkv_gate:
+        _check(a_logit.dtype == torch.float32, "the log-decay gate must be float32.")
+    else:
+        _check(a_logit.dtype == v.dtype, "all tensors must share one dtype.")
     _check(L % 16 == 0, "Length L must be multiple of 16")
     _check_layout("a_logit", a_logit, (B, L, heads))
     _check_layout("b_logit", b_logit, (B, L, kv_heads * 16))
@@ -314,7 +322,7 @@ def mix_forward(
     with torch.cuda.device(v.device):
         rc = lib.spear_phalanx_mix_forward(
             a_logit.data_ptr(), b_logit.data_ptr(), c.data_ptr(), v.data_ptr(), out.data_ptr(),
-            B, L, heads, kv_heads, _tag(v.dtype), 0, _stream_ptr(v.device),
+            B, L, heads, kv_heads, _tag(v.dtype), FLAG_MIX_QKV_GATE if qkv_gate else 0, _stream_ptr(v.device),
         )
     if rc != 0:
         _raise_native(lib, rc)
@@ -338,12 +346,14 @@ def mix_backward(
     heads: int,
     kv_heads: int,
     sums: tuple[torch.Tensor, torch.Tensor, torch.Tensor] | None = None,
+    qkv_gate: bool = False,
 ) -> None:
     """Gradients of :func:`mix_forward`, written in place; ``heads // kv_heads`` must be 1, 2, 4 or 8
     (see ``spear_phalanx_mix_backward`` in the C header). ``sums``: three fp32 tensors
     ``[mix_backward_sum_rows(B, L, heads), heads | kv_heads*16 | kv_heads*16]`` that receive the per-chunk
     column sums of ``da_logit``, ``db_logit`` and ``dc``. The four gradient tensors may be column blocks of one
-    wider ``[B, L, ld]`` buffer (``spear_phalanx_mix_backward_ex``)."""
+    wider ``[B, L, ld]`` buffer (``spear_phalanx_mix_backward_ex``). ``qkv_gate`` as in :func:`mix_forward`;
+    ``da_logit`` is then the fp32 gradient of the gate."""
     tensors = (a_logit, b_logit, c, v, dout, da_logit, db_logit, dc, dv)
     _check(all(t.is_cuda for t in tensors), "All tensors must be CUDA.")
     _check(v.dim() == 3, "v must be [B, L, heads * 16].")
@@ -353,7 +363,11 @@ def mix_backward(
     _check(kv_heads > 0 and heads % kv_heads == 0, "heads must be divisible by kv_heads.")
     _check(heads // kv_heads in (1, 2, 4, 8), "heads / kv_heads must be 1, 2, 4 or 8.")
     _check(v.dtype in (torch.float16, torch.bfloat16), "tensors must be float16 or bfloat16.")
-    _check(all(t.dtype == v.dtype for t in tensors), "all tensors must share one dtype.")
+    gate_like = (a_logit, da_logit)
+    _check(all(t.dtype == v.dtype for t in tensors if all(t is not g for g in gate_like)), "all tensors must share one dtype.")
+    _check(all(t.dtype == (torch.float32 if qkv_gate else v.dtype) for t in gate_like),
+           "the log-decay gate and its gradient must be float32." if qkv_gate else "all tensors must share one dtype.")
+    _check(sums is None or not qkv_gate, "column sums belong to the layer form, not to qkv_gate.")
     _check(L % 16 == 0, "Length L must be multiple of 16")
     Fkv = kv_heads * 16
     for name, t, shape in (
@@ -377,7 +391,7 @@ def mix_backward(
             a_logit.data_ptr(), b_logit.data_ptr(), c.data_ptr(), v.data_ptr(), dout.data_ptr(),
             da_logit.data_ptr(), db_logit.data_ptr(), dc.data_ptr(), dv.data_ptr(), *lds,
             *sum_ptrs, rows,
-            B, L, heads, kv_heads, _tag(v.dtype), 0, _stream_ptr(v.device),
+            B, L, heads, kv_heads, _tag(v.dtype), FLAG_MIX_QKV_GATE if qkv_gate else 0, _stream_ptr(v.device),
         )
     if rc != 0:
         _raise_native(lib, rc)

@@ -138,7 +138,7 @@ int spear_phalanx_mix_forward(const void* a_logit, const void* b_logit, const vo
     return fail(SPEAR_BTP_EINVAL, "%s: heads (%d) must be divisible by kv_heads (%d)", who, H, kv_heads);
   if (dtype != SPEAR_BTP_BF16 && dtype != SPEAR_BTP_F16)
     return fail(SPEAR_BTP_EINVAL, "%s: tensors must be float16 or bfloat16.", who);
-  if (flags != 0) return fail(SPEAR_BTP_EINVAL, "%s: unknown flag bits 0x%x", who, flags);
+  if (flags & ~SPEAR_MIX_QKV_GATE) return fail(SPEAR_BTP_EINVAL, "%s: unknown flag bits 0x%x", who, flags);
   if ((long long)B * L * H * 16ll >= (1ll << 40)) return fail(SPEAR_BTP_EINVAL, "%s: tensor too large", who);
   if ((long long)L * H * 32ll >= (1ll << 31))  // a batch row is addressed through one 32-bit buffer resource
     return fail(SPEAR_BTP_EINVAL, "%s: one batch row (L * H * 16 elements) must stay below 2 GiB", who);
@@ -146,7 +146,7 @@ int spear_phalanx_mix_forward(const void* a_logit, const void* b_logit, const vo
   if (!a_logit || !b_logit || !c || !v || !out) return fail(SPEAR_BTP_ENULL, "%s: NULL tensor pointer", who);
   if (!aligned16(a_logit) || !aligned16(b_logit) || !aligned16(c) || !aligned16(v) || !aligned16(out))
     return fail(SPEAR_BTP_EINVAL, "%s: tensor pointers must be 16-byte aligned", who);
-  spear_btp::MixArgs a{a_logit, b_logit, c, v, out, B, L, H, H / kv_heads, dtype};
+  spear_btp::MixArgs a{a_logit, b_logit, c, v, out, B, L, H, H / kv_heads, dtype, (flags & SPEAR_MIX_QKV_GATE) != 0};
   const hipError_t err = spear_btp::fused_mix_forward(a, static_cast<hipStream_t>(stream));
   if (err != hipSuccess) return fail(SPEAR_BTP_ELAUNCH, "%s: launch failed: %s", who, hipGetErrorString(err));
   return 0;
@@ -183,7 +183,8 @@ int spear_phalanx_mix_backward_ex(const void* a_logit, const void* b_logit, cons
     return fail(SPEAR_BTP_EINVAL, "%s: groups of 8 heads need heads divisible by 8 (got %d)", who, H);
   if (dtype != SPEAR_BTP_BF16 && dtype != SPEAR_BTP_F16)
     return fail(SPEAR_BTP_EINVAL, "%s: tensors must be float16 or bfloat16.", who);
-  if (flags != 0) return fail(SPEAR_BTP_EINVAL, "%s: unknown flag bits 0x%x", who, flags);
+  if (flags & ~SPEAR_MIX_QKV_GATE) return fail(SPEAR_BTP_EINVAL, "%s: unknown flag bits 0x%x", who, flags);
+  const bool qkv = (flags & SPEAR_MIX_QKV_GATE) != 0;
   if ((long long)B * L * H * 16ll >= (1ll << 40)) return fail(SPEAR_BTP_EINVAL, "%s: tensor too large", who);
   if ((long long)L * H * 32ll >= (1ll << 31))  // a batch row is addressed through one 32-bit buffer resource
     return fail(SPEAR_BTP_EINVAL, "%s: one batch row (L * H * 16 elements) must stay below 2 GiB", who);
@@ -198,10 +199,11 @@ int spear_phalanx_mix_backward_ex(const void* a_logit, const void* b_logit, cons
     if (lds[i] == 0) continue;
     if (lds[i] < widths[i] || lds[i] % 2 != 0)
       return fail(SPEAR_BTP_EINVAL, "%s: a gradient's row stride must be 0 (dense) or an even number of elements not below its width (got %d for width %d)", who, lds[i], widths[i]);
-    if ((long long)L * lds[i] * 2ll >= (1ll << 31))
+    if ((long long)L * lds[i] * (i == 0 && qkv ? 4ll : 2ll) >= (1ll << 31))
       return fail(SPEAR_BTP_EINVAL, "%s: one batch row (L * row stride) must stay below 2 GiB", who);
   }
   const bool sums = sum_da || sum_db || sum_dc;
+  if (sums && qkv) return fail(SPEAR_BTP_EINVAL, "%s: column sums are for the layer form, not SPEAR_MIX_QKV_GATE", who);
   if (sums) {
     if (!sum_da || !sum_db || !sum_dc) return fail(SPEAR_BTP_ENULL, "%s: the three sum arrays must be given together", who);
     if (!aligned16(sum_da) || !aligned16(sum_db) || !aligned16(sum_dc))
@@ -211,7 +213,7 @@ int spear_phalanx_mix_backward_ex(const void* a_logit, const void* b_logit, cons
       return fail(SPEAR_BTP_EINVAL, "%s: sum arrays must have %lld rows for this shape (got %lld)", who, want, sum_rows);
   }
   spear_btp::MixBwdArgs a{a_logit, b_logit, c, v, dout, da_logit, db_logit, dc, dv, B, L, H, groups, dtype,
-                          sum_da, sum_db, sum_dc, ld_da, ld_db, ld_dc, ld_dv};
+                          sum_da, sum_db, sum_dc, ld_da, ld_db, ld_dc, ld_dv, qkv};
   const hipError_t err = spear_btp::fused_mix_backward(a, static_cast<hipStream_t>(stream));
   if (err != hipSuccess) return fail(SPEAR_BTP_ELAUNCH, "%s: launch failed: %s", who, hipGetErrorString(err));
   return 0;

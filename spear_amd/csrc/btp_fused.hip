@@ -31,6 +31,8 @@
 #include <stdint.h>
 #include <stdlib.h>
 
+#include <type_traits>
+
 #include "btp_device.h"
 #include "btp_launch.h"
 
@@ -47,10 +49,35 @@ __device__ __forceinline__ float fast_sigmoid(float z) {
   return __builtin_amdgcn_rcpf(1.0f + __expf(-z));
 }
 
+// The kernels come in two operand conventions (kQkv):
+//   false  layer form:  a = sigmoid(a_logit), a_logit 16-bit;  input gate G = sigmoid(b_logit)
+//   true   q/k/v/gate form:  a = exp(gate), gate fp32 log-decay [B, L, H];  the b operand is k itself
+//          (G = k), the c operand is q:   out = q * btp(exp(gate), k * v) + v
+// Everything else (layout, work split, recurrences) is shared.
+struct GateWords {
+  uint32_t lo, hi;  // layer form: lo = two 16-bit logits; q/k/v form: two fp32 log-decays
+};
+
+template <class E, bool kQkv>
+__device__ __forceinline__ float2 decay_pair(GateWords w) {
+  if constexpr (kQkv) {
+    const float a0 = __expf(__uint_as_float(w.lo)), a1 = __expf(__uint_as_float(w.hi));
+    return make_float2(clamp_coeff<E>(a0), clamp_coeff<E>(a1));
+  } else {
+    return make_float2(clamp_coeff<E>(fast_sigmoid(E::lo(w.lo))), clamp_coeff<E>(fast_sigmoid(E::hi(w.lo))));
+  }
+}
+
+template <bool kQkv>
+__device__ __forceinline__ float input_gate(float b) {
+  if constexpr (kQkv) return b;
+  else return fast_sigmoid(b);
+}
+
 constexpr int kHeadsPerWave = 8;
 constexpr int kGateRow = 20;  // floats per head in the decay tile: 16 steps + 4 of padding (bank spread)
 
-template <class E, int kFwdWaves>
+template <class E, int kFwdWaves, bool kQkv>
 __global__ __launch_bounds__(64 * kFwdWaves) void phalanx_mix_fwd_kernel(
     const uint16_t* __restrict__ a_logit, const uint16_t* __restrict__ b_logit, const uint16_t* __restrict__ c_in,
     const uint16_t* __restrict__ v_in, uint16_t* __restrict__ out, int L, int H, int kv_groups, int chunk_steps,
@@ -89,14 +116,16 @@ __global__ __launch_bounds__(64 * kFwdWaves) void phalanx_mix_fwd_kernel(
       __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(b_logit + brow * L * Fkv), 0, L * kv_stride, kRsrcFlags);
   const __amdgpu_buffer_rsrc_t rc =
       __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(c_in + brow * L * Fkv), 0, L * kv_stride, kRsrcFlags);
-  const __amdgpu_buffer_rsrc_t ra =
-      __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(a_logit + brow * L * H), 0, L * H * 2, kRsrcFlags);
+  constexpr int kGateBytes = kQkv ? 4 : 2;
+  const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<char*>(reinterpret_cast<const char*>(a_logit) + brow * L * H * kGateBytes), 0, L * H * kGateBytes,
+      kRsrcFlags);
   const int v_lane = 2 * (head * kChan + d0), kv_lane = 2 * ((head / kv_groups) * kChan + d0);
   // A lane without a head stores at an offset beyond the resource, which the buffer unit drops.
   const int o_lane = real ? v_lane : 0x7ffffff0;
   // gate logits: lane (hg, t) = (lane / 16, lane % 16) converts heads ho + 2 hg, + 1 of step t
   const int gt = lane & 15, ghead = min(ho + 2 * (lane >> 4), H - 2);
-  const int a_lane = 2 * (gt * H + ghead);
+  const int a_lane = kGateBytes * (gt * H + ghead);
   float* at = a_tile[wave];
 #ifndef SPEAR_FUSED_LD_AUX
 #define SPEAR_FUSED_LD_AUX 2
@@ -132,14 +161,20 @@ __global__ __launch_bounds__(64 * kFwdWaves) void phalanx_mix_fwd_kernel(
       wd.c[r] = 0u;
     }
   };
-  auto issue_gate = [&](int t) -> uint32_t { return __builtin_amdgcn_raw_buffer_load_b32(ra, a_lane, t * H * 2, 0); };
+  auto issue_gate = [&](int t) -> GateWords {
+    GateWords w;
+    w.lo = __builtin_amdgcn_raw_buffer_load_b32(ra, a_lane, t * H * kGateBytes, 0);
+    w.hi = kQkv ? __builtin_amdgcn_raw_buffer_load_b32(ra, a_lane + 4, t * H * kGateBytes, 0) : 0u;
+    return w;
+  };
 
   float carry0 = 0.0f, carry1 = 0.0f;  // terminal local state of the previous block
 
-  auto process = [&](const Words& wd, uint32_t araw, int t0) {
+  auto process = [&](const Words& wd, GateWords araw, int t0) {
     const int o_off = (t0 >= t_begin) ? o_lane : 0x7ffffff0;  // run-in block: store nowhere
-    at[(2 * (lane >> 4)) * kGateRow + gt] = clamp_coeff<E>(fast_sigmoid(E::lo(araw)));
-    at[(2 * (lane >> 4) + 1) * kGateRow + gt] = clamp_coeff<E>(fast_sigmoid(E::hi(araw)));
+    const float2 a01 = decay_pair<E, kQkv>(araw);
+    at[(2 * (lane >> 4)) * kGateRow + gt] = a01.x;
+    at[(2 * (lane >> 4) + 1) * kGateRow + gt] = a01.y;
     wave_lds_handover();
     float a[16];
 #pragma unroll
@@ -154,8 +189,8 @@ __global__ __launch_bounds__(64 * kFwdWaves) void phalanx_mix_fwd_kernel(
     float l0 = 0.0f, l1 = 0.0f;
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
-      x0[r] = fast_sigmoid(E::lo(wd.b[r])) * E::lo(wd.v[r]);
-      x1[r] = fast_sigmoid(E::hi(wd.b[r])) * E::hi(wd.v[r]);
+      x0[r] = input_gate<kQkv>(E::lo(wd.b[r])) * E::lo(wd.v[r]);
+      x1[r] = input_gate<kQkv>(E::hi(wd.b[r])) * E::hi(wd.v[r]);
       l0 = fmaf(a[r], l0, x0[r]);
       l1 = fmaf(a[r], l1, x1[r]);
     }
@@ -176,7 +211,7 @@ __global__ __launch_bounds__(64 * kFwdWaves) void phalanx_mix_fwd_kernel(
   Words w0, w1;
   if (t_first < t_begin) issue_run_in(w0, t_first);
   else issue(w0, t_first);
-  uint32_t g0 = issue_gate(t_first), g1 = 0u;
+  GateWords g0 = issue_gate(t_first), g1 = {0u, 0u};
   for (int t0 = t_first; t0 < t_end; t0 += 2 * kTile) {
     // the scheduling barriers keep the look-ahead loads in front of the arithmetic (left alone,
     // the scheduler sinks them next to their uses to save registers, which serialises the two)
@@ -225,14 +260,14 @@ __global__ __launch_bounds__(64 * kFwdWaves) void phalanx_mix_fwd_kernel(
 // ==========================================================================================
 struct MixSet {
   uint32_t b[16], c[16], v[16], g[16];  // g: dout words
-  uint32_t araw;
+  GateWords araw;
 };
 
 // kSums: also leave, per (batch row, time chunk), the sums over the chunk's time steps of da_logit, db_logit
 // and dc in fp32 (before their rounding to 16 bits) -- the bias gradients of the projections that produced
 // a_logit, b_logit and c, up to a sum over those few rows. A lane keeps its features for the whole walk, so
 // this is five accumulators per lane and one store at the end.
-template <class E, bool kSums>
+template <class E, bool kSums, bool kQkv>
 __global__ __launch_bounds__(64 * kWaves) void phalanx_mix_bwd_kernel(
     const uint16_t* __restrict__ a_logit, const uint16_t* __restrict__ b_logit, const uint16_t* __restrict__ c_in,
     const uint16_t* __restrict__ v_in, const uint16_t* __restrict__ dout, uint16_t* __restrict__ da_logit,
@@ -259,19 +294,20 @@ __global__ __launch_bounds__(64 * kWaves) void phalanx_mix_bwd_kernel(
   const int F = H * kChan, Fkv = (H / kv_groups) * kChan;
   const int stride = 2 * F, kv_stride = 2 * Fkv;  // bytes per time step of the [B, L, F] / [B, L, Fkv] tensors
   constexpr int kRsrcFlags = 0x00020000;          // raw 32-bit buffer, gfx9 encoding
+  constexpr int kGateBytes = kQkv ? 4 : 2;        // element size of the a operand and of its gradient
   const long big = brow * L * F, kvbig = brow * L * Fkv, small = brow * L * H;
   auto rsrc = [&](const uint16_t* p, long off, int bytes) {
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(p + off), 0, bytes, kRsrcFlags);
   };
   const __amdgpu_buffer_rsrc_t rb = rsrc(b_logit, kvbig, L * kv_stride), rc = rsrc(c_in, kvbig, L * kv_stride),
                                rv = rsrc(v_in, big, L * stride), rg = rsrc(dout, big, L * stride),
-                               ra = rsrc(a_logit, small, L * H * 2),
+                               ra = rsrc(a_logit, small * (kGateBytes / 2), L * H * kGateBytes),
                                // the four gradients may sit side by side in one wider buffer: each has its
                                // own elements-per-time-step (ld_*), equal to its width when it is dense
                                rdb = rsrc(db_logit, brow * L * ld_db, L * ld_db * 2),
                                rdc = rsrc(dc, brow * L * ld_dc, L * ld_dc * 2),
                                rdv = rsrc(dv, brow * L * ld_dv, L * ld_dv * 2),
-                               rda = rsrc(da_logit, brow * L * ld_da, L * ld_da * 2);
+                               rda = rsrc(da_logit, brow * L * ld_da * (kGateBytes / 2), L * ld_da * kGateBytes);
   const int f_lane = 2 * (head * kChan + d0);
   const int kv_lane = 2 * ((head / kv_groups) * kChan + d0);
   const int o_lane = real ? f_lane : 0x7ffffff0;  // lanes without a head store nowhere
@@ -279,15 +315,16 @@ __global__ __launch_bounds__(64 * kWaves) void phalanx_mix_bwd_kernel(
   // gradients of b and c are summed over the group's lanes and stored by its first head only.
   const int okv_lane = (real && (head % kv_groups) == 0) ? kv_lane : 0x7ffffff0;
   const int gt = lane & 15, ghead = min(ho + 2 * (lane >> 4), H - 2);
-  const int a_lane = 2 * (gt * H + ghead);
+  const int a_lane = kGateBytes * (gt * H + ghead);
   // da_logit: lane k of a head (k = lane % 8) ends up with steps 2k and 2k+1 of that head
-  const int da_lane = real ? 2 * ((2 * (lane & 7)) * ld_da + head) : 0x7ffffff0;
+  const int da_lane = real ? kGateBytes * ((2 * (lane & 7)) * ld_da + head) : 0x7ffffff0;
   constexpr int kNt = 2;
 
   auto issue = [&](MixSet& m, int t) {
     // b, v and the gate logits first: the look-ahead pass needs them before pass R of the next
     // iteration needs dout and c
-    m.araw = __builtin_amdgcn_raw_buffer_load_b32(ra, a_lane, t * H * 2, 0);
+    m.araw.lo = __builtin_amdgcn_raw_buffer_load_b32(ra, a_lane, t * H * kGateBytes, 0);
+    m.araw.hi = kQkv ? __builtin_amdgcn_raw_buffer_load_b32(ra, a_lane + 4, t * H * kGateBytes, 0) : 0u;
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
       m.b[r] = __builtin_amdgcn_raw_buffer_load_b32(rb, kv_lane, (t + r) * kv_stride, kNt);
@@ -299,9 +336,10 @@ __global__ __launch_bounds__(64 * kWaves) void phalanx_mix_bwd_kernel(
       m.c[r] = __builtin_amdgcn_raw_buffer_load_b32(rc, kv_lane, (t + r) * kv_stride, kNt);
     }
   };
-  auto write_gate_tile = [&](float* tile, uint32_t araw) {
-    tile[(2 * (lane >> 4)) * kGateRow + gt] = clamp_coeff<E>(fast_sigmoid(E::lo(araw)));
-    tile[(2 * (lane >> 4) + 1) * kGateRow + gt] = clamp_coeff<E>(fast_sigmoid(E::hi(araw)));
+  auto write_gate_tile = [&](float* tile, GateWords araw) {
+    const float2 a01 = decay_pair<E, kQkv>(araw);
+    tile[(2 * (lane >> 4)) * kGateRow + gt] = a01.x;
+    tile[(2 * (lane >> 4) + 1) * kGateRow + gt] = a01.y;
   };
   auto read_gates = [&](const float* tile, float (&a)[16]) {
 #pragma unroll
@@ -360,8 +398,8 @@ __global__ __launch_bounds__(64 * kWaves) void phalanx_mix_bwd_kernel(
       read_gates(tn, ap);
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        cin0 = fmaf(ap[r], cin0, fast_sigmoid(E::lo(nxt.b[r])) * E::lo(nxt.v[r]));
-        cin1 = fmaf(ap[r], cin1, fast_sigmoid(E::hi(nxt.b[r])) * E::hi(nxt.v[r]));
+        cin0 = fmaf(ap[r], cin0, input_gate<kQkv>(E::lo(nxt.b[r])) * E::lo(nxt.v[r]));
+        cin1 = fmaf(ap[r], cin1, input_gate<kQkv>(E::hi(nxt.b[r])) * E::hi(nxt.v[r]));
       }
     } else {
       wave_lds_handover();
@@ -377,7 +415,7 @@ __global__ __launch_bounds__(64 * kWaves) void phalanx_mix_bwd_kernel(
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
       const float4 pk = my_park[r * 64];  // R0, R1, dX0, dX1
-      const float G0 = fast_sigmoid(E::lo(cur.b[r])), G1 = fast_sigmoid(E::hi(cur.b[r]));
+      const float G0 = input_gate<kQkv>(E::lo(cur.b[r])), G1 = input_gate<kQkv>(E::hi(cur.b[r]));
       const float v0 = E::lo(cur.v[r]), v1 = E::hi(cur.v[r]);
       const float go0 = E::lo(cur.g[r]), go1 = E::hi(cur.g[r]);
       my_e[r * 256] = fmaf(pk.z, vp0, pk.x * z0) + fmaf(pk.w, vp1, pk.y * z1);
@@ -385,7 +423,11 @@ __global__ __launch_bounds__(64 * kWaves) void phalanx_mix_bwd_kernel(
       vp0 = fmaf(a[r], vp0, G0 * v0);
       vp1 = fmaf(a[r], vp1, G1 * v1);
       float dc0 = go0 * (vp0 + az0), dc1 = go1 * (vp1 + az1);
-      float db0 = pk.z * v0 * G0 * (1.0f - G0), db1 = pk.w * v1 * G1 * (1.0f - G1);
+      float db0 = pk.z * v0, db1 = pk.w * v1;  // dX * v: the gradient of k in the q/k/v form
+      if constexpr (!kQkv) {
+        db0 *= G0 * (1.0f - G0);
+        db1 *= G1 * (1.0f - G1);
+      }
       if (kv_groups > 1) {  // wave-uniform: sum over the heads that share this kv head
         dc0 += row_xor<8>(dc0); dc1 += row_xor<8>(dc1); db0 += row_xor<8>(db0); db1 += row_xor<8>(db1);
         if (kv_groups > 2) {
@@ -440,12 +482,18 @@ __global__ __launch_bounds__(64 * kWaves) void phalanx_mix_bwd_kernel(
       s1 = k1 + row_xor<1>(n1);
     }
     const float2 aa = *reinterpret_cast<const float2*>(tc + head_local * kGateRow + 2 * kk);
-    const float da0 = s0 * aa.x * (1.0f - aa.x), da1 = s1 * aa.y * (1.0f - aa.y);
+    // d/d a_logit = dA a (1 - a);  d/d gate = dA a  (gate = log a)
+    const float da0 = kQkv ? s0 * aa.x : s0 * aa.x * (1.0f - aa.x), da1 = kQkv ? s1 * aa.y : s1 * aa.y * (1.0f - aa.y);
     if constexpr (kSums) acc_a += da0 + da1;
     const int da_off = (t0 >= t_begin) ? da_lane : 0x7ffffff0;
-    const uint32_t dap = E::pack2(da0, da1);
-    __builtin_amdgcn_raw_buffer_store_b16((unsigned short)(dap & 0xffffu), rda, da_off, t0 * ld_da * 2, 0);
-    __builtin_amdgcn_raw_buffer_store_b16((unsigned short)(dap >> 16), rda, da_off + 2 * ld_da, t0 * ld_da * 2, 0);
+    if constexpr (kQkv) {
+      __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(da0), rda, da_off, t0 * ld_da * 4, 0);
+      __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(da1), rda, da_off + 4 * ld_da, t0 * ld_da * 4, 0);
+    } else {
+      const uint32_t dap = E::pack2(da0, da1);
+      __builtin_amdgcn_raw_buffer_store_b16((unsigned short)(dap & 0xffffu), rda, da_off, t0 * ld_da * 2, 0);
+      __builtin_amdgcn_raw_buffer_store_b16((unsigned short)(dap >> 16), rda, da_off + 2 * ld_da, t0 * ld_da * 2, 0);
+    }
     wave_lds_handover();  // tile `tc` and the parking slots are free for the iteration after next
   };
 
@@ -525,11 +573,11 @@ MixPlan plan_mix(long B, int H, int L) {
   return m;
 }
 
-template <class E, int kW>
+template <class E, int kW, bool kQkv>
 void launch_mix_fwd(const MixArgs& p, const MixPlan& m, hipStream_t s) {
   const long total = (long)p.B * m.chunks * ((p.H + 7) / 8);
   const unsigned blocks = (unsigned)((total + kW - 1) / kW);
-  hipLaunchKernelGGL((phalanx_mix_fwd_kernel<E, kW>), dim3(blocks), dim3(64 * kW), 0, s,
+  hipLaunchKernelGGL((phalanx_mix_fwd_kernel<E, kW, kQkv>), dim3(blocks), dim3(64 * kW), 0, s,
                      static_cast<const uint16_t*>(p.a_logit), static_cast<const uint16_t*>(p.b_logit),
                      static_cast<const uint16_t*>(p.c), static_cast<const uint16_t*>(p.v), static_cast<uint16_t*>(p.out),
                      p.L, p.H, p.kv_groups, m.chunk_blocks * kTile, m.chunks, total);
@@ -539,12 +587,17 @@ void launch_mix_fwd(const MixArgs& p, const MixPlan& m, hipStream_t s) {
 
 hipError_t fused_mix_forward(const MixArgs& p, hipStream_t s) {
   const MixPlan m = plan_mix(p.B, p.H, p.L);
+  auto by_waves = [&](auto e, auto q) {
+    using E = decltype(e);
+    if (m.wg_waves == 8) launch_mix_fwd<E, 8, decltype(q)::value>(p, m, s);
+    else launch_mix_fwd<E, 4, decltype(q)::value>(p, m, s);
+  };
   if (p.dtype == kBf16) {
-    if (m.wg_waves == 8) launch_mix_fwd<Bf16, 8>(p, m, s);
-    else launch_mix_fwd<Bf16, 4>(p, m, s);
+    if (p.qkv) by_waves(Bf16{}, std::true_type{});
+    else by_waves(Bf16{}, std::false_type{});
   } else {
-    if (m.wg_waves == 8) launch_mix_fwd<Fp16, 8>(p, m, s);
-    else launch_mix_fwd<Fp16, 4>(p, m, s);
+    if (p.qkv) by_waves(Fp16{}, std::true_type{});
+    else by_waves(Fp16{}, std::false_type{});
   }
   return hipGetLastError();
 }
@@ -569,14 +622,14 @@ MixPlan plan_mix_bwd(long B, int H, int L) {
   return m;
 }
 
-template <class E, bool kSums>
+template <class E, bool kSums, bool kQkv>
 void launch_mix_bwd(const MixBwdArgs& p, const MixPlan& m, hipStream_t s) {
   const long total = (long)p.B * m.chunks * ((p.H + 7) / 8);
   const unsigned blocks = (unsigned)((total + kWaves - 1) / kWaves);
   auto u = [](const void* q) { return static_cast<const uint16_t*>(q); };
   auto w = [](void* q) { return static_cast<uint16_t*>(q); };
   const int Fkv = (p.H / p.kv_groups) * kChan;
-  hipLaunchKernelGGL((phalanx_mix_bwd_kernel<E, kSums>), dim3(blocks), dim3(64 * kWaves), 0, s, u(p.a_logit),
+  hipLaunchKernelGGL((phalanx_mix_bwd_kernel<E, kSums, kQkv>), dim3(blocks), dim3(64 * kWaves), 0, s, u(p.a_logit),
                      u(p.b_logit), u(p.c), u(p.v), u(p.dout), w(p.da_logit), w(p.db_logit), w(p.dc), w(p.dv), p.sum_da,
                      p.sum_db, p.sum_dc, p.ld_da ? p.ld_da : p.H, p.ld_db ? p.ld_db : Fkv, p.ld_dc ? p.ld_dc : Fkv,
                      p.ld_dv ? p.ld_dv : p.H * kChan, p.L, p.H, p.kv_groups, m.chunk_blocks * kTile, m.chunks, total);
@@ -592,12 +645,15 @@ long fused_mix_backward_sum_rows(long B, int H, int L) {
 hipError_t fused_mix_backward(const MixBwdArgs& p, hipStream_t s) {
   const MixPlan m = plan_mix_bwd(p.B, p.H, p.L);
   const bool sums = p.sum_da != nullptr;
+  if (sums && p.qkv) return hipErrorInvalidValue;  // the caller has checked: sums belong to the layer form
   if (p.dtype == kBf16) {
-    if (sums) launch_mix_bwd<Bf16, true>(p, m, s);
-    else launch_mix_bwd<Bf16, false>(p, m, s);
+    if (p.qkv) launch_mix_bwd<Bf16, false, true>(p, m, s);
+    else if (sums) launch_mix_bwd<Bf16, true, false>(p, m, s);
+    else launch_mix_bwd<Bf16, false, false>(p, m, s);
   } else {
-    if (sums) launch_mix_bwd<Fp16, true>(p, m, s);
-    else launch_mix_bwd<Fp16, false>(p, m, s);
+    if (p.qkv) launch_mix_bwd<Fp16, false, true>(p, m, s);
+    else if (sums) launch_mix_bwd<Fp16, true, false>(p, m, s);
+    else launch_mix_bwd<Fp16, false, false>(p, m, s);
   }
   return hipGetLastError();
 }

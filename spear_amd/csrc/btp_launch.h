@@ -47,6 +47,8 @@ struct MixArgs {
   void* out;            // [B, L, H * 16]
   int B, L, H, kv_groups;
   int dtype;
+  // q/k/v/gate form: a_logit is an fp32 log-decay gate (a = exp(gate)), b_logit is k (used as it is), c is q
+  bool qkv = false;
 };
 hipError_t fused_mix_forward(const MixArgs& p, hipStream_t s);
 
@@ -60,6 +62,7 @@ struct MixBwdArgs {
   float *sum_da = nullptr, *sum_db = nullptr, *sum_dc = nullptr;
   // elements per time step of each gradient tensor; 0 = dense (its own width)
   int ld_da = 0, ld_db = 0, ld_dc = 0, ld_dv = 0;
+  bool qkv = false;  // as in MixArgs; da_logit is then the fp32 gradient of the gate
 };
 hipError_t fused_mix_backward(const MixBwdArgs& p, hipStream_t s);
 long fused_mix_backward_sum_rows(long B, int H, int L);

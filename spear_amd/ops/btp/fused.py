@@ -23,7 +23,7 @@ from spear_amd import _btp
 
 from .interface import lib, register_traceable_op
 
-__all__ = ["phalanx_mix"]
+__all__ = ["phalanx_mix", "btp_qkv"]
 
 
 def _mix_forward_impl(
@@ -57,6 +57,38 @@ def _mix_backward_fake(
 register_traceable_op(lib, "mix_forward", _mix_forward_impl, _mix_forward_fake, mutates_args=["out"])
 register_traceable_op(
     lib, "mix_backward", _mix_backward_impl, _mix_backward_fake, mutates_args=["da", "db", "dc", "dv"]
+)
+
+
+def _qkv_forward_impl(
+    gate: torch.Tensor, k: torch.Tensor, q: torch.Tensor, v: torch.Tensor, out: torch.Tensor, heads: int, kv_heads: int
+) -> None:
+    _btp.mix_forward(gate, k, q, v, out, heads, kv_heads, qkv_gate=True)
+
+
+def _qkv_forward_fake(
+    gate: torch.Tensor, k: torch.Tensor, q: torch.Tensor, v: torch.Tensor, out: torch.Tensor, heads: int, kv_heads: int
+) -> None:
+    return None
+
+
+def _qkv_backward_impl(
+    gate: torch.Tensor, k: torch.Tensor, q: torch.Tensor, v: torch.Tensor, dout: torch.Tensor,
+    dgate: torch.Tensor, dk: torch.Tensor, dq: torch.Tensor, dv: torch.Tensor, heads: int, kv_heads: int,
+) -> None:
+    _btp.mix_backward(gate, k, q, v, dout, dgate, dk, dq, dv, heads, kv_heads, qkv_gate=True)
+
+
+def _qkv_backward_fake(
+    gate: torch.Tensor, k: torch.Tensor, q: torch.Tensor, v: torch.Tensor, dout: torch.Tensor,
+    dgate: torch.Tensor, dk: torch.Tensor, dq: torch.Tensor, dv: torch.Tensor, heads: int, kv_heads: int,
+) -> None:
+    return None
+
+
+register_traceable_op(lib, "qkv_forward", _qkv_forward_impl, _qkv_forward_fake, mutates_args=["out"])
+register_traceable_op(
+    lib, "qkv_backward", _qkv_backward_impl, _qkv_backward_fake, mutates_args=["dgate", "dk", "dq", "dv"]
 )
 
 
@@ -153,3 +185,51 @@ def phalanx_mix(
     """
     kv = heads if kv_heads is None else kv_heads
     return _PhalanxMix.apply(a_logits.contiguous(), b_logits.contiguous(), c.contiguous(), v.contiguous(), heads, kv)
+
+
+class _BtpQkv(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, q, k, v, gate, heads: int, kv_heads: int):
+        out = torch.empty_like(v)
+        torch.ops.spear_btp.qkv_forward(gate, k, q, v, out, heads, kv_heads)
+        ctx.save_for_backward(q, k, v, gate)
+        ctx.heads, ctx.kv_heads = heads, kv_heads
+        return out
+
+    @staticmethod
+    def backward(ctx, dout):
+        q, k, v, gate = ctx.saved_tensors
+        dq, dk, dv, dgate = (torch.empty_like(t) for t in (q, k, v, gate))
+        torch.ops.spear_btp.qkv_backward(gate, k, q, v, dout.contiguous(), dgate, dk, dq, dv, ctx.heads, ctx.kv_heads)
+        return dq, dk, dv, dgate, None, None
+
+
+def btp_qkv(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, gate: torch.Tensor) -> torch.Tensor:
+    """The operator in linear-attention terms, time-major:
+
+        out = q * btp(exp(gate), k * v) + v
+
+    one fused kernel forward and one backward (``dq, dk, dv, dgate``), no transposes.
+
+    Args:
+        q, k: ``[B, L, kv_heads, 16]`` bf16 / fp16 (``kv_heads`` divides ``heads``; ``heads // kv_heads`` in
+            1, 2, 4, 8; head ``h`` uses q/k of kv head ``h // (heads // kv_heads)``).
+        v: ``[B, L, heads, 16]``, same dtype; ``heads`` a multiple of 4, ``L`` a multiple of 16.
+        gate: ``[B, L, heads]`` float32 log-decay (``<= 0``, e.g. ``-softplus(logit)``); the decay
+            ``exp(gate)`` is formed in fp32 inside the kernel, and the gradient is w.r.t. ``gate``.
+
+    Returns ``[B, L, heads, 16]`` in ``v``'s dtype. This is what the Phalanx layer computes
+    (spear/nn/phalanx/swr.py:196-221, 311-327) with ``k = sigmoid(proj_b(x))``, ``q = proj_c(x)``,
+    ``gate = log sigmoid(proj_a(x))``.
+    """
+    if v.dim() != 4 or v.shape[-1] != 16 or q.dim() != 4 or q.shape != k.shape or q.shape[-1] != 16:
+        raise RuntimeError("q, k must be [B, L, kv_heads, 16] and v [B, L, heads, 16].")
+    B, L, H, _ = v.shape
+    Hkv = q.shape[2]
+    if Hkv == 0 or H % Hkv != 0 or H // Hkv not in (1, 2, 4, 8) or (H // Hkv == 8 and H % 8 != 0):
+        raise RuntimeError("heads / kv_heads must be 1, 2, 4 or 8.")
+    out = _BtpQkv.apply(
+        q.reshape(B, L, Hkv * 16).contiguous(), k.reshape(B, L, Hkv * 16).contiguous(),
+        v.reshape(B, L, H * 16).contiguous(), gate.contiguous(), H, Hkv,
+    )
+    return out.view(B, L, H, 16)

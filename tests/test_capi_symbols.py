@@ -100,6 +100,11 @@ def test_host_side_validation_needs_no_gpu():
     # fused layer kernels: a batch row must fit one 32-bit buffer resource
     assert lib.spear_phalanx_mix_forward(p, p, p, p, p, 1, 1 << 20, 128, 128, 0, 0, None) == -1
     assert b"below 2 GiB" in lib.spear_btp_last_error()
+    # SPEAR_MIX_QKV_GATE (0x1) is the only flag of the fused entry points
+    assert lib.spear_phalanx_mix_forward(p, p, p, p, p, 1, 32, 4, 4, 0, 0x2, None) == -1
+    assert b"unknown flag" in lib.spear_btp_last_error()
+    assert lib.spear_phalanx_mix_backward(p, p, p, p, p, p, p, p, p, 1, 32, 4, 4, 0, 0x4, None) == -1
+    assert _btp.FLAG_MIX_QKV_GATE == int(re.search(r"#define SPEAR_MIX_QKV_GATE (0x[0-9a-f]+)u", open(HEADER).read()).group(1), 16)
     # backward with column sums: the three arrays come together and with the row count the library states
     rows = lib.spear_phalanx_mix_backward_sum_rows(2, 64, 8)
     assert rows >= 2 and rows % 2 == 0
@@ -111,6 +116,8 @@ def test_host_side_validation_needs_no_gpu():
     assert sums(p, p, p, rows + 1) == -1
     assert b"rows for this shape" in lib.spear_btp_last_error()
     assert sums(p + 4, p, p, rows) == -1
+    assert lib.spear_phalanx_mix_backward_ex(p, p, p, p, p, p, p, p, p, 0, 0, 0, 0, p, p, p, rows, 2, 64, 8, 8, 0, 0x1, None) == -1
+    assert b"layer form" in lib.spear_btp_last_error()
     # output row strides: 0 or an even number of elements not below the tensor's width
     assert sums(None, None, None, 0, (4, 0, 0, 0)) == -1
     assert b"row stride" in lib.spear_btp_last_error()

@@ -279,6 +279,33 @@ def test_oracle_fused_backward_matches_torch_autograd():
         np.testing.assert_allclose(gg, t.grad.numpy(), rtol=1e-10, atol=1e-12, err_msg=f"d{name}")
 
 
+def test_oracle_qkv_gate_form_matches_torch_composition_and_autograd():
+    """out = q * btp(exp(gate), k * v) + v and its gradients (dgate w.r.t. the LOG decay), against the
+    same expression in torch ops on the float64 reference recurrence, differentiated by autograd."""
+    import numpy as np
+
+    from oracle import btp_oracle as orc
+    from spear_amd.ops.btp.reference import block_two_pass_ref
+
+    B, L, H, Hkv = 2, 48, 8, 4
+    g = torch.Generator().manual_seed(10)
+    q, k = (torch.randn(B, L, Hkv * 16, generator=g, dtype=torch.float64, requires_grad=True) for _ in range(2))
+    v = torch.randn(B, L, H * 16, generator=g, dtype=torch.float64, requires_grad=True)
+    gate = (-torch.nn.functional.softplus(torch.randn(B, L, H, generator=g, dtype=torch.float64))).requires_grad_(True)
+    dout = torch.randn(B, L, H * 16, generator=g, dtype=torch.float64)
+    heads = lambda t, h: t.view(B, L, h, 16).permute(0, 2, 3, 1)
+    A = torch.exp(gate).transpose(1, 2).contiguous()
+    K = heads(k, Hkv).repeat_interleave(H // Hkv, 1)
+    Q = heads(q, Hkv).repeat_interleave(H // Hkv, 1)
+    out = (block_two_pass_ref(A, (K * heads(v, H)).contiguous()) * Q + heads(v, H)).permute(0, 3, 1, 2).reshape(B, L, H * 16)
+    out.backward(dout)
+    args = [t.detach().numpy() for t in (q, k, v, gate)]
+    np.testing.assert_allclose(orc.qkv_gate_forward(*args, H, Hkv), out.detach().numpy(), rtol=1e-11, atol=1e-12)
+    dgate, dk, dq, dv = orc.qkv_gate_backward(*args, dout.numpy(), H, Hkv)
+    for name, got, t in (("dgate", dgate, gate), ("dk", dk, k), ("dq", dq, q), ("dv", dv, v)):
+        np.testing.assert_allclose(got, t.grad.numpy(), rtol=1e-10, atol=1e-12, err_msg=name)
+
+
 def test_streaming_module_surface_and_state_dataclass():
     from spear_amd.nn.phalanx import inference as inf
 
