@@ -11,6 +11,8 @@ import os
 import shutil
 import subprocess
 import sys
+import tempfile
+from concurrent.futures import ThreadPoolExecutor
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 PKG = os.path.dirname(HERE)
@@ -25,7 +27,6 @@ HIPCC_FLAGS = [
     "-O3",
     "-std=c++17",
     "-fPIC",
-    "-shared",
     "-ffp-contract=off",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wall",
@@ -44,9 +45,7 @@ def lib_path() -> str:
     return os.path.join(PKG, LIB_NAME)
 
 
-def build(verbose: bool = False, extra_flags: list[str] | None = None, out: str | None = None) -> str:
-    out = out or lib_path()
-    cmd = [hipcc_path(), *HIPCC_FLAGS, *(extra_flags or []), "-o", out, *[os.path.join(HERE, s) for s in SOURCES]]
+def _run(cmd: list[str], verbose: bool) -> None:
     if verbose:
         print(" ".join(cmd), flush=True)
     proc = subprocess.run(cmd, cwd=HERE, capture_output=True, text=True)
@@ -56,6 +55,19 @@ def build(verbose: bool = False, extra_flags: list[str] | None = None, out: str 
         raise RuntimeError(f"hipcc failed ({proc.returncode}):\n{proc.stdout}\n{err}")
     if verbose and err.strip():
         print(err, file=sys.stderr)
+
+
+def build(verbose: bool = False, extra_flags: list[str] | None = None, out: str | None = None) -> str:
+    """One object per source, compiled side by side (the files are independent and the kernels'
+    template instances make each take tens of seconds), then one link."""
+    out = out or lib_path()
+    hipcc, flags = hipcc_path(), [*HIPCC_FLAGS, *(extra_flags or [])]
+    with tempfile.TemporaryDirectory(prefix="spear_btp_build_") as tmp:
+        objects = [os.path.join(tmp, os.path.splitext(s)[0] + ".o") for s in SOURCES]
+        jobs = [[hipcc, *flags, "-c", os.path.join(HERE, s), "-o", o] for s, o in zip(SOURCES, objects)]
+        with ThreadPoolExecutor(max_workers=min(len(jobs), os.cpu_count() or 1, 8)) as pool:
+            list(pool.map(lambda cmd: _run(cmd, verbose), jobs))
+        _run([hipcc, *flags, "-shared", "-o", out, *objects], verbose)
     return out
 
 

@@ -303,3 +303,44 @@ def test_measurement_aids_move_the_bytes_they_are_timed_for(slabs):
     assert lib.spear_btp_copy(a.data_ptr(), out.data_ptr(), ctypes.c_ulonglong(n), sp) == 0
     torch.cuda.synchronize()
     assert torch.equal(out[:n], a) and bool((out[n:] == 0xA5).all())
+
+
+def test_concurrent_callers_on_their_own_streams():
+    """The library keeps no state between calls (the error string is per thread): two host threads
+    launching on two streams at once get the results they get alone."""
+    import threading
+
+    from spear_amd import _btp
+
+    cases = []
+    for seed in (501, 502):
+        coeff, x, dy = make_inputs(8, 8, 1024, seed=seed)
+        cases.append([t.to(DEV) for t in (coeff, x, dy)])
+    alone = [(run_forward(c.cpu(), x.cpu()), run_backward(c.cpu(), x.cpu(), g.cpu())) for c, x, g in cases]
+    results, errors = [None, None], []
+
+    def worker(i):
+        try:
+            c, x, g = cases[i]
+            stream = torch.cuda.Stream()
+            with torch.cuda.stream(stream):
+                for _ in range(25):
+                    y = torch.empty_like(x)
+                    dx = torch.empty_like(x)
+                    dA = torch.empty(c.shape, device=DEV, dtype=torch.float32)
+                    ck = torch.empty(8, 8, 64, 16, device=DEV, dtype=torch.float32)
+                    _btp.forward(c, x, y, ck, 2, 32, flags=0)
+                    _btp.backward(c, x, g, ck, dx, dA, 2, 32)
+                stream.synchronize()
+            results[i] = (y.cpu(), dx.cpu(), dA.cpu())
+        except Exception as e:  # surfaced below: an exception in a thread would otherwise pass silently
+            errors.append(e)
+
+    threads = [threading.Thread(target=worker, args=(i,)) for i in range(2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+    for (y, dx, dA), (y0, (dx0, dA0)) in zip(results, alone):
+        assert torch.equal(y, y0) and torch.equal(dx, dx0) and torch.equal(dA, dA0)
