@@ -406,8 +406,8 @@ def main() -> int:
                 xl.grad = None
                 mod(xl).backward(gout)
 
-            def layer_ms(fn, n=10):
-                for _ in range(2):
+            def layer_ms(fn, n=20):
+                for _ in range(4):
                     fn()
                 torch.cuda.synchronize()
                 e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
