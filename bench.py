@@ -267,8 +267,15 @@ def main() -> int:
 
     # fused layer-layout forward (gates + recurrence + y*C+V on [B, L, features] tensors) against the
     # same stage built from PyTorch ops around the stand-alone kernel
-    fused = None
-    if H % 4 == 0 and not args.no_fused:
+    def guarded(leg):
+        """Run an auxiliary leg; if it raises, the headline measurement above still gets reported."""
+        try:
+            return leg()
+        except Exception as exc:  # noqa: BLE001 - reported in the JSON line instead of propagating
+            torch.cuda.synchronize()
+            return {"error": f"{type(exc).__name__}: {exc}"}
+
+    def fused_leg():
         from spear_amd.ops.btp import btp as btp_op
 
         F = H * 16
@@ -376,11 +383,13 @@ def main() -> int:
             },
         }
         del msets
+        return fused
+
+    fused = guarded(fused_leg) if (H % 4 == 0 and not args.no_fused) else None
 
     # the Phalanx layer end to end (five projections + mixing stage) on x[B, L, H*16], forward and
     # forward+backward, for the reference's PyTorch-ops method, its kernel method and the fused method
-    layer = None
-    if H % 4 == 0 and not args.no_layer:
+    def layer_leg():
         from spear_amd import Phalanx
 
         dim = H * 16
@@ -422,11 +431,13 @@ def main() -> int:
             del mod
         del xl, gout
         torch.cuda.empty_cache()
+        return layer
+
+    layer = guarded(layer_leg) if (H % 4 == 0 and not args.no_layer) else None
 
     # streaming form: prompt prefill (recurrence + y*C+V + state hand-over) on the same tensors, and
     # the one-token decode step on [B, H, 16] operands with fp32 state
-    streaming = None
-    if not args.no_streaming:
+    def streaming_leg():
         st_h = torch.zeros(B, H, 16, device=dev)
         st_c = torch.zeros(B, H, 16, device=dev)
         st_r = torch.ones(B, H, device=dev)
@@ -531,6 +542,9 @@ def main() -> int:
                             "same_step_from_pytorch_ops_ms": step_torch_ms, "speedup": step_torch_ms / step_ms,
                             "avg_launch_ms_in_hip_graph": step_graph_ms},
         }
+        return streaming
+
+    streaming = None if args.no_streaming else guarded(streaming_leg)
 
     units = B * H * L
     tokens = B * L
