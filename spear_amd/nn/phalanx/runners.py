@@ -9,6 +9,7 @@ from spear_amd.testing.numerics import (
     DEFAULT_INPUT_DISTRIBUTION,
     InputDistributionConfig,
     compute_error_metrics,
+    extract_layer_gradients,
     make_generator,
     manual_seed,
     maybe_synchronize,
@@ -26,19 +27,16 @@ __all__ = [
 ]
 
 
+def _pick_device(device) -> torch.device:
+    return torch.device(device or ("cuda" if torch.cuda.is_available() else "cpu"))
+
+
 def sample_layer_inputs(
-    B: int,
-    L: int,
-    dim: int,
-    *,
-    dtype: torch.dtype = torch.bfloat16,
-    device: torch.device | None = None,
-    seed: int | None = None,
-    stress_scale: float = 1.0,
-    distribution: InputDistributionConfig | None = None,
+    B: int, L: int, dim: int, *, dtype: torch.dtype = torch.bfloat16, device: torch.device | None = None,
+    seed: int | None = None, stress_scale: float = 1.0, distribution: InputDistributionConfig | None = None,
 ) -> torch.Tensor:
     """``[B, L, dim]`` activations, drawn on a CPU generator and moved to ``device``."""
-    device = torch.device(device or ("cuda" if torch.cuda.is_available() else "cpu"))
+    device = _pick_device(device)
     if seed is not None:
         manual_seed(seed, device)
     cpu = torch.device("cpu")
@@ -51,35 +49,23 @@ def sample_layer_inputs(
 
 
 def create_phalanx_layers(
-    dim: int,
-    length: int,
-    *,
-    methods: tuple[str, ...] = ("default", "pytorch", "pytorch_linspace"),
-    dtype: torch.dtype = torch.bfloat16,
-    k: int = 2,
-    wpb: int = 32,
-    output_dtype: torch.dtype | None = None,
-    block_size: int = 16,
-    kv_heads: int | None = None,
-    device: torch.device | None = None,
-    seed: int | None = None,
+    dim: int, length: int, *, methods: tuple[str, ...] = ("default", "pytorch", "pytorch_linspace"),
+    dtype: torch.dtype = torch.bfloat16, k: int = 2, wpb: int = 32, output_dtype: torch.dtype | None = None,
+    block_size: int = 16, kv_heads: int | None = None, device: torch.device | None = None, seed: int | None = None,
 ) -> dict[str, Phalanx]:
     """One layer per method; every layer after the first receives the first one's weights."""
-    device = torch.device(device or ("cuda" if torch.cuda.is_available() else "cpu"))
+    device = _pick_device(device)
     if seed is not None:
         manual_seed(seed, device)
-    layers: dict[str, Phalanx] = {}
-    first: Phalanx | None = None
-    for method in methods:
-        layer = Phalanx(
-            dim=dim, length=length, method=method, dtype=dtype, k=k, wpb=wpb, output_dtype=output_dtype,
-            block_size=block_size, kv_heads=kv_heads,
-        ).to(device)
-        if first is None:
-            first = layer
+    shared = dict(dim=dim, length=length, dtype=dtype, k=k, wpb=wpb, output_dtype=output_dtype,
+                  block_size=block_size, kv_heads=kv_heads)
+    layers = {method: Phalanx(method=method, **shared).to(device) for method in methods}
+    weights = None
+    for layer in layers.values():
+        if weights is None:
+            weights = layer.state_dict()
         else:
-            layer.load_state_dict(first.state_dict())
-        layers[method] = layer
+            layer.load_state_dict(weights)
     return layers
 
 
@@ -123,15 +109,14 @@ def compare_layer_gradients(
         gen = torch.Generator().manual_seed(0)
         grad_out = torch.randn(x.shape, generator=gen, dtype=torch.float32).to(x.device)
 
-    grads: dict[str, dict[str, torch.Tensor]] = {}
-    for method, layer in layers.items():
+    def gradients_of(layer: Phalanx) -> dict[str, torch.Tensor]:
         layer.zero_grad(set_to_none=True)
-        xin = x.clone().detach().requires_grad_(True)
-        torch.autograd.backward(run_layer_forward(layer, xin, compile=compile, compile_opts=compile_opts), grad_out)
-        g = {"x": xin.grad.detach().clone() if xin.grad is not None else torch.zeros_like(xin)}
-        for name, p in layer.named_parameters():
-            g[name] = p.grad.detach().clone() if p.grad is not None else torch.zeros_like(p)
-        grads[method] = g
+        xin = x.detach().clone().requires_grad_(True)
+        run_layer_forward(layer, xin, compile=compile, compile_opts=compile_opts).backward(grad_out)
+        wrt_input = torch.zeros_like(xin) if xin.grad is None else xin.grad.detach().clone()
+        return {"x": wrt_input, **extract_layer_gradients(layer)}
+
+    grads = {method: gradients_of(layer) for method, layer in layers.items()}
     maybe_synchronize(x.device)
 
     ref = grads[reference_method]

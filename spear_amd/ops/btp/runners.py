@@ -43,15 +43,8 @@ __all__ = [
 
 
 def sample_inputs(
-    B: int,
-    H: int,
-    L: int,
-    *,
-    dtype: torch.dtype = torch.bfloat16,
-    device: torch.device | None = None,
-    seed: int | None = None,
-    stress_scale: float = 1.0,
-    distribution: InputDistributionConfig | None = None,
+    B: int, H: int, L: int, *, dtype: torch.dtype = torch.bfloat16, device: torch.device | None = None,
+    seed: int | None = None, stress_scale: float = 1.0, distribution: InputDistributionConfig | None = None,
 ) -> tuple[torch.Tensor, torch.Tensor]:
     """``(coeff [H, L], x [B, H, 16, L])`` in ``dtype`` on ``device`` (default: the GPU)."""
     device = torch.device(device or ("cuda" if torch.cuda.is_available() else "cpu"))
@@ -80,14 +73,8 @@ def _maybe_compiled(compile: bool, compile_opts: dict | None):
 
 
 def run_kernel_forward(
-    coeff: torch.Tensor,
-    x: torch.Tensor,
-    *,
-    k: int = 2,
-    output_dtype: torch.dtype = torch.float32,
-    wpb: int | None = None,
-    compile: bool = False,
-    compile_opts: dict | None = None,
+    coeff: torch.Tensor, x: torch.Tensor, *, k: int = 2, output_dtype: torch.dtype = torch.float32,
+    wpb: int | None = None, compile: bool = False, compile_opts: dict | None = None,
 ) -> torch.Tensor:
     fn = _maybe_compiled(compile, compile_opts)
     return fn(_broadcast_coeff(coeff, x.shape[0]).contiguous(), x, k=k, wpb=wpb, output_dtype=output_dtype)
@@ -104,14 +91,8 @@ def run_reference_logbtp(coeff: torch.Tensor, x: torch.Tensor, BL: int = 16) -> 
 
 
 def compare_backward_gradients(
-    coeff: torch.Tensor,
-    x: torch.Tensor,
-    *,
-    grad_out: torch.Tensor | None = None,
-    k: int = 2,
-    output_dtype: torch.dtype = torch.float32,
-    compile: bool = False,
-    compile_opts: dict | None = None,
+    coeff: torch.Tensor, x: torch.Tensor, *, grad_out: torch.Tensor | None = None, k: int = 2,
+    output_dtype: torch.dtype = torch.float32, compile: bool = False, compile_opts: dict | None = None,
 ) -> dict[str, dict[str, float]]:
     """Error metrics of the kernel's ``d coeff`` and ``dx`` against autograd through the float64
     reference, for the same upstream gradient."""
@@ -140,14 +121,13 @@ def compare_backward_gradients(
     }
 
 
-RUNNERS: dict[str, Callable[..., torch.Tensor]] = {
-    "kernel": run_kernel_forward,
-    "reference_logbtp": run_reference_logbtp,
-    "reference": run_reference,
-}
+RUNNERS: dict[str, Callable[..., torch.Tensor]] = dict(
+    kernel=run_kernel_forward, reference_logbtp=run_reference_logbtp, reference=run_reference
+)
 
 
 def get_runner(name: str) -> Callable[..., torch.Tensor]:
-    if name not in RUNNERS:
-        raise ValueError(f"Unknown BTP runner '{name}'")
-    return RUNNERS[name]
+    try:
+        return RUNNERS[name]
+    except KeyError:
+        raise ValueError(f"Unknown BTP runner '{name}'") from None
