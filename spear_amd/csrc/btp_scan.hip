@@ -209,9 +209,15 @@ __global__ __launch_bounds__(64 * kWaves) SPEAR_BTP_FWD_OCC void btp_fwd_scan_ke
 // Wavefronts per workgroup of the backward kernels: the larger workgroup for rows of several spans
 // where 4 waves per SIMD fit (16-bit dy, 16-bit coefficients). The other variants need more than
 // 128 registers, and two 8-wave workgroups would then no longer fit a CU (measured: -33 %).
+// Wavefronts per workgroup of the lean backward kernel on rows of one span (no hand-over there, so the
+// size is free): 4 measured best at B*H = 32768 rows of L = 128 (1, 2 and 8 are 0.6-1.9 % slower).
+#ifndef SPEAR_BTP_BWD_SHORT_ROW_WAVES
+#define SPEAR_BTP_BWD_SHORT_ROW_WAVES kWaves
+#endif
 template <bool kLean, bool kStreamIn>
 constexpr int bwd_waves() {
-  return (kStreamIn || !kLean) ? kWaves : kWavesLong;
+  if (!kLean) return kWaves;
+  return kStreamIn ? SPEAR_BTP_BWD_SHORT_ROW_WAVES : kWavesLong;
 }
 
 template <class E, class C, class GradT, bool kStreamIn, int kW>
@@ -507,7 +513,7 @@ void launch_bwd_as(const BwdArgs& p, const Grid& g, hipStream_t s) {
 template <class E, class C, class GradT>
 hipError_t launch_bwd(const BwdArgs& p, hipStream_t s) {
   constexpr bool kLean = !(std::is_same<GradT, float>::value || C::kLog);  // the kernel launch_bwd_as picks
-  const Grid g = make_grid((long)p.B * p.H, p.L, bwd_waves<kLean, false>());
+  const Grid g = make_grid((long)p.B * p.H, p.L, bwd_waves<kLean, false>(), bwd_waves<kLean, true>());
   if (stream_inputs(g)) launch_bwd_as<E, C, GradT, true>(p, g, s);
   else launch_bwd_as<E, C, GradT, false>(p, g, s);
   return hipGetLastError();

@@ -459,12 +459,12 @@ struct Grid {
 // Rows that fit one span are read exactly once and can be streamed; longer rows are re-read by
 // neighbouring spans' halo loads, so their lines should stay in L2. `waves_long` is the workgroup
 // size (in wavefronts) the calling kernel family uses for those longer rows.
-inline Grid make_grid(long rows, int L, int waves_long = kWaves) {
+inline Grid make_grid(long rows, int L, int waves_long = kWaves, int waves_short = kWaves) {
   Grid g;
   g.spans_per_row = (L + kSpan - 1) / kSpan;
   g.total_spans = rows * g.spans_per_row;
   g.stream = g.spans_per_row == 1;  // template argument kStreamIn of the kernels: rows of a single span
-  g.waves = g.stream ? kWaves : waves_long;
+  g.waves = g.stream ? waves_short : waves_long;
   g.blocks = (unsigned)((g.total_spans + g.waves - 1) / g.waves);
   return g;
 }
