@@ -16,7 +16,10 @@ initialises identical weights).
   ``"pytorch_linspace"``  the linear-space PyTorch statement
   ``"fused"``             (addition) one HIP kernel for gates + recurrence + ``* C + V`` working
                           directly on the projection outputs; needs ``heads % 4 == 0``, ``k == 2``
-The choice is explicit; ``"default"`` and ``"fused"`` never degrade to a PyTorch path.
+The choice is explicit; ``"default"`` and ``"fused"`` never degrade to a PyTorch path. Code written
+against the reference says ``method="default"``; with ``SPEAR_PHALANX_DEFAULT=fused`` in the environment
+such a layer runs the fused kernels wherever they apply (``heads % 4 == 0``, ``k == 2``, bf16 output) and
+the stand-alone kernels elsewhere, without a change to the calling code.
 
 On a GPU, from 8192 tokens per call on, the ``"default"`` and ``"fused"`` layers run their five
 projections through :mod:`.projections` (same forward; weight gradients cut along the token axis, one
@@ -25,6 +28,8 @@ other two are compared with.
 """
 
 from __future__ import annotations
+
+import os
 
 import torch
 import torch.nn as nn
@@ -180,12 +185,16 @@ class Phalanx(nn.Module):
         self.proj_out = nn.Linear(dim, dim, bias=False, dtype=dtype)
         self.param.token_sliced_backward = method in ("default", "fused")
 
-        if method == "default":
+        runs_fused = method == "fused" or (
+            method == "default" and os.environ.get("SPEAR_PHALANX_DEFAULT", "") == "fused"
+            and heads % 4 == 0 and k == 2 and self.output_dtype == self.compute_dtype
+        )
+        if method == "default" and not runs_fused:
             from spear_amd.ops.btp import btp
 
             self.btp_module = btp
             self._forward_fn = self._forward_default
-        elif method == "fused":
+        elif runs_fused:
             from spear_amd.ops.btp import phalanx_mix
 
             self.mix_module = phalanx_mix

@@ -235,3 +235,15 @@ def test_fused_rejects_unsupported_shapes():
     a, b, c, v = make_mix_inputs(1, 32, 6, 6, seed=0)
     with pytest.raises(RuntimeError, match="multiple of 4"):
         _btp.mix_forward(a.to(DEV), b.to(DEV), c.to(DEV), v.to(DEV), torch.empty_like(v, device=DEV), 6, 6)
+
+
+def test_default_method_rerouted_by_environment_gives_the_fused_results(monkeypatch):
+    from spear_amd import Phalanx
+
+    torch.manual_seed(3)
+    fused = Phalanx(dim=128, length=64, method="fused", dtype=torch.bfloat16).to(DEV)
+    monkeypatch.setenv("SPEAR_PHALANX_DEFAULT", "fused")
+    rerouted = Phalanx(dim=128, length=64, dtype=torch.bfloat16).to(DEV)
+    rerouted.load_state_dict(fused.state_dict())
+    x = torch.randn(2, 64, 128, generator=torch.Generator().manual_seed(4)).bfloat16().to(DEV)
+    assert torch.equal(rerouted(x), fused(x))

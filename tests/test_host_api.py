@@ -306,6 +306,24 @@ def test_oracle_qkv_gate_form_matches_torch_composition_and_autograd():
         np.testing.assert_allclose(got, t.grad.numpy(), rtol=1e-10, atol=1e-12, err_msg=name)
 
 
+def test_default_method_can_be_sent_to_the_fused_kernels_by_environment(monkeypatch):
+    from spear_amd import Phalanx
+
+    plain = Phalanx(dim=64, dtype=torch.bfloat16)
+    assert plain._forward_fn == plain._forward_default
+    monkeypatch.setenv("SPEAR_PHALANX_DEFAULT", "fused")
+    sent = Phalanx(dim=64, dtype=torch.bfloat16)
+    assert sent.method == "default" and sent._forward_fn == sent._forward_fused
+    assert list(sent.state_dict()) == list(plain.state_dict())
+    # where the fused kernels do not apply the stand-alone kernels stay: k = 1, heads not a multiple of 4, fp32 output
+    for kwargs in (dict(dim=64, k=1), dict(dim=32), dict(dim=64, output_dtype=torch.float32)):
+        layer = Phalanx(dtype=torch.bfloat16, **kwargs)
+        assert layer._forward_fn == layer._forward_default
+    # the explicit PyTorch methods are never rerouted
+    layer = Phalanx(dim=64, dtype=torch.bfloat16, method="pytorch")
+    assert layer._forward_fn == layer._forward_pytorch
+
+
 def test_streaming_module_surface_and_state_dataclass():
     from spear_amd.nn.phalanx import inference as inf
 
