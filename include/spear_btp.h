@@ -47,8 +47,8 @@ extern "C" {
 
 /* flags */
 #define SPEAR_BTP_WRITE_CHECKPOINT 0x1u /* forward: also store the carry checkpoint            */
-#define SPEAR_BTP_PATH_MFMA 0x2u        /* use the bf16-MFMA tile kernels (decay matrix rounded */
-                                        /* to bf16) instead of the exact-fp32 recurrence kernels */
+#define SPEAR_BTP_PATH_MFMA 0x2u        /* forward: use the MFMA tile kernel (decay matrix rounded */
+                                        /* to the input dtype) instead of the exact-fp32 recurrence */
 
 /* error codes */
 #define SPEAR_BTP_EINVAL (-1)  /* bad shape, dtype, k, flag or alignment                       */

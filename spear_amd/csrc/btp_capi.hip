@@ -61,8 +61,6 @@ int spear_btp_forward(const void* coeff, const void* x, void* y, float* checkpoi
   if (!aligned16(coeff) || !aligned16(x) || !aligned16(y) || (want_ckpt && !aligned16(checkpoint)))
     return fail(SPEAR_BTP_EINVAL, "spear_btp_forward: tensor pointers must be 16-byte aligned");
   const bool mfma = (flags & SPEAR_BTP_PATH_MFMA) != 0;
-  if (mfma && in_dtype != SPEAR_BTP_BF16)
-    return fail(SPEAR_BTP_EINVAL, "spear_btp_forward: the MFMA path takes bfloat16 inputs only");
   if (mfma && want_ckpt)
     return fail(SPEAR_BTP_EINVAL, "spear_btp_forward: the MFMA path does not store the carry checkpoint");
 

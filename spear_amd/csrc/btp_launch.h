@@ -35,7 +35,7 @@ struct BwdArgs {
 hipError_t scan_forward(const FwdArgs& p, hipStream_t s);
 hipError_t scan_backward(const BwdArgs& p, hipStream_t s);
 
-// bf16-MFMA tile kernels (btp_mfma.hip). bf16 inputs only; the forward one stores no checkpoint.
+// MFMA tile kernel (btp_mfma.hip), forward only, bf16 or fp16 inputs; it stores no checkpoint.
 hipError_t mfma_forward(const FwdArgs& p, hipStream_t s);
 
 // Fused layer-layout forward (btp_fused.hip): all operands [B, L, features], 16-bit.

@@ -1,7 +1,7 @@
-// bf16-MFMA tile kernels for the Block Two-Pass operator on gfx950 (MI355X): the formulation the
+// MFMA tile kernel for the Block Two-Pass operator on gfx950 (MI355X), bf16 and fp16: the formulation the
 // reference uses on sm90 -- materialise the block's decay matrix, multiply it with the activation
 // tile on the matrix cores (csrc/btp/btp-forward.cu:214-274, WarpMma in csrc/btp/btp_common.h:35-45)
-// -- rebuilt around v_mfma_f32_16x16x32_bf16. Selected with SPEAR_BTP_PATH_MFMA; the default path
+// -- rebuilt around v_mfma_f32_16x16x32_bf16 / _f16. Selected with SPEAR_BTP_PATH_MFMA; the default path
 // is the exact-fp32 recurrence (btp_scan.hip), which is at least as fast (both are HBM-bound) and
 // does not round the decay matrix to bf16.
 //
@@ -63,12 +63,20 @@ __device__ __forceinline__ float lane_broadcast(float v, int src_lane) {
   return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), src_lane));
 }
 
-__device__ __forceinline__ bf16x8_t pack_bf16x8(const float (&e)[8]) {
-  uint4 q = pack8<Bf16>(e);
-  return __builtin_bit_cast(bf16x8_t, q);
+typedef _Float16 halfx8_t __attribute__((ext_vector_type(8)));
+
+// One 16x16x32 matrix instruction on eight 16-bit elements per lane and operand (raw bits), fp32 accumulate.
+template <class E>
+__device__ __forceinline__ floatx4_t mfma_16x16x32(uint4 a, uint4 b, floatx4_t acc) {
+  if constexpr (std::is_same<E, Bf16>::value)
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), acc,
+                                                   0, 0, 0);
+  else
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(halfx8_t, a), __builtin_bit_cast(halfx8_t, b), acc,
+                                                  0, 0, 0);
 }
 
-template <class OutT, bool kStreamIn>
+template <class E, class OutT, bool kStreamIn>
 __global__ __launch_bounds__(64 * kWaves) void btp_fwd_mfma_kernel(const uint16_t* __restrict__ coeff,
                                                                    const uint16_t* __restrict__ x,
                                                                    OutT* __restrict__ y, int L, int spans_per_row,
@@ -97,7 +105,7 @@ __global__ __launch_bounds__(64 * kWaves) void btp_fwd_mfma_kernel(const uint16_
   // ---- global -> LDS
   uint4 xin[4];
   slab16_global_to_regs<kStreamIn>(xslab, L, sc.nvalid, lane, xin);
-  const uint32_t ain = coeff_global_to_reg<LinCoeff<Bf16>>(arow, sc.nvalid, lane);
+  const uint32_t ain = coeff_global_to_reg<LinCoeff<E>>(arow, sc.nvalid, lane);
   const bool halo = (k == 2) && (sc.sp > 0);  // wave-uniform
   uint4 hx = zero4();
   uint32_t ha = 0u;
@@ -109,12 +117,12 @@ __global__ __launch_bounds__(64 * kWaves) void btp_fwd_mfma_kernel(const uint16_
   if (lane < 32) *reinterpret_cast<uint4*>(halo_x + (lane >> 1) * 32 + ((lane & 1) << 4)) = hx;
   {
     float2 f;
-    f.x = clamp_coeff<Bf16>(Bf16::lo(ain));
-    f.y = clamp_coeff<Bf16>(Bf16::hi(ain));
+    f.x = clamp_coeff<E>(E::lo(ain));
+    f.y = clamp_coeff<E>(E::hi(ain));
     *reinterpret_cast<float2*>(a_ext + kTile + (lane << 1)) = f;
     if (lane < 8) {
-      f.x = clamp_coeff<Bf16>(Bf16::lo(ha));
-      f.y = clamp_coeff<Bf16>(Bf16::hi(ha));
+      f.x = clamp_coeff<E>(E::lo(ha));
+      f.y = clamp_coeff<E>(E::hi(ha));
       *reinterpret_cast<float2*>(a_ext + (lane << 1)) = f;
     }
   }
@@ -148,7 +156,7 @@ __global__ __launch_bounds__(64 * kWaves) void btp_fwd_mfma_kernel(const uint16_
       e[jj] = above ? 0.0f : val;
       val *= above ? 1.0f : av[jj];
     }
-    const bf16x8_t A = pack_bf16x8(e);
+    const uint4 A = pack8<E>(e);
 
     // B: steps 16(i-1) + 8q .. +7 of channel n
     const int cidx = 2 * i - 2 + q;
@@ -160,15 +168,15 @@ __global__ __launch_bounds__(64 * kWaves) void btp_fwd_mfma_kernel(const uint16_
       braw = *reinterpret_cast<const uint4*>(img_x + swz<256>(n, cidx));
     }
     floatx4_t acc = {0.0f, 0.0f, 0.0f, 0.0f};
-    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(A, __builtin_bit_cast(bf16x8_t, braw), acc, 0, 0, 0);
+    acc = mfma_16x16x32<E>(A, braw, acc);
 
     // D: y[channel n][16 i + 4 q .. + 3]
     if constexpr (kOutF32) {
       *reinterpret_cast<float4*>(img_y + swz<512>(n, 4 * i + q)) = make_float4(acc[0], acc[1], acc[2], acc[3]);
     } else {
       uint2 o;
-      o.x = Bf16::pack2(acc[0], acc[1]);
-      o.y = Bf16::pack2(acc[2], acc[3]);
+      o.x = E::pack2(acc[0], acc[1]);
+      o.y = E::pack2(acc[2], acc[3]);
       *reinterpret_cast<uint2*>(img_y + swz<256>(n, 2 * i + (q >> 1)) + ((q & 1) << 3)) = o;
     }
     g_prev = s15;
@@ -184,9 +192,9 @@ __global__ __launch_bounds__(64 * kWaves) void btp_fwd_mfma_kernel(const uint16_
   }
 }
 
-template <class OutT, bool kStreamIn>
+template <class E, class OutT, bool kStreamIn>
 void launch_fwd_mfma(const FwdArgs& p, const Grid& g, hipStream_t s) {
-  hipLaunchKernelGGL((btp_fwd_mfma_kernel<OutT, kStreamIn>), dim3(g.blocks), dim3(64 * kWaves), 0, s,
+  hipLaunchKernelGGL((btp_fwd_mfma_kernel<E, OutT, kStreamIn>), dim3(g.blocks), dim3(64 * kWaves), 0, s,
                      static_cast<const uint16_t*>(p.coeff), static_cast<const uint16_t*>(p.x),
                      static_cast<OutT*>(p.y), p.L, g.spans_per_row, g.total_spans, p.k);
 }
@@ -196,13 +204,18 @@ void launch_fwd_mfma(const FwdArgs& p, const Grid& g, hipStream_t s) {
 hipError_t mfma_forward(const FwdArgs& p, hipStream_t s) {
   const Grid g = make_grid((long)p.B * p.H, p.L);
   const bool st = stream_inputs(g);
-  if (p.out_dtype == kF32) {
-    if (st) launch_fwd_mfma<float, true>(p, g, s);
-    else launch_fwd_mfma<float, false>(p, g, s);
-  } else {
-    if (st) launch_fwd_mfma<uint16_t, true>(p, g, s);
-    else launch_fwd_mfma<uint16_t, false>(p, g, s);
-  }
+  auto by_out = [&](auto e) {
+    using E = decltype(e);
+    if (p.out_dtype == kF32) {
+      if (st) launch_fwd_mfma<E, float, true>(p, g, s);
+      else launch_fwd_mfma<E, float, false>(p, g, s);
+    } else {
+      if (st) launch_fwd_mfma<E, uint16_t, true>(p, g, s);
+      else launch_fwd_mfma<E, uint16_t, false>(p, g, s);
+    }
+  };
+  if (p.in_dtype == kBf16) by_out(Bf16{});
+  else by_out(Fp16{});
   return hipGetLastError();
 }
 

@@ -75,6 +75,16 @@ def test_forward_mfma_path_matches_oracle(B, H, L, k, out_dtype):
     assert_close(f64(y), orc.forward(f64(coeff), f64(x), k=k), BF16_ATOL, BF16_RTOL, "y")
 
 
+@pytest.mark.parametrize("B,H,L,k", [(2, 3, 64, 2), (1, 2, 400, 2), (2, 2, 144, 1)])
+def test_forward_mfma_path_fp16(B, H, L, k):
+    coeff, x, _ = make_inputs(B, H, L, seed=900 + L, dtype=torch.float16)
+    y = run_forward(coeff, x, k=k, out_dtype=torch.float16, mfma=True)
+    # fp16 storage (11 significant bits) of the decay matrix and of y
+    assert_close(f64(y), orc.forward(f64(coeff), f64(x), k=k), 4e-3, 4e-3, "y mfma fp16")
+    y32 = run_forward(coeff, x, k=k, out_dtype=torch.float32, mfma=True)
+    assert_close(f64(y32), orc.forward(f64(coeff), f64(x), k=k), 4e-3, 4e-3, "y32 mfma fp16")
+
+
 def test_forward_mfma_path_stress_and_zero_coefficients():
     coeff, x, _ = make_inputs(2, 8, 2048, seed=1236, gate="mixed")
     y = run_forward(coeff, x, mfma=True)
@@ -88,12 +98,12 @@ def test_forward_mfma_path_stress_and_zero_coefficients():
 def test_mfma_path_rejects_what_it_does_not_do():
     from spear_amd import _btp
 
-    coeff, x, dy = make_inputs(1, 2, 32, seed=1, dtype=torch.float16)
+    coeff, x, dy = make_inputs(1, 2, 32, seed=1)
     c, xx = coeff.to(DEV), x.to(DEV)
     y = torch.empty_like(xx)
     ck = torch.empty(1, 2, 2, 16, device=DEV)
-    with pytest.raises(RuntimeError, match="bfloat16 inputs only"):
-        _btp.forward(c, xx, y, ck, 2, 32, flags=_btp.FLAG_PATH_MFMA)
+    with pytest.raises(RuntimeError, match="does not store the carry checkpoint"):
+        _btp.forward(c, xx, y, ck, 2, 32, flags=_btp.FLAG_PATH_MFMA | _btp.FLAG_WRITE_CHECKPOINT)
     with pytest.raises(RuntimeError, match="no MFMA variant"):
         _btp.backward(c, xx, dy.to(DEV), ck, torch.empty_like(xx), torch.empty(1, 2, 32, device=DEV), 2, 32, flags=_btp.FLAG_PATH_MFMA)
 
