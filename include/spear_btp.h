@@ -140,6 +140,28 @@ int spear_phalanx_mix_backward_ex(const void* a_logit, const void* b_logit, cons
                                   long long sum_rows, int B, int L, int H, int kv_heads, int dtype, unsigned flags,
                                   void* stream);
 
+/* The same backward for callers that cannot allocate device memory -- code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc -- and therefore cannot bring the partial-sum arrays of
+ * spear_phalanx_mix_backward_ex. It has no counterpart in the reference. The partial column sums pass through
+ * a device array the library holds statically (SPEAR_MIX_BIAS_SCRATCH_FLOATS floats = 8 MiB on every GPU the
+ * library is used on, until the process ends), a second kernel finishes them, and the caller receives the
+ * finished bias gradients of proj_a, proj_b and proj_c (spear/nn/phalanx/swr.py:157-163):
+ *     bias_da [H],  bias_db [kv_heads * 16],  bias_dc [kv_heads * 16]      fp32, sums over batch and time,
+ * taken before the gradients are rounded to `dtype`; all three are required and 16-byte aligned. Everything
+ * else is as in spear_phalanx_mix_backward_ex (layer form only, no SPEAR_MIX_QKV_GATE). The call makes no
+ * hipMalloc / hipFree and no allocating library call. Limit:
+ *     spear_phalanx_mix_backward_sum_rows(B, L, H) * (H + 2 * kv_heads * 16) <= SPEAR_MIX_BIAS_SCRATCH_FLOATS
+ * (B = 1024, L = 128, H = kv_heads = 32 needs 1,081,344), otherwise SPEAR_BTP_EINVAL. All calls on one GPU
+ * share that GPU's array: calls that overlap in time on one GPU (two streams, two threads) race, so
+ * serialise them. Nothing in the array has to be cleared between calls -- each call overwrites all it later
+ * reads. The array's address is looked up on the first call on each device; make that first call outside
+ * stream capture. */
+#define SPEAR_MIX_BIAS_SCRATCH_FLOATS 2097152
+int spear_phalanx_mix_backward_bias(const void* a_logit, const void* b_logit, const void* c, const void* v,
+                                    const void* dout, void* da_logit, void* db_logit, void* dc, void* dv, int ld_da,
+                                    int ld_db, int ld_dc, int ld_dv, float* bias_da, float* bias_db, float* bias_dc,
+                                    int B, int L, int H, int kv_heads, int dtype, unsigned flags, void* stream);
+
 /* ---- streaming form: prompt prefill with state hand-over, and the one-token decode step --------
  * They replace the PyTorch loops of spear/nn/phalanx/inference.py. Tensors are dense, row-major:
  *     a         [B, H, L]      a_dtype (x_dtype or fp32)   a_t, or log(a_t) with SPEAR_JAGGED_LOG_A

@@ -18,7 +18,7 @@ import threading
 
 import torch
 
-__all__ = ["forward", "backward", "forward_log", "backward_log", "mix_forward", "mix_backward", "jagged_prefill", "jagged_step", "library_path", "load_library", "FLAG_WRITE_CHECKPOINT", "FLAG_PATH_MFMA", "FLAG_JAGGED_LOG_A", "FLAG_JAGGED_LOG_R", "FLAG_MIX_QKV_GATE", "mix_backward_sum_rows"]
+__all__ = ["forward", "backward", "forward_log", "backward_log", "mix_forward", "mix_backward", "jagged_prefill", "jagged_step", "library_path", "load_library", "FLAG_WRITE_CHECKPOINT", "FLAG_PATH_MFMA", "FLAG_JAGGED_LOG_A", "FLAG_JAGGED_LOG_R", "FLAG_MIX_QKV_GATE", "mix_backward_sum_rows", "mix_backward_bias"]
 
 _BF16, _F16, _F32 = 0, 1, 2
 FLAG_WRITE_CHECKPOINT = 0x1
@@ -26,7 +26,7 @@ FLAG_PATH_MFMA = 0x2
 FLAG_JAGGED_LOG_A = 0x4
 FLAG_JAGGED_LOG_R = 0x8
 FLAG_MIX_QKV_GATE = 0x1
-_ABI_VERSION = 8
+_ABI_VERSION = 9
 _SUPPORTED_WPB = (4, 8, 16, 32)
 
 _lock = threading.Lock()
@@ -57,6 +57,8 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.spear_phalanx_mix_backward.restype = ci
     lib.spear_phalanx_mix_backward_ex.argtypes = [vp] * 9 + [ci] * 4 + [vp] * 3 + [ctypes.c_longlong, ci, ci, ci, ci, ci, cu, vp]
     lib.spear_phalanx_mix_backward_ex.restype = ci
+    lib.spear_phalanx_mix_backward_bias.argtypes = [vp] * 9 + [ci] * 4 + [vp] * 3 + [ci, ci, ci, ci, ci, cu, vp]
+    lib.spear_phalanx_mix_backward_bias.restype = ci
     lib.spear_phalanx_mix_backward_sum_rows.argtypes = [ci, ci, ci]
     lib.spear_phalanx_mix_backward_sum_rows.restype = ctypes.c_longlong
     lib.spear_jagged_prefill.argtypes = [vp] * 9 + [ci] * 9 + [cu, vp]
@@ -392,6 +394,57 @@ def mix_backward(
             da_logit.data_ptr(), db_logit.data_ptr(), dc.data_ptr(), dv.data_ptr(), *lds,
             *sum_ptrs, rows,
             B, L, heads, kv_heads, _tag(v.dtype), FLAG_MIX_QKV_GATE if qkv_gate else 0, _stream_ptr(v.device),
+        )
+    if rc != 0:
+        _raise_native(lib, rc)
+
+
+def mix_backward_bias(
+    a_logit: torch.Tensor,
+    b_logit: torch.Tensor,
+    c: torch.Tensor,
+    v: torch.Tensor,
+    dout: torch.Tensor,
+    da_logit: torch.Tensor,
+    db_logit: torch.Tensor,
+    dc: torch.Tensor,
+    dv: torch.Tensor,
+    bias: tuple[torch.Tensor, torch.Tensor, torch.Tensor],
+    heads: int,
+    kv_heads: int,
+) -> None:
+    """:func:`mix_backward` plus the finished column sums of ``da_logit``, ``db_logit`` and ``dc`` over batch
+    and time in ``bias`` (fp32 ``[heads]``, ``[kv_heads*16]``, ``[kv_heads*16]``), with no device memory
+    allocated anywhere on the way: the partial sums pass through an array the library holds statically
+    (``spear_phalanx_mix_backward_bias`` in the C header; shapes beyond its size raise). Calls on one GPU
+    must not overlap in time."""
+    tensors = (a_logit, b_logit, c, v, dout, da_logit, db_logit, dc, dv, *bias)
+    _check(all(t.is_cuda for t in tensors), "All tensors must be CUDA.")
+    _check(len({t.device for t in tensors}) == 1, "All tensors must be on the same device.")
+    _check(v.dim() == 3, "v must be [B, L, heads * 16].")
+    B, L, F = v.shape
+    _check(F == heads * 16, "v must be [B, L, heads * 16].")
+    _check(kv_heads > 0 and heads % kv_heads == 0, "heads must be divisible by kv_heads.")
+    _check(v.dtype in (torch.float16, torch.bfloat16), "tensors must be float16 or bfloat16.")
+    _check(all(t.dtype == v.dtype for t in tensors[:9]), "all tensors must share one dtype.")
+    Fkv = kv_heads * 16
+    for name, t, shape in (
+        ("a_logit", a_logit, (B, L, heads)), ("b_logit", b_logit, (B, L, Fkv)), ("c", c, (B, L, Fkv)),
+        ("v", v, (B, L, F)), ("dout", dout, (B, L, F)),
+    ):
+        _check_layout(name, t, shape)
+    lds = [_row_stride(name, t, (B, L, width)) for name, t, width in
+           (("da_logit", da_logit, heads), ("db_logit", db_logit, Fkv), ("dc", dc, Fkv), ("dv", dv, F))]
+    for name, t, width in (("bias_da", bias[0], heads), ("bias_db", bias[1], Fkv), ("bias_dc", bias[2], Fkv)):
+        _check(t.dtype == torch.float32, f"{name} must be float32.")
+        _check_layout(name, t, (width,))
+    lib = load_library()
+    with torch.cuda.device(v.device):
+        rc = lib.spear_phalanx_mix_backward_bias(
+            a_logit.data_ptr(), b_logit.data_ptr(), c.data_ptr(), v.data_ptr(), dout.data_ptr(),
+            da_logit.data_ptr(), db_logit.data_ptr(), dc.data_ptr(), dv.data_ptr(), *lds,
+            bias[0].data_ptr(), bias[1].data_ptr(), bias[2].data_ptr(),
+            B, L, heads, kv_heads, _tag(v.dtype), 0, _stream_ptr(v.device),
         )
     if rc != 0:
         _raise_native(lib, rc)

@@ -44,7 +44,7 @@ int check_common(const char* who, int B, int H, int L, int k, int in_dtype, int 
 
 extern "C" {
 
-int spear_btp_abi_version(void) { return 8; }
+int spear_btp_abi_version(void) { return 9; }
 
 const char* spear_btp_last_error(void) { return g_error; }
 
@@ -162,13 +162,9 @@ int spear_phalanx_mix_backward(const void* a_logit, const void* b_logit, const v
                                        nullptr, nullptr, 0, B, L, H, kv_heads, dtype, flags, stream);
 }
 
-int spear_phalanx_mix_backward_ex(const void* a_logit, const void* b_logit, const void* c, const void* v,
-                                  const void* dout, void* da_logit, void* db_logit, void* dc, void* dv, int ld_da,
-                                  int ld_db, int ld_dc, int ld_dv, float* sum_da, float* sum_db, float* sum_dc,
-                                  long long sum_rows, int B, int L, int H, int kv_heads, int dtype, unsigned flags,
-                                  void* stream) {
-  g_error[0] = '\0';
-  const char* who = "spear_phalanx_mix_backward";
+// Checks shared by the fused backward entry points; 1 = nothing to do (empty tensors), 0 = go on.
+static int check_mix_backward(const char* who, const void* const (&ptrs)[9], const int (&lds)[4], int B, int L, int H,
+                              int kv_heads, int dtype, unsigned flags, unsigned allowed_flags) {
   if (B < 0 || L < 0 || H < 0) return fail(SPEAR_BTP_EINVAL, "%s: negative dimension (B=%d L=%d H=%d)", who, B, L, H);
   if (L % 16 != 0) return fail(SPEAR_BTP_EINVAL, "%s: Length L must be multiple of 16 (got %d)", who, L);
   if (H % 4 != 0) return fail(SPEAR_BTP_EINVAL, "%s: heads must be a multiple of 4 (got %d)", who, H);
@@ -181,18 +177,17 @@ int spear_phalanx_mix_backward_ex(const void* a_logit, const void* b_logit, cons
     return fail(SPEAR_BTP_EINVAL, "%s: groups of 8 heads need heads divisible by 8 (got %d)", who, H);
   if (dtype != SPEAR_BTP_BF16 && dtype != SPEAR_BTP_F16)
     return fail(SPEAR_BTP_EINVAL, "%s: tensors must be float16 or bfloat16.", who);
-  if (flags & ~SPEAR_MIX_QKV_GATE) return fail(SPEAR_BTP_EINVAL, "%s: unknown flag bits 0x%x", who, flags);
+  if (flags & ~allowed_flags) return fail(SPEAR_BTP_EINVAL, "%s: unknown flag bits 0x%x", who, flags & ~allowed_flags);
   const bool qkv = (flags & SPEAR_MIX_QKV_GATE) != 0;
   if ((long long)B * L * H * 16ll >= (1ll << 40)) return fail(SPEAR_BTP_EINVAL, "%s: tensor too large", who);
   if ((long long)L * H * 32ll >= (1ll << 31))  // a batch row is addressed through one 32-bit buffer resource
     return fail(SPEAR_BTP_EINVAL, "%s: one batch row (L * H * 16 elements) must stay below 2 GiB", who);
-  if ((long long)B * H == 0 || L == 0) return 0;
-  const void* ptrs[] = {a_logit, b_logit, c, v, dout, da_logit, db_logit, dc, dv};
+  if ((long long)B * H == 0 || L == 0) return 1;
   for (const void* q : ptrs) {
     if (!q) return fail(SPEAR_BTP_ENULL, "%s: NULL tensor pointer", who);
     if (!aligned16(q)) return fail(SPEAR_BTP_EINVAL, "%s: tensor pointers must be 16-byte aligned", who);
   }
-  const int widths[4] = {H, kv_heads * 16, kv_heads * 16, H * 16}, lds[4] = {ld_da, ld_db, ld_dc, ld_dv};
+  const int widths[4] = {H, kv_heads * 16, kv_heads * 16, H * 16};
   for (int i = 0; i < 4; ++i) {
     if (lds[i] == 0) continue;
     if (lds[i] < widths[i] || lds[i] % 2 != 0)
@@ -200,6 +195,20 @@ int spear_phalanx_mix_backward_ex(const void* a_logit, const void* b_logit, cons
     if ((long long)L * lds[i] * (i == 0 && qkv ? 4ll : 2ll) >= (1ll << 31))
       return fail(SPEAR_BTP_EINVAL, "%s: one batch row (L * row stride) must stay below 2 GiB", who);
   }
+  return 0;
+}
+
+int spear_phalanx_mix_backward_ex(const void* a_logit, const void* b_logit, const void* c, const void* v,
+                                  const void* dout, void* da_logit, void* db_logit, void* dc, void* dv, int ld_da,
+                                  int ld_db, int ld_dc, int ld_dv, float* sum_da, float* sum_db, float* sum_dc,
+                                  long long sum_rows, int B, int L, int H, int kv_heads, int dtype, unsigned flags,
+                                  void* stream) {
+  g_error[0] = '\0';
+  const char* who = "spear_phalanx_mix_backward";
+  const void* const ptrs[9] = {a_logit, b_logit, c, v, dout, da_logit, db_logit, dc, dv};
+  const int lds[4] = {ld_da, ld_db, ld_dc, ld_dv};
+  if (int rc = check_mix_backward(who, ptrs, lds, B, L, H, kv_heads, dtype, flags, SPEAR_MIX_QKV_GATE)) return rc < 0 ? rc : 0;
+  const bool qkv = (flags & SPEAR_MIX_QKV_GATE) != 0;
   const bool sums = sum_da || sum_db || sum_dc;
   if (sums && qkv) return fail(SPEAR_BTP_EINVAL, "%s: column sums are for the layer form, not SPEAR_MIX_QKV_GATE", who);
   if (sums) {
@@ -210,9 +219,37 @@ int spear_phalanx_mix_backward_ex(const void* a_logit, const void* b_logit, cons
     if (sum_rows != want)
       return fail(SPEAR_BTP_EINVAL, "%s: sum arrays must have %lld rows for this shape (got %lld)", who, want, sum_rows);
   }
-  spear_btp::MixBwdArgs a{a_logit, b_logit, c, v, dout, da_logit, db_logit, dc, dv, B, L, H, groups, dtype,
+  spear_btp::MixBwdArgs a{a_logit, b_logit, c, v, dout, da_logit, db_logit, dc, dv, B, L, H, H / kv_heads, dtype,
                           sum_da, sum_db, sum_dc, ld_da, ld_db, ld_dc, ld_dv, qkv};
   const hipError_t err = spear_btp::fused_mix_backward(a, static_cast<hipStream_t>(stream));
+  if (err != hipSuccess) return fail(SPEAR_BTP_ELAUNCH, "%s: launch failed: %s", who, hipGetErrorString(err));
+  return 0;
+}
+
+int spear_phalanx_mix_backward_bias(const void* a_logit, const void* b_logit, const void* c, const void* v,
+                                    const void* dout, void* da_logit, void* db_logit, void* dc, void* dv, int ld_da,
+                                    int ld_db, int ld_dc, int ld_dv, float* bias_da, float* bias_db, float* bias_dc,
+                                    int B, int L, int H, int kv_heads, int dtype, unsigned flags, void* stream) {
+  g_error[0] = '\0';
+  const char* who = "spear_phalanx_mix_backward_bias";
+  const void* const ptrs[9] = {a_logit, b_logit, c, v, dout, da_logit, db_logit, dc, dv};
+  const int lds[4] = {ld_da, ld_db, ld_dc, ld_dv};
+  const int rc = check_mix_backward(who, ptrs, lds, B, L, H, kv_heads, dtype, flags, 0u);
+  if (rc < 0) return rc;
+  if (!bias_da || !bias_db || !bias_dc) return fail(SPEAR_BTP_ENULL, "%s: the three bias gradient arrays are required", who);
+  if (!aligned16(bias_da) || !aligned16(bias_db) || !aligned16(bias_dc))
+    return fail(SPEAR_BTP_EINVAL, "%s: bias gradient arrays must be 16-byte aligned", who);
+  if (rc == 1) return 0;  // empty tensors: nothing is read or written, as in the other entry points
+  const long long need = spear_btp::fused_mix_backward_bias_scratch_floats(B, H, H / kv_heads, L);
+  if (need > (long long)SPEAR_MIX_BIAS_SCRATCH_FLOATS)
+    return fail(SPEAR_BTP_EINVAL,
+                "%s: this shape needs %lld floats of partial sums, the library's static array holds %lld; use "
+                "spear_phalanx_mix_backward_ex with caller-allocated sum arrays",
+                who, need, (long long)SPEAR_MIX_BIAS_SCRATCH_FLOATS);
+  spear_btp::MixBwdArgs a{a_logit, b_logit, c, v, dout, da_logit, db_logit, dc, dv, B, L, H, H / kv_heads, dtype,
+                          nullptr, nullptr, nullptr, ld_da, ld_db, ld_dc, ld_dv, false};
+  const hipError_t err =
+      spear_btp::fused_mix_backward_bias(a, bias_da, bias_db, bias_dc, static_cast<hipStream_t>(stream));
   if (err != hipSuccess) return fail(SPEAR_BTP_ELAUNCH, "%s: launch failed: %s", who, hipGetErrorString(err));
   return 0;
 }

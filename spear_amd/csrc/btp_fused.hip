@@ -31,10 +31,20 @@
 #include <stdint.h>
 #include <stdlib.h>
 
+#include <mutex>
 #include <type_traits>
 
+#include "../../include/spear_btp.h"
 #include "btp_device.h"
 #include "btp_launch.h"
+
+// Device memory owned by the library, for the one entry point that must not allocate
+// (fused_mix_backward_bias below): the per-(batch row, time chunk) partial column sums of the fused
+// backward kernel park here between that kernel and the kernel that finishes the sums. Every GPU the
+// library runs on holds its own copy until the process ends. In host code the name stands for the
+// symbol, not for a device address: the address is looked up once per device and only that pointer
+// is handed to kernels.
+static __device__ __align__(256) float scratch[SPEAR_MIX_BIAS_SCRATCH_FLOATS];
 
 namespace spear_btp {
 
@@ -655,6 +665,99 @@ hipError_t fused_mix_backward(const MixBwdArgs& p, hipStream_t s) {
     else if (sums) launch_mix_bwd<Fp16, true, false>(p, m, s);
     else launch_mix_bwd<Fp16, false, false>(p, m, s);
   }
+  return hipGetLastError();
+}
+
+namespace {
+
+// Finishes the column sums: out[col] = sum over `rows` of part[row * cols + col], for three arrays at once
+// (blockIdx.y picks one). A workgroup owns 64 columns; its 16 wavefronts each add up every 16th row (a
+// wave-level load is one contiguous 256-byte run of a row), then the 16 partial results meet in LDS. The
+// order of the additions is fixed, so equal inputs give equal bits.
+constexpr int kSumWaves = 16;
+struct SumJob {
+  const float* part;
+  float* out;
+  int cols;
+};
+__global__ __launch_bounds__(64 * kSumWaves) void finish_column_sums_kernel(SumJob j0, SumJob j1, SumJob j2, long rows) {
+  __shared__ float partial[kSumWaves][64];
+  const SumJob job = blockIdx.y == 0 ? j0 : (blockIdx.y == 1 ? j1 : j2);
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int col = blockIdx.x * 64 + lane;
+  const bool live = col < job.cols;  // whole workgroups beyond the array's width fall through to the barrier
+  float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+  if (live) {
+    const float* p = job.part + col;
+    long r = wave;
+    for (; r + 3 * kSumWaves < rows; r += 4 * kSumWaves) {
+#pragma unroll
+      for (int u = 0; u < 4; ++u) acc[u] += p[(r + u * kSumWaves) * job.cols];
+    }
+    for (; r < rows; r += kSumWaves) acc[0] += p[r * job.cols];
+  }
+  partial[wave][lane] = (acc[0] + acc[1]) + (acc[2] + acc[3]);
+  __syncthreads();
+  if (wave == 0 && live) {
+    float total = 0.0f;
+#pragma unroll
+    for (int w = 0; w < kSumWaves; ++w) total += partial[w][lane];
+    job.out[col] = total;
+  }
+}
+
+// Device address of `scratch` on the current device, looked up once per device.
+constexpr int kMaxDevices = 64;
+struct ScratchSlot {
+  std::once_flag once;
+  float* ptr = nullptr;
+  hipError_t err = hipSuccess;
+};
+ScratchSlot g_scratch[kMaxDevices];
+
+hipError_t scratch_of_current_device(float** out) {
+  int dev = -1;
+  hipError_t err = hipGetDevice(&dev);
+  if (err != hipSuccess) return err;
+  if (dev < 0 || dev >= kMaxDevices) return hipErrorInvalidDevice;
+  ScratchSlot& slot = g_scratch[dev];
+  std::call_once(slot.once, [&slot] {
+    void* p = nullptr;
+    slot.err = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    slot.ptr = slot.err == hipSuccess ? static_cast<float*>(p) : nullptr;
+  });
+  if (slot.err != hipSuccess) return slot.err;
+  if (slot.ptr == nullptr) return hipErrorInvalidSymbol;
+  *out = slot.ptr;
+  return hipSuccess;
+}
+
+}  // namespace
+
+long fused_mix_backward_bias_scratch_floats(long B, int H, int kv_groups, int L) {
+  if (B <= 0 || H <= 0 || L <= 0 || kv_groups <= 0) return 0;
+  const long Fkv = (long)(H / kv_groups) * kChan;
+  return fused_mix_backward_sum_rows(B, H, L) * (H + 2 * Fkv);
+}
+
+hipError_t fused_mix_backward_bias(const MixBwdArgs& p, float* bias_da, float* bias_db, float* bias_dc, hipStream_t s) {
+  if (p.qkv) return hipErrorInvalidValue;
+  const long rows = fused_mix_backward_sum_rows(p.B, p.H, p.L);
+  const long Fkv = (long)(p.H / p.kv_groups) * kChan;
+  if (rows * (p.H + 2 * Fkv) > (long)SPEAR_MIX_BIAS_SCRATCH_FLOATS) return hipErrorInvalidValue;  // the caller has checked
+  float* base = nullptr;
+  if (hipError_t err = scratch_of_current_device(&base); err != hipSuccess) return err;
+  // Nothing has to be cleared: the backward kernel writes every element of the three partial-sum arrays
+  // of this shape, and the finishing kernel reads only those.
+  MixBwdArgs q = p;
+  q.sum_da = base;
+  q.sum_db = base + rows * p.H;
+  q.sum_dc = q.sum_db + rows * Fkv;
+  if (hipError_t err = fused_mix_backward(q, s); err != hipSuccess) return err;
+  const SumJob ja{q.sum_da, bias_da, p.H}, jb{q.sum_db, bias_db, (int)Fkv}, jc{q.sum_dc, bias_dc, (int)Fkv};
+  const unsigned gx = (unsigned)((Fkv + 63) / 64);  // H <= Fkv * kv_groups / 16: the gate array is never the widest
+  const unsigned gxa = (unsigned)((p.H + 63) / 64);
+  hipLaunchKernelGGL(finish_column_sums_kernel, dim3(gx > gxa ? gx : gxa, 3), dim3(64 * kSumWaves), 0, s, ja, jb, jc, rows);
   return hipGetLastError();
 }
 

@@ -66,6 +66,11 @@ struct MixBwdArgs {
 };
 hipError_t fused_mix_backward(const MixBwdArgs& p, hipStream_t s);
 long fused_mix_backward_sum_rows(long B, int H, int L);
+// The same backward with the column sums finished inside the library: the per-chunk partial sums go through
+// a static device array instead of caller memory, and bias_da [H], bias_db / bias_dc [(H / kv_groups) * 16]
+// receive the sums over batch and time. Allocates nothing. `p.sum_*` are ignored.
+hipError_t fused_mix_backward_bias(const MixBwdArgs& p, float* bias_da, float* bias_db, float* bias_dc, hipStream_t s);
+long fused_mix_backward_bias_scratch_floats(long B, int H, int kv_groups, int L);
 
 // Streaming form (btp_jagged.hip). Tensors [B, H, D, L] / [B, H, L]; state vectors [B, H, D] / [B, H].
 struct JagPrefillArgs {

@@ -29,6 +29,7 @@ def test_header_declares_the_expected_entry_points():
         "spear_jagged_prefill",
         "spear_jagged_step",
         "spear_phalanx_mix_backward",
+        "spear_phalanx_mix_backward_bias",
         "spear_phalanx_mix_backward_ex",
         "spear_phalanx_mix_backward_sum_rows",
         "spear_phalanx_mix_forward",
@@ -66,7 +67,7 @@ def test_host_side_validation_needs_no_gpu():
     from spear_amd import _btp
 
     lib = _btp.load_library()
-    assert lib.spear_btp_abi_version() == 8
+    assert lib.spear_btp_abi_version() == _btp._ABI_VERSION
     buf = ctypes.create_string_buffer(4096)
     p = ctypes.addressof(buf)
     p -= p % 16

@@ -1,0 +1,113 @@
+"""spear_phalanx_mix_backward_bias -- the entry point that allocates nothing (its partial column sums pass
+through a device array the library holds statically) -- against spear_phalanx_mix_backward_ex, whose
+partial sums pass through arrays the caller allocates. Two calls in a row share the static array, the second
+on a smaller input; the gradients must be the same bits, and the finished sums must equal the caller-side
+sum of the other entry point's partial sums."""
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import f64
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+# fp32 sums of fp32 partial sums, compared with their float64 sum: |got - want| <= 1e-4 * sum|terms| + 1e-6
+SUM_RTOL, SUM_ATOL = 1e-4, 1e-6
+
+
+def _inputs(B, L, H, Hkv, seed):
+    g = torch.Generator().manual_seed(seed)
+    a = torch.randn(B, L, H, generator=g).bfloat16()
+    b = torch.randn(B, L, Hkv * 16, generator=g).bfloat16()
+    c = torch.randn(B, L, Hkv * 16, generator=g).bfloat16()
+    v = torch.randn(B, L, H * 16, generator=g).bfloat16()
+    dout = torch.randn(B, L, H * 16, generator=g).bfloat16()
+    return [t.to(DEV) for t in (a, b, c, v, dout)]
+
+
+def _with_caller_arrays(ins, H, Hkv):
+    from spear_amd import _btp
+
+    B, L, _ = ins[3].shape
+    grads = [torch.full(t.shape, float("nan"), device=DEV, dtype=t.dtype) for t in ins[:4]]
+    rows = _btp.mix_backward_sum_rows(B, L, H)
+    sums = tuple(torch.full((rows, w), float("nan"), device=DEV) for w in (H, Hkv * 16, Hkv * 16))
+    _btp.mix_backward(*ins, *grads, H, Hkv, sums=sums)
+    torch.cuda.synchronize()
+    return grads, sums
+
+
+def _without_allocation(ins, grads, bias, H, Hkv):
+    """The call itself: every buffer it touches exists before it, and the caching allocator must not move."""
+    from spear_amd import _btp
+
+    torch.cuda.synchronize()
+    before = torch.cuda.memory_stats(DEV)["allocation.all.allocated"]
+    _btp.mix_backward_bias(*ins, *grads, bias, H, Hkv)
+    torch.cuda.synchronize()
+    assert torch.cuda.memory_stats(DEV)["allocation.all.allocated"] == before
+
+
+@pytest.mark.parametrize("first,second", [
+    ((6, 256, 32, 32), (3, 64, 8, 4)),       # one chunk per row, then a smaller shape with shared kv heads
+    ((2, 4096, 8, 8), (1, 48, 4, 4)),        # rows cut into several chunks (several partial rows per batch row)
+])
+def test_two_calls_in_a_row_match_the_allocating_entry_point(first, second):
+    for call, (B, L, H, Hkv) in enumerate((first, second)):
+        print(f"no-alloc call {call}: B={B} L={L} H={H} Hkv={Hkv}", flush=True)
+        ins = _inputs(B, L, H, Hkv, seed=7000 + 13 * call + L)
+        want_grads, partial = _with_caller_arrays(ins, H, Hkv)
+        grads = [torch.full(t.shape, float("nan"), device=DEV, dtype=t.dtype) for t in ins[:4]]
+        bias = tuple(torch.full((w,), float("nan"), device=DEV) for w in (H, Hkv * 16, Hkv * 16))
+        _without_allocation(ins, grads, bias, H, Hkv)
+        for name, got, want in zip(("da", "db", "dc", "dv"), grads, want_grads):
+            assert torch.equal(got, want), name
+        for name, got, part in zip(("bias_da", "bias_db", "bias_dc"), bias, partial):
+            p = f64(part)
+            want, mass = p.sum(0), np.abs(p).sum(0)
+            err = np.abs(f64(got) - want)
+            assert np.isfinite(f64(got)).all(), name
+            assert (err <= SUM_RTOL * mass + SUM_ATOL).all(), (name, err.max(), mass.max())
+
+
+def test_strided_gradients_and_repeatability():
+    """Gradients written as column blocks of one buffer; a second call on the same input gives the same bits."""
+    from spear_amd import _btp
+
+    B, L, H, Hkv = 4, 128, 16, 4
+    ins = _inputs(B, L, H, Hkv, seed=7100)
+    want_grads, _ = _with_caller_arrays(ins, H, Hkv)
+    widths = (H, Hkv * 16, Hkv * 16, H * 16)
+    ld = sum(widths) + 16
+    packed = torch.full((B, L, ld), float("nan"), device=DEV, dtype=torch.bfloat16)
+    cols = np.cumsum((0,) + widths)
+    grads = [packed[:, :, cols[i]:cols[i + 1]] for i in range(4)]
+    runs = []
+    for _ in range(2):
+        bias = tuple(torch.full((w,), float("nan"), device=DEV) for w in widths[:3])
+        _without_allocation(ins, grads, bias, H, Hkv)
+        runs.append([t.clone() for t in bias])
+        for name, got, want in zip(("da", "db", "dc", "dv"), grads, want_grads):
+            assert torch.equal(got, want), name
+    assert torch.isnan(packed[:, :, cols[4]:]).all()  # the padding columns are not touched
+    for x, y in zip(*runs):
+        assert torch.equal(x, y)
+
+
+def test_shapes_beyond_the_static_array_are_refused():
+    from spear_amd import _btp
+
+    lib = _btp.load_library()
+    B, L, H = 2048, 128, 32  # 2048 partial rows x (32 + 2 * 512) floats > 2 Mi floats
+    assert _btp.mix_backward_sum_rows(B, L, H) * (H + 2 * H * 16) > 2097152
+    t = torch.zeros(64, device=DEV)
+    p = t.data_ptr()
+    rc = lib.spear_phalanx_mix_backward_bias(p, p, p, p, p, p, p, p, p, 0, 0, 0, 0, p, p, p, B, L, H, H, 0, 0, None)
+    assert rc == -1 and b"static array" in lib.spear_btp_last_error()
+    # the q/k/v/gate form has no bias gradients
+    rc = lib.spear_phalanx_mix_backward_bias(p, p, p, p, p, p, p, p, p, 0, 0, 0, 0, p, p, p, 1, 16, 4, 4, 0, 1, None)
+    assert rc == -1 and b"unknown flag" in lib.spear_btp_last_error()
+    rc = lib.spear_phalanx_mix_backward_bias(p, p, p, p, p, p, p, p, p, 0, 0, 0, 0, None, p, p, 1, 16, 4, 4, 0, 0, None)
+    assert rc == -2
