@@ -50,6 +50,9 @@ extern "C" {
 #define SPEAR_BTP_PATH_MFMA 0x2u        /* forward: use the MFMA tile kernel (decay matrix rounded */
                                         /* to the input dtype) instead of the exact-fp32 recurrence */
 
+#define SPEAR_BTP_DX_F32 0x10u          /* backward: check mode, `dx` is fp32 [B, H, 16, L] and receives the    */
+                                        /* kernel's fp32 values instead of their rounding to in_dtype           */
+
 /* error codes */
 #define SPEAR_BTP_EINVAL (-1)  /* bad shape, dtype, k, flag or alignment                       */
 #define SPEAR_BTP_ENULL (-2)   /* a required pointer is NULL                                   */
@@ -63,7 +66,9 @@ int spear_btp_forward(const void* coeff, const void* x, void* y, float* checkpoi
 
 /* Replaces spear._btp.backward -> sss::launch_btp_backward (csrc/btp/_bindings.cu:152-229,
  * csrc/btp/btp-backwards.cu:811-884).  `checkpoint` is accepted for signature compatibility and
- * never read: the carries are recomputed from `coeff` and `x`. */
+ * never read: the carries are recomputed from `coeff` and `x`. The reference fixes dx.dtype == x.dtype
+ * (_bindings.cu:52-54), which stays the default; SPEAR_BTP_DX_F32 is the fp32 check mode (arithmetic is fp32
+ * either way, the flag only drops the final rounding so that dx can be compared at fp32 tolerances). */
 int spear_btp_backward(const void* coeff, const void* x, const void* dy, const float* checkpoint,
                        void* dx, float* dA, int B, int H, int L, int k, int in_dtype, int dy_dtype,
                        unsigned flags, void* stream);
@@ -105,6 +110,12 @@ int spear_phalanx_mix_forward(const void* a_logit, const void* b_logit, const vo
  * This is the composition written out at spear/nn/phalanx/swr.py:196-221, 311-327 with the two sigmoids
  * left to the caller; the reference has no single function for it. */
 #define SPEAR_MIX_QKV_GATE 0x1u
+
+/* Flag for the same three entry points: fp32 check mode. The kernels compute in fp32 either way; with this
+ * flag the results are stored as fp32 instead of being rounded to `dtype`, so that they can be held to fp32
+ * tolerances: forward `out`; backward `da_logit`, `db_logit`, `dc`, `dv` (row strides then count fp32
+ * elements). Inputs keep their types. Not combinable with the column sums of _backward_ex. */
+#define SPEAR_MIX_F32_RESULTS 0x2u
 
 /* Backward of spear_phalanx_mix_forward: reads a_logit, b_logit, c, v and the upstream gradient
  * dout [B, L, H * 16]; writes da_logit [B, L, H], db_logit and dc [B, L, kv_heads * 16] (summed over

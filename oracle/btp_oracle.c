@@ -2,8 +2,8 @@
  * btp_oracle.c -- CPU restatement (fp64, plain C) of SPEAR's Block Two-Pass (BTP) operator.
  *
  * THIS FILE IS TEST INFRASTRUCTURE. It is the checker the HIP kernels are compared against.
- * Nothing in the shipped package may import, link or call it; only tests/, the smoke check and
- * the cpu_baseline leg of bench.py do.
+ * Nothing in the shipped package may import, link or call it; only tests/ and the smoke check do
+ * (the CPU baseline timed by bench.py is the package's own PyTorch restatement, not this file).
  *
  * What it restates (paths relative to the reference repository):
  *   - spear/ops/btp/reference.py:55-77   construct_L_ref              -> build_L(mode 0)

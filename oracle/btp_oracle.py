@@ -1,7 +1,8 @@
 """numpy front-end of the C oracle (oracle/btp_oracle.c) plus bf16 helpers.
 
-TEST INFRASTRUCTURE ONLY: imported by tests/, by ``__graft_entry__.smoke`` and by the
-``cpu_baseline`` leg of ``bench.py``; the shipped package never imports it.
+TEST INFRASTRUCTURE ONLY: imported by tests/ and by ``__graft_entry__.smoke``; the shipped package and
+``bench.py`` never import it (the CPU baseline that ``bench.py`` times is the package's own PyTorch
+restatement, ``spear_amd.ops.btp.reference``).
 
 The protocol mirrors the reference's gold-standard runner (spear/ops/btp/runners.py:111-116):
 inputs are first rounded to the kernel's storage dtype (bf16), then promoted to float64, and the

@@ -18,7 +18,7 @@ import threading
 
 import torch
 
-__all__ = ["forward", "backward", "forward_log", "backward_log", "mix_forward", "mix_backward", "jagged_prefill", "jagged_step", "library_path", "load_library", "FLAG_WRITE_CHECKPOINT", "FLAG_PATH_MFMA", "FLAG_JAGGED_LOG_A", "FLAG_JAGGED_LOG_R", "FLAG_MIX_QKV_GATE", "mix_backward_sum_rows", "mix_backward_bias"]
+__all__ = ["forward", "backward", "forward_log", "backward_log", "mix_forward", "mix_backward", "jagged_prefill", "jagged_step", "library_path", "load_library", "FLAG_WRITE_CHECKPOINT", "FLAG_PATH_MFMA", "FLAG_JAGGED_LOG_A", "FLAG_JAGGED_LOG_R", "FLAG_MIX_QKV_GATE", "FLAG_MIX_F32_RESULTS", "FLAG_DX_F32", "mix_backward_sum_rows", "mix_backward_bias"]
 
 _BF16, _F16, _F32 = 0, 1, 2
 FLAG_WRITE_CHECKPOINT = 0x1
@@ -26,7 +26,9 @@ FLAG_PATH_MFMA = 0x2
 FLAG_JAGGED_LOG_A = 0x4
 FLAG_JAGGED_LOG_R = 0x8
 FLAG_MIX_QKV_GATE = 0x1
-_ABI_VERSION = 9
+FLAG_MIX_F32_RESULTS = 0x2
+FLAG_DX_F32 = 0x10
+_ABI_VERSION = 10
 _SUPPORTED_WPB = (4, 8, 16, 32)
 
 _lock = threading.Lock()
@@ -175,7 +177,8 @@ def forward(
     _check_layout("coeff", coeff, (B, H, L))
     _check_layout("x", x, (B, H, 16, L))
     _check_layout("y", y, (B, H, 16, L))
-    _check_layout("checkpoint", checkpoint, (B, H, L // 16, 16))
+    if flags & FLAG_WRITE_CHECKPOINT or checkpoint.numel() != 0:  # a zero-element placeholder when it is not stored
+        _check_layout("checkpoint", checkpoint, (B, H, L // 16, 16))
     _check(coeff.device == x.device == y.device == checkpoint.device, "All tensors must be on the same device.")
 
     lib = load_library()
@@ -202,7 +205,8 @@ def backward(
     """``dx, dA <- vjp of btp at (coeff, x) applied to dy``, in place (csrc/btp/_bindings.cu:152-229).
 
     Every element of ``dA`` is written, so it need not arrive zero-filled. ``checkpoint`` is
-    accepted for signature compatibility and not read.
+    accepted for signature compatibility and not read. ``flags`` is an extension: with ``FLAG_DX_F32``
+    ``dx`` is a float32 tensor and receives the kernel's fp32 values unrounded (fp32 check mode).
     """
     _check(
         coeff.is_cuda and x.is_cuda and dy.is_cuda and checkpoint.is_cuda,
@@ -210,7 +214,10 @@ def backward(
     )
     _check(dx.is_cuda and dA.is_cuda, "dx and dA must be CUDA.")
     _check_common(x, coeff, k, wpb, "Unsupported WPB value for backward: ")
-    _check(dx.dtype == x.dtype, "dx dtype must match x.")
+    if flags & FLAG_DX_F32:
+        _check(dx.dtype == torch.float32, "dx must be float32 in the fp32 check mode.")
+    else:
+        _check(dx.dtype == x.dtype, "dx dtype must match x.")
     _check(dA.dtype == torch.float32, "dA must be float32.")
     _check(dy.dtype == torch.float32 or dy.dtype == x.dtype, "dy must be float32 or match x dtype.")
     B, H, _, L = x.shape
@@ -267,10 +274,11 @@ def forward_log(gate: torch.Tensor, x: torch.Tensor, y: torch.Tensor, k: int) ->
 def backward_log(
     gate: torch.Tensor, x: torch.Tensor, dy: torch.Tensor, dx: torch.Tensor, dgate: torch.Tensor, k: int
 ) -> None:
-    """``dx, dgate <- vjp of btp(exp(gate), x)``; ``dgate`` is the gradient w.r.t. the log-space gate."""
+    """``dx, dgate <- vjp of btp(exp(gate), x)``; ``dgate`` is the gradient w.r.t. the log-space gate.
+    A float32 ``dx`` selects the fp32 check mode (``SPEAR_BTP_DX_F32``)."""
     B, H, L = _check_log_common(gate, x, k)
     _check(dy.is_cuda and dx.is_cuda and dgate.is_cuda, "All tensors must be CUDA.")
-    _check(dx.dtype == x.dtype, "dx dtype must match x.")
+    _check(dx.dtype in (x.dtype, torch.float32), "dx must be float32 or match x dtype.")
     _check(dgate.dtype == torch.float32, "dgate must be float32.")
     _check(dy.dtype == torch.float32 or dy.dtype == x.dtype, "dy must be float32 or match x dtype.")
     _check_layout("dy", dy, (B, H, 16, L))
@@ -281,7 +289,7 @@ def backward_log(
     with torch.cuda.device(x.device):
         rc = lib.spear_btp_backward_loggate(
             gate.data_ptr(), x.data_ptr(), dy.data_ptr(), dx.data_ptr(), dgate.data_ptr(), B, H, L, int(k),
-            _tag(x.dtype), _tag(dy.dtype), 0, _stream_ptr(x.device),
+            _tag(x.dtype), _tag(dy.dtype), FLAG_DX_F32 if dx.dtype == torch.float32 else 0, _stream_ptr(x.device),
         )
     if rc != 0:
         _raise_native(lib, rc)
@@ -308,7 +316,9 @@ def mix_forward(
     _check(heads % 4 == 0, "heads must be a multiple of 4.")
     _check(kv_heads > 0 and heads % kv_heads == 0, "heads must be divisible by kv_heads.")
     _check(v.dtype in (torch.float16, torch.bfloat16), "tensors must be float16 or bfloat16.")
-    _check(b_logit.dtype == c.dtype == out.dtype == v.dtype, "all tensors must share one dtype.")
+    _check(b_logit.dtype == c.dtype == v.dtype, "all tensors must share one dtype.")
+    _check(out.dtype in (v.dtype, torch.float32), "out must be float32 (fp32 check mode) or match v dtype.")
+    f32 = out.dtype == torch.float32
     if qkv_gate:
         _check(a_logit.dtype == torch.float32, "the log-decay gate must be float32.")
     else:
@@ -324,7 +334,8 @@ def mix_forward(
     with torch.cuda.device(v.device):
         rc = lib.spear_phalanx_mix_forward(
             a_logit.data_ptr(), b_logit.data_ptr(), c.data_ptr(), v.data_ptr(), out.data_ptr(),
-            B, L, heads, kv_heads, _tag(v.dtype), FLAG_MIX_QKV_GATE if qkv_gate else 0, _stream_ptr(v.device),
+            B, L, heads, kv_heads, _tag(v.dtype),
+            (FLAG_MIX_QKV_GATE if qkv_gate else 0) | (FLAG_MIX_F32_RESULTS if f32 else 0), _stream_ptr(v.device),
         )
     if rc != 0:
         _raise_native(lib, rc)
@@ -355,7 +366,8 @@ def mix_backward(
     ``[mix_backward_sum_rows(B, L, heads), heads | kv_heads*16 | kv_heads*16]`` that receive the per-chunk
     column sums of ``da_logit``, ``db_logit`` and ``dc``. The four gradient tensors may be column blocks of one
     wider ``[B, L, ld]`` buffer (``spear_phalanx_mix_backward_ex``). ``qkv_gate`` as in :func:`mix_forward`;
-    ``da_logit`` is then the fp32 gradient of the gate."""
+    ``da_logit`` is then the fp32 gradient of the gate. Float32 ``db_logit, dc, dv`` (and ``da_logit``) select
+    the fp32 check mode (``SPEAR_MIX_F32_RESULTS``)."""
     tensors = (a_logit, b_logit, c, v, dout, da_logit, db_logit, dc, dv)
     _check(all(t.is_cuda for t in tensors), "All tensors must be CUDA.")
     _check(v.dim() == 3, "v must be [B, L, heads * 16].")
@@ -365,10 +377,15 @@ def mix_backward(
     _check(kv_heads > 0 and heads % kv_heads == 0, "heads must be divisible by kv_heads.")
     _check(heads // kv_heads in (1, 2, 4, 8), "heads / kv_heads must be 1, 2, 4 or 8.")
     _check(v.dtype in (torch.float16, torch.bfloat16), "tensors must be float16 or bfloat16.")
-    gate_like = (a_logit, da_logit)
-    _check(all(t.dtype == v.dtype for t in tensors if all(t is not g for g in gate_like)), "all tensors must share one dtype.")
-    _check(all(t.dtype == (torch.float32 if qkv_gate else v.dtype) for t in gate_like),
-           "the log-decay gate and its gradient must be float32." if qkv_gate else "all tensors must share one dtype.")
+    f32 = dv.dtype == torch.float32  # fp32 check mode: the four gradients are stored unrounded
+    _check(all(t.dtype == v.dtype for t in (b_logit, c, dout)), "all tensors must share one dtype.")
+    _check(all(t.dtype == dv.dtype for t in (db_logit, dc)) and dv.dtype in (v.dtype, torch.float32),
+           "db_logit, dc and dv must all be float32 (fp32 check mode) or all match v dtype.")
+    _check(a_logit.dtype == (torch.float32 if qkv_gate else v.dtype),
+           "the log-decay gate must be float32." if qkv_gate else "all tensors must share one dtype.")
+    _check(da_logit.dtype == (torch.float32 if (qkv_gate or f32) else v.dtype),
+           "the gradient of the gate must be float32." if (qkv_gate or f32) else "all tensors must share one dtype.")
+    _check(sums is None or not f32, "column sums are not available in the fp32 check mode.")
     _check(sums is None or not qkv_gate, "column sums belong to the layer form, not to qkv_gate.")
     _check(L % 16 == 0, "Length L must be multiple of 16")
     Fkv = kv_heads * 16
@@ -393,7 +410,8 @@ def mix_backward(
             a_logit.data_ptr(), b_logit.data_ptr(), c.data_ptr(), v.data_ptr(), dout.data_ptr(),
             da_logit.data_ptr(), db_logit.data_ptr(), dc.data_ptr(), dv.data_ptr(), *lds,
             *sum_ptrs, rows,
-            B, L, heads, kv_heads, _tag(v.dtype), FLAG_MIX_QKV_GATE if qkv_gate else 0, _stream_ptr(v.device),
+            B, L, heads, kv_heads, _tag(v.dtype),
+            (FLAG_MIX_QKV_GATE if qkv_gate else 0) | (FLAG_MIX_F32_RESULTS if f32 else 0), _stream_ptr(v.device),
         )
     if rc != 0:
         _raise_native(lib, rc)

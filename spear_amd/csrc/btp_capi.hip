@@ -44,7 +44,7 @@ int check_common(const char* who, int B, int H, int L, int k, int in_dtype, int 
 
 extern "C" {
 
-int spear_btp_abi_version(void) { return 9; }
+int spear_btp_abi_version(void) { return 10; }
 
 const char* spear_btp_last_error(void) { return g_error; }
 
@@ -75,7 +75,8 @@ int spear_btp_backward(const void* coeff, const void* x, const void* dy, const f
                        int B, int H, int L, int k, int in_dtype, int dy_dtype, unsigned flags, void* stream) {
   (void)checkpoint;  // carries are recomputed from coeff and x
   g_error[0] = '\0';
-  if (int rc = check_common("spear_btp_backward", B, H, L, k, in_dtype, dy_dtype, "dy", flags, SPEAR_BTP_PATH_MFMA))
+  if (int rc = check_common("spear_btp_backward", B, H, L, k, in_dtype, dy_dtype, "dy", flags,
+                            SPEAR_BTP_PATH_MFMA | SPEAR_BTP_DX_F32))
     return rc;
   if ((long long)B * H == 0 || L == 0) return 0;
   if (!coeff || !x || !dy || !dx || !dA) return fail(SPEAR_BTP_ENULL, "spear_btp_backward: NULL tensor pointer");
@@ -84,7 +85,7 @@ int spear_btp_backward(const void* coeff, const void* x, const void* dy, const f
   if (flags & SPEAR_BTP_PATH_MFMA)
     return fail(SPEAR_BTP_EINVAL, "spear_btp_backward: there is no MFMA variant of the backward kernel");
 
-  spear_btp::BwdArgs a{coeff, x, dy, dx, dA, B, H, L, k, in_dtype, dy_dtype};
+  spear_btp::BwdArgs a{coeff, x, dy, dx, dA, B, H, L, k, in_dtype, dy_dtype, false, (flags & SPEAR_BTP_DX_F32) != 0};
   const hipError_t err = spear_btp::scan_backward(a, static_cast<hipStream_t>(stream));
   if (err != hipSuccess) return fail(SPEAR_BTP_ELAUNCH, "spear_btp_backward: launch failed: %s", hipGetErrorString(err));
   return 0;
@@ -112,13 +113,14 @@ int spear_btp_forward_loggate(const float* gate, const void* x, void* y, float* 
 int spear_btp_backward_loggate(const float* gate, const void* x, const void* dy, void* dx, float* dgate, int B, int H,
                                int L, int k, int x_dtype, int dy_dtype, unsigned flags, void* stream) {
   g_error[0] = '\0';
-  if (int rc = check_common("spear_btp_backward_loggate", B, H, L, k, x_dtype, dy_dtype, "dy", flags, 0u)) return rc;
+  if (int rc = check_common("spear_btp_backward_loggate", B, H, L, k, x_dtype, dy_dtype, "dy", flags, SPEAR_BTP_DX_F32))
+    return rc;
   if ((long long)B * H == 0 || L == 0) return 0;
   if (!gate || !x || !dy || !dx || !dgate)
     return fail(SPEAR_BTP_ENULL, "spear_btp_backward_loggate: NULL tensor pointer");
   if (!aligned16(gate) || !aligned16(x) || !aligned16(dy) || !aligned16(dx) || !aligned16(dgate))
     return fail(SPEAR_BTP_EINVAL, "spear_btp_backward_loggate: tensor pointers must be 16-byte aligned");
-  spear_btp::BwdArgs a{gate, x, dy, dx, dgate, B, H, L, k, x_dtype, dy_dtype, true};
+  spear_btp::BwdArgs a{gate, x, dy, dx, dgate, B, H, L, k, x_dtype, dy_dtype, true, (flags & SPEAR_BTP_DX_F32) != 0};
   const hipError_t err = spear_btp::scan_backward(a, static_cast<hipStream_t>(stream));
   if (err != hipSuccess)
     return fail(SPEAR_BTP_ELAUNCH, "spear_btp_backward_loggate: launch failed: %s", hipGetErrorString(err));
@@ -136,15 +138,17 @@ int spear_phalanx_mix_forward(const void* a_logit, const void* b_logit, const vo
     return fail(SPEAR_BTP_EINVAL, "%s: heads (%d) must be divisible by kv_heads (%d)", who, H, kv_heads);
   if (dtype != SPEAR_BTP_BF16 && dtype != SPEAR_BTP_F16)
     return fail(SPEAR_BTP_EINVAL, "%s: tensors must be float16 or bfloat16.", who);
-  if (flags & ~SPEAR_MIX_QKV_GATE) return fail(SPEAR_BTP_EINVAL, "%s: unknown flag bits 0x%x", who, flags);
+  const unsigned known = SPEAR_MIX_QKV_GATE | SPEAR_MIX_F32_RESULTS;
+  if (flags & ~known) return fail(SPEAR_BTP_EINVAL, "%s: unknown flag bits 0x%x", who, flags & ~known);
+  const bool f32 = (flags & SPEAR_MIX_F32_RESULTS) != 0;
   if ((long long)B * L * H * 16ll >= (1ll << 40)) return fail(SPEAR_BTP_EINVAL, "%s: tensor too large", who);
-  if ((long long)L * H * 32ll >= (1ll << 31))  // a batch row is addressed through one 32-bit buffer resource
+  if ((long long)L * H * (f32 ? 64ll : 32ll) >= (1ll << 31))  // a batch row is addressed through one 32-bit buffer resource
     return fail(SPEAR_BTP_EINVAL, "%s: one batch row (L * H * 16 elements) must stay below 2 GiB", who);
   if ((long long)B * H == 0 || L == 0) return 0;
   if (!a_logit || !b_logit || !c || !v || !out) return fail(SPEAR_BTP_ENULL, "%s: NULL tensor pointer", who);
   if (!aligned16(a_logit) || !aligned16(b_logit) || !aligned16(c) || !aligned16(v) || !aligned16(out))
     return fail(SPEAR_BTP_EINVAL, "%s: tensor pointers must be 16-byte aligned", who);
-  spear_btp::MixArgs a{a_logit, b_logit, c, v, out, B, L, H, H / kv_heads, dtype, (flags & SPEAR_MIX_QKV_GATE) != 0};
+  spear_btp::MixArgs a{a_logit, b_logit, c, v, out, B, L, H, H / kv_heads, dtype, (flags & SPEAR_MIX_QKV_GATE) != 0, f32};
   const hipError_t err = spear_btp::fused_mix_forward(a, static_cast<hipStream_t>(stream));
   if (err != hipSuccess) return fail(SPEAR_BTP_ELAUNCH, "%s: launch failed: %s", who, hipGetErrorString(err));
   return 0;
@@ -178,9 +182,9 @@ static int check_mix_backward(const char* who, const void* const (&ptrs)[9], con
   if (dtype != SPEAR_BTP_BF16 && dtype != SPEAR_BTP_F16)
     return fail(SPEAR_BTP_EINVAL, "%s: tensors must be float16 or bfloat16.", who);
   if (flags & ~allowed_flags) return fail(SPEAR_BTP_EINVAL, "%s: unknown flag bits 0x%x", who, flags & ~allowed_flags);
-  const bool qkv = (flags & SPEAR_MIX_QKV_GATE) != 0;
+  const bool qkv = (flags & SPEAR_MIX_QKV_GATE) != 0, f32 = (flags & SPEAR_MIX_F32_RESULTS) != 0;
   if ((long long)B * L * H * 16ll >= (1ll << 40)) return fail(SPEAR_BTP_EINVAL, "%s: tensor too large", who);
-  if ((long long)L * H * 32ll >= (1ll << 31))  // a batch row is addressed through one 32-bit buffer resource
+  if ((long long)L * H * (f32 ? 64ll : 32ll) >= (1ll << 31))  // a batch row is addressed through one 32-bit buffer resource
     return fail(SPEAR_BTP_EINVAL, "%s: one batch row (L * H * 16 elements) must stay below 2 GiB", who);
   if ((long long)B * H == 0 || L == 0) return 1;
   for (const void* q : ptrs) {
@@ -192,7 +196,7 @@ static int check_mix_backward(const char* who, const void* const (&ptrs)[9], con
     if (lds[i] == 0) continue;
     if (lds[i] < widths[i] || lds[i] % 2 != 0)
       return fail(SPEAR_BTP_EINVAL, "%s: a gradient's row stride must be 0 (dense) or an even number of elements not below its width (got %d for width %d)", who, lds[i], widths[i]);
-    if ((long long)L * lds[i] * (i == 0 && qkv ? 4ll : 2ll) >= (1ll << 31))
+    if ((long long)L * lds[i] * ((i == 0 && qkv) || f32 ? 4ll : 2ll) >= (1ll << 31))
       return fail(SPEAR_BTP_EINVAL, "%s: one batch row (L * row stride) must stay below 2 GiB", who);
   }
   return 0;
@@ -207,10 +211,12 @@ int spear_phalanx_mix_backward_ex(const void* a_logit, const void* b_logit, cons
   const char* who = "spear_phalanx_mix_backward";
   const void* const ptrs[9] = {a_logit, b_logit, c, v, dout, da_logit, db_logit, dc, dv};
   const int lds[4] = {ld_da, ld_db, ld_dc, ld_dv};
-  if (int rc = check_mix_backward(who, ptrs, lds, B, L, H, kv_heads, dtype, flags, SPEAR_MIX_QKV_GATE)) return rc < 0 ? rc : 0;
-  const bool qkv = (flags & SPEAR_MIX_QKV_GATE) != 0;
+  if (int rc = check_mix_backward(who, ptrs, lds, B, L, H, kv_heads, dtype, flags, SPEAR_MIX_QKV_GATE | SPEAR_MIX_F32_RESULTS))
+    return rc < 0 ? rc : 0;
+  const bool qkv = (flags & SPEAR_MIX_QKV_GATE) != 0, f32 = (flags & SPEAR_MIX_F32_RESULTS) != 0;
   const bool sums = sum_da || sum_db || sum_dc;
   if (sums && qkv) return fail(SPEAR_BTP_EINVAL, "%s: column sums are for the layer form, not SPEAR_MIX_QKV_GATE", who);
+  if (sums && f32) return fail(SPEAR_BTP_EINVAL, "%s: column sums are not available with SPEAR_MIX_F32_RESULTS", who);
   if (sums) {
     if (!sum_da || !sum_db || !sum_dc) return fail(SPEAR_BTP_ENULL, "%s: the three sum arrays must be given together", who);
     if (!aligned16(sum_da) || !aligned16(sum_db) || !aligned16(sum_dc))
@@ -220,7 +226,7 @@ int spear_phalanx_mix_backward_ex(const void* a_logit, const void* b_logit, cons
       return fail(SPEAR_BTP_EINVAL, "%s: sum arrays must have %lld rows for this shape (got %lld)", who, want, sum_rows);
   }
   spear_btp::MixBwdArgs a{a_logit, b_logit, c, v, dout, da_logit, db_logit, dc, dv, B, L, H, H / kv_heads, dtype,
-                          sum_da, sum_db, sum_dc, ld_da, ld_db, ld_dc, ld_dv, qkv};
+                          sum_da, sum_db, sum_dc, ld_da, ld_db, ld_dc, ld_dv, qkv, f32};
   const hipError_t err = spear_btp::fused_mix_backward(a, static_cast<hipStream_t>(stream));
   if (err != hipSuccess) return fail(SPEAR_BTP_ELAUNCH, "%s: launch failed: %s", who, hipGetErrorString(err));
   return 0;

@@ -87,7 +87,10 @@ __device__ __forceinline__ float input_gate(float b) {
 constexpr int kHeadsPerWave = 8;
 constexpr int kGateRow = 20;  // floats per head in the decay tile: 16 steps + 4 of padding (bank spread)
 
-template <class E, int kFwdWaves, bool kQkv>
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+
+// kF32: check mode, the result leaves as fp32 (the kernel's own values, not rounded to 16 bits).
+template <class E, int kFwdWaves, bool kQkv, bool kF32>
 __global__ __launch_bounds__(64 * kFwdWaves) void phalanx_mix_fwd_kernel(
     const uint16_t* __restrict__ a_logit, const uint16_t* __restrict__ b_logit, const uint16_t* __restrict__ c_in,
     const uint16_t* __restrict__ v_in, uint16_t* __restrict__ out, int L, int H, int kv_groups, int chunk_steps,
@@ -121,7 +124,9 @@ __global__ __launch_bounds__(64 * kFwdWaves) void phalanx_mix_fwd_kernel(
   constexpr int kRsrcFlags = 0x00020000;            // raw 32-bit buffer, gfx9 encoding
   const __amdgpu_buffer_rsrc_t rv =
       __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(v_in + brow * L * F), 0, L * v_stride, kRsrcFlags);
-  const __amdgpu_buffer_rsrc_t ro = __builtin_amdgcn_make_buffer_rsrc(out + brow * L * F, 0, L * v_stride, kRsrcFlags);
+  constexpr int kOutScale = kF32 ? 2 : 1;  // bytes of an output element over bytes of an input element
+  const __amdgpu_buffer_rsrc_t ro =
+      __builtin_amdgcn_make_buffer_rsrc(out + brow * L * F * kOutScale, 0, L * v_stride * kOutScale, kRsrcFlags);
   const __amdgpu_buffer_rsrc_t rb =
       __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(b_logit + brow * L * Fkv), 0, L * kv_stride, kRsrcFlags);
   const __amdgpu_buffer_rsrc_t rc =
@@ -132,7 +137,7 @@ __global__ __launch_bounds__(64 * kFwdWaves) void phalanx_mix_fwd_kernel(
       kRsrcFlags);
   const int v_lane = 2 * (head * kChan + d0), kv_lane = 2 * ((head / kv_groups) * kChan + d0);
   // A lane without a head stores at an offset beyond the resource, which the buffer unit drops.
-  const int o_lane = real ? v_lane : 0x7ffffff0;
+  const int o_lane = real ? v_lane * kOutScale : 0x7ffffff0;
   // gate logits: lane (hg, t) = (lane / 16, lane % 16) converts heads ho + 2 hg, + 1 of step t
   const int gt = lane & 15, ghead = min(ho + 2 * (lane >> 4), H - 2);
   const int a_lane = kGateBytes * (gt * H + ghead);
@@ -210,9 +215,13 @@ __global__ __launch_bounds__(64 * kFwdWaves) void phalanx_mix_fwd_kernel(
     for (int r = 0; r < 16; ++r) {
       y0 = fmaf(a[r], y0, x0[r]);
       y1 = fmaf(a[r], y1, x1[r]);
-      const uint32_t ow =
-          E::pack2(fmaf(y0, E::lo(wd.c[r]), E::lo(wd.v[r])), fmaf(y1, E::hi(wd.c[r]), E::hi(wd.v[r])));
-      __builtin_amdgcn_raw_buffer_store_b32(ow, ro, o_off, (t0 + r) * v_stride, kNtS);
+      const float o0 = fmaf(y0, E::lo(wd.c[r]), E::lo(wd.v[r])), o1 = fmaf(y1, E::hi(wd.c[r]), E::hi(wd.v[r]));
+      if constexpr (kF32) {
+        const u32x2_t ow = {__float_as_uint(o0), __float_as_uint(o1)};
+        __builtin_amdgcn_raw_buffer_store_b64(ow, ro, o_off, (t0 + r) * v_stride * 2, kNtS);
+      } else {
+        __builtin_amdgcn_raw_buffer_store_b32(E::pack2(o0, o1), ro, o_off, (t0 + r) * v_stride, kNtS);
+      }
     }
     carry0 = l0;
     carry1 = l1;
@@ -277,7 +286,8 @@ struct MixSet {
 // and dc in fp32 (before their rounding to 16 bits) -- the bias gradients of the projections that produced
 // a_logit, b_logit and c, up to a sum over those few rows. A lane keeps its features for the whole walk, so
 // this is five accumulators per lane and one store at the end.
-template <class E, bool kSums, bool kQkv>
+// kF32: check mode, the four gradients leave as fp32 (the kernel's own values, not rounded to 16 bits).
+template <class E, bool kSums, bool kQkv, bool kF32>
 __global__ __launch_bounds__(64 * kWaves) void phalanx_mix_bwd_kernel(
     const uint16_t* __restrict__ a_logit, const uint16_t* __restrict__ b_logit, const uint16_t* __restrict__ c_in,
     const uint16_t* __restrict__ v_in, const uint16_t* __restrict__ dout, uint16_t* __restrict__ da_logit,
@@ -304,7 +314,9 @@ __global__ __launch_bounds__(64 * kWaves) void phalanx_mix_bwd_kernel(
   const int F = H * kChan, Fkv = (H / kv_groups) * kChan;
   const int stride = 2 * F, kv_stride = 2 * Fkv;  // bytes per time step of the [B, L, F] / [B, L, Fkv] tensors
   constexpr int kRsrcFlags = 0x00020000;          // raw 32-bit buffer, gfx9 encoding
-  constexpr int kGateBytes = kQkv ? 4 : 2;        // element size of the a operand and of its gradient
+  constexpr int kGateBytes = kQkv ? 4 : 2;        // element size of the a operand
+  constexpr int kDaBytes = (kQkv || kF32) ? 4 : 2;  // element size of its gradient
+  constexpr int kGradBytes = kF32 ? 4 : 2;          // element size of db, dc, dv
   const long big = brow * L * F, kvbig = brow * L * Fkv, small = brow * L * H;
   auto rsrc = [&](const uint16_t* p, long off, int bytes) {
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(p + off), 0, bytes, kRsrcFlags);
@@ -314,20 +326,20 @@ __global__ __launch_bounds__(64 * kWaves) void phalanx_mix_bwd_kernel(
                                ra = rsrc(a_logit, small * (kGateBytes / 2), L * H * kGateBytes),
                                // the four gradients may sit side by side in one wider buffer: each has its
                                // own elements-per-time-step (ld_*), equal to its width when it is dense
-                               rdb = rsrc(db_logit, brow * L * ld_db, L * ld_db * 2),
-                               rdc = rsrc(dc, brow * L * ld_dc, L * ld_dc * 2),
-                               rdv = rsrc(dv, brow * L * ld_dv, L * ld_dv * 2),
-                               rda = rsrc(da_logit, brow * L * ld_da * (kGateBytes / 2), L * ld_da * kGateBytes);
+                               rdb = rsrc(db_logit, brow * L * ld_db * (kGradBytes / 2), L * ld_db * kGradBytes),
+                               rdc = rsrc(dc, brow * L * ld_dc * (kGradBytes / 2), L * ld_dc * kGradBytes),
+                               rdv = rsrc(dv, brow * L * ld_dv * (kGradBytes / 2), L * ld_dv * kGradBytes),
+                               rda = rsrc(da_logit, brow * L * ld_da * (kDaBytes / 2), L * ld_da * kDaBytes);
   const int f_lane = 2 * (head * kChan + d0);
   const int kv_lane = 2 * ((head / kv_groups) * kChan + d0);
-  const int o_lane = real ? f_lane : 0x7ffffff0;  // lanes without a head store nowhere
+  const int o_lane = real ? f_lane * (kGradBytes / 2) : 0x7ffffff0;  // lanes without a head store nowhere
   // With shared kv heads (kv_groups = 2, 4 or 8 consecutive heads, all inside this wavefront) the
   // gradients of b and c are summed over the group's lanes and stored by its first head only.
-  const int okv_lane = (real && (head % kv_groups) == 0) ? kv_lane : 0x7ffffff0;
+  const int okv_lane = (real && (head % kv_groups) == 0) ? kv_lane * (kGradBytes / 2) : 0x7ffffff0;
   const int gt = lane & 15, ghead = min(ho + 2 * (lane >> 4), H - 2);
   const int a_lane = kGateBytes * (gt * H + ghead);
   // da_logit: lane k of a head (k = lane % 8) ends up with steps 2k and 2k+1 of that head
-  const int da_lane = real ? kGateBytes * ((2 * (lane & 7)) * ld_da + head) : 0x7ffffff0;
+  const int da_lane = real ? kDaBytes * ((2 * (lane & 7)) * ld_da + head) : 0x7ffffff0;
   constexpr int kNt = 2;
 
   auto issue = [&](MixSet& m, int t) {
@@ -452,14 +464,20 @@ __global__ __launch_bounds__(64 * kWaves) void phalanx_mix_bwd_kernel(
       if constexpr (kSums) {
         acc_b0 += db0; acc_b1 += db1; acc_c0 += dc0; acc_c1 += dc1;
       }
-      const uint32_t wdc = E::pack2(dc0, dc1);
-      const uint32_t wdv = E::pack2(fmaf(pk.z, G0, go0), fmaf(pk.w, G1, go1));
-      const uint32_t wdb = E::pack2(db0, db1);
+      const float dv0 = fmaf(pk.z, G0, go0), dv1 = fmaf(pk.w, G1, go1);
       z0 = az0;
       z1 = az1;
-      __builtin_amdgcn_raw_buffer_store_b32(wdc, rdc, okv_off, (t0 + r) * 2 * ld_dc, kNt);
-      __builtin_amdgcn_raw_buffer_store_b32(wdv, rdv, o_off, (t0 + r) * 2 * ld_dv, kNt);
-      __builtin_amdgcn_raw_buffer_store_b32(wdb, rdb, okv_off, (t0 + r) * 2 * ld_db, kNt);
+      if constexpr (kF32) {
+        const u32x2_t wdc = {__float_as_uint(dc0), __float_as_uint(dc1)}, wdv = {__float_as_uint(dv0), __float_as_uint(dv1)},
+                      wdb = {__float_as_uint(db0), __float_as_uint(db1)};
+        __builtin_amdgcn_raw_buffer_store_b64(wdc, rdc, okv_off, (t0 + r) * 4 * ld_dc, kNt);
+        __builtin_amdgcn_raw_buffer_store_b64(wdv, rdv, o_off, (t0 + r) * 4 * ld_dv, kNt);
+        __builtin_amdgcn_raw_buffer_store_b64(wdb, rdb, okv_off, (t0 + r) * 4 * ld_db, kNt);
+      } else {
+        __builtin_amdgcn_raw_buffer_store_b32(E::pack2(dc0, dc1), rdc, okv_off, (t0 + r) * 2 * ld_dc, kNt);
+        __builtin_amdgcn_raw_buffer_store_b32(E::pack2(dv0, dv1), rdv, o_off, (t0 + r) * 2 * ld_dv, kNt);
+        __builtin_amdgcn_raw_buffer_store_b32(E::pack2(db0, db1), rdb, okv_off, (t0 + r) * 2 * ld_db, kNt);
+      }
     }
 
     // ---- dA: sum over the 8 lanes (16 channels) of the head, transposing: lane k keeps steps 2k, 2k+1
@@ -496,7 +514,7 @@ __global__ __launch_bounds__(64 * kWaves) void phalanx_mix_bwd_kernel(
     const float da0 = kQkv ? s0 * aa.x : s0 * aa.x * (1.0f - aa.x), da1 = kQkv ? s1 * aa.y : s1 * aa.y * (1.0f - aa.y);
     if constexpr (kSums) acc_a += da0 + da1;
     const int da_off = (t0 >= t_begin) ? da_lane : 0x7ffffff0;
-    if constexpr (kQkv) {
+    if constexpr (kDaBytes == 4) {
       __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(da0), rda, da_off, t0 * ld_da * 4, 0);
       __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(da1), rda, da_off + 4 * ld_da, t0 * ld_da * 4, 0);
     } else {
@@ -583,11 +601,11 @@ MixPlan plan_mix(long B, int H, int L) {
   return m;
 }
 
-template <class E, int kW, bool kQkv>
+template <class E, int kW, bool kQkv, bool kF32 = false>
 void launch_mix_fwd(const MixArgs& p, const MixPlan& m, hipStream_t s) {
   const long total = (long)p.B * m.chunks * ((p.H + 7) / 8);
   const unsigned blocks = (unsigned)((total + kW - 1) / kW);
-  hipLaunchKernelGGL((phalanx_mix_fwd_kernel<E, kW, kQkv>), dim3(blocks), dim3(64 * kW), 0, s,
+  hipLaunchKernelGGL((phalanx_mix_fwd_kernel<E, kW, kQkv, kF32>), dim3(blocks), dim3(64 * kW), 0, s,
                      static_cast<const uint16_t*>(p.a_logit), static_cast<const uint16_t*>(p.b_logit),
                      static_cast<const uint16_t*>(p.c), static_cast<const uint16_t*>(p.v), static_cast<uint16_t*>(p.out),
                      p.L, p.H, p.kv_groups, m.chunk_blocks * kTile, m.chunks, total);
@@ -599,7 +617,8 @@ hipError_t fused_mix_forward(const MixArgs& p, hipStream_t s) {
   const MixPlan m = plan_mix(p.B, p.H, p.L);
   auto by_waves = [&](auto e, auto q) {
     using E = decltype(e);
-    if (m.wg_waves == 8) launch_mix_fwd<E, 8, decltype(q)::value>(p, m, s);
+    if (p.f32_out) launch_mix_fwd<E, 4, decltype(q)::value, true>(p, m, s);  // check mode: one instance per form
+    else if (m.wg_waves == 8) launch_mix_fwd<E, 8, decltype(q)::value>(p, m, s);
     else launch_mix_fwd<E, 4, decltype(q)::value>(p, m, s);
   };
   if (p.dtype == kBf16) {
@@ -632,14 +651,14 @@ MixPlan plan_mix_bwd(long B, int H, int L) {
   return m;
 }
 
-template <class E, bool kSums, bool kQkv>
+template <class E, bool kSums, bool kQkv, bool kF32 = false>
 void launch_mix_bwd(const MixBwdArgs& p, const MixPlan& m, hipStream_t s) {
   const long total = (long)p.B * m.chunks * ((p.H + 7) / 8);
   const unsigned blocks = (unsigned)((total + kWaves - 1) / kWaves);
   auto u = [](const void* q) { return static_cast<const uint16_t*>(q); };
   auto w = [](void* q) { return static_cast<uint16_t*>(q); };
   const int Fkv = (p.H / p.kv_groups) * kChan;
-  hipLaunchKernelGGL((phalanx_mix_bwd_kernel<E, kSums, kQkv>), dim3(blocks), dim3(64 * kWaves), 0, s, u(p.a_logit),
+  hipLaunchKernelGGL((phalanx_mix_bwd_kernel<E, kSums, kQkv, kF32>), dim3(blocks), dim3(64 * kWaves), 0, s, u(p.a_logit),
                      u(p.b_logit), u(p.c), u(p.v), u(p.dout), w(p.da_logit), w(p.db_logit), w(p.dc), w(p.dv), p.sum_da,
                      p.sum_db, p.sum_dc, p.ld_da ? p.ld_da : p.H, p.ld_db ? p.ld_db : Fkv, p.ld_dc ? p.ld_dc : Fkv,
                      p.ld_dv ? p.ld_dv : p.H * kChan, p.L, p.H, p.kv_groups, m.chunk_blocks * kTile, m.chunks, total);
@@ -655,7 +674,17 @@ long fused_mix_backward_sum_rows(long B, int H, int L) {
 hipError_t fused_mix_backward(const MixBwdArgs& p, hipStream_t s) {
   const MixPlan m = plan_mix_bwd(p.B, p.H, p.L);
   const bool sums = p.sum_da != nullptr;
-  if (sums && p.qkv) return hipErrorInvalidValue;  // the caller has checked: sums belong to the layer form
+  if (sums && (p.qkv || p.f32_grads)) return hipErrorInvalidValue;  // the caller has checked: layer form, 16-bit results
+  if (p.f32_grads) {
+    if (p.dtype == kBf16) {
+      if (p.qkv) launch_mix_bwd<Bf16, false, true, true>(p, m, s);
+      else launch_mix_bwd<Bf16, false, false, true>(p, m, s);
+    } else {
+      if (p.qkv) launch_mix_bwd<Fp16, false, true, true>(p, m, s);
+      else launch_mix_bwd<Fp16, false, false, true>(p, m, s);
+    }
+    return hipGetLastError();
+  }
   if (p.dtype == kBf16) {
     if (p.qkv) launch_mix_bwd<Bf16, false, true>(p, m, s);
     else if (sums) launch_mix_bwd<Bf16, true, false>(p, m, s);

@@ -29,6 +29,7 @@ struct BwdArgs {
   int B, H, L, k;
   int in_dtype, dy_dtype;
   bool log_gate = false;
+  bool dx_f32 = false;  // check mode: dx is fp32 [B, H, 16, L] (the kernel's fp32 values, not rounded to in_dtype)
 };
 
 // Exact-fp32 recurrence kernels (btp_scan.hip).
@@ -49,6 +50,7 @@ struct MixArgs {
   int dtype;
   // q/k/v/gate form: a_logit is an fp32 log-decay gate (a = exp(gate)), b_logit is k (used as it is), c is q
   bool qkv = false;
+  bool f32_out = false;  // check mode: `out` is fp32
 };
 hipError_t fused_mix_forward(const MixArgs& p, hipStream_t s);
 
@@ -63,6 +65,7 @@ struct MixBwdArgs {
   // elements per time step of each gradient tensor; 0 = dense (its own width)
   int ld_da = 0, ld_db = 0, ld_dc = 0, ld_dv = 0;
   bool qkv = false;  // as in MixArgs; da_logit is then the fp32 gradient of the gate
+  bool f32_grads = false;  // check mode: da_logit, db_logit, dc, dv are fp32
 };
 hipError_t fused_mix_backward(const MixBwdArgs& p, hipStream_t s);
 long fused_mix_backward_sum_rows(long B, int H, int L);

@@ -220,13 +220,14 @@ constexpr int bwd_waves() {
   return kStreamIn ? SPEAR_BTP_BWD_SHORT_ROW_WAVES : kWavesLong;
 }
 
-template <class E, class C, class GradT, bool kStreamIn, int kW>
+template <class E, class C, class GradT, class DxT, bool kStreamIn, int kW>
 __device__ __forceinline__ void btp_bwd_scan_body(
     unsigned char (*lds)[4096 + (std::is_same<GradT, float>::value ? 8192 : 4096) + kCoeffLdsBytes],
     const typename C::elem* __restrict__ coeff, const uint16_t* __restrict__ x, const GradT* __restrict__ dy,
-    uint16_t* __restrict__ dx, float* __restrict__ dA, int L, int spans_per_row, long total_spans,
+    DxT* __restrict__ dx, float* __restrict__ dA, int L, int spans_per_row, long total_spans,
     int k) {
   constexpr bool kGradF32 = std::is_same<GradT, float>::value;
+  constexpr bool kDxF32 = std::is_same<DxT, float>::value;  // check mode: dx leaves unrounded
   constexpr int kGradBytes = kGradF32 ? 8192 : 4096;
 
   // Rows longer than one span: the carries that cross a span boundary inside the workgroup (the
@@ -416,10 +417,18 @@ __device__ __forceinline__ void btp_bwd_scan_body(
   if (32 * j < sc.nvalid) __builtin_nontemporal_store(dA_A, dArow);
   if (32 * j + 16 < sc.nvalid) __builtin_nontemporal_store(dA_B, dArow + 16);
 
-  // dx goes back through the x image: every lane overwrites exactly the chunks it read
-  lane_write16<E>(img_x, j, d, dxv);
-  wave_lds_handover();
-  slab16_lds_to_global<kStreamOut>(img_x, dx + slab_off, L, sc.nvalid, lane);
+  if constexpr (kDxF32) {
+    // fp32 dx: an 8 KiB image (512 B per channel row) laid over the x and dy images, both dead by now
+    wave_lds_handover();
+    lane_write32(img_x, j, d, dxv);
+    wave_lds_handover();
+    slab32_lds_to_global<kStreamOut>(img_x, dx + slab_off, L, sc.nvalid, lane);
+  } else {
+    // dx goes back through the x image: every lane overwrites exactly the chunks it read
+    lane_write16<E>(img_x, j, d, dxv);
+    wave_lds_handover();
+    slab16_lds_to_global<kStreamOut>(img_x, dx + slab_off, L, sc.nvalid, lane);
+  }
 }
 
 // 16-bit dy and 16-bit coefficients (the reference's operands): the body fits 128 VGPRs, so four
@@ -430,19 +439,19 @@ __global__ __launch_bounds__((64 * bwd_waves<true, kStreamIn>())) SPEAR_BTP_BWD_
     uint16_t* __restrict__ dx, float* __restrict__ dA, int L, int spans_per_row, long total_spans, int k) {
   constexpr int kW = bwd_waves<true, kStreamIn>();
   __shared__ __align__(16) unsigned char lds[kW][4096 + 4096 + kCoeffLdsBytes];
-  btp_bwd_scan_body<E, C, uint16_t, kStreamIn, kW>(lds, coeff, x, dy, dx, dA, L, spans_per_row, total_spans, k);
+  btp_bwd_scan_body<E, C, uint16_t, uint16_t, kStreamIn, kW>(lds, coeff, x, dy, dx, dA, L, spans_per_row, total_spans, k);
 }
 
-// fp32 dy (twice the staging registers and LDS) and log-space gates (an exponential per
-// coefficient): occupancy is left to the compiler.
-template <class E, class C, class GradT, bool kStreamIn>
+// fp32 dy (twice the staging registers and LDS), log-space gates (an exponential per coefficient)
+// and the fp32-dx check mode: occupancy is left to the compiler.
+template <class E, class C, class GradT, class DxT, bool kStreamIn>
 __global__ __launch_bounds__((64 * bwd_waves<false, kStreamIn>())) void btp_bwd_scan_kernel_relaxed(
     const typename C::elem* __restrict__ coeff, const uint16_t* __restrict__ x, const GradT* __restrict__ dy,
-    uint16_t* __restrict__ dx, float* __restrict__ dA, int L, int spans_per_row, long total_spans, int k) {
+    DxT* __restrict__ dx, float* __restrict__ dA, int L, int spans_per_row, long total_spans, int k) {
   constexpr int kGradBytes = std::is_same<GradT, float>::value ? 8192 : 4096;
   constexpr int kW = bwd_waves<false, kStreamIn>();
   __shared__ __align__(16) unsigned char lds[kW][4096 + kGradBytes + kCoeffLdsBytes];
-  btp_bwd_scan_body<E, C, GradT, kStreamIn, kW>(lds, coeff, x, dy, dx, dA, L, spans_per_row, total_spans, k);
+  btp_bwd_scan_body<E, C, GradT, DxT, kStreamIn, kW>(lds, coeff, x, dy, dx, dA, L, spans_per_row, total_spans, k);
 }
 
 __global__ __launch_bounds__(256) void copy_kernel(const uint4* __restrict__ src, uint4* __restrict__ dst,
@@ -501,8 +510,14 @@ void launch_bwd_as(const BwdArgs& p, const Grid& g, hipStream_t s) {
   const auto* c = static_cast<const typename C::elem*>(p.coeff);
   const auto* x = static_cast<const uint16_t*>(p.x);
   auto* dx = static_cast<uint16_t*>(p.dx);
+  if (p.dx_f32) {
+    hipLaunchKernelGGL((btp_bwd_scan_kernel_relaxed<E, C, GradT, float, kStreamIn>), dim3(g.blocks), dim3(64 * g.waves),
+                       0, s, c, x, static_cast<const GradT*>(p.dy), static_cast<float*>(p.dx), p.dA, p.L,
+                       g.spans_per_row, g.total_spans, p.k);
+    return;
+  }
   if constexpr (std::is_same<GradT, float>::value || C::kLog) {
-    hipLaunchKernelGGL((btp_bwd_scan_kernel_relaxed<E, C, GradT, kStreamIn>), dim3(g.blocks), dim3(64 * g.waves), 0, s,
+    hipLaunchKernelGGL((btp_bwd_scan_kernel_relaxed<E, C, GradT, uint16_t, kStreamIn>), dim3(g.blocks), dim3(64 * g.waves), 0, s,
                        c, x, static_cast<const GradT*>(p.dy), dx, p.dA, p.L, g.spans_per_row, g.total_spans, p.k);
   } else {
     hipLaunchKernelGGL((btp_bwd_scan_kernel<E, C, kStreamIn>), dim3(g.blocks), dim3(64 * g.waves), 0, s, c, x,
@@ -512,8 +527,10 @@ void launch_bwd_as(const BwdArgs& p, const Grid& g, hipStream_t s) {
 
 template <class E, class C, class GradT>
 hipError_t launch_bwd(const BwdArgs& p, hipStream_t s) {
-  constexpr bool kLean = !(std::is_same<GradT, float>::value || C::kLog);  // the kernel launch_bwd_as picks
-  const Grid g = make_grid((long)p.B * p.H, p.L, bwd_waves<kLean, false>(), bwd_waves<kLean, true>());
+  constexpr bool kLeanIo = !(std::is_same<GradT, float>::value || C::kLog);
+  const bool lean = kLeanIo && !p.dx_f32;  // the kernel launch_bwd_as picks
+  const Grid g = lean ? make_grid((long)p.B * p.H, p.L, bwd_waves<true, false>(), bwd_waves<true, true>())
+                      : make_grid((long)p.B * p.H, p.L, bwd_waves<false, false>(), bwd_waves<false, true>());
   if (stream_inputs(g)) launch_bwd_as<E, C, GradT, true>(p, g, s);
   else launch_bwd_as<E, C, GradT, false>(p, g, s);
   return hipGetLastError();

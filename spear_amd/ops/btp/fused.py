@@ -118,10 +118,16 @@ class _PhalanxMix(torch.autograd.Function):
         a_logits, b_logits, c, v = ctx.saved_tensors
         H, Hkv = ctx.heads, ctx.kv_heads
         groups = H // Hkv
+        dout = dout.contiguous()
         if groups in (1, 2, 4, 8) and (groups < 8 or H % 8 == 0):
             da, db, dc, dv = (torch.empty_like(t) for t in (a_logits, b_logits, c, v))
-            torch.ops.spear_btp.mix_backward(a_logits, b_logits, c, v, dout.contiguous(), da, db, dc, dv, H, Hkv)
+            torch.ops.spear_btp.mix_backward(a_logits, b_logits, c, v, dout, da, db, dc, dv, H, Hkv)
             return da, db, dc, dv, None, None
+
+        # Head groups that span wavefronts: gates recomputed with PyTorch ops, stand-alone kernels for the
+        # recurrence. The decay and the gated input are rounded to the tensors' 16-bit type on the way (the
+        # stand-alone op takes 16-bit operands), so these gradients differ from the fused kernel's in the last
+        # bits of that rounding.
 
         B, L, _ = v.shape
         dt = v.dtype

@@ -11,9 +11,10 @@ Differences that do not change results:
     without a GPU (the reference imports its extension unconditionally, interface.py:16);
   * ``dA`` is allocated uninitialised, because the kernel writes every element
     (the reference zero-fills it, interface.py:158);
-  * the carry checkpoint is allocated (the op schema requires it) but not stored by default,
-    because this backward recomputes the carries; set ``SPEAR_BTP_WRITE_CHECKPOINT=1`` or call
-    ``spear_amd._btp.forward`` directly to have it written.
+  * the carry checkpoint is not stored by default, because this backward recomputes the carries:
+    the op then receives a zero-element placeholder (its schema requires a tensor) and nothing of
+    that size is kept alive for backward. Set ``SPEAR_BTP_WRITE_CHECKPOINT=1`` before importing this
+    module (the variable is read once) or call ``spear_amd._btp.forward`` directly to have it written.
 """
 
 from __future__ import annotations
@@ -35,14 +36,14 @@ WPB_K1_DEFAULT = 8
 WPB_K2_DEFAULT = 32
 
 
-def _forward_flags() -> int:
-    return _btp.FLAG_WRITE_CHECKPOINT if os.environ.get("SPEAR_BTP_WRITE_CHECKPOINT", "0") == "1" else 0
+# Read once: the op sits on the hot path of every layer call.
+_FORWARD_FLAGS = _btp.FLAG_WRITE_CHECKPOINT if os.environ.get("SPEAR_BTP_WRITE_CHECKPOINT", "0") == "1" else 0
 
 
 def _forward_impl(
     coeff: torch.Tensor, x: torch.Tensor, y: torch.Tensor, checkpoint: torch.Tensor, k: int, wpb: int
 ) -> None:
-    _btp.forward(coeff, x, y, checkpoint, k, wpb, flags=_forward_flags())
+    _btp.forward(coeff, x, y, checkpoint, k, wpb, flags=_FORWARD_FLAGS)
 
 
 def _forward_fake(
@@ -132,7 +133,8 @@ class _BTPFunction(torch.autograd.Function):
         assert wpb in SUPPORTED_WPB, f"WPB must be one of {SUPPORTED_WPB}"
 
         y = torch.empty_like(x, dtype=output_dtype)
-        checkpoint = torch.empty((B, H, L // BLK, DH), device=x.device, dtype=torch.float32)
+        ckpt_shape = (B, H, L // BLK, DH) if _FORWARD_FLAGS & _btp.FLAG_WRITE_CHECKPOINT else (0,)
+        checkpoint = torch.empty(ckpt_shape, device=x.device, dtype=torch.float32)
         torch.ops.spear_btp.forward(coeff, x, y, checkpoint, int(k), int(wpb))
 
         ctx.save_for_backward(coeff, x, checkpoint)

@@ -8,7 +8,7 @@ import numpy as np
 import pytest
 import torch
 
-from helpers import BF16_ATOL, BF16_RTOL, assert_close, f64
+from helpers import BF16_ATOL, BF16_RTOL, F32_ATOL, F32_RTOL, assert_close, f64
 from oracle import btp_oracle as orc
 
 pytestmark = pytest.mark.gpu
@@ -103,19 +103,87 @@ def test_same_numbers_as_the_log_gate_operator_with_glue():
     assert float(err.max()) <= 0
 
 
-def test_benchmark_shape_properties():
-    """B=1024, L=128, H=32 (the headline shape in this form): q = 0 returns v, batch rows are independent."""
+# The benchmark configurations in the terms they are worded in (q, k, v bf16, fp32 log-decay gate; check out,
+# dq, dk, dv, dgate), at full size: B1024 L128 H32 with gate = -softplus(N(0,1)) and q/k/v ~ N(0, 1/16); the long
+# rows B16 L8192 H64; and B64 L2048 H128 with q/k/v ~ N(0,1) and per head either U[-20,-5] or U[-1e-4,0] gates.
+BENCH_SHAPES = {
+    "c3_B1024_L128_H32": dict(B=1024, L=128, H=32, seed=1234, std=0.25, gates="softplus"),
+    "c4_B16_L8192_H64": dict(B=16, L=8192, H=64, seed=1235, std=0.25, gates="softplus"),
+    "c5_B64_L2048_H128": dict(B=64, L=2048, H=128, seed=1236, std=1.0, gates="mixed"),
+}
+
+
+@pytest.mark.parametrize("name", list(BENCH_SHAPES))
+def test_benchmark_shapes_forward_and_backward(name):
+    """Full-size forward and backward; the oracle on sampled batch rows (rows are independent), and the
+    properties that need no oracle: q = 0 returns v, a slice of the batch run alone gives the same bits."""
     from spear_amd import btp_qkv
 
-    q, k, v, gate, _ = make_qkv(1024, 128, 32, 32, seed=75)
-    qd, kd, vd, gd = (t.to(DEV) for t in (q, k, v, gate))
-    out = btp_qkv(qd, kd, vd, gd)
+    cfg = BENCH_SHAPES[name]
+    B, L, H = cfg["B"], cfg["L"], cfg["H"]
+    print(f"{name}: generating inputs", flush=True)
+    q, k, v, gate, dout = make_qkv(B, L, H, H, seed=cfg["seed"], std=cfg["std"], gates=cfg["gates"])
+    print(f"{name}: forward/backward", flush=True)
+    leaves = [t.to(DEV).requires_grad_(True) for t in (q, k, v, gate)]
+    out = btp_qkv(*leaves)
+    out.backward(dout.to(DEV))
+    torch.cuda.synchronize()
+    qd, kd, vd, gd = (t.detach() for t in leaves)
+    grads = [t.grad for t in leaves]
+    assert all(bool(torch.isfinite(t.float()).all()) for t in (out, *grads))
     assert torch.equal(btp_qkv(torch.zeros_like(qd), kd, vd, gd), vd)     # q = 0 leaves v
-    part = btp_qkv(qd[1000:1003].contiguous(), kd[1000:1003].contiguous(), vd[1000:1003].contiguous(), gd[1000:1003].contiguous())
-    assert torch.equal(part, out[1000:1003])
-    sample = [0, 517, 1023]
+    lo = B - 3
+    part = [t[lo:].contiguous().requires_grad_(True) for t in (qd, kd, vd, gd)]
+    out_part = btp_qkv(*part)
+    out_part.backward(dout[lo:].to(DEV))
+    assert torch.equal(out_part.detach(), out.detach()[lo:])
+    for name_g, gp, gall in zip(("dq", "dk", "dv", "dgate"), part, grads):
+        assert torch.equal(gp.grad, gall[lo:]), name_g
+
+    print(f"{name}: oracle on sampled batch rows", flush=True)
+    rng = np.random.default_rng(cfg["seed"])
+    sample = sorted(set([0, B - 1] + [int(i) for i in rng.integers(0, B, size=2)]))
     args = [f64(flat(t[sample])) for t in (q, k, v)] + [f64(gate[sample])]
-    assert_close(f64(flat(out[sample].cpu())), orc.qkv_gate_forward(*args, 32, 32), BF16_ATOL, BF16_RTOL, "out sample")
+    assert_close(f64(flat(out.detach()[sample].cpu())), orc.qkv_gate_forward(*args, H, H), BF16_ATOL, BF16_RTOL, "out")
+    rgate, rk, rq, rv = orc.qkv_gate_backward(*args, f64(flat(dout[sample])), H, H)
+    dq, dk, dv, dgate = (t[sample].cpu() for t in grads)
+    assert_close(f64(flat(dv)), rv, BF16_ATOL, BF16_RTOL, "dv")
+    assert_close(f64(flat(dq)), rq, BF16_ATOL, BF16_RTOL, "dq")
+    assert_close(f64(flat(dk)), rk, BF16_ATOL, BF16_RTOL, "dk")
+    assert_close(f64(dgate), rgate, F32_ATOL, F32_RTOL, "dgate")
+
+
+def test_log_gate_operator_at_the_log_space_stress_shape():
+    """btp_log (fp32 log-space gates in the op's own [B, H, 16, L] layout) at B64 H128 L2048 with the per-head
+    forgetting / near-identity mixture: y, dx, dgate on sampled rows against the oracle at a = exp(gate)."""
+    from spear_amd import btp_log
+
+    B, H, L = 64, 128, 2048
+    g = torch.Generator().manual_seed(1236)
+    print("btp_log c5: generating inputs", flush=True)
+    forget = torch.rand(B, H, 1, generator=g) < 0.5
+    u = torch.rand(B, H, L, generator=g)
+    gate = torch.where(forget, -20.0 + 15.0 * u, -1e-4 * u).float()
+    x = torch.randn(B, H, 16, L, generator=g).bfloat16()
+    dy = torch.randn(B, H, 16, L, generator=g).bfloat16()
+    gd, xd = gate.to(DEV).requires_grad_(True), x.to(DEV).requires_grad_(True)
+    print("btp_log c5: forward/backward", flush=True)
+    y = btp_log(gd, xd, output_dtype=torch.float32)
+    y.backward(dy.to(DEV).float())
+    torch.cuda.synchronize()
+    assert all(bool(torch.isfinite(t.float()).all()) for t in (y, gd.grad, xd.grad))
+    rng = np.random.default_rng(1236)
+    rows = list(zip(rng.integers(0, B, size=6), rng.integers(0, H, size=6)))
+    rows += [(int(b), int(h)) for b, h in zip(*np.nonzero(~forget[:, :, 0].numpy()))][:2]  # two near-identity heads for sure
+    print("btp_log c5: oracle on sampled rows", flush=True)
+    for b, h in rows:
+        sl = (slice(b, b + 1), slice(h, h + 1))
+        a = np.exp(f64(gate[sl]))
+        ry = orc.forward(a, f64(x[sl]))
+        rdx, rdA = orc.backward(a, f64(x[sl]), f64(dy[sl]))
+        assert_close(f64(y.detach()[sl]), ry, F32_ATOL, F32_RTOL, f"y[{b},{h}]")
+        assert_close(f64(xd.grad[sl]), rdx, BF16_ATOL, BF16_RTOL, f"dx[{b},{h}]")
+        assert_close(f64(gd.grad[sl]), rdA * a, F32_ATOL, F32_RTOL, f"dgate[{b},{h}]")
 
 
 def test_rejects_what_it_cannot_do():
