@@ -249,6 +249,20 @@ def main() -> int:
     ceil_copy = 2 * nbytes / (probe_copy_ms * 1e-3) / 1e9
     ceil_2r1w = 3 * nbytes / (probe_2r1w_ms * 1e-3) / 1e9
 
+    # the same traffic in other launch shapes: is there a shape the kernels could borrow that moves more?
+    shape_names = ["one_slab_per_wave", "two_slabs_per_wave", "loop_4_slabs_prefetch", "persistent_grid_prefetch",
+                   "one_16B_element_per_thread"]
+    probe_shapes = {}
+    for shape, name in enumerate(shape_names):
+        def shaped(s, second, shape=shape):
+            rc = lib.spear_btp_stream_probe_shape(s["x"].data_ptr(), s["dy"].data_ptr() if second else None,
+                                                  s["dx"].data_ptr(), ctypes.c_ulonglong(nbytes), shape, sp)
+            assert rc == 0, lib.spear_btp_last_error()
+        t1, t2 = kernel_ms(lambda s: shaped(s, False)), kernel_ms(lambda s: shaped(s, True))
+        probe_shapes[name] = {"copy_1r1w": 2 * nbytes / (t1 * 1e-3) / 1e9, "nt_2r1w": 3 * nbytes / (t2 * 1e-3) / 1e9}
+    best_copy = max(v["copy_1r1w"] for v in probe_shapes.values())
+    best_2r1w = max(v["nt_2r1w"] for v in probe_shapes.values())
+
     # log-space gate entry points on the same shape (fp32 gate in, fp32 dgate out: 68 + 108 B per unit)
     for s_ in sets:
         s_["gate"] = torch.log(s_["coeff"].float()).contiguous()
@@ -546,6 +560,57 @@ def main() -> int:
 
     streaming = None if args.no_streaming else guarded(streaming_leg)
 
+    # what a caller of the public op gets: y = btp(coeff, x); y.backward(dy) through autograd, torch.library
+    # dispatch and the compiled binding, eager (host-bound on small shapes) and as a HIP-graph replay of the
+    # same two ops, at this shape and at the batch of configuration 1 (B = 8)
+    def public_op_leg():
+        from spear_amd.ops.btp import btp as btp_op
+
+        def measure(bs):
+            s = sets[0]
+            c, xx, g = (s[k][:bs].contiguous() for k in ("coeff", "x", "dy"))
+            ck = torch.empty(0, device=dev)
+            y, dx = torch.empty_like(xx), torch.empty_like(xx)
+            dA = torch.empty(bs, H, L, device=dev)
+
+            def eager():
+                cl, xl = c.detach().requires_grad_(True), xx.detach().requires_grad_(True)
+                btp_op(cl, xl, 2, 32, torch.bfloat16).backward(g)
+
+            def ops_only():  # the two custom ops on preallocated outputs (what a graph can hold)
+                torch.ops.spear_btp.forward(c, xx, y, ck, 2, 32)
+                torch.ops.spear_btp.backward(c, xx, g, ck, dx, dA, 2, 32)
+
+            def timed(fn, n):
+                for _ in range(5):
+                    fn()
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                for _ in range(n):
+                    fn()
+                torch.cuda.synchronize()
+                return (time.perf_counter() - t0) * 1e3 / n
+
+            n = max(20, args.steps // 2)
+            eager_ms, ops_ms = timed(eager, n), timed(ops_only, n)
+            side = torch.cuda.Stream()
+            side.wait_stream(stream)
+            with torch.cuda.stream(side):
+                ops_only()
+            stream.wait_stream(side)
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=side):
+                ops_only()
+            torch.cuda.synchronize()
+            graph_ms = timed(graph.replay, n)
+            return {"B": bs, "eager_autograd_ms": eager_ms, "two_ops_preallocated_ms": ops_ms, "hip_graph_replay_ms": graph_ms,
+                    "eager_over_graph": eager_ms / graph_ms, "two_ops_over_graph": ops_ms / graph_ms}
+
+        return {"what": "btp(coeff, x, output_dtype=bf16) + backward through the public op (wall clock per fwd+bwd)",
+                "this_shape": measure(B), "config1_batch": measure(min(B, 8))}
+
+    public_op = guarded(public_op_leg)
+
     units = B * H * L
     tokens = B * L
     bwd_gbps = units * BWD_BYTES / (bwd_ms * 1e-3) / 1e9
@@ -604,7 +669,11 @@ def main() -> int:
             "nt_2r1w": {"avg_launch_ms": probe_2r1w_ms, "achieved": ceil_2r1w, "unit": "GB/s"},
             "forward_kernel_vs_nt_copy": fwd_gbps / ceil_copy,
             "backward_kernel_vs_nt_2r1w": bwd_gbps / ceil_2r1w,
+            "other_launch_shapes_GBps": probe_shapes,
+            "forward_kernel_vs_best_copy_shape": fwd_gbps / best_copy,
+            "backward_kernel_vs_best_2r1w_shape": bwd_gbps / best_2r1w,
         },
+        "public_op": public_op,
     }
     if not args.no_cpu_baseline:
         base = cpu_baseline(B, H, L, seed, x_std, gate)

@@ -233,6 +233,15 @@ int spear_btp_copy(const void* src, void* dst, unsigned long long bytes, void* s
  * compared with beside the 8 TB/s peak. */
 int spear_btp_stream_probe(const void* src_a, const void* src_b, void* dst, unsigned long long bytes, void* stream);
 
+/* The same traffic in other launch shapes, to show where the kernels' own shape stands among the
+ * alternatives: shape 0 = spear_btp_stream_probe (one 4 KiB slab per wavefront); 1 = two slabs per
+ * wavefront, all loads issued before the first store; 2 = four slabs per wavefront in a loop that issues
+ * the next slab's loads before the current slab's stores; 3 = that loop as a persistent grid striding over
+ * the buffer; 4 = one 16-byte element per thread. Same arguments and result as spear_btp_stream_probe. */
+#define SPEAR_BTP_PROBE_SHAPES 5
+int spear_btp_stream_probe_shape(const void* src_a, const void* src_b, void* dst, unsigned long long bytes, int shape,
+                                 void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,5 +1,5 @@
-"""`pip install -e .` builds spear_amd/libspear_btp.so with hipcc for gfx950 and installs the
-pure-Python package around it. There is no CUDA path and no architecture detection."""
+"""`pip install -e .` builds spear_amd/libspear_btp.so and its torch binding spear_amd/_btp_ext.so with
+hipcc for gfx950 and installs the Python package around them. There is no CUDA path and no architecture detection."""
 
 import os
 import sys
@@ -15,6 +15,7 @@ class BuildWithHip(build_py):
         from spear_amd.csrc import build as hip_build
 
         print("building", hip_build.build(verbose=True))
+        print("building", hip_build.build_extension(verbose=True))
         super().run()
 
 
@@ -22,8 +23,9 @@ setup(
     name="spear-amd",
     version="0.1.0",
     description="SPEAR Block Two-Pass kernels and Phalanx layer for AMD MI355X (gfx950)",
-    packages=find_packages(include=["spear_amd", "spear_amd.*"]),
-    package_data={"spear_amd": ["libspear_btp.so", "csrc/*.hip", "csrc/*.h"]},
+    # `spear` is the reference's import name: an alias package without code of its own
+    packages=find_packages(include=["spear_amd", "spear_amd.*", "spear"]),
+    package_data={"spear_amd": ["libspear_btp.so", "_btp_ext.so", "csrc/*.hip", "csrc/*.h", "csrc/*.cpp"]},
     python_requires=">=3.10",
     install_requires=["torch>=2.0.0"],
     cmdclass={"build_py": BuildWithHip},

@@ -1,7 +1,9 @@
 """Host shim between torch tensors and the C ABI of ``libspear_btp.so``.
 
-Takes the place of the reference's compiled extension module ``spear._btp``
-(csrc/btp/_bindings.cu:240-243): it exports ``forward(coeff, x, y, checkpoint, k, wpb)`` and
+ctypes view of the whole C ABI, used by the tests, the benchmark and the host code of the streaming
+and layer paths. The custom ops themselves go through the compiled binding ``spear_amd._btp_ext``
+(:func:`load_extension`), which takes the place of the reference's extension module ``spear._btp``
+(csrc/btp/_bindings.cu:240-243). Like it, this module exports ``forward(coeff, x, y, checkpoint, k, wpb)`` and
 ``backward(coeff, x, dy, checkpoint, dx, dA, k, wpb)`` with the same positional arguments, the
 same in-place semantics (the caller allocates every output) and the same argument checks and
 messages (csrc/btp/_bindings.cu:19-60, raised as ``RuntimeError`` like ``TORCH_CHECK``).
@@ -18,7 +20,7 @@ import threading
 
 import torch
 
-__all__ = ["forward", "backward", "forward_log", "backward_log", "mix_forward", "mix_backward", "jagged_prefill", "jagged_step", "library_path", "load_library", "FLAG_WRITE_CHECKPOINT", "FLAG_PATH_MFMA", "FLAG_JAGGED_LOG_A", "FLAG_JAGGED_LOG_R", "FLAG_MIX_QKV_GATE", "FLAG_MIX_F32_RESULTS", "FLAG_DX_F32", "mix_backward_sum_rows", "mix_backward_bias"]
+__all__ = ["forward", "backward", "forward_log", "backward_log", "mix_forward", "mix_backward", "jagged_prefill", "jagged_step", "library_path", "load_library", "load_extension", "FLAG_WRITE_CHECKPOINT", "FLAG_PATH_MFMA", "FLAG_JAGGED_LOG_A", "FLAG_JAGGED_LOG_R", "FLAG_MIX_QKV_GATE", "FLAG_MIX_F32_RESULTS", "FLAG_DX_F32", "mix_backward_sum_rows", "mix_backward_bias"]
 
 _BF16, _F16, _F32 = 0, 1, 2
 FLAG_WRITE_CHECKPOINT = 0x1
@@ -28,7 +30,7 @@ FLAG_JAGGED_LOG_R = 0x8
 FLAG_MIX_QKV_GATE = 0x1
 FLAG_MIX_F32_RESULTS = 0x2
 FLAG_DX_F32 = 0x10
-_ABI_VERSION = 10
+_ABI_VERSION = 11
 _SUPPORTED_WPB = (4, 8, 16, 32)
 
 _lock = threading.Lock()
@@ -75,6 +77,8 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.spear_btp_copy.restype = ci
     lib.spear_btp_stream_probe.argtypes = [vp, vp, vp, ctypes.c_ulonglong, vp]
     lib.spear_btp_stream_probe.restype = ci
+    lib.spear_btp_stream_probe_shape.argtypes = [vp, vp, vp, ctypes.c_ulonglong, ci, vp]
+    lib.spear_btp_stream_probe_shape.restype = ci
 
 
 def load_library() -> ctypes.CDLL:
@@ -101,6 +105,33 @@ def load_library() -> ctypes.CDLL:
             ) from exc
         _lib = lib
     return _lib
+
+
+_ext = None
+
+
+def load_extension():
+    """Import (once) and return ``spear_amd._btp_ext``, the compiled torch binding over the same C ABI
+    (``spear_amd/csrc/btp_torch_ext.cpp``): the custom ops call it so that a hot call carries no Python
+    argument checks. Raises ``RuntimeError`` if it is not built or does not match this package."""
+    global _ext
+    if _ext is not None:
+        return _ext
+    with _lock:
+        if _ext is None:
+            try:
+                import importlib
+
+                ext = importlib.import_module("spear_amd._btp_ext")
+            except ImportError as exc:
+                raise RuntimeError(
+                    f"spear_amd: the compiled torch binding spear_amd/_btp_ext.so could not be imported ({exc}). "
+                    "Build it with `python -m spear_amd.csrc.build` (needs hipcc); there is no fallback."
+                ) from exc
+            if ext.abi_version() != _ABI_VERSION:
+                raise RuntimeError(f"spear_amd._btp_ext speaks C ABI {ext.abi_version()}, this package needs {_ABI_VERSION}")
+            _ext = ext
+    return _ext
 
 
 def _check(cond: bool, msg: str) -> None:

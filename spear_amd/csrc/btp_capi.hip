@@ -44,7 +44,7 @@ int check_common(const char* who, int B, int H, int L, int k, int in_dtype, int 
 
 extern "C" {
 
-int spear_btp_abi_version(void) { return 10; }
+int spear_btp_abi_version(void) { return 11; }
 
 const char* spear_btp_last_error(void) { return g_error; }
 
@@ -337,6 +337,20 @@ int spear_btp_stream_probe(const void* src_a, const void* src_b, void* dst, unsi
   const hipError_t err = spear_btp::stream_probe(src_a, src_b, dst, bytes, static_cast<hipStream_t>(stream));
   if (err != hipSuccess)
     return fail(SPEAR_BTP_ELAUNCH, "spear_btp_stream_probe: launch failed: %s", hipGetErrorString(err));
+  return 0;
+}
+
+int spear_btp_stream_probe_shape(const void* src_a, const void* src_b, void* dst, unsigned long long bytes, int shape,
+                                 void* stream) {
+  g_error[0] = '\0';
+  if (!src_a || !dst) return fail(SPEAR_BTP_ENULL, "spear_btp_stream_probe_shape: NULL pointer");
+  if (bytes % 4096 != 0 || !aligned16(src_a) || !aligned16(src_b) || !aligned16(dst))
+    return fail(SPEAR_BTP_EINVAL, "spear_btp_stream_probe_shape: size must be a multiple of 4096, pointers of 16 bytes");
+  if (shape < 0 || shape >= SPEAR_BTP_PROBE_SHAPES)
+    return fail(SPEAR_BTP_EINVAL, "spear_btp_stream_probe_shape: shape must be 0..%d (got %d)", SPEAR_BTP_PROBE_SHAPES - 1, shape);
+  const hipError_t err = spear_btp::stream_probe_shape(src_a, src_b, dst, bytes, shape, static_cast<hipStream_t>(stream));
+  if (err != hipSuccess)
+    return fail(SPEAR_BTP_ELAUNCH, "spear_btp_stream_probe_shape: launch failed: %s", hipGetErrorString(err));
   return 0;
 }
 

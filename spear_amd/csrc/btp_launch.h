@@ -109,5 +109,7 @@ hipError_t device_copy(const void* src, void* dst, unsigned long long bytes, hip
 // Slab-shaped non-temporal copy (b == nullptr) or two-input combine, for measuring what the memory
 // system gives the operator's access pattern (btp_scan.hip).
 hipError_t stream_probe(const void* a, const void* b, void* dst, unsigned long long bytes, hipStream_t s);
+// The same traffic in other launch shapes (0 = the one above, 1..4 see stream_probe_shape_kernel).
+hipError_t stream_probe_shape(const void* a, const void* b, void* dst, unsigned long long bytes, int shape, hipStream_t s);
 
 }  // namespace spear_btp

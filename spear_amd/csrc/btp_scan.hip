@@ -484,6 +484,68 @@ __global__ __launch_bounds__(64 * kWaves) void stream_probe_kernel(const uint4* 
   }
 }
 
+// Other launch shapes for the same traffic, to show where the shape above stands (measured on MI355X: none
+// of them is faster). kShape 1: two slabs per wavefront, every load issued before the first store (twice
+// the bytes in flight per wavefront); 2: a loop over `iters` slabs per wavefront with the next slab's loads
+// issued before the current slab's stores (a workgroup covers kWaves * iters consecutive slabs); 3: the
+// same loop as a persistent grid striding over the buffer; 4: one 16-byte element per thread.
+template <int kReads, int kShape>
+__global__ __launch_bounds__(64 * kWaves) void stream_probe_shape_kernel(const uint4* __restrict__ a,
+                                                                         const uint4* __restrict__ b,
+                                                                         uint4* __restrict__ dst,
+                                                                         unsigned long long slabs, int iters) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  auto load = [&](unsigned long long slab, uint4 (&q)[4], uint4 (&r)[4]) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      q[i] = stream_load16(a + slab * 256 + lane + 64 * i);
+      if constexpr (kReads == 2) r[i] = stream_load16(b + slab * 256 + lane + 64 * i);
+    }
+  };
+  auto store = [&](unsigned long long slab, uint4 (&q)[4], const uint4 (&r)[4]) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      if constexpr (kReads == 2) q[i] = make_uint4(q[i].x ^ r[i].x, q[i].y ^ r[i].y, q[i].z ^ r[i].z, q[i].w ^ r[i].w);
+      stream_store16(dst + slab * 256 + lane + 64 * i, q[i]);
+    }
+  };
+  if constexpr (kShape == 1) {
+    const unsigned long long s0 = (unsigned long long)blockIdx.x * kWaves * 2 + wave, s1 = s0 + kWaves;
+    uint4 q0[4], r0[4], q1[4], r1[4];
+    if (s0 < slabs) load(s0, q0, r0);
+    if (s1 < slabs) load(s1, q1, r1);
+    if (s0 < slabs) store(s0, q0, r0);
+    if (s1 < slabs) store(s1, q1, r1);
+  } else if constexpr (kShape == 2 || kShape == 3) {
+    const unsigned long long step = kShape == 2 ? kWaves : (unsigned long long)gridDim.x * kWaves;
+    unsigned long long slab = kShape == 2 ? (unsigned long long)blockIdx.x * kWaves * iters + wave
+                                          : (unsigned long long)blockIdx.x * kWaves + wave;
+    const unsigned long long end = kShape == 2 ? slab + step * iters : slabs;
+    uint4 q[4], r[4], nq[4], nr[4];
+    if (slab < slabs) load(slab, nq, nr);
+    for (; slab < slabs && slab < end; slab += step) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) { q[i] = nq[i]; r[i] = nr[i]; }
+      const unsigned long long next = slab + step;
+      if (next < slabs && next < end) load(next, nq, nr);
+      __builtin_amdgcn_sched_barrier(0);
+      store(slab, q, r);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  } else {
+    static_assert(kShape == 4, "unknown probe shape");
+    const unsigned long long i = (unsigned long long)blockIdx.x * (64 * kWaves) + threadIdx.x;
+    if (i < slabs * 256) {
+      uint4 q = stream_load16(a + i);
+      if constexpr (kReads == 2) {
+        const uint4 r = stream_load16(b + i);
+        q = make_uint4(q.x ^ r.x, q.y ^ r.y, q.z ^ r.z, q.w ^ r.w);
+      }
+      stream_store16(dst + i, q);
+    }
+  }
+}
+
 template <class E, class C, class OutT, bool kCheckpoint, bool kStreamIn>
 void launch_fwd_as(const FwdArgs& p, const Grid& g, hipStream_t s) {
   hipLaunchKernelGGL((btp_fwd_scan_kernel<E, C, OutT, kCheckpoint, kStreamIn>), dim3(g.blocks), dim3(64 * g.waves), 0,
@@ -570,6 +632,37 @@ hipError_t stream_probe(const void* a, const void* b, void* dst, unsigned long l
   else
     hipLaunchKernelGGL(stream_probe_kernel<2>, dim3(blocks), dim3(64 * kWaves), 0, s, static_cast<const uint4*>(a),
                        static_cast<const uint4*>(b), static_cast<uint4*>(dst), slabs);
+  return hipGetLastError();
+}
+
+namespace {
+template <int kReads>
+void launch_probe_shape(const void* a, const void* b, void* dst, unsigned long long slabs, int shape, hipStream_t s) {
+  const auto* pa = static_cast<const uint4*>(a);
+  const auto* pb = static_cast<const uint4*>(b);
+  auto* pd = static_cast<uint4*>(dst);
+  const dim3 wg(64 * kWaves);
+  auto blocks_for = [&](unsigned long long per) { return dim3((unsigned)((slabs + per - 1) / per)); };
+  constexpr int kLoopIters = 4;
+  switch (shape) {
+    case 1: hipLaunchKernelGGL((stream_probe_shape_kernel<kReads, 1>), blocks_for(2 * kWaves), wg, 0, s, pa, pb, pd, slabs, 2); break;
+    case 2: hipLaunchKernelGGL((stream_probe_shape_kernel<kReads, 2>), blocks_for(kLoopIters * kWaves), wg, 0, s, pa, pb, pd, slabs, kLoopIters); break;
+    case 3: {
+      const unsigned long long want = (slabs + kWaves - 1) / kWaves;
+      hipLaunchKernelGGL((stream_probe_shape_kernel<kReads, 3>), dim3((unsigned)(want < 2048 ? want : 2048)), wg, 0, s, pa, pb, pd, slabs, 0);
+      break;
+    }
+    default: hipLaunchKernelGGL((stream_probe_shape_kernel<kReads, 4>), blocks_for(1), wg, 0, s, pa, pb, pd, slabs, 1); break;
+  }
+}
+}  // namespace
+
+hipError_t stream_probe_shape(const void* a, const void* b, void* dst, unsigned long long bytes, int shape, hipStream_t s) {
+  if (shape == 0) return stream_probe(a, b, dst, bytes, s);
+  const unsigned long long slabs = bytes / 4096;
+  if (slabs == 0) return hipSuccess;
+  if (b == nullptr) launch_probe_shape<1>(a, b, dst, slabs, shape, s);
+  else launch_probe_shape<2>(a, b, dst, slabs, shape, s);
   return hipGetLastError();
 }
 

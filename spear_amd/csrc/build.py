@@ -1,8 +1,9 @@
 """Builds ``spear_amd/libspear_btp.so`` (HIP kernels + C ABI) for gfx950 with hipcc.
 
-Usage: ``python -m spear_amd.csrc.build`` or ``spear_amd.csrc.build.build()``. hipcc
-cross-compiles without a GPU present. The CMake target in the repository root builds the same
-library from the same sources.
+Usage: ``python -m spear_amd.csrc.build`` or ``spear_amd.csrc.build.build()`` followed by
+``build_extension()`` (``spear_amd/_btp_ext.so``, the compiled torch binding over the C ABI). hipcc
+cross-compiles without a GPU present. The CMake targets in the repository root build the same
+two files from the same sources.
 """
 
 from __future__ import annotations
@@ -71,6 +72,40 @@ def build(verbose: bool = False, extra_flags: list[str] | None = None, out: str 
     return out
 
 
+EXT_NAME = "_btp_ext"
+EXT_SOURCE = "btp_torch_ext.cpp"
+
+
+def ext_path() -> str:
+    return os.path.join(PKG, EXT_NAME + ".so")
+
+
+def build_extension(verbose: bool = False, out: str | None = None) -> str:
+    """``spear_amd/_btp_ext.so``: the compiled torch binding over the C ABI (host code only, no kernels),
+    linked against ``libspear_btp.so`` beside it. Needs the library built first."""
+    import sysconfig
+
+    import torch
+    from torch.utils import cpp_extension
+
+    out = out or ext_path()
+    if not os.path.exists(lib_path()):
+        raise RuntimeError(f"{lib_path()} is missing; build the C-ABI library before its torch binding")
+    rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
+    includes = [*cpp_extension.include_paths(), sysconfig.get_paths()["include"], os.path.join(rocm, "include")]
+    torch_lib = os.path.join(os.path.dirname(torch.__file__), "lib")
+    cmd = [
+        hipcc_path(), "-x", "c++", "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-Wno-unused-command-line-argument",
+        "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1", f"-DTORCH_EXTENSION_NAME={EXT_NAME}", "-DTORCH_API_INCLUDE_EXTENSION_H",
+        f"-D_GLIBCXX_USE_CXX11_ABI={int(torch._C._GLIBCXX_USE_CXX11_ABI)}",
+        *[f"-I{p}" for p in includes], os.path.join(HERE, EXT_SOURCE), "-o", out,
+        f"-L{torch_lib}", "-lc10", "-lc10_hip", "-ltorch_cpu", "-ltorch_hip", "-ltorch", "-ltorch_python",
+        f"-L{PKG}", "-lspear_btp", "-Wl,-rpath,$ORIGIN",
+    ]
+    _run(cmd, verbose)
+    return out
+
+
 def is_stale() -> bool:
     out = lib_path()
     if not os.path.exists(out):
@@ -82,3 +117,4 @@ def is_stale() -> bool:
 
 if __name__ == "__main__":
     print(build(verbose=True))
+    print(build_extension(verbose=True))

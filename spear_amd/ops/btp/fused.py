@@ -30,7 +30,7 @@ def _mix_forward_impl(
     a_logits: torch.Tensor, b_logits: torch.Tensor, c: torch.Tensor, v: torch.Tensor, out: torch.Tensor,
     heads: int, kv_heads: int,
 ) -> None:
-    _btp.mix_forward(a_logits, b_logits, c, v, out, heads, kv_heads)
+    _btp.load_extension().mix_forward(a_logits, b_logits, c, v, out, heads, kv_heads)
 
 
 def _mix_forward_fake(
@@ -44,7 +44,7 @@ def _mix_backward_impl(
     a_logits: torch.Tensor, b_logits: torch.Tensor, c: torch.Tensor, v: torch.Tensor, dout: torch.Tensor,
     da: torch.Tensor, db: torch.Tensor, dc: torch.Tensor, dv: torch.Tensor, heads: int, kv_heads: int,
 ) -> None:
-    _btp.mix_backward(a_logits, b_logits, c, v, dout, da, db, dc, dv, heads, kv_heads)
+    _btp.load_extension().mix_backward(a_logits, b_logits, c, v, dout, da, db, dc, dv, heads, kv_heads)
 
 
 def _mix_backward_fake(
@@ -63,7 +63,7 @@ register_traceable_op(
 def _qkv_forward_impl(
     gate: torch.Tensor, k: torch.Tensor, q: torch.Tensor, v: torch.Tensor, out: torch.Tensor, heads: int, kv_heads: int
 ) -> None:
-    _btp.mix_forward(gate, k, q, v, out, heads, kv_heads, qkv_gate=True)
+    _btp.load_extension().mix_forward(gate, k, q, v, out, heads, kv_heads, True)
 
 
 def _qkv_forward_fake(
@@ -76,7 +76,7 @@ def _qkv_backward_impl(
     gate: torch.Tensor, k: torch.Tensor, q: torch.Tensor, v: torch.Tensor, dout: torch.Tensor,
     dgate: torch.Tensor, dk: torch.Tensor, dq: torch.Tensor, dv: torch.Tensor, heads: int, kv_heads: int,
 ) -> None:
-    _btp.mix_backward(gate, k, q, v, dout, dgate, dk, dq, dv, heads, kv_heads, qkv_gate=True)
+    _btp.load_extension().mix_backward(gate, k, q, v, dout, dgate, dk, dq, dv, heads, kv_heads, [], True)
 
 
 def _qkv_backward_fake(

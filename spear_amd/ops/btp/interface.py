@@ -7,8 +7,9 @@ function, same constants, the same two custom ops ``torch.ops.spear_btp.forward`
 (interface.py:126-161): backward returns ``(dA fp32 [B,H,L], dx [B,H,16,L] in x.dtype)``.
 
 Differences that do not change results:
-  * the native library is loaded on first use, so importing this module works on a machine
-    without a GPU (the reference imports its extension unconditionally, interface.py:16);
+  * the compiled binding (``spear_amd._btp_ext``, the counterpart of ``spear._btp``) is imported on
+    first use, so importing this module works before anything is built (the reference imports its
+    extension unconditionally, interface.py:16); a call without it raises, there is no fallback;
   * ``dA`` is allocated uninitialised, because the kernel writes every element
     (the reference zero-fills it, interface.py:158);
   * the carry checkpoint is not stored by default, because this backward recomputes the carries:
@@ -43,7 +44,7 @@ _FORWARD_FLAGS = _btp.FLAG_WRITE_CHECKPOINT if os.environ.get("SPEAR_BTP_WRITE_C
 def _forward_impl(
     coeff: torch.Tensor, x: torch.Tensor, y: torch.Tensor, checkpoint: torch.Tensor, k: int, wpb: int
 ) -> None:
-    _btp.forward(coeff, x, y, checkpoint, k, wpb, flags=_FORWARD_FLAGS)
+    _btp.load_extension().forward(coeff, x, y, checkpoint, k, wpb, _FORWARD_FLAGS)
 
 
 def _forward_fake(
@@ -62,7 +63,7 @@ def _backward_impl(
     k: int,
     wpb: int,
 ) -> None:
-    _btp.backward(coeff, x, dy, checkpoint, dx, dA, k, wpb)
+    _btp.load_extension().backward(coeff, x, dy, checkpoint, dx, dA, k, wpb)
 
 
 def _backward_fake(
@@ -98,7 +99,7 @@ def register_traceable_op(
 
 
 def _forward_log_impl(gate: torch.Tensor, x: torch.Tensor, y: torch.Tensor, k: int) -> None:
-    _btp.forward_log(gate, x, y, k)
+    _btp.load_extension().forward_log(gate, x, y, k)
 
 
 def _forward_log_fake(gate: torch.Tensor, x: torch.Tensor, y: torch.Tensor, k: int) -> None:
@@ -108,7 +109,7 @@ def _forward_log_fake(gate: torch.Tensor, x: torch.Tensor, y: torch.Tensor, k: i
 def _backward_log_impl(
     gate: torch.Tensor, x: torch.Tensor, dy: torch.Tensor, dx: torch.Tensor, dgate: torch.Tensor, k: int
 ) -> None:
-    _btp.backward_log(gate, x, dy, dx, dgate, k)
+    _btp.load_extension().backward_log(gate, x, dy, dx, dgate, k)
 
 
 def _backward_log_fake(

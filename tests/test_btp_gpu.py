@@ -309,6 +309,16 @@ def test_measurement_aids_move_the_bytes_they_are_timed_for(slabs):
         torch.cuda.synchronize()
         assert torch.equal(out[:n], want)
         assert bool((out[n:] == 0xA5).all())
+    for shape in range(5):  # the alternative launch shapes of the probe move the same bytes
+        for second, want in ((None, a), (b, a ^ b)):
+            out.fill_(0xA5)
+            rc = lib.spear_btp_stream_probe_shape(a.data_ptr(), None if second is None else second.data_ptr(),
+                                                  out.data_ptr(), ctypes.c_ulonglong(n), shape, sp)
+            assert rc == 0, lib.spear_btp_last_error()
+            torch.cuda.synchronize()
+            assert torch.equal(out[:n], want), shape
+            assert bool((out[n:] == 0xA5).all()), shape
+    assert lib.spear_btp_stream_probe_shape(a.data_ptr(), None, out.data_ptr(), ctypes.c_ulonglong(n), 5, sp) == -1
     out.fill_(0xA5)
     assert lib.spear_btp_copy(a.data_ptr(), out.data_ptr(), ctypes.c_ulonglong(n), sp) == 0
     torch.cuda.synchronize()

@@ -258,3 +258,46 @@ def test_layer_forward_replays_as_a_hip_graph(method):
             # same kernels on the same data; a library GEMM is allowed its last bit
             err = float((static_y.float() - want.float()).abs().max())
             assert err <= 2.0 ** -7 * float(want.float().abs().max()), f"replay {i}: {err}"
+
+
+def test_compiled_binding_matches_the_ctypes_route_and_the_reference_messages():
+    """`spear._btp.forward / backward` (the compiled binding, reference signature) give the same bits as the
+    ctypes route over the same C ABI, and refuse what the reference's binding refuses, in its words
+    (csrc/btp/_bindings.cu:19-60)."""
+    import spear._btp as ext
+
+    from helpers import make_inputs
+    from spear_amd import _btp
+
+    coeff, x, dy = (t.to(DEV) for t in make_inputs(3, 5, 272, seed=99))
+    B, H, _, L = x.shape
+    ck = torch.empty(B, H, L // 16, 16, device=DEV)
+    y1, y2 = torch.empty_like(x), torch.empty_like(x)
+    ext.forward(coeff, x, y1, ck, 2, 32)
+    _btp.forward(coeff, x, y2, ck, 2, 32)
+    dx1, dx2 = torch.empty_like(x), torch.empty_like(x)
+    dA1, dA2 = torch.empty(B, H, L, device=DEV), torch.empty(B, H, L, device=DEV)
+    ext.backward(coeff, x, dy, ck, dx1, dA1, 2, 32)
+    _btp.backward(coeff, x, dy, ck, dx2, dA2, 2, 32)
+    torch.cuda.synchronize()
+    assert torch.equal(y1, y2) and torch.equal(dx1, dx2) and torch.equal(dA1, dA2)
+    for args, msg in (
+        ((coeff, x, y1, ck, 3, 32), "k must be 1 or 2."),
+        ((coeff, x, y1, ck, 2, 5), "Unsupported WPB value: 5"),
+        ((coeff.float(), x, y1, ck, 2, 32), "coeff must be float16 or bfloat16."),
+        ((coeff, x.half(), y1, ck, 2, 32), "x dtype must match coeff."),
+        ((coeff, x, y1.half(), ck, 2, 32), "y must be float32 or match x dtype."),
+        ((coeff, x, y1, ck.half(), 2, 32), "checkpoint must be float32."),
+        ((coeff, x[:, :, :8], y1, ck, 2, 32), r"Channel dim \(DH\) must be 16."),
+        ((coeff[:, :, :100], x[..., :100], y1[..., :100], ck, 2, 32), "Length L must be multiple of 16"),
+        ((coeff[:, :1], x, y1, ck, 2, 32), "coeff must have shape"),
+        ((coeff, x.transpose(0, 1).contiguous().transpose(0, 1), y1, ck, 2, 32), "x must be contiguous"),
+    ):
+        with pytest.raises(RuntimeError, match=msg):
+            ext.forward(*args)
+    with pytest.raises(RuntimeError, match="dx dtype must match x."):
+        ext.backward(coeff, x, dy, ck, dx1.float(), dA1, 2, 32)
+    with pytest.raises(RuntimeError, match="dA must be float32."):
+        ext.backward(coeff, x, dy, ck, dx1, dA1.half(), 2, 32)
+    with pytest.raises(RuntimeError, match="Unsupported WPB value for backward: 7"):
+        ext.backward(coeff, x, dy, ck, dx1, dA1, 2, 7)
