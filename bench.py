@@ -263,6 +263,20 @@ def main() -> int:
     best_copy = max(v["copy_1r1w"] for v in probe_shapes.values())
     best_2r1w = max(v["nt_2r1w"] for v in probe_shapes.values())
 
+    # one direction at a time: HBM serves reads and writes one after the other, so a kernel that reads R bytes
+    # and writes W bytes takes at least R / read_rate + W / write_rate; this is the floor the kernels are up against
+    def one_way(shape, second):
+        def fn(s):
+            rc = lib.spear_btp_stream_probe_shape(s["x"].data_ptr(), s["dy"].data_ptr() if second else None,
+                                                  s["dx"].data_ptr(), ctypes.c_ulonglong(nbytes), shape, sp)
+            assert rc == 0, lib.spear_btp_last_error()
+        return kernel_ms(fn)
+    read_rate = 2 * nbytes / (one_way(5, True) * 1e-3) / 1e9
+    write_rate = nbytes / (one_way(6, False) * 1e-3) / 1e9
+    def serial_floor(read_bytes, write_bytes):  # GB/s of algorithmic bytes if reads and writes just add up
+        return (read_bytes + write_bytes) / (read_bytes / read_rate + write_bytes / write_rate)
+    floor_fwd, floor_bwd = serial_floor(34, 32), serial_floor(66, 36)
+
     # log-space gate entry points on the same shape (fp32 gate in, fp32 dgate out: 68 + 108 B per unit)
     for s_ in sets:
         s_["gate"] = torch.log(s_["coeff"].float()).contiguous()
@@ -321,6 +335,13 @@ def main() -> int:
                                                 B, L, H, H, 0, 0, sp)
             assert rc == 0, lib.spear_btp_last_error()
 
+        def mix_bwd_tile(s):  # the other work split of the same backward (SPEAR_MIX_TILE_SPLIT)
+            rc = lib.spear_phalanx_mix_backward(s["a"].data_ptr(), s["b"].data_ptr(), s["c"].data_ptr(),
+                                                s["v"].data_ptr(), s["dout"].data_ptr(), s["da"].data_ptr(),
+                                                s["db"].data_ptr(), s["dc"].data_ptr(), s["dv"].data_ptr(),
+                                                B, L, H, H, 0, 0x4, sp)
+            assert rc == 0, lib.spear_btp_last_error()
+
         def unfused_stage(a, b, c, v):  # what the layer does around the stand-alone kernel (swr.py)
             A = torch.sigmoid(a).transpose(1, 2)
             V = v.transpose(1, 2).view(B, H, 16, L)
@@ -374,6 +395,7 @@ def main() -> int:
 
         mix_ms, unfused_ms = kernel_ms_over(mix, msets), kernel_ms_over(mix_unfused, msets)
         mix_bwd_ms, unfused_train_ms = kernel_ms_over(mix_bwd, msets), kernel_ms_over(mix_unfused_train, msets)
+        mix_bwd_tile_ms = kernel_ms_over(mix_bwd_tile, msets)
         mix_bytes = B * L * H * (2 + 3 * 32 + 32)          # a, b, c, v read; out written
         mix_bwd_bytes = B * L * H * (2 + 4 * 32 + 2 + 3 * 32)  # a, b, c, v, dout read; da, db, dc, dv written
         fused = {
@@ -384,6 +406,8 @@ def main() -> int:
                 "avg_launch_ms": mix_bwd_ms, "algorithmic_bytes_per_launch": mix_bwd_bytes,
                 "achieved": mix_bwd_bytes / (mix_bwd_ms * 1e-3) / 1e9,
                 "frac": mix_bwd_bytes / (mix_bwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+                "tile_split_avg_launch_ms": mix_bwd_tile_ms,
+                "tile_split_frac": mix_bwd_bytes / (mix_bwd_tile_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
             },
             "fwd_plus_bwd_ms": mix_ms + mix_bwd_ms,
             "same_stage_fwd_plus_bwd_from_pytorch_ops_plus_btp_kernels_ms": unfused_train_ms,
@@ -672,6 +696,13 @@ def main() -> int:
             "other_launch_shapes_GBps": probe_shapes,
             "forward_kernel_vs_best_copy_shape": fwd_gbps / best_copy,
             "backward_kernel_vs_best_2r1w_shape": bwd_gbps / best_2r1w,
+            "read_only_GBps": read_rate, "write_only_GBps": write_rate,
+            "serial_read_plus_write_model": {
+                "what": "algorithmic GB/s if a kernel's reads and writes run one after the other at the two rates above",
+                "forward_34R_32W": floor_fwd, "backward_66R_36W": floor_bwd,
+                "forward_kernel_vs_model": fwd_gbps / floor_fwd, "backward_kernel_vs_model": bwd_gbps / floor_bwd,
+                "fused_forward_98R_32W": serial_floor(98, 32), "fused_backward_130R_98W": serial_floor(130, 98),
+            },
         },
         "public_op": public_op,
     }

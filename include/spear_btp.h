@@ -117,6 +117,13 @@ int spear_phalanx_mix_forward(const void* a_logit, const void* b_logit, const vo
  * elements). Inputs keep their types. Not combinable with the column sums of _backward_ex. */
 #define SPEAR_MIX_F32_RESULTS 0x2u
 
+/* Flag for spear_phalanx_mix_backward / _backward_ex: the other work split of the same backward -- one
+ * wavefront per 16-step block with the two carries handed between neighbouring blocks through LDS, instead of
+ * wavefronts that walk through time. Same results up to fp32 rounding; 3 % faster at B=1024 L=128 H=32, within
+ * 1 % elsewhere, so it is not the default (SPEAR_BTP_FUSED_BWD=tile in the environment makes it the default for
+ * calls it can serve). Not combinable with column sums or SPEAR_MIX_F32_RESULTS. */
+#define SPEAR_MIX_TILE_SPLIT 0x4u
+
 /* Backward of spear_phalanx_mix_forward: reads a_logit, b_logit, c, v and the upstream gradient
  * dout [B, L, H * 16]; writes da_logit [B, L, H], db_logit and dc [B, L, kv_heads * 16] (summed over
  * the heads sharing a kv head) and dv [B, L, H * 16] -- every element, no accumulation, all in
@@ -237,8 +244,12 @@ int spear_btp_stream_probe(const void* src_a, const void* src_b, void* dst, unsi
  * alternatives: shape 0 = spear_btp_stream_probe (one 4 KiB slab per wavefront); 1 = two slabs per
  * wavefront, all loads issued before the first store; 2 = four slabs per wavefront in a loop that issues
  * the next slab's loads before the current slab's stores; 3 = that loop as a persistent grid striding over
- * the buffer; 4 = one 16-byte element per thread. Same arguments and result as spear_btp_stream_probe. */
-#define SPEAR_BTP_PROBE_SHAPES 5
+ * the buffer; 4 = one 16-byte element per thread; 5 = reads only (src_a, and src_b if given; `dst` is not
+ * written unless every input word is all ones); 6 = writes only (`dst` is filled, nothing is read). HBM serves
+ * reads and writes one after the other, so shapes 5 and 6 give the two rates from which the floor of a mixed
+ * kernel follows: R bytes read and W bytes written take at least R / read rate + W / write rate. Same arguments
+ * and result as spear_btp_stream_probe. */
+#define SPEAR_BTP_PROBE_SHAPES 7
 int spear_btp_stream_probe_shape(const void* src_a, const void* src_b, void* dst, unsigned long long bytes, int shape,
                                  void* stream);
 

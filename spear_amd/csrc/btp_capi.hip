@@ -6,6 +6,7 @@
 #include <stdarg.h>
 #include <stdint.h>
 #include <stdio.h>
+#include <stdlib.h>
 
 #include "../../include/spear_btp.h"
 #include "btp_launch.h"
@@ -44,7 +45,7 @@ int check_common(const char* who, int B, int H, int L, int k, int in_dtype, int 
 
 extern "C" {
 
-int spear_btp_abi_version(void) { return 11; }
+int spear_btp_abi_version(void) { return 12; }
 
 const char* spear_btp_last_error(void) { return g_error; }
 
@@ -211,12 +212,23 @@ int spear_phalanx_mix_backward_ex(const void* a_logit, const void* b_logit, cons
   const char* who = "spear_phalanx_mix_backward";
   const void* const ptrs[9] = {a_logit, b_logit, c, v, dout, da_logit, db_logit, dc, dv};
   const int lds[4] = {ld_da, ld_db, ld_dc, ld_dv};
-  if (int rc = check_mix_backward(who, ptrs, lds, B, L, H, kv_heads, dtype, flags, SPEAR_MIX_QKV_GATE | SPEAR_MIX_F32_RESULTS))
+  if (int rc = check_mix_backward(who, ptrs, lds, B, L, H, kv_heads, dtype, flags,
+                                  SPEAR_MIX_QKV_GATE | SPEAR_MIX_F32_RESULTS | SPEAR_MIX_TILE_SPLIT))
     return rc < 0 ? rc : 0;
   const bool qkv = (flags & SPEAR_MIX_QKV_GATE) != 0, f32 = (flags & SPEAR_MIX_F32_RESULTS) != 0;
+  // the tile split is a flag, or the process-wide default when SPEAR_BTP_FUSED_BWD=tile is set (read once)
+  static const bool tile_default = [] {
+    const char* e = getenv("SPEAR_BTP_FUSED_BWD");
+    return e != nullptr && e[0] == 't';
+  }();
+  const bool tile_asked = (flags & SPEAR_MIX_TILE_SPLIT) != 0;
   const bool sums = sum_da || sum_db || sum_dc;
   if (sums && qkv) return fail(SPEAR_BTP_EINVAL, "%s: column sums are for the layer form, not SPEAR_MIX_QKV_GATE", who);
   if (sums && f32) return fail(SPEAR_BTP_EINVAL, "%s: column sums are not available with SPEAR_MIX_F32_RESULTS", who);
+  if (tile_asked && (sums || f32))
+    return fail(SPEAR_BTP_EINVAL, "%s: SPEAR_MIX_TILE_SPLIT has neither column sums nor fp32 results", who);
+  const bool tile = (tile_asked || (tile_default && !sums && !f32)) &&
+                    (long long)B * ((L / 16 + 3) / 4) * ((H + 7) / 8) < (1ll << 31);
   if (sums) {
     if (!sum_da || !sum_db || !sum_dc) return fail(SPEAR_BTP_ENULL, "%s: the three sum arrays must be given together", who);
     if (!aligned16(sum_da) || !aligned16(sum_db) || !aligned16(sum_dc))
@@ -226,7 +238,7 @@ int spear_phalanx_mix_backward_ex(const void* a_logit, const void* b_logit, cons
       return fail(SPEAR_BTP_EINVAL, "%s: sum arrays must have %lld rows for this shape (got %lld)", who, want, sum_rows);
   }
   spear_btp::MixBwdArgs a{a_logit, b_logit, c, v, dout, da_logit, db_logit, dc, dv, B, L, H, H / kv_heads, dtype,
-                          sum_da, sum_db, sum_dc, ld_da, ld_db, ld_dc, ld_dv, qkv, f32};
+                          sum_da, sum_db, sum_dc, ld_da, ld_db, ld_dc, ld_dv, qkv, f32, tile};
   const hipError_t err = spear_btp::fused_mix_backward(a, static_cast<hipStream_t>(stream));
   if (err != hipSuccess) return fail(SPEAR_BTP_ELAUNCH, "%s: launch failed: %s", who, hipGetErrorString(err));
   return 0;

@@ -557,6 +557,382 @@ __global__ __launch_bounds__(64 * kWaves) void phalanx_mix_bwd_kernel(
 }
 
 
+// ==========================================================================================
+// Backward of the fused mixing stage, tile form (SPEAR_MIX_TILE_SPLIT; not the default): the same
+// mathematics with a different work split. Measured against the walking kernel above at B=1024 L=128 H=32 it is
+// 3 % faster (180.6 against 186 us), at B=16 L=8192 H=64 1 % slower, at B=64 L=2048 H=128 1 % faster; it stays in
+// the library as the measured alternative. One
+// wavefront owns ONE 16-step block of 128 features and runs no loop: every load is issued at the start, every
+// store at the end, and a workgroup (8 wavefronts = octs_w head groups x nb_w consecutive blocks of one batch
+// row) lives for a few microseconds. Copy loops with this kernel's traffic show why: wavefronts that walk
+// through time with two register sets reach 0.65 of the HBM peak whatever the chunking, short-lived tiles
+// 0.71-0.74 (reads and writes do not overlap on the memory bus, so what counts is how quickly a wavefront
+// turns from its read phase to its write phase and makes room for the next one).
+//
+// The one-hop structure makes tiles independent up to two neighbour quantities, both LOCAL to a block:
+//   c_out(i)  = terminal value of the zero-started forward recurrence over block i      (carry into block i+1)
+//   dC_out(i) = a_0 R_0 of the zero-started reverse recurrence over block i             (gradient carry into block i-1)
+// Every wavefront computes both for its own block first and leaves them in LDS; after the kernel's single
+// barrier its neighbours pick them up. The first and last block of a workgroup have no neighbour inside it:
+// those wavefronts read two operands of the block beyond the edge as well (b, v for the forward carry or dout,
+// c for the gradient carry; cacheable loads, the neighbouring workgroup reads the same lines at about the
+// same time) and run the one recurrence they need on them.
+//
+// With h the state of the carry-started recurrence (h_{-1} = c_in, h_r = a_r h_{r-1} + x_r) and
+// dX_r = R_r + (prod_{j>r} a_j) dC, per step
+//   dc_r = dout_r h_r ;  dv_r = dout_r + dX_r G_r ;  db_r = dX_r v_r G_r (1 - G_r)
+//   dA_r = sum over the head's channels of dX_r h_{r-1}  -  (prod_{j != r} a_j) sum over channels of dC c_in
+// (the second term takes out the two-hop path c_in -> dC that h carries but the operator does not have).
+// ==========================================================================================
+#ifndef SPEAR_FUSED_TILE_WAVES
+#define SPEAR_FUSED_TILE_WAVES 8
+#endif
+constexpr int kTileWaves = SPEAR_FUSED_TILE_WAVES;
+
+// v of the lane `kCtrl` names within the lane's DPP row of 16, or 1.0 where that lane does not exist
+template <int kCtrl>
+__device__ __forceinline__ float dpp_or_one(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0x3f800000, __float_as_int(v), kCtrl, 0xF, 0xF, false));
+}
+
+// For a value held by the 16 lanes of a DPP row (lane t = step t): the product over all OTHER lanes' values.
+__device__ __forceinline__ float product_of_the_others(float a) {
+  float p = a, q = a;  // inclusive prefix and suffix products (row_shr / row_shl by 1, 2, 4, 8)
+  p *= dpp_or_one<0x111>(p); p *= dpp_or_one<0x112>(p); p *= dpp_or_one<0x114>(p); p *= dpp_or_one<0x118>(p);
+  q *= dpp_or_one<0x101>(q); q *= dpp_or_one<0x102>(q); q *= dpp_or_one<0x104>(q); q *= dpp_or_one<0x108>(q);
+  return dpp_or_one<0x111>(p) * dpp_or_one<0x101>(q);
+}
+
+#ifndef SPEAR_FUSED_TILE_WAVES_PER_EU  // 4 waves per SIMD (two workgroups per CU) need <= 128 VGPRs
+#define SPEAR_FUSED_TILE_WAVES_PER_EU 4
+#endif
+template <class E, bool kQkv>
+__global__ __launch_bounds__(64 * kTileWaves) __attribute__((amdgpu_waves_per_eu(SPEAR_FUSED_TILE_WAVES_PER_EU)))
+void phalanx_mix_bwd_tile_kernel(
+    const uint16_t* __restrict__ a_logit, const uint16_t* __restrict__ b_logit, const uint16_t* __restrict__ c_in,
+    const uint16_t* __restrict__ v_in, const uint16_t* __restrict__ dout, uint16_t* __restrict__ da_logit,
+    uint16_t* __restrict__ db_logit, uint16_t* __restrict__ dc, uint16_t* __restrict__ dv, int ld_da, int ld_db, int ld_dc,
+    int ld_dv, int L, int H, int kv_groups, int octs_w, int nb_w, int tiles, int oct_groups) {
+  // per wavefront: decay of its block, product of the block's other decays per step, decay of the block beyond the edge
+  __shared__ __align__(16) float gate_tiles[kTileWaves][3][kHeadsPerWave * kGateRow];
+  __shared__ float2 carry_out[kTileWaves][2][64];  // [0] dC_out, [1] c_out of the wavefront's block, per lane
+
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+  // workgroup -> (batch row, time tile, group of octs_w head groups); head groups fastest, so that workgroups
+  // next to each other in launch order read neighbouring features of the same time steps
+  const unsigned wg = blockIdx.x;
+  const int og = (int)(wg % (unsigned)oct_groups);
+  const unsigned tt = wg / (unsigned)oct_groups;
+  const int tile = (int)(tt % (unsigned)tiles);
+  const long brow = tt / (unsigned)tiles;
+  const int o = wave % octs_w, bl = wave / octs_w;  // octs_w * nb_w == kTileWaves
+  const int octs = (H + kHeadsPerWave - 1) / kHeadsPerWave;
+  const int ho = (og * octs_w + o) * kHeadsPerWave;
+  const int t0 = (tile * nb_w + bl) * kTile;
+  const bool valid = ho < H && t0 < L;  // wave-uniform; a wavefront without a block only joins the barrier
+  (void)octs;
+
+  const int head_local = lane >> 3;
+  const bool real = ho + head_local < H;
+  const int head = real ? ho + head_local : H - 1;
+  const int d0 = (lane & 7) << 1;
+  const int F = H * kChan, Fkv = (H / kv_groups) * kChan;
+  const int stride = 2 * F, kv_stride = 2 * Fkv;
+  constexpr int kRsrcFlags = 0x00020000;
+  constexpr int kGateBytes = kQkv ? 4 : 2;
+  constexpr int kDaBytes = kQkv ? 4 : 2;
+  constexpr int kGradBytes = 2;
+  const long big = brow * L * F, kvbig = brow * L * Fkv, small = brow * L * H;
+  auto rsrc = [&](const uint16_t* p, long off, int bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(p + off), 0, bytes, kRsrcFlags);
+  };
+  const __amdgpu_buffer_rsrc_t rb = rsrc(b_logit, kvbig, L * kv_stride), rc = rsrc(c_in, kvbig, L * kv_stride),
+                               rv = rsrc(v_in, big, L * stride), rg = rsrc(dout, big, L * stride),
+                               ra = rsrc(a_logit, small * (kGateBytes / 2), L * H * kGateBytes),
+                               rdb = rsrc(db_logit, brow * L * ld_db * (kGradBytes / 2), L * ld_db * kGradBytes),
+                               rdc = rsrc(dc, brow * L * ld_dc * (kGradBytes / 2), L * ld_dc * kGradBytes),
+                               rdv = rsrc(dv, brow * L * ld_dv * (kGradBytes / 2), L * ld_dv * kGradBytes),
+                               rda = rsrc(da_logit, brow * L * ld_da * (kDaBytes / 2), L * ld_da * kDaBytes);
+  const int f_lane = 2 * (head * kChan + d0);
+  const int kv_lane = 2 * ((head / kv_groups) * kChan + d0);
+  const int o_lane = real ? f_lane * (kGradBytes / 2) : 0x7ffffff0;
+  const int okv_lane = (real && (head % kv_groups) == 0) ? kv_lane * (kGradBytes / 2) : 0x7ffffff0;
+  const int gt = lane & 15, ghead = min(ho + 2 * (lane >> 4), H - 2);
+  const int a_lane = kGateBytes * (gt * H + ghead);
+  const int da_lane = real ? kDaBytes * ((2 * (lane & 7)) * ld_da + head) : 0x7ffffff0;
+  constexpr int kNt = 2;
+
+  // the block beyond the workgroup's edge that this wavefront has to look at (at most one: nb_w >= 2)
+  const bool halo_prev = valid && bl == 0 && t0 > 0;                    // needs c_out of block t0 - 16
+  const bool halo_next = valid && bl == nb_w - 1 && t0 + kTile < L;     // needs dC_out of block t0 + 16
+  const int th = halo_prev ? t0 - kTile : t0 + kTile;
+
+  // ---- every global read, before anything waits
+  uint32_t b[16], c[16], v[16], g[16], h0[16], h1[16];
+  GateWords araw = {0u, 0u}, haraw = {0u, 0u};
+  auto load_gate = [&](int t) {
+    GateWords w;
+    w.lo = __builtin_amdgcn_raw_buffer_load_b32(ra, a_lane, t * H * kGateBytes, 0);
+    w.hi = kQkv ? __builtin_amdgcn_raw_buffer_load_b32(ra, a_lane + 4, t * H * kGateBytes, 0) : 0u;
+    return w;
+  };
+  // Wavefronts at a workgroup edge read the block beyond the edge first and their own b, v only once those 32
+  // registers are free again (b and v are not needed before the local forward recurrence); the other
+  // wavefronts issue everything at once. That keeps the kernel within 128 registers = two workgroups per CU.
+  const bool halo = halo_prev || halo_next;
+  auto load_bv = [&]() {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      b[r] = __builtin_amdgcn_raw_buffer_load_b32(rb, kv_lane, (t0 + r) * kv_stride, kNt);
+      v[r] = __builtin_amdgcn_raw_buffer_load_b32(rv, f_lane, (t0 + r) * stride, kNt);
+    }
+  };
+  if (valid) {
+    araw = load_gate(t0);
+    if (halo) haraw = load_gate(th);
+    if (halo_prev) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        h0[r] = __builtin_amdgcn_raw_buffer_load_b32(rb, kv_lane, (th + r) * kv_stride, 0);
+        h1[r] = __builtin_amdgcn_raw_buffer_load_b32(rv, f_lane, (th + r) * stride, 0);
+      }
+    } else if (halo_next) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        h0[r] = __builtin_amdgcn_raw_buffer_load_b32(rg, f_lane, (th + r) * stride, 0);
+        h1[r] = __builtin_amdgcn_raw_buffer_load_b32(rc, kv_lane, (th + r) * kv_stride, 0);
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      g[r] = __builtin_amdgcn_raw_buffer_load_b32(rg, f_lane, (t0 + r) * stride, kNt);
+      c[r] = __builtin_amdgcn_raw_buffer_load_b32(rc, kv_lane, (t0 + r) * kv_stride, kNt);
+    }
+    if (!halo) load_bv();
+  }
+  __builtin_amdgcn_sched_barrier(0);
+
+  float* ta = gate_tiles[wave][0];
+  float* te = gate_tiles[wave][1];
+  float* tn = gate_tiles[wave][2];
+  auto write_tile = [&](float* tile_, float x0, float x1) {
+    tile_[(2 * (lane >> 4)) * kGateRow + gt] = x0;
+    tile_[(2 * (lane >> 4) + 1) * kGateRow + gt] = x1;
+  };
+
+  float cin0 = 0.0f, cin1 = 0.0f, dC0 = 0.0f, dC1 = 0.0f;
+  float R[32];  // local reverse states, later dX, channel pair interleaved: R[2 r], R[2 r + 1]
+  if (valid) {
+    const float2 a01 = decay_pair<E, kQkv>(araw);
+    write_tile(ta, a01.x, a01.y);
+    write_tile(te, product_of_the_others(a01.x), product_of_the_others(a01.y));
+    if (halo) {
+      const float2 n01 = decay_pair<E, kQkv>(haraw);
+      write_tile(tn, n01.x, n01.y);
+    }
+    wave_lds_handover();
+
+    // ---- the block beyond the edge first, so that its 32 registers are free again before R is formed
+    if (halo_prev) {
+#pragma unroll
+      for (int c4 = 0; c4 < 4; ++c4) {
+        const float4 q = *reinterpret_cast<const float4*>(tn + head_local * kGateRow + 4 * c4);
+        const float a4[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int r = 4 * c4 + i;
+          cin0 = fmaf(a4[i], cin0, input_gate<kQkv>(E::lo(h0[r])) * E::lo(h1[r]));
+          cin1 = fmaf(a4[i], cin1, input_gate<kQkv>(E::hi(h0[r])) * E::hi(h1[r]));
+        }
+        asm volatile("" ::: "memory");
+      }
+    } else if (halo_next) {
+      float r0 = 0.0f, r1 = 0.0f, up = 0.0f;
+#pragma unroll
+      for (int c4 = 3; c4 >= 0; --c4) {
+        const float4 q = *reinterpret_cast<const float4*>(tn + head_local * kGateRow + 4 * c4);
+        const float a4[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+        for (int i = 3; i >= 0; --i) {
+          const int r = 4 * c4 + i;
+          r0 = fmaf(up, r0, E::lo(h0[r]) * E::lo(h1[r]));
+          r1 = fmaf(up, r1, E::hi(h0[r]) * E::hi(h1[r]));
+          up = a4[i];
+        }
+        asm volatile("" ::: "memory");
+      }
+      dC0 = up * r0;
+      dC1 = up * r1;
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    if (halo) load_bv();
+    __builtin_amdgcn_sched_barrier(0);
+
+    // Decays are read from the LDS tile four steps at a time, next to their use (a broadcast read for the 8
+    // lanes of a head), rather than held in 16 registers through every pass; the compiler barriers keep the
+    // reads where they are written.
+    // ---- local reverse recurrence (upstream gradient of the recurrence: dout * c)
+    {
+      float r0 = 0.0f, r1 = 0.0f, up = 0.0f;  // up: decay of the step after the current one
+#pragma unroll
+      for (int c4 = 3; c4 >= 0; --c4) {
+        const float4 q = *reinterpret_cast<const float4*>(ta + head_local * kGateRow + 4 * c4);
+        const float a4[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+        for (int i = 3; i >= 0; --i) {
+          const int r = 4 * c4 + i;
+          r0 = fmaf(up, r0, E::lo(g[r]) * E::lo(c[r]));
+          r1 = fmaf(up, r1, E::hi(g[r]) * E::hi(c[r]));
+          R[2 * r] = r0;
+          R[2 * r + 1] = r1;
+          up = a4[i];
+        }
+        asm volatile("" ::: "memory");
+      }
+      carry_out[wave][0][lane] = make_float2(up * r0, up * r1);
+    }
+    // ---- local forward recurrence: only its terminal value is needed here
+    {
+      float l0 = 0.0f, l1 = 0.0f;
+#pragma unroll
+      for (int c4 = 0; c4 < 4; ++c4) {
+        const float4 q = *reinterpret_cast<const float4*>(ta + head_local * kGateRow + 4 * c4);
+        const float a4[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int r = 4 * c4 + i;
+          l0 = fmaf(a4[i], l0, input_gate<kQkv>(E::lo(b[r])) * E::lo(v[r]));
+          l1 = fmaf(a4[i], l1, input_gate<kQkv>(E::hi(b[r])) * E::hi(v[r]));
+        }
+        asm volatile("" ::: "memory");
+      }
+      carry_out[wave][1][lane] = make_float2(l0, l1);
+    }
+  }
+  __syncthreads();  // the kernel's only workgroup barrier; wavefronts without a block arrive here directly
+  if (!valid) return;
+
+  if (bl > 0) {  // the block before this one belongs to the wavefront octs_w places down
+    const float2 q = carry_out[wave - octs_w][1][lane];
+    cin0 = q.x;
+    cin1 = q.y;
+  }
+  if (bl < nb_w - 1 && t0 + kTile < L) {
+    const float2 q = carry_out[wave + octs_w][0][lane];
+    dC0 = q.x;
+    dC1 = q.y;
+  }
+
+  // dX_r = R_r + (prod_{j > r} a_j) dC, in place
+  {
+    float q0 = dC0, q1 = dC1;
+#pragma unroll
+    for (int c4 = 3; c4 >= 0; --c4) {
+      const float4 q = *reinterpret_cast<const float4*>(ta + head_local * kGateRow + 4 * c4);
+      const float a4[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+      for (int i = 3; i >= 0; --i) {
+        const int r = 4 * c4 + i;
+        R[2 * r] += q0;
+        R[2 * r + 1] += q1;
+        q0 *= a4[i];
+        q1 *= a4[i];
+      }
+      asm volatile("" ::: "memory");
+    }
+  }
+
+  // ---- forward pass: state, gradients, per-step partial sums of dA
+  float e[16];
+  float hs0 = cin0, hs1 = cin1;  // h_{r-1}
+#pragma unroll
+  for (int c4 = 0; c4 < 4; ++c4) {
+    const float4 qa = *reinterpret_cast<const float4*>(ta + head_local * kGateRow + 4 * c4);
+    const float a4[4] = {qa.x, qa.y, qa.z, qa.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int r = 4 * c4 + i;
+      const float G0 = input_gate<kQkv>(E::lo(b[r])), G1 = input_gate<kQkv>(E::hi(b[r]));
+      const float v0 = E::lo(v[r]), v1 = E::hi(v[r]);
+      const float go0 = E::lo(g[r]), go1 = E::hi(g[r]);
+      const float dX0 = R[2 * r], dX1 = R[2 * r + 1];
+      e[r] = fmaf(dX0, hs0, dX1 * hs1);
+      hs0 = fmaf(a4[i], hs0, G0 * v0);
+      hs1 = fmaf(a4[i], hs1, G1 * v1);
+      float dc0 = go0 * hs0, dc1 = go1 * hs1;
+      float db0 = dX0 * v0, db1 = dX1 * v1;  // dX * v: the gradient of k in the q/k/v form
+      if constexpr (!kQkv) {
+        db0 *= G0 * (1.0f - G0);
+        db1 *= G1 * (1.0f - G1);
+      }
+      if (kv_groups > 1) {  // wave-uniform: sum over the heads that share this kv head
+        dc0 += row_xor<8>(dc0); dc1 += row_xor<8>(dc1); db0 += row_xor<8>(db0); db1 += row_xor<8>(db1);
+        if (kv_groups > 2) {
+          dc0 += lane_xor(dc0, lane, 16); dc1 += lane_xor(dc1, lane, 16);
+          db0 += lane_xor(db0, lane, 16); db1 += lane_xor(db1, lane, 16);
+        }
+        if (kv_groups > 4) {
+          dc0 += lane_xor(dc0, lane, 32); dc1 += lane_xor(dc1, lane, 32);
+          db0 += lane_xor(db0, lane, 32); db1 += lane_xor(db1, lane, 32);
+        }
+      }
+      const float dv0 = fmaf(dX0, G0, go0), dv1 = fmaf(dX1, G1, go1);
+      __builtin_amdgcn_raw_buffer_store_b32(E::pack2(dc0, dc1), rdc, okv_lane, (t0 + r) * 2 * ld_dc, kNt);
+      __builtin_amdgcn_raw_buffer_store_b32(E::pack2(dv0, dv1), rdv, o_lane, (t0 + r) * 2 * ld_dv, kNt);
+      __builtin_amdgcn_raw_buffer_store_b32(E::pack2(db0, db1), rdb, okv_lane, (t0 + r) * 2 * ld_db, kNt);
+    }
+    asm volatile("" ::: "memory");
+  }
+
+  // ---- dA: sum over the 8 lanes (16 channels) of the head, transposing: lane k keeps steps 2k, 2k+1
+  const int kk = lane & 7;
+  float f8[8], f4[4];
+  {
+    const bool hi = kk & 4;
+#pragma unroll
+    for (int t = 0; t < 8; ++t) {
+      const float keep = hi ? e[t + 8] : e[t], send = hi ? e[t] : e[t + 8];
+      f8[t] = keep + row_xor<4>(send);
+    }
+  }
+  {
+    const bool hi = kk & 2;
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      const float keep = hi ? f8[t + 4] : f8[t], send = hi ? f8[t] : f8[t + 4];
+      f4[t] = keep + row_xor<2>(send);
+    }
+  }
+  float s0, s1;
+  {
+    const bool hi = kk & 1;
+    const float k0 = hi ? f4[2] : f4[0], n0 = hi ? f4[0] : f4[2];
+    const float k1 = hi ? f4[3] : f4[1], n1 = hi ? f4[1] : f4[3];
+    s0 = k0 + row_xor<1>(n0);
+    s1 = k1 + row_xor<1>(n1);
+  }
+  // the two-hop path c_in -> dC, summed over the head's channels
+  float two_hop = fmaf(dC0, cin0, dC1 * cin1);
+  two_hop += row_xor<1>(two_hop);
+  two_hop += row_xor<2>(two_hop);
+  two_hop += row_xor<4>(two_hop);
+  const float2 aa = *reinterpret_cast<const float2*>(ta + head_local * kGateRow + 2 * kk);
+  const float2 ee = *reinterpret_cast<const float2*>(te + head_local * kGateRow + 2 * kk);
+  s0 = fmaf(-ee.x, two_hop, s0);
+  s1 = fmaf(-ee.y, two_hop, s1);
+  // d/d a_logit = dA a (1 - a);  d/d gate = dA a  (gate = log a)
+  const float da0 = kQkv ? s0 * aa.x : s0 * aa.x * (1.0f - aa.x), da1 = kQkv ? s1 * aa.y : s1 * aa.y * (1.0f - aa.y);
+  if constexpr (kDaBytes == 4) {
+    __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(da0), rda, da_lane, t0 * ld_da * 4, 0);
+    __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(da1), rda, da_lane + 4 * ld_da, t0 * ld_da * 4, 0);
+  } else {
+    const uint32_t dap = E::pack2(da0, da1);
+    __builtin_amdgcn_raw_buffer_store_b16((unsigned short)(dap & 0xffffu), rda, da_lane, t0 * ld_da * 2, 0);
+    __builtin_amdgcn_raw_buffer_store_b16((unsigned short)(dap >> 16), rda, da_lane + 2 * ld_da, t0 * ld_da * 2, 0);
+  }
+}
+
+
 // How a row is cut into time chunks and how many wavefronts share a workgroup (measured on MI355X).
 //   * HBM serves this layout best when the wavefronts of a workgroup together read whole
 //     feature rows and the workgroups, taken in launch order, advance through memory: chunks of a
@@ -664,6 +1040,22 @@ void launch_mix_bwd(const MixBwdArgs& p, const MixPlan& m, hipStream_t s) {
                      p.ld_dv ? p.ld_dv : p.H * kChan, p.L, p.H, p.kv_groups, m.chunk_blocks * kTile, m.chunks, total);
 }
 
+template <class E, bool kQkv>
+void launch_mix_bwd_tile(const MixBwdArgs& p, hipStream_t s) {
+  const int octs = (p.H + 7) / 8, nb = p.L / kTile;
+  const int octs_w = octs % 2 == 0 ? 2 : 1;  // measured with copy loops: 2 head groups x 4 blocks moves the most
+  const int nb_w = kTileWaves / octs_w;
+  const int oct_groups = octs / octs_w, tiles = (nb + nb_w - 1) / nb_w;
+  const long wgs = (long)p.B * tiles * oct_groups;
+  auto u = [](const void* q) { return static_cast<const uint16_t*>(q); };
+  auto w = [](void* q) { return static_cast<uint16_t*>(q); };
+  const int Fkv = (p.H / p.kv_groups) * kChan;
+  hipLaunchKernelGGL((phalanx_mix_bwd_tile_kernel<E, kQkv>), dim3((unsigned)wgs), dim3(64 * kTileWaves), 0, s,
+                     u(p.a_logit), u(p.b_logit), u(p.c), u(p.v), u(p.dout), w(p.da_logit), w(p.db_logit), w(p.dc), w(p.dv),
+                     p.ld_da ? p.ld_da : p.H, p.ld_db ? p.ld_db : Fkv, p.ld_dc ? p.ld_dc : Fkv,
+                     p.ld_dv ? p.ld_dv : p.H * kChan, p.L, p.H, p.kv_groups, octs_w, nb_w, tiles, oct_groups);
+}
+
 }  // namespace
 
 long fused_mix_backward_sum_rows(long B, int H, int L) {
@@ -675,6 +1067,17 @@ hipError_t fused_mix_backward(const MixBwdArgs& p, hipStream_t s) {
   const MixPlan m = plan_mix_bwd(p.B, p.H, p.L);
   const bool sums = p.sum_da != nullptr;
   if (sums && (p.qkv || p.f32_grads)) return hipErrorInvalidValue;  // the caller has checked: layer form, 16-bit results
+  if (p.tile_split) {  // the caller has checked: no sums, 16-bit results, a grid that fits
+    if (sums || p.f32_grads) return hipErrorInvalidValue;
+    if (p.dtype == kBf16) {
+      if (p.qkv) launch_mix_bwd_tile<Bf16, true>(p, s);
+      else launch_mix_bwd_tile<Bf16, false>(p, s);
+    } else {
+      if (p.qkv) launch_mix_bwd_tile<Fp16, true>(p, s);
+      else launch_mix_bwd_tile<Fp16, false>(p, s);
+    }
+    return hipGetLastError();
+  }
   if (p.f32_grads) {
     if (p.dtype == kBf16) {
       if (p.qkv) launch_mix_bwd<Bf16, false, true, true>(p, m, s);

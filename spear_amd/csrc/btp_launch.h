@@ -66,6 +66,7 @@ struct MixBwdArgs {
   int ld_da = 0, ld_db = 0, ld_dc = 0, ld_dv = 0;
   bool qkv = false;  // as in MixArgs; da_logit is then the fp32 gradient of the gate
   bool f32_grads = false;  // check mode: da_logit, db_logit, dc, dv are fp32
+  bool tile_split = false;  // one wavefront per 16-step block instead of wavefronts that walk through time
 };
 hipError_t fused_mix_backward(const MixBwdArgs& p, hipStream_t s);
 long fused_mix_backward_sum_rows(long B, int H, int L);

@@ -61,6 +61,14 @@
 #ifndef SPEAR_BTP_HANDOVER  // 1: carries between the spans of a workgroup go through LDS; 0: every span reads its halo
 #define SPEAR_BTP_HANDOVER 1
 #endif
+#ifndef SPEAR_BTP_SETPRIO  // 1: wavefronts run at raised priority while they issue their global loads / stores
+#define SPEAR_BTP_SETPRIO 0
+#endif
+#if SPEAR_BTP_SETPRIO
+#define SPEAR_BTP_PRIO(n) __builtin_amdgcn_s_setprio(n)
+#else
+#define SPEAR_BTP_PRIO(n) ((void)0)
+#endif
 #if SPEAR_BTP_FWD_WAVES_PER_EU > 0
 #define SPEAR_BTP_FWD_OCC __attribute__((amdgpu_waves_per_eu(SPEAR_BTP_FWD_WAVES_PER_EU)))
 #else
@@ -236,6 +244,7 @@ __device__ __forceinline__ void btp_bwd_scan_body(
   constexpr bool kHandOver = SPEAR_BTP_HANDOVER && !kStreamIn && kW > 1;
   __shared__ float edge_state[kHandOver ? kW : 1][2][kChan];
 
+  SPEAR_BTP_PRIO(3);
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const long span = first_span_of_workgroup(kW) + wave;
   if (span >= total_spans) {  // wave-uniform
@@ -304,6 +313,7 @@ __device__ __forceinline__ void btp_bwd_scan_body(
     dc_halo = ah[0] * h;
   }
 
+  SPEAR_BTP_PRIO(0);
   slab16_regs_to_lds(img_x, lane, xin);
   if constexpr (kGradF32) {
     slab32_regs_to_lds(img_g, lane, gin);
@@ -413,6 +423,7 @@ __device__ __forceinline__ void btp_bwd_scan_body(
     dA_A *= a_lds[coeff_slot(32 * j) + d];
     dA_B *= a_lds[coeff_slot(32 * j) + 16 + d];
   }
+  SPEAR_BTP_PRIO(3);
   float* dArow = dA + sc.row * (long)L + sc.s0 + 32 * j + d;
   if (32 * j < sc.nvalid) __builtin_nontemporal_store(dA_A, dArow);
   if (32 * j + 16 < sc.nvalid) __builtin_nontemporal_store(dA_B, dArow + 16);
@@ -488,7 +499,10 @@ __global__ __launch_bounds__(64 * kWaves) void stream_probe_kernel(const uint4* 
 // of them is faster). kShape 1: two slabs per wavefront, every load issued before the first store (twice
 // the bytes in flight per wavefront); 2: a loop over `iters` slabs per wavefront with the next slab's loads
 // issued before the current slab's stores (a workgroup covers kWaves * iters consecutive slabs); 3: the
-// same loop as a persistent grid striding over the buffer; 4: one 16-byte element per thread.
+// same loop as a persistent grid striding over the buffer; 4: one 16-byte element per thread; 5 and 6: one
+// direction only (reads without writes, writes without reads), which gives the two rates a mixed kernel's
+// time is made of -- HBM serves reads and writes one after the other, so a kernel that reads R bytes and
+// writes W bytes cannot finish before R / read rate + W / write rate.
 template <int kReads, int kShape>
 __global__ __launch_bounds__(64 * kWaves) void stream_probe_shape_kernel(const uint4* __restrict__ a,
                                                                          const uint4* __restrict__ b,
@@ -531,6 +545,28 @@ __global__ __launch_bounds__(64 * kWaves) void stream_probe_shape_kernel(const u
       __builtin_amdgcn_sched_barrier(0);
       store(slab, q, r);
       __builtin_amdgcn_sched_barrier(0);
+    }
+  } else if constexpr (kShape == 5 || kShape == 6) {
+    // one direction only, in the kernels' own shape: 5 reads the inputs and writes nothing (the store below
+    // never happens for real data: it needs all-ones words), 6 writes `dst` and reads nothing
+    const unsigned long long slab = (unsigned long long)blockIdx.x * kWaves + wave;
+    if (slab >= slabs) return;
+    uint4 q[4], r[4];
+    if constexpr (kShape == 5) {
+      load(slab, q, r);
+      uint32_t all = 0xffffffffu;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        all &= q[i].x & q[i].y & q[i].z & q[i].w;
+        if constexpr (kReads == 2) all &= r[i].x & r[i].y & r[i].z & r[i].w;
+      }
+      if (all == 0xffffffffu) stream_store16(dst + slab * 256 + lane, q[0]);
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        q[i] = make_uint4((uint32_t)slab, (uint32_t)lane, (uint32_t)i, 0u);
+        stream_store16(dst + slab * 256 + lane + 64 * i, q[i]);
+      }
     }
   } else {
     static_assert(kShape == 4, "unknown probe shape");
@@ -652,6 +688,8 @@ void launch_probe_shape(const void* a, const void* b, void* dst, unsigned long l
       hipLaunchKernelGGL((stream_probe_shape_kernel<kReads, 3>), dim3((unsigned)(want < 2048 ? want : 2048)), wg, 0, s, pa, pb, pd, slabs, 0);
       break;
     }
+    case 5: hipLaunchKernelGGL((stream_probe_shape_kernel<kReads, 5>), blocks_for(kWaves), wg, 0, s, pa, pb, pd, slabs, 1); break;
+    case 6: hipLaunchKernelGGL((stream_probe_shape_kernel<kReads, 6>), blocks_for(kWaves), wg, 0, s, pa, pb, pd, slabs, 1); break;
     default: hipLaunchKernelGGL((stream_probe_shape_kernel<kReads, 4>), blocks_for(1), wg, 0, s, pa, pb, pd, slabs, 1); break;
   }
 }

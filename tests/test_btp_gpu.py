@@ -318,7 +318,18 @@ def test_measurement_aids_move_the_bytes_they_are_timed_for(slabs):
             torch.cuda.synchronize()
             assert torch.equal(out[:n], want), shape
             assert bool((out[n:] == 0xA5).all()), shape
-    assert lib.spear_btp_stream_probe_shape(a.data_ptr(), None, out.data_ptr(), ctypes.c_ulonglong(n), 5, sp) == -1
+    # one-way shapes: 5 reads only and leaves dst alone, 6 writes every byte of dst and nothing beyond
+    out.fill_(0xA5)
+    assert lib.spear_btp_stream_probe_shape(a.data_ptr(), b.data_ptr(), out.data_ptr(), ctypes.c_ulonglong(n), 5, sp) == 0
+    torch.cuda.synchronize()
+    assert bool((out == 0xA5).all())
+    assert lib.spear_btp_stream_probe_shape(a.data_ptr(), None, out.data_ptr(), ctypes.c_ulonglong(n), 6, sp) == 0
+    torch.cuda.synchronize()
+    words = out[:n].view(torch.int32).view(slabs, 4, 64, 4)
+    assert bool((words[..., 1] == torch.arange(64, device=DEV, dtype=torch.int32).view(1, 1, 64)).all())
+    assert bool((words[..., 0] == torch.arange(slabs, device=DEV, dtype=torch.int32).view(slabs, 1, 1)).all())
+    assert bool((out[n:] == 0xA5).all())
+    assert lib.spear_btp_stream_probe_shape(a.data_ptr(), None, out.data_ptr(), ctypes.c_ulonglong(n), 7, sp) == -1
     out.fill_(0xA5)
     assert lib.spear_btp_copy(a.data_ptr(), out.data_ptr(), ctypes.c_ulonglong(n), sp) == 0
     torch.cuda.synchronize()

@@ -52,22 +52,29 @@ def test_fused_forward_fp16_and_steep_gates():
     assert_close(f64(out), ref, 4e-3, 4e-3, "out fp16")
 
 
-def run_mix_backward(a, b, c, v, dout, H, Hkv=None):
+def run_mix_backward(a, b, c, v, dout, H, Hkv=None, tile_split=False):
     from spear_amd import _btp
 
     dev = [t.to(DEV) for t in (a, b, c, v, dout)]
     outs = [torch.full(t.shape, float("nan"), device=DEV, dtype=t.dtype) for t in (a, b, c, v)]
-    _btp.mix_backward(*dev, *outs, H, H if Hkv is None else Hkv)
+    _btp.mix_backward(*dev, *outs, H, H if Hkv is None else Hkv, tile_split=tile_split)
     torch.cuda.synchronize()
     return [t.cpu() for t in outs]
 
 
-@pytest.mark.parametrize("B,L,H", [(1, 16, 4), (2, 32, 4), (2, 48, 8), (1, 80, 12), (3, 128, 8), (2, 144, 16), (1, 512, 32), (1, 1040, 4), (1, 4096, 8), (2, 2064, 16)])
-def test_fused_backward_matches_oracle(B, L, H):
+# the backward kernel comes in two work splits: wavefronts that walk through time (default) and one wavefront
+# per 16-step block (SPEAR_MIX_TILE_SPLIT); both are held to the same oracle
+SPLITS = pytest.mark.parametrize("tile_split", [False, True], ids=["walk", "tile"])
+
+
+@SPLITS
+@pytest.mark.parametrize("B,L,H", [(1, 16, 4), (2, 32, 4), (2, 48, 8), (1, 80, 12), (3, 128, 8), (2, 144, 16), (1, 512, 32), (1, 1040, 4), (1, 4096, 8), (2, 2064, 16),
+                                   (5, 64, 32), (2, 112, 24), (3, 272, 64)])
+def test_fused_backward_matches_oracle(B, L, H, tile_split):
     a, b, c, v = make_mix_inputs(B, L, H, H, seed=2000 + L + H)
     dout = torch.randn(B, L, H * 16, generator=torch.Generator().manual_seed(L)).bfloat16()
-    print(f"fused bwd B={B} L={L} H={H}", flush=True)
-    da, db, dc, dv = run_mix_backward(a, b, c, v, dout, H)
+    print(f"fused bwd B={B} L={L} H={H} tile={tile_split}", flush=True)
+    da, db, dc, dv = run_mix_backward(a, b, c, v, dout, H, tile_split=tile_split)
     rda, rdb, rdc, rdv = orc.phalanx_mix_backward(f64(a), f64(b), f64(c), f64(v), f64(dout), H, H)
     assert_close(f64(dv), rdv, BF16_ATOL, BF16_RTOL, "dv")
     assert_close(f64(dc), rdc, BF16_ATOL, BF16_RTOL, "dc")
@@ -75,12 +82,13 @@ def test_fused_backward_matches_oracle(B, L, H):
     assert_close(f64(da), rda, BF16_ATOL, BF16_RTOL, "da")
 
 
+@SPLITS
 @pytest.mark.parametrize("B,L,H,Hkv", [(2, 48, 8, 4), (1, 80, 12, 3), (2, 144, 16, 2), (1, 272, 32, 8), (2, 64, 4, 2), (1, 2064, 8, 1)])
-def test_fused_backward_with_shared_kv_heads(B, L, H, Hkv):
+def test_fused_backward_with_shared_kv_heads(B, L, H, Hkv, tile_split):
     a, b, c, v = make_mix_inputs(B, L, H, Hkv, seed=3000 + L + H)
     dout = torch.randn(B, L, H * 16, generator=torch.Generator().manual_seed(L + 1)).bfloat16()
-    print(f"fused bwd kv B={B} L={L} H={H} Hkv={Hkv}", flush=True)
-    da, db, dc, dv = run_mix_backward(a, b, c, v, dout, H, Hkv)
+    print(f"fused bwd kv B={B} L={L} H={H} Hkv={Hkv} tile={tile_split}", flush=True)
+    da, db, dc, dv = run_mix_backward(a, b, c, v, dout, H, Hkv, tile_split=tile_split)
     rda, rdb, rdc, rdv = orc.phalanx_mix_backward(f64(a), f64(b), f64(c), f64(v), f64(dout), H, Hkv)
     assert_close(f64(dv), rdv, BF16_ATOL, BF16_RTOL, "dv")
     # sums over up to 8 heads: magnitudes grow, the relative term carries the tolerance
@@ -149,12 +157,13 @@ def test_fused_backward_into_column_blocks_of_one_buffer(B, L, H, Hkv):
         _btp.mix_backward(*dev, views[0], views[1], views[2], every_other, H, Hkv)
 
 
-def test_fused_backward_fp16_and_steep_gates():
+@SPLITS
+def test_fused_backward_fp16_and_steep_gates(tile_split):
     a, b, c, v = make_mix_inputs(2, 96, 8, 4, seed=6, dtype=torch.float16, scale=3.0)
     a[0, :10, :] = -30.0  # decay ~ 1e-13: counts as zero
     a[1, 20:40, 3] = 30.0  # decay -> 1
     dout = torch.randn(2, 96, 128, generator=torch.Generator().manual_seed(7)).half()
-    da, db, dc, dv = run_mix_backward(a, b, c, v, dout, 8, 4)
+    da, db, dc, dv = run_mix_backward(a, b, c, v, dout, 8, 4, tile_split=tile_split)
     rda, rdb, rdc, rdv = orc.phalanx_mix_backward(f64(a), f64(b), f64(c), f64(v), f64(dout), 8, 4)
     # fp16 storage: 11 significant bits; sums over two heads and up to 32 steps of undamped states
     for name, got, want in (("dv", dv, rdv), ("dc", dc, rdc), ("db", db, rdb), ("da", da, rda)):
@@ -247,3 +256,46 @@ def test_default_method_rerouted_by_environment_gives_the_fused_results(monkeypa
     rerouted.load_state_dict(fused.state_dict())
     x = torch.randn(2, 64, 128, generator=torch.Generator().manual_seed(4)).bfloat16().to(DEV)
     assert torch.equal(rerouted(x), fused(x))
+
+
+def test_tile_split_strided_outputs_qkv_form_and_what_it_refuses():
+    """The tile work split writes into column blocks of a wider buffer like the default kernel, serves the
+    q/k/v/gate form, and refuses the options it does not have."""
+    from spear_amd import _btp
+
+    B, L, H, Hkv = 3, 176, 16, 4
+    a, b, c, v = make_mix_inputs(B, L, H, Hkv, seed=8100)
+    dout = torch.randn(B, L, H * 16, generator=torch.Generator().manual_seed(8101)).bfloat16()
+    dense = run_mix_backward(a, b, c, v, dout, H, Hkv, tile_split=True)
+    widths = (H, Hkv * 16, Hkv * 16, H * 16)
+    ld = sum(widths) + 32
+    packed = torch.full((B, L, ld), float("nan"), device=DEV, dtype=torch.bfloat16)
+    cols = np.cumsum((0,) + widths)
+    views = [packed[:, :, cols[i]:cols[i + 1]] for i in range(4)]
+    dev = [t.to(DEV) for t in (a, b, c, v, dout)]
+    _btp.mix_backward(*dev, *views, H, Hkv, tile_split=True)
+    torch.cuda.synchronize()
+    for got, want in zip(views, dense):
+        assert torch.equal(got.cpu(), want)
+    assert torch.isnan(packed[:, :, cols[4]:]).all()
+
+    # q/k/v/gate form against the oracle
+    g = torch.Generator().manual_seed(8102)
+    gate = -torch.nn.functional.softplus(torch.randn(B, L, H, generator=g))
+    q, k, vv, dd = ((0.5 * torch.randn(B, L, w, generator=g)).bfloat16() for w in (Hkv * 16, Hkv * 16, H * 16, H * 16))
+    outs = [torch.full(t.shape, float("nan"), device=DEV, dtype=t.dtype) for t in (gate, k, q, vv)]
+    _btp.mix_backward(gate.to(DEV), k.to(DEV), q.to(DEV), vv.to(DEV), dd.to(DEV), *outs, H, Hkv, qkv_gate=True, tile_split=True)
+    torch.cuda.synchronize()
+    rgate, rk, rq, rv = orc.qkv_gate_backward(f64(q), f64(k), f64(vv), f64(gate), f64(dd), H, Hkv)
+    assert_close(f64(outs[0]), rgate, 1e-4, 1e-4, "dgate")
+    assert_close(f64(outs[1]), rk, 3e-2, BF16_RTOL, "dk")
+    assert_close(f64(outs[2]), rq, 3e-2, BF16_RTOL, "dq")
+    assert_close(f64(outs[3]), rv, BF16_ATOL, BF16_RTOL, "dv")
+
+    rows = _btp.mix_backward_sum_rows(B, L, H)
+    sums = tuple(torch.empty(rows, w, device=DEV) for w in widths[:3])
+    grads = [torch.empty_like(t) for t in dev[:4]]
+    with pytest.raises(RuntimeError, match="neither column sums nor fp32 results"):
+        _btp.mix_backward(*dev, *grads, H, Hkv, sums=sums, tile_split=True)
+    with pytest.raises(RuntimeError, match="neither column sums nor fp32 results"):
+        _btp.mix_backward(*dev, *[torch.empty(t.shape, device=DEV) for t in dev[:4]], H, Hkv, tile_split=True)
