@@ -568,6 +568,57 @@ def main() -> int:
         e1.record(stream)
         torch.cuda.synchronize()
         step_graph_ms = e0.elapsed_time(e1) / (16 * n_rep)
+        # the whole layer for one token: four projections, the layer-layout step kernel (gates + state update +
+        # y*C+V on the projections' [B, features] outputs, block position on the device), output projection;
+        # eager and as ONE HIP graph replayed per token
+        def layer_decode():
+            from spear_amd import Phalanx
+            from spear_amd.nn.phalanx.inference import PhalanxStepState, phalanx_step
+
+            dim = H * 16
+            torch.manual_seed(seed)
+            mod = Phalanx(dim=dim, length=L, method="fused", dtype=torch.bfloat16).to(dev)
+            gl = torch.Generator(device="cpu").manual_seed(seed + 17)
+            xs = torch.randn(16, B, dim, generator=gl).to(torch.bfloat16).to(dev)
+            st8 = PhalanxStepState.zeros(B, H, dev)
+            y_buf = torch.empty(B, dim, device=dev, dtype=torch.bfloat16)
+            x_buf = xs[0].clone()
+
+            def timed(fn, n):
+                for i in range(16):
+                    fn(i)
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                for i in range(n):
+                    fn(i)
+                torch.cuda.synchronize()
+                return (time.perf_counter() - t0) * 1e3 / n
+
+            n_tok = 16 * max(4, args.steps // 16)
+            eager_ms = timed(lambda i: phalanx_step(mod, xs[i % 16], st8, out=y_buf), n_tok)
+            side2 = torch.cuda.Stream()
+            side2.wait_stream(stream)
+            with torch.cuda.stream(side2):
+                phalanx_step(mod, x_buf, st8, out=y_buf)
+            stream.wait_stream(side2)
+            g2 = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g2, stream=side2):
+                phalanx_step(mod, x_buf, st8, out=y_buf)
+            torch.cuda.synchronize()
+            graph_ms = timed(lambda i: g2.replay(), n_tok)
+
+            def step_only(i):  # the mixing-stage kernel alone on precomputed projections
+                _btp.mix_step(pa, pb, pc, pv, mixed, st8.h_loc, st8.r_pref, st8.c_prev_loc, st8.pos, False, 16, H, H)
+
+            xc = xs[0]
+            pa, pb, pc, pv = (q(xc) for q in (mod.param.proj_a, mod.param.proj_b, mod.param.proj_c, mod.param.proj_v))
+            mixed = torch.empty_like(pv)
+            kernel_ms_ = timed(step_only, n_tok)
+            return {"what": "one token through the Phalanx layer at this batch: 4 projections + layer-layout step kernel + proj_out",
+                    "eager_ms_per_token": eager_ms, "hip_graph_ms_per_token": graph_ms,
+                    "tokens_per_s_graph": B / (graph_ms * 1e-3), "step_kernel_call_ms": kernel_ms_}
+
+        layer_step = guarded(layer_decode) if H % 4 == 0 else None
         step_bytes = B * H * (2 + 8 + 3 * 32 + 32 + 2 * 64 + 64)  # a, r in/out, x c v, y, h in/out, c_prev
         streaming = {
             "prefill": {"avg_launch_ms": prefill_ms, "algorithmic_bytes_per_launch": prefill_bytes,
@@ -579,6 +630,7 @@ def main() -> int:
                             "tokens_per_s": B / (step_ms * 1e-3),
                             "same_step_from_pytorch_ops_ms": step_torch_ms, "speedup": step_torch_ms / step_ms,
                             "avg_launch_ms_in_hip_graph": step_graph_ms},
+            "layer_decode_step": layer_step,
         }
         return streaming
 

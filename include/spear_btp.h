@@ -180,6 +180,24 @@ int spear_phalanx_mix_backward_bias(const void* a_logit, const void* b_logit, co
                                     int ld_db, int ld_dc, int ld_dv, float* bias_da, float* bias_db, float* bias_dc,
                                     int B, int L, int H, int kv_heads, int dtype, unsigned flags, void* stream);
 
+/* One decode token of the mixing stage in the layer's own layout: the four projections' outputs for one time step,
+ * [B, features] in `dtype`, and the fp32 streaming state, updated in place. It stands for step_jagged
+ * (spear/nn/phalanx/inference.py:178-278) fed by the layer's gates (spear/nn/phalanx/swr.py:196-221): the reference
+ * has no single function for it (its step takes A_t, X_t, C_t, V_t already gated, expanded over kv heads and
+ * reshaped to [B, H, D]).
+ *     a_logit [B, H]     b_logit, c [B, kv_heads * 16]     v, out [B, H * 16]
+ *     h, c_prev [B, H, 16] fp32     r [B, H] fp32           (zero state: h = 0, r = 1, c_prev = 0)
+ *     A = sigmoid(a_logit);  h = A h + sigmoid(b_logit) v;  r = A r;  out = (h + r c_prev) c + v
+ *     a token that completes a block:  c_prev = h, h = 0, r = 1
+ * Which tokens complete a block: with `pos` (device int32 [B], the position of each batch row's token inside its
+ * block, 0 .. block_len-1) every row decides for itself (pos[b] == block_len - 1) and the call advances pos by one
+ * step (wrapping to 0), so that one captured HIP graph serves every token and batch rows may be at different
+ * positions; with pos == NULL the host decides for all rows through `boundary`. Calls on one state must not
+ * overlap. Nothing is allocated; with `pos` the call launches two kernels. */
+int spear_phalanx_mix_step(const void* a_logit, const void* b_logit, const void* c, const void* v, void* out, float* h,
+                           float* r, float* c_prev, int* pos, int boundary, int block_len, int B, int H, int kv_heads,
+                           int dtype, unsigned flags, void* stream);
+
 /* ---- streaming form: prompt prefill with state hand-over, and the one-token decode step --------
  * They replace the PyTorch loops of spear/nn/phalanx/inference.py. Tensors are dense, row-major:
  *     a         [B, H, L]      a_dtype (x_dtype or fp32)   a_t, or log(a_t) with SPEAR_JAGGED_LOG_A

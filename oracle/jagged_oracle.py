@@ -8,6 +8,7 @@ What follows what (paths relative to the reference repository):
     step()        spear/nn/phalanx/inference.py:178-278  step_jagged (also JaggedBandState.step, :121-140,
                                                           which is the same update without ``* C + V``)
     prefill()     spear/nn/phalanx/inference.py:281-360  parallel_jagged: outputs and the hand-over state
+    layer_step()  spear/nn/phalanx/swr.py:196-221 (the layer's gates and kv-head expansion) feeding step()
 
 How each is pinned (tests/test_jagged_oracle.py); none of the tests imports the reference:
     sequential    equals the committed closed-form vectors at block length 16 and a windowed brute-force
@@ -21,6 +22,8 @@ How each is pinned (tests/test_jagged_oracle.py); none of the tests imports the 
                   identity fixes (stepping from it counts that state twice); that case, like the others,
                   is pinned by vectors computed with the reference's own parallel_jagged / step_jagged
                   (tests/golden/make_jagged_vectors.py -> jagged_reference_vectors.npz).
+    layer_step    L steps from the zero state equal the two-pass statement of the same stage on the whole
+                  sequence (oracle.btp_oracle.phalanx_mix_forward, itself pinned), with shared kv heads
 """
 
 from __future__ import annotations
@@ -119,3 +122,20 @@ def prefill(A, X, C, V, *, block_len: int, use_log_a: bool = False):
     done = L // block_len
     c_prev = local_at(done * block_len - 1)[0] if done > 0 else np.zeros((B, H, D))
     return Y, State(h_tail, r_tail, c_prev, (L - 1) % block_len + 1, block_len)
+
+
+def layer_step(a_logit, b_logit, c, v, state: State, heads: int, kv_heads: int | None = None):
+    """One token of the Phalanx mixing stage on the projections' outputs for that token: a_logit [B, H],
+    b_logit / c [B, kv_heads * D], v [B, H * D]. The gates and the kv-head expansion are the layer's
+    (swr.py:196-221: A = sigmoid(a), X = sigmoid(b) * v, head h uses b / c of kv head h // (H // kv_heads)), the
+    update is step(). Returns (out [B, H * D], new State)."""
+    kv = heads if kv_heads is None else kv_heads
+    a64, b64, c64, v64 = (np.asarray(t, dtype=np.float64) for t in (a_logit, b_logit, c, v))
+    B = v64.shape[0]
+    D = v64.shape[1] // heads
+    sig = lambda z: 1.0 / (1.0 + np.exp(-z))
+    V = v64.reshape(B, heads, D)
+    G = np.repeat(sig(b64).reshape(B, kv, D), heads // kv, axis=1)
+    C = np.repeat(c64.reshape(B, kv, D), heads // kv, axis=1)
+    y, new = step(sig(a64), G * V, C, V, state)
+    return y.reshape(B, heads * D), new

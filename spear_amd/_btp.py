@@ -20,7 +20,7 @@ import threading
 
 import torch
 
-__all__ = ["forward", "backward", "forward_log", "backward_log", "mix_forward", "mix_backward", "jagged_prefill", "jagged_step", "library_path", "load_library", "load_extension", "FLAG_WRITE_CHECKPOINT", "FLAG_PATH_MFMA", "FLAG_JAGGED_LOG_A", "FLAG_JAGGED_LOG_R", "FLAG_MIX_QKV_GATE", "FLAG_MIX_F32_RESULTS", "FLAG_DX_F32", "mix_backward_sum_rows", "mix_backward_bias"]
+__all__ = ["forward", "backward", "forward_log", "backward_log", "mix_forward", "mix_backward", "jagged_prefill", "jagged_step", "library_path", "load_library", "load_extension", "FLAG_WRITE_CHECKPOINT", "FLAG_PATH_MFMA", "FLAG_JAGGED_LOG_A", "FLAG_JAGGED_LOG_R", "FLAG_MIX_QKV_GATE", "FLAG_MIX_F32_RESULTS", "FLAG_DX_F32", "mix_backward_sum_rows", "mix_backward_bias", "mix_step"]
 
 _BF16, _F16, _F32 = 0, 1, 2
 FLAG_WRITE_CHECKPOINT = 0x1
@@ -31,7 +31,7 @@ FLAG_MIX_QKV_GATE = 0x1
 FLAG_MIX_F32_RESULTS = 0x2
 FLAG_MIX_TILE_SPLIT = 0x4
 FLAG_DX_F32 = 0x10
-_ABI_VERSION = 12
+_ABI_VERSION = 13
 _SUPPORTED_WPB = (4, 8, 16, 32)
 
 _lock = threading.Lock()
@@ -66,6 +66,8 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.spear_phalanx_mix_backward_bias.restype = ci
     lib.spear_phalanx_mix_backward_sum_rows.argtypes = [ci, ci, ci]
     lib.spear_phalanx_mix_backward_sum_rows.restype = ctypes.c_longlong
+    lib.spear_phalanx_mix_step.argtypes = [vp] * 9 + [ci] * 6 + [cu, vp]
+    lib.spear_phalanx_mix_step.restype = ci
     lib.spear_jagged_prefill.argtypes = [vp] * 9 + [ci] * 9 + [cu, vp]
     lib.spear_jagged_prefill.restype = ci
     lib.spear_jagged_step.argtypes = [vp] * 11 + [ci] * 8 + [cu, ctypes.c_float, vp]
@@ -498,6 +500,55 @@ def mix_backward_bias(
             da_logit.data_ptr(), db_logit.data_ptr(), dc.data_ptr(), dv.data_ptr(), *lds,
             bias[0].data_ptr(), bias[1].data_ptr(), bias[2].data_ptr(),
             B, L, heads, kv_heads, _tag(v.dtype), 0, _stream_ptr(v.device),
+        )
+    if rc != 0:
+        _raise_native(lib, rc)
+
+
+def mix_step(
+    a_logit: torch.Tensor,
+    b_logit: torch.Tensor,
+    c: torch.Tensor,
+    v: torch.Tensor,
+    out: torch.Tensor,
+    h: torch.Tensor,
+    r: torch.Tensor,
+    c_prev: torch.Tensor,
+    pos: torch.Tensor | None,
+    boundary: bool,
+    block_len: int,
+    heads: int,
+    kv_heads: int,
+) -> None:
+    """One decode token of the mixing stage on the projections' ``[B, features]`` outputs; the fp32 state
+    ``h, r, c_prev`` is updated in place (see ``spear_phalanx_mix_step`` in the C header). ``pos``: int32 ``[B]``
+    positions inside the block (advanced by the call) or ``None`` to let ``boundary`` decide for all rows."""
+    tensors = [a_logit, b_logit, c, v, out, h, r, c_prev] + ([pos] if pos is not None else [])
+    _check(all(t.is_cuda for t in tensors), "All tensors must be CUDA.")
+    _check(len({t.device for t in tensors}) == 1, "All tensors must be on the same device.")
+    _check(v.dim() == 2 and v.shape[1] == heads * 16, "v must be [B, heads * 16].")
+    B = v.shape[0]
+    _check(kv_heads > 0 and heads % kv_heads == 0, "heads must be divisible by kv_heads.")
+    _check(v.dtype in (torch.float16, torch.bfloat16), "tensors must be float16 or bfloat16.")
+    _check(all(t.dtype == v.dtype for t in (a_logit, b_logit, c, out)), "all tensors must share one dtype.")
+    _check(all(t.dtype == torch.float32 for t in (h, r, c_prev)), "the state must be float32.")
+    _check_layout("a_logit", a_logit, (B, heads))
+    _check_layout("b_logit", b_logit, (B, kv_heads * 16))
+    _check_layout("c", c, (B, kv_heads * 16))
+    _check_layout("v", v, (B, heads * 16))
+    _check_layout("out", out, (B, heads * 16))
+    _check_layout("h", h, (B, heads, 16))
+    _check_layout("c_prev", c_prev, (B, heads, 16))
+    _check_layout("r", r, (B, heads))
+    if pos is not None:
+        _check(pos.dtype == torch.int32, "pos must be int32.")
+        _check_layout("pos", pos, (B,))
+    lib = load_library()
+    with torch.cuda.device(v.device):
+        rc = lib.spear_phalanx_mix_step(
+            a_logit.data_ptr(), b_logit.data_ptr(), c.data_ptr(), v.data_ptr(), out.data_ptr(), h.data_ptr(),
+            r.data_ptr(), c_prev.data_ptr(), _ptr(pos), int(bool(boundary)), int(block_len), B, heads, kv_heads,
+            _tag(v.dtype), 0, _stream_ptr(v.device),
         )
     if rc != 0:
         _raise_native(lib, rc)

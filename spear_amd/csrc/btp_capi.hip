@@ -45,7 +45,7 @@ int check_common(const char* who, int B, int H, int L, int k, int in_dtype, int 
 
 extern "C" {
 
-int spear_btp_abi_version(void) { return 12; }
+int spear_btp_abi_version(void) { return 13; }
 
 const char* spear_btp_last_error(void) { return g_error; }
 
@@ -268,6 +268,32 @@ int spear_phalanx_mix_backward_bias(const void* a_logit, const void* b_logit, co
                           nullptr, nullptr, nullptr, ld_da, ld_db, ld_dc, ld_dv, false};
   const hipError_t err =
       spear_btp::fused_mix_backward_bias(a, bias_da, bias_db, bias_dc, static_cast<hipStream_t>(stream));
+  if (err != hipSuccess) return fail(SPEAR_BTP_ELAUNCH, "%s: launch failed: %s", who, hipGetErrorString(err));
+  return 0;
+}
+
+int spear_phalanx_mix_step(const void* a_logit, const void* b_logit, const void* c, const void* v, void* out, float* h,
+                           float* r, float* c_prev, int* pos, int boundary, int block_len, int B, int H, int kv_heads,
+                           int dtype, unsigned flags, void* stream) {
+  g_error[0] = '\0';
+  const char* who = "spear_phalanx_mix_step";
+  if (B < 0 || H < 0) return fail(SPEAR_BTP_EINVAL, "%s: negative dimension (B=%d H=%d)", who, B, H);
+  if (block_len <= 0) return fail(SPEAR_BTP_EINVAL, "%s: block_len must be positive (got %d)", who, block_len);
+  if (kv_heads <= 0 || H % kv_heads != 0)
+    return fail(SPEAR_BTP_EINVAL, "%s: heads (%d) must be divisible by kv_heads (%d)", who, H, kv_heads);
+  if (dtype != SPEAR_BTP_BF16 && dtype != SPEAR_BTP_F16)
+    return fail(SPEAR_BTP_EINVAL, "%s: tensors must be float16 or bfloat16.", who);
+  if (flags != 0u) return fail(SPEAR_BTP_EINVAL, "%s: unknown flag bits 0x%x", who, flags);
+  if ((long long)B * H * 16ll >= (1ll << 40)) return fail(SPEAR_BTP_EINVAL, "%s: tensor too large", who);
+  if ((long long)B * H == 0) return 0;
+  const void* ptrs[] = {a_logit, b_logit, c, v, out, h, r, c_prev};
+  for (const void* q : ptrs) {
+    if (!q) return fail(SPEAR_BTP_ENULL, "%s: NULL tensor pointer", who);
+    if (!aligned16(q)) return fail(SPEAR_BTP_EINVAL, "%s: tensor pointers must be 16-byte aligned", who);
+  }
+  if (pos && (reinterpret_cast<uintptr_t>(pos) & 3u)) return fail(SPEAR_BTP_EINVAL, "%s: pos must be 4-byte aligned", who);
+  spear_btp::MixStepArgs a{a_logit, b_logit, c, v, out, h, r, c_prev, pos, boundary ? 1 : 0, block_len, B, H, H / kv_heads, dtype};
+  const hipError_t err = spear_btp::fused_mix_step(a, static_cast<hipStream_t>(stream));
   if (err != hipSuccess) return fail(SPEAR_BTP_ELAUNCH, "%s: launch failed: %s", who, hipGetErrorString(err));
   return 0;
 }

@@ -933,6 +933,68 @@ void phalanx_mix_bwd_tile_kernel(
 }
 
 
+// ==========================================================================================
+// One decode token of the mixing stage in the layer's own layout: the projections' outputs for ONE time step,
+// [B, features], and the streaming state of every (batch row, head). It is step_jagged of the reference
+// (spear/nn/phalanx/inference.py:178-278) with the gates of the layer (spear/nn/phalanx/swr.py:196-221) applied
+// in the same pass and the kv-head sharing resolved by indexing:
+//   A = sigmoid(a_logit), G = sigmoid(b_logit);   h = A h + G v;   r = A r;   out = (h + r c_prev) c + v
+//   a token that completes a block:  c_prev = h, h = 0, r = 1
+// A thread owns 8 consecutive features (16-byte accesses); the two threads of a head sit in neighbouring lanes,
+// so the head's scalar r is read by both before one of them writes it back (in-place state).
+// ==========================================================================================
+template <class E>
+__global__ __launch_bounds__(256) void phalanx_mix_step_kernel(
+    const uint16_t* __restrict__ a_logit, const uint16_t* __restrict__ b_logit, const uint16_t* __restrict__ c_in,
+    const uint16_t* __restrict__ v_in, uint16_t* __restrict__ out, float* __restrict__ h, float* __restrict__ r,
+    float* __restrict__ c_prev, const int* __restrict__ pos, int boundary_all, int block_len, long total, int H,
+    int kv_groups) {
+  const long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total) return;
+  const int per_row = 2 * H;  // 8-feature pieces per batch row
+  const long brow = idx / per_row;
+  const int piece = (int)(idx - brow * per_row);
+  const int head = piece >> 1, half = piece & 1;
+  const long kv_piece = brow * (2 * (H / kv_groups)) + 2 * (head / kv_groups) + half;
+  const bool boundary = pos != nullptr ? (pos[brow] == block_len - 1) : (boundary_all != 0);
+
+  const uint32_t aw = a_logit[brow * H + head];
+  const float a = clamp_coeff<E>(fast_sigmoid(E::lo(aw)));
+  const float r_new = a * r[brow * H + head];
+  float bf[8], cf[8], vf[8], hf[8], pf[8], of[8];
+  unpack8<E>(*reinterpret_cast<const uint4*>(b_logit + kv_piece * 8), bf);
+  unpack8<E>(*reinterpret_cast<const uint4*>(c_in + kv_piece * 8), cf);
+  unpack8<E>(*reinterpret_cast<const uint4*>(v_in + idx * 8), vf);
+  const float4 h0 = *reinterpret_cast<const float4*>(h + idx * 8), h1 = *reinterpret_cast<const float4*>(h + idx * 8 + 4);
+  const float4 p0 = *reinterpret_cast<const float4*>(c_prev + idx * 8), p1 = *reinterpret_cast<const float4*>(c_prev + idx * 8 + 4);
+  hf[0] = h0.x; hf[1] = h0.y; hf[2] = h0.z; hf[3] = h0.w; hf[4] = h1.x; hf[5] = h1.y; hf[6] = h1.z; hf[7] = h1.w;
+  pf[0] = p0.x; pf[1] = p0.y; pf[2] = p0.z; pf[3] = p0.w; pf[4] = p1.x; pf[5] = p1.y; pf[6] = p1.z; pf[7] = p1.w;
+#pragma unroll
+  for (int q = 0; q < 8; ++q) {
+    hf[q] = fmaf(a, hf[q], fast_sigmoid(bf[q]) * vf[q]);
+    of[q] = fmaf(fmaf(r_new, pf[q], hf[q]), cf[q], vf[q]);
+  }
+  *reinterpret_cast<uint4*>(out + idx * 8) = pack8<E>(of);
+  if (boundary) {
+    *reinterpret_cast<float4*>(c_prev + idx * 8) = make_float4(hf[0], hf[1], hf[2], hf[3]);
+    *reinterpret_cast<float4*>(c_prev + idx * 8 + 4) = make_float4(hf[4], hf[5], hf[6], hf[7]);
+#pragma unroll
+    for (int q = 0; q < 8; ++q) hf[q] = 0.0f;
+  }
+  *reinterpret_cast<float4*>(h + idx * 8) = make_float4(hf[0], hf[1], hf[2], hf[3]);
+  *reinterpret_cast<float4*>(h + idx * 8 + 4) = make_float4(hf[4], hf[5], hf[6], hf[7]);
+  if (half == 0) r[brow * H + head] = boundary ? 1.0f : r_new;
+}
+
+// pos[b] <- position of the next token inside its block
+__global__ __launch_bounds__(256) void advance_block_positions_kernel(int* __restrict__ pos, int B, int block_len) {
+  const int b = blockIdx.x * blockDim.x + threadIdx.x;
+  if (b >= B) return;
+  const int next = pos[b] + 1;
+  pos[b] = next >= block_len ? 0 : next;
+}
+
+
 // How a row is cut into time chunks and how many wavefronts share a workgroup (measured on MI355X).
 //   * HBM serves this layout best when the wavefronts of a workgroup together read whole
 //     feature rows and the workgroups, taken in launch order, advance through memory: chunks of a
@@ -1165,6 +1227,24 @@ hipError_t scratch_of_current_device(float** out) {
 }
 
 }  // namespace
+
+hipError_t fused_mix_step(const MixStepArgs& p, hipStream_t s) {
+  const long total = (long)p.B * p.H * 2;
+  const unsigned blocks = (unsigned)((total + 255) / 256);
+  auto u = [](const void* q) { return static_cast<const uint16_t*>(q); };
+  if (p.dtype == kBf16)
+    hipLaunchKernelGGL(phalanx_mix_step_kernel<Bf16>, dim3(blocks), dim3(256), 0, s, u(p.a_logit), u(p.b_logit), u(p.c), u(p.v),
+                       static_cast<uint16_t*>(p.out), p.h, p.r, p.c_prev, p.pos, p.boundary, p.block_len, total, p.H, p.kv_groups);
+  else
+    hipLaunchKernelGGL(phalanx_mix_step_kernel<Fp16>, dim3(blocks), dim3(256), 0, s, u(p.a_logit), u(p.b_logit), u(p.c), u(p.v),
+                       static_cast<uint16_t*>(p.out), p.h, p.r, p.c_prev, p.pos, p.boundary, p.block_len, total, p.H, p.kv_groups);
+  if (hipError_t err = hipGetLastError(); err != hipSuccess) return err;
+  if (p.pos != nullptr) {  // stream order puts this after every read of pos above
+    hipLaunchKernelGGL(advance_block_positions_kernel, dim3((unsigned)((p.B + 255) / 256)), dim3(256), 0, s, p.pos, p.B, p.block_len);
+    return hipGetLastError();
+  }
+  return hipSuccess;
+}
 
 long fused_mix_backward_bias_scratch_floats(long B, int H, int kv_groups, int L) {
   if (B <= 0 || H <= 0 || L <= 0 || kv_groups <= 0) return 0;

@@ -76,6 +76,20 @@ long fused_mix_backward_sum_rows(long B, int H, int L);
 hipError_t fused_mix_backward_bias(const MixBwdArgs& p, float* bias_da, float* bias_db, float* bias_dc, hipStream_t s);
 long fused_mix_backward_bias_scratch_floats(long B, int H, int kv_groups, int L);
 
+// One decode token of the mixing stage in the layer's layout (btp_fused.hip): 16-bit [B, features] operands,
+// fp32 state updated in place. pos: null, or the position inside its block of every batch row's token (device
+// int32 [B]), which decides the block boundary per row and is advanced by the call; else `boundary` decides.
+struct MixStepArgs {
+  const void *a_logit, *b_logit, *c, *v;  // [B, H], [B, Hkv*16] x 2, [B, H*16]
+  void* out;                              // [B, H*16]
+  float *h, *r, *c_prev;                  // [B, H, 16], [B, H], [B, H, 16]
+  int* pos;
+  int boundary, block_len;
+  int B, H, kv_groups;
+  int dtype;
+};
+hipError_t fused_mix_step(const MixStepArgs& p, hipStream_t s);
+
 // Streaming form (btp_jagged.hip). Tensors [B, H, D, L] / [B, H, L]; state vectors [B, H, D] / [B, H].
 struct JagPrefillArgs {
   const void *a, *x, *c, *v;  // c and v both null: no "* C + V" epilogue

@@ -23,6 +23,13 @@ What differs from the reference, none of it in the values beyond rounding:
     the first updates the state's own tensors instead of allocating new ones each token, the
     second keeps the hand-over state in fp32 when the tensors are 16-bit.
 
+Additions for decoding with the whole layer (no counterpart in the reference, whose step function takes
+gated, kv-expanded ``[B, H, D]`` operands): ``phalanx_step(layer, x_t, state)`` runs one token through a
+``Phalanx`` layer -- four projections, ONE kernel for gates + recurrence step + ``* C + V`` on the projections'
+``[B, features]`` outputs (``spear_phalanx_mix_step``), output projection -- with the block position kept on the
+device, so that the step records into one HIP graph that serves every token; ``phalanx_prefill`` runs a prompt
+through the layer and hands over the state to continue from.
+
 The state ``parallel_jagged`` returns for a prompt whose length is a multiple of ``block_len``
 follows the reference as written (inference.py:327-341): ``h_loc`` is the last block's terminal
 local state, not zero, so a decode step taken from that state counts it twice. Prompts of any
@@ -43,6 +50,9 @@ __all__ = [
     "JagState",
     "step_jagged",
     "parallel_jagged",
+    "PhalanxStepState",
+    "phalanx_prefill",
+    "phalanx_step",
 ]
 
 
@@ -268,3 +278,71 @@ def parallel_jagged(
         log_r_pref=None,
     )
     return Y, state
+
+
+# ---- decoding with the whole layer ------------------------------------------------------------------
+
+@dataclass
+class PhalanxStepState:
+    """Streaming state of a ``Phalanx`` layer, fp32, updated in place by :func:`phalanx_step`:
+    ``h_loc`` [B, H, 16] block-local state, ``r_pref`` [B, H] in-block gate product, ``c_prev_loc`` [B, H, 16]
+    terminal local state of the last completed block, ``pos`` [B] int32 position of the next token inside
+    its block (on the device: a captured step needs no host decision)."""
+
+    h_loc: torch.Tensor
+    r_pref: torch.Tensor
+    c_prev_loc: torch.Tensor
+    pos: torch.Tensor
+    block_len: int = 16
+
+    @classmethod
+    def zeros(cls, batch: int, heads: int, device, block_len: int = 16) -> "PhalanxStepState":
+        return cls(
+            torch.zeros(batch, heads, 16, device=device),
+            torch.ones(batch, heads, device=device),
+            torch.zeros(batch, heads, 16, device=device),
+            torch.zeros(batch, device=device, dtype=torch.int32),
+            block_len,
+        )
+
+
+@torch.no_grad()
+def phalanx_step(layer, x_t: torch.Tensor, state: PhalanxStepState, out: torch.Tensor | None = None) -> torch.Tensor:
+    """One token through ``layer`` (a ``Phalanx``): ``x_t`` [B, dim] -> [B, dim]; ``state`` is updated in place.
+    Equals position t of ``layer(x)`` for the sequence fed so far. Every op is stream-ordered and allocation
+    apart, so the call can be recorded into a HIP graph (``torch.cuda.graph``) with fixed ``x_t`` / ``out``
+    buffers and replayed once per token."""
+    _need_gpu(x_t, state.h_loc)
+    p = layer.param
+    xc = x_t.to(p.compute_dtype)
+    a, b, c, v = p.proj_a(xc), p.proj_b(xc), p.proj_c(xc), p.proj_v(xc)
+    mixed = torch.empty_like(v)
+    _btp.mix_step(a, b, c, v, mixed, state.h_loc, state.r_pref, state.c_prev_loc, state.pos, False,
+                  state.block_len, layer.heads, layer.kv_heads)
+    y = layer.proj_out(mixed)
+    if out is not None:
+        out.copy_(y)
+        return out
+    return y
+
+
+@torch.no_grad()
+def phalanx_prefill(layer, x: torch.Tensor) -> tuple[torch.Tensor, PhalanxStepState]:
+    """A prompt ``x`` [B, L, dim] (any L >= 1) through ``layer``: returns ``layer``'s output for it and the
+    state after its last token, from which :func:`phalanx_step` continues. The output of the whole blocks comes
+    from the layer's own forward; the state depends only on the last completed block and the partial block
+    after it (the carry is one hop), so it is rebuilt by stepping through those at most 31 tokens from the zero
+    state; a partial last block's outputs are taken from those steps."""
+    _need_gpu(x)
+    B, L, _ = x.shape
+    bl = 16
+    full = (L // bl) * bl
+    start = max(0, full - bl) if L > full else max(0, L - bl)  # a block boundary: stepping from zero there is exact
+    state = PhalanxStepState.zeros(B, layer.heads, x.device, bl)
+    tail = torch.empty(B, L - start, layer.dim, device=x.device, dtype=layer.proj_out.weight.dtype)
+    for t in range(start, L):
+        phalanx_step(layer, x[:, t], state, out=tail[:, t - start])
+    if full == 0:
+        return tail, state
+    y_full = layer(x[:, :full])
+    return (y_full if L == full else torch.cat([y_full, tail[:, full - start:]], dim=1)), state

@@ -144,3 +144,25 @@ def test_oracle_reproduces_the_reference_vectors(case):
         np.testing.assert_allclose(y, v["y_steps"][..., k], rtol=1e-11, atol=1e-12)
     final = np.concatenate([st.h_loc.ravel(), st.r_pref.ravel(), st.c_prev_loc.ravel(), [st.i]])
     np.testing.assert_allclose(final, v["final"], rtol=1e-11, atol=1e-12)
+
+
+@pytest.mark.parametrize("H,Hkv,L", [(4, 4, 40), (8, 2, 33), (12, 3, 64)])
+def test_layer_steps_equal_the_two_pass_statement_of_the_stage(H, Hkv, L):
+    """Stepping the layer-layout token update through a sequence gives what the two-pass (block) statement of
+    the same stage gives for the whole sequence: the gates, the kv-head sharing and the layout of layer_step
+    are pinned by an algorithm that shares none of its code."""
+    from oracle import btp_oracle as orc
+
+    rng = np.random.default_rng(H * 100 + L)
+    B = 2
+    Lp = -(-L // 16) * 16  # the block statement needs whole blocks; the extra steps do not touch earlier outputs
+    a = rng.normal(size=(B, Lp, H))
+    b = rng.normal(size=(B, Lp, Hkv * 16))
+    c = rng.normal(size=(B, Lp, Hkv * 16))
+    v = rng.normal(size=(B, Lp, H * 16))
+    want = orc.phalanx_mix_forward(a, b, c, v, H, Hkv)
+    state = jag.zero_state(B, H, 16, 16)
+    for t in range(L):
+        out, state = jag.layer_step(a[:, t], b[:, t], c[:, t], v[:, t], state, H, Hkv)
+        np.testing.assert_allclose(out, want[:, t], rtol=1e-10, atol=1e-10)
+    assert state.i == L % 16
