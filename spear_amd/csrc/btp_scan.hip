@@ -104,7 +104,7 @@ __global__ __launch_bounds__(64 * kWaves) SPEAR_BTP_FWD_OCC void btp_fwd_scan_ke
   __shared__ float left_state[kHandOver ? kW : 1][kChan];
 
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const long span = first_span_of_workgroup(kW) + wave;
+  const long span = first_span_of_workgroup<(SPEAR_BTP_XCD_REMAP == 2) || (SPEAR_BTP_XCD_REMAP == 1 && !kStreamIn)>(kW) + wave;
   if (span >= total_spans) {  // wave-uniform
     if constexpr (kHandOver) __syncthreads();  // keep the barrier count equal for every wavefront
     return;

@@ -327,7 +327,9 @@ def test_default_method_can_be_sent_to_the_fused_kernels_by_environment(monkeypa
 def test_streaming_module_surface_and_state_dataclass():
     from spear_amd.nn.phalanx import inference as inf
 
-    assert inf.__all__ == ["jagged_band_infer_sequential", "JaggedBandState", "JagState", "step_jagged", "parallel_jagged"]
+    # the reference's five names first, then the additions for decoding with the whole layer
+    assert inf.__all__[:5] == ["jagged_band_infer_sequential", "JaggedBandState", "JagState", "step_jagged", "parallel_jagged"]
+    assert inf.__all__[5:] == ["PhalanxStepState", "phalanx_prefill", "phalanx_step"]
     st = inf.JagState(torch.zeros(1, 2, 3), torch.ones(1, 2), torch.zeros(1, 2, 3), 5, 16)
     assert (st.use_log_r, st.log_r_pref) == (False, None)
     cl = st.clone_detached()
