@@ -33,7 +33,7 @@ FWD_BYTES, BWD_BYTES = 66, 102  # per (token, head), bf16 y / dy
 # WRITE_SIZE and scaled by what the same counters read for the copy kernel (x1.9997 / x1.0000);
 # figures and commands are in profiles/btp_kernels_c3_B1024_H32_L128.txt (and the c4 / c5 files beside it). Counters cannot be read
 # from inside this script, so the value is recorded here; it is null for shapes never profiled.
-MEASURED_BWD_TRAFFIC_BYTES = {"c3": 429.29e6, "c4": 891.20e6, "c5": 1756.40e6}
+MEASURED_BWD_TRAFFIC_BYTES = {"c3": 429.2e6, "c4": 891.4e6, "c5": 1756.4e6}
 
 CONFIGS = {
     # name: (B, H, L, seed, x_std, gate)
@@ -653,6 +653,10 @@ def main() -> int:
                 cl, xl = c.detach().requires_grad_(True), xx.detach().requires_grad_(True)
                 btp_op(cl, xl, 2, 32, torch.bfloat16).backward(g)
 
+            def eager_forward():  # inference: no autograd node
+                with torch.no_grad():
+                    btp_op(c, xx, 2, 32, torch.bfloat16)
+
             def ops_only():  # the two custom ops on preallocated outputs (what a graph can hold)
                 torch.ops.spear_btp.forward(c, xx, y, ck, 2, 32)
                 torch.ops.spear_btp.backward(c, xx, g, ck, dx, dA, 2, 32)
@@ -668,7 +672,19 @@ def main() -> int:
                 return (time.perf_counter() - t0) * 1e3 / n
 
             n = max(20, args.steps // 2)
-            eager_ms, ops_ms = timed(eager, n), timed(ops_only, n)
+            eager_ms, ops_ms, eager_fwd_ms = timed(eager, n), timed(ops_only, n), timed(eager_forward, n)
+            def fwd_op_only():
+                torch.ops.spear_btp.forward(c, xx, y, ck, 2, 32)
+            gside = torch.cuda.Stream()
+            gside.wait_stream(stream)
+            with torch.cuda.stream(gside):
+                fwd_op_only()
+            stream.wait_stream(gside)
+            fgraph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(fgraph, stream=gside):
+                fwd_op_only()
+            torch.cuda.synchronize()
+            fwd_graph_ms = timed(fgraph.replay, n)
             side = torch.cuda.Stream()
             side.wait_stream(stream)
             with torch.cuda.stream(side):
@@ -680,7 +696,9 @@ def main() -> int:
             torch.cuda.synchronize()
             graph_ms = timed(graph.replay, n)
             return {"B": bs, "eager_autograd_ms": eager_ms, "two_ops_preallocated_ms": ops_ms, "hip_graph_replay_ms": graph_ms,
-                    "eager_over_graph": eager_ms / graph_ms, "two_ops_over_graph": ops_ms / graph_ms}
+                    "eager_over_graph": eager_ms / graph_ms, "two_ops_over_graph": ops_ms / graph_ms,
+                    "forward_only": {"eager_no_grad_ms": eager_fwd_ms, "hip_graph_replay_ms": fwd_graph_ms,
+                                     "eager_over_graph": eager_fwd_ms / fwd_graph_ms}}
 
         return {"what": "btp(coeff, x, output_dtype=bf16) + backward through the public op (wall clock per fwd+bwd)",
                 "this_shape": measure(B), "config1_batch": measure(min(B, 8))}

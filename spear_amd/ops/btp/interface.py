@@ -125,6 +125,14 @@ register_traceable_op(lib, "forward_log", _forward_log_impl, _forward_log_fake, 
 register_traceable_op(lib, "backward_log", _backward_log_impl, _backward_log_fake, mutates_args=["dx", "dgate"])
 
 
+def _no_checkpoint(x: torch.Tensor) -> torch.Tensor:
+    """The carry checkpoint argument of the forward op: a zero-element placeholder unless the store is on."""
+    if _FORWARD_FLAGS & _btp.FLAG_WRITE_CHECKPOINT:
+        B, H, _, L = x.shape
+        return torch.empty((B, H, L // BLK, DH), device=x.device, dtype=torch.float32)
+    return torch.empty((0,), device=x.device, dtype=torch.float32)
+
+
 class _BTPFunction(torch.autograd.Function):
     @staticmethod
     def forward(ctx, coeff: torch.Tensor, x: torch.Tensor, k: int, output_dtype: torch.dtype, wpb: int):
@@ -134,8 +142,7 @@ class _BTPFunction(torch.autograd.Function):
         assert wpb in SUPPORTED_WPB, f"WPB must be one of {SUPPORTED_WPB}"
 
         y = torch.empty_like(x, dtype=output_dtype)
-        ckpt_shape = (B, H, L // BLK, DH) if _FORWARD_FLAGS & _btp.FLAG_WRITE_CHECKPOINT else (0,)
-        checkpoint = torch.empty(ckpt_shape, device=x.device, dtype=torch.float32)
+        checkpoint = _no_checkpoint(x)
         torch.ops.spear_btp.forward(coeff, x, y, checkpoint, int(k), int(wpb))
 
         ctx.save_for_backward(coeff, x, checkpoint)
@@ -173,7 +180,16 @@ def btp(
     """
     out_dtype = output_dtype or torch.float32
     wpb_val = wpb if wpb is not None else (WPB_K2_DEFAULT if k == 2 else WPB_K1_DEFAULT)
-    return _BTPFunction.apply(coeff.contiguous(), x.contiguous(), k, out_dtype, wpb_val)
+    coeff, x = coeff.contiguous(), x.contiguous()
+    if not (torch.is_grad_enabled() and (coeff.requires_grad or x.requires_grad)):
+        # nothing to differentiate (inference): the op itself, without the autograd node and its bookkeeping
+        assert x.dim() == 4 and x.shape[2] == DH, f"Channel dimension must be {DH}"
+        assert x.shape[3] % BLK == 0, f"Length L must be multiple of {BLK}"
+        assert wpb_val in SUPPORTED_WPB, f"WPB must be one of {SUPPORTED_WPB}"
+        y = torch.empty_like(x, dtype=out_dtype)
+        torch.ops.spear_btp.forward(coeff, x, y, _no_checkpoint(x), int(k), int(wpb_val))
+        return y
+    return _BTPFunction.apply(coeff, x, k, out_dtype, wpb_val)
 
 
 class _BTPLogFunction(torch.autograd.Function):
