@@ -276,6 +276,8 @@ def main() -> int:
     def serial_floor(read_bytes, write_bytes):  # GB/s of algorithmic bytes if reads and writes just add up
         return (read_bytes + write_bytes) / (read_bytes / read_rate + write_bytes / write_rate)
     floor_fwd, floor_bwd = serial_floor(34, 32), serial_floor(66, 36)
+    # the 2R:1W probe with a compute phase of the backward kernel's length (640 dependent FMAs) between loads and stores
+    with_compute_2r1w = 3 * nbytes / (one_way(7, True) * 1e-3) / 1e9
 
     # log-space gate entry points on the same shape (fp32 gate in, fp32 dgate out: 68 + 108 B per unit)
     for s_ in sets:
@@ -767,6 +769,8 @@ def main() -> int:
             "forward_kernel_vs_best_copy_shape": fwd_gbps / best_copy,
             "backward_kernel_vs_best_2r1w_shape": bwd_gbps / best_2r1w,
             "read_only_GBps": read_rate, "write_only_GBps": write_rate,
+            "nt_2r1w_with_640_dependent_fma_GBps": with_compute_2r1w,
+            "backward_kernel_vs_2r1w_with_compute": bwd_gbps / with_compute_2r1w,
             "serial_read_plus_write_model": {
                 "what": "algorithmic GB/s if a kernel's reads and writes run one after the other at the two rates above",
                 "forward_34R_32W": floor_fwd, "backward_66R_36W": floor_bwd,

@@ -265,9 +265,10 @@ int spear_btp_stream_probe(const void* src_a, const void* src_b, void* dst, unsi
  * the buffer; 4 = one 16-byte element per thread; 5 = reads only (src_a, and src_b if given; `dst` is not
  * written unless every input word is all ones); 6 = writes only (`dst` is filled, nothing is read). HBM serves
  * reads and writes one after the other, so shapes 5 and 6 give the two rates from which the floor of a mixed
- * kernel follows: R bytes read and W bytes written take at least R / read rate + W / write rate. Same arguments
- * and result as spear_btp_stream_probe. */
-#define SPEAR_BTP_PROBE_SHAPES 7
+ * kernel follows: R bytes read and W bytes written take at least R / read rate + W / write rate; 7 = shape 0
+ * with 640 dependent FMAs between loads and stores (the output's last word may differ from shape 0's in its
+ * lowest bit). Same arguments and result as spear_btp_stream_probe. */
+#define SPEAR_BTP_PROBE_SHAPES 8
 int spear_btp_stream_probe_shape(const void* src_a, const void* src_b, void* dst, unsigned long long bytes, int shape,
                                  void* stream);
 

@@ -79,7 +79,7 @@ __global__ __launch_bounds__(64 * kWaves) void jagged_prefill_kernel(
   constexpr bool kHandOver = !kStreamIn && kWaves > 1;
   __shared__ float left_state[kHandOver ? kWaves : 1][kChan];
 
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const long span = first_span_of_workgroup() + wave;
   if (span >= total_spans) {  // wave-uniform
     if constexpr (kHandOver) __syncthreads();  // keep the barrier count equal for every wavefront

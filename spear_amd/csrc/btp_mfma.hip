@@ -88,7 +88,7 @@ __global__ __launch_bounds__(64 * kWaves) void btp_fwd_mfma_kernel(const uint16_
   constexpr int kWaveBytes = 4096 + 512 + kOutBytes + (kTile + kSpan) * 4;
   __shared__ __align__(16) unsigned char lds[kWaves][kWaveBytes];
 
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const long span = first_span_of_workgroup() + wave;
   if (span >= total_spans) return;
   const SpanCoord sc = span_coord(span, spans_per_row, L);

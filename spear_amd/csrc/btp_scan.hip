@@ -103,7 +103,7 @@ __global__ __launch_bounds__(64 * kWaves) SPEAR_BTP_FWD_OCC void btp_fwd_scan_ke
   constexpr bool kHandOver = SPEAR_BTP_HANDOVER && !kStreamIn && kW > 1;
   __shared__ float left_state[kHandOver ? kW : 1][kChan];
 
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const long span = first_span_of_workgroup<(SPEAR_BTP_XCD_REMAP == 2) || (SPEAR_BTP_XCD_REMAP == 1 && !kStreamIn)>(kW) + wave;
   if (span >= total_spans) {  // wave-uniform
     if constexpr (kHandOver) __syncthreads();  // keep the barrier count equal for every wavefront
@@ -245,7 +245,7 @@ __device__ __forceinline__ void btp_bwd_scan_body(
   __shared__ float edge_state[kHandOver ? kW : 1][2][kChan];
 
   SPEAR_BTP_PRIO(3);
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const long span = first_span_of_workgroup(kW) + wave;
   if (span >= total_spans) {  // wave-uniform
     if constexpr (kHandOver) __syncthreads();  // keep the barrier count equal for every wavefront
@@ -502,7 +502,9 @@ __global__ __launch_bounds__(64 * kWaves) void stream_probe_kernel(const uint4* 
 // same loop as a persistent grid striding over the buffer; 4: one 16-byte element per thread; 5 and 6: one
 // direction only (reads without writes, writes without reads), which gives the two rates a mixed kernel's
 // time is made of -- HBM serves reads and writes one after the other, so a kernel that reads R bytes and
-// writes W bytes cannot finish before R / read rate + W / write rate.
+// writes W bytes cannot finish before R / read rate + W / write rate; 7: shape 0 with a chain of 640 dependent
+// FMAs between the loads and the stores (what a compute phase of the backward kernel's length costs even
+// though the vector units are far from busy: every wavefront holds its slot that much longer).
 template <int kReads, int kShape>
 __global__ __launch_bounds__(64 * kWaves) void stream_probe_shape_kernel(const uint4* __restrict__ a,
                                                                          const uint4* __restrict__ b,
@@ -568,6 +570,21 @@ __global__ __launch_bounds__(64 * kWaves) void stream_probe_shape_kernel(const u
         stream_store16(dst + slab * 256 + lane + 64 * i, q[i]);
       }
     }
+  } else if constexpr (kShape == 7) {
+    // the kernels' own shape with arithmetic between the loads and the stores: a chain of 640 dependent FMAs,
+    // about the backward kernel's instruction count, whose result flips one bit of the output's last word
+    const unsigned long long slab = (unsigned long long)blockIdx.x * kWaves + wave;
+    if (slab >= slabs) return;
+    uint4 q[4], r[4];
+    load(slab, q, r);
+    float acc = __uint_as_float(q[0].x & 0x3fffffffu);
+#pragma unroll 1
+    for (int s = 0; s < 80; ++s) {
+#pragma unroll
+      for (int u = 0; u < 8; ++u) acc = __builtin_fmaf(acc, 0.999f, 0.001f);
+    }
+    q[3].w ^= __float_as_uint(acc) & 1u;
+    store(slab, q, r);
   } else {
     static_assert(kShape == 4, "unknown probe shape");
     const unsigned long long i = (unsigned long long)blockIdx.x * (64 * kWaves) + threadIdx.x;
@@ -690,6 +707,7 @@ void launch_probe_shape(const void* a, const void* b, void* dst, unsigned long l
     }
     case 5: hipLaunchKernelGGL((stream_probe_shape_kernel<kReads, 5>), blocks_for(kWaves), wg, 0, s, pa, pb, pd, slabs, 1); break;
     case 6: hipLaunchKernelGGL((stream_probe_shape_kernel<kReads, 6>), blocks_for(kWaves), wg, 0, s, pa, pb, pd, slabs, 1); break;
+    case 7: hipLaunchKernelGGL((stream_probe_shape_kernel<kReads, 7>), blocks_for(kWaves), wg, 0, s, pa, pb, pd, slabs, 1); break;
     default: hipLaunchKernelGGL((stream_probe_shape_kernel<kReads, 4>), blocks_for(1), wg, 0, s, pa, pb, pd, slabs, 1); break;
   }
 }

@@ -329,7 +329,12 @@ def test_measurement_aids_move_the_bytes_they_are_timed_for(slabs):
     assert bool((words[..., 1] == torch.arange(64, device=DEV, dtype=torch.int32).view(1, 1, 64)).all())
     assert bool((words[..., 0] == torch.arange(slabs, device=DEV, dtype=torch.int32).view(slabs, 1, 1)).all())
     assert bool((out[n:] == 0xA5).all())
-    assert lib.spear_btp_stream_probe_shape(a.data_ptr(), None, out.data_ptr(), ctypes.c_ulonglong(n), 7, sp) == -1
+    out.fill_(0xA5)  # shape 7: the 2R:1W combine, up to the lowest bit of every fourth word of a lane's last 16 bytes
+    assert lib.spear_btp_stream_probe_shape(a.data_ptr(), b.data_ptr(), out.data_ptr(), ctypes.c_ulonglong(n), 7, sp) == 0
+    torch.cuda.synchronize()
+    diff = (out[:n] ^ (a ^ b)).view(torch.int32)
+    assert bool(((diff & ~1) == 0).all()) and bool((out[n:] == 0xA5).all())
+    assert lib.spear_btp_stream_probe_shape(a.data_ptr(), None, out.data_ptr(), ctypes.c_ulonglong(n), 8, sp) == -1
     out.fill_(0xA5)
     assert lib.spear_btp_copy(a.data_ptr(), out.data_ptr(), ctypes.c_ulonglong(n), sp) == 0
     torch.cuda.synchronize()
