@@ -180,6 +180,16 @@ int spear_phalanx_mix_backward_bias(const void* a_logit, const void* b_logit, co
                                     int ld_db, int ld_dc, int ld_dv, float* bias_da, float* bias_db, float* bias_dc,
                                     int B, int L, int H, int kv_heads, int dtype, unsigned flags, void* stream);
 
+/* spear_phalanx_mix_forward for a prompt that token-by-token decoding will continue: the same kernel also leaves
+ * the part of the streaming state that depends on the prompt,
+ *     c_prev_tail [B, H, 16] fp32   terminal local state of every row's last block
+ * (after a whole number of blocks the block-local state is 0 and the gate product 1, so this is all of it).
+ * It stands for what parallel_jagged returns beside Y (spear/nn/phalanx/inference.py:327-357) when the layer's gates
+ * are applied in the same pass; layer form only. */
+int spear_phalanx_mix_prefill(const void* a_logit, const void* b_logit, const void* c, const void* v, void* out,
+                              float* c_prev_tail, int B, int L, int H, int kv_heads, int dtype, unsigned flags,
+                              void* stream);
+
 /* One decode token of the mixing stage in the layer's own layout: the four projections' outputs for one time step,
  * [B, features] in `dtype`, and the fp32 streaming state, updated in place. It stands for step_jagged
  * (spear/nn/phalanx/inference.py:178-278) fed by the layer's gates (spear/nn/phalanx/swr.py:196-221): the reference

@@ -31,7 +31,7 @@ FLAG_MIX_QKV_GATE = 0x1
 FLAG_MIX_F32_RESULTS = 0x2
 FLAG_MIX_TILE_SPLIT = 0x4
 FLAG_DX_F32 = 0x10
-_ABI_VERSION = 13
+_ABI_VERSION = 14
 _SUPPORTED_WPB = (4, 8, 16, 32)
 
 _lock = threading.Lock()
@@ -66,6 +66,8 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.spear_phalanx_mix_backward_bias.restype = ci
     lib.spear_phalanx_mix_backward_sum_rows.argtypes = [ci, ci, ci]
     lib.spear_phalanx_mix_backward_sum_rows.restype = ctypes.c_longlong
+    lib.spear_phalanx_mix_prefill.argtypes = [vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, cu, vp]
+    lib.spear_phalanx_mix_prefill.restype = ci
     lib.spear_phalanx_mix_step.argtypes = [vp] * 9 + [ci] * 6 + [cu, vp]
     lib.spear_phalanx_mix_step.restype = ci
     lib.spear_jagged_prefill.argtypes = [vp] * 9 + [ci] * 9 + [cu, vp]
@@ -338,11 +340,14 @@ def mix_forward(
     heads: int,
     kv_heads: int,
     qkv_gate: bool = False,
+    c_prev_tail: torch.Tensor | None = None,
 ) -> None:
     """``out <- btp(sigmoid(a_logit), sigmoid(b_logit) * v) * c + v`` with every operand in the
     layer's ``[B, L, features]`` layout (see ``spear_phalanx_mix_forward`` in the C header).
     ``qkv_gate``: ``a_logit`` is an fp32 log-decay gate, ``b_logit`` is k, ``c`` is q:
-    ``out <- c * btp(exp(a_logit), b_logit * v) + v`` (``SPEAR_MIX_QKV_GATE``)."""
+    ``out <- c * btp(exp(a_logit), b_logit * v) + v`` (``SPEAR_MIX_QKV_GATE``). ``c_prev_tail``: fp32
+    ``[B, heads, 16]`` that receives the terminal local state of every row's last block, the hand-over state
+    for decoding after this prompt (``spear_phalanx_mix_prefill``)."""
     _check(all(t.is_cuda for t in (a_logit, b_logit, c, v, out)), "All tensors must be CUDA.")
     _check(v.dim() == 3, "v must be [B, L, heads * 16].")
     B, L, F = v.shape
@@ -364,10 +369,14 @@ def mix_forward(
     _check_layout("v", v, (B, L, F))
     _check_layout("out", out, (B, L, F))
     _check(len({t.device for t in (a_logit, b_logit, c, v, out)}) == 1, "All tensors must be on the same device.")
+    if c_prev_tail is not None:
+        _check(c_prev_tail.is_cuda and c_prev_tail.device == v.device and c_prev_tail.dtype == torch.float32,
+               "c_prev_tail must be float32 on v's device.")
+        _check_layout("c_prev_tail", c_prev_tail, (B, heads, 16))
     lib = load_library()
     with torch.cuda.device(v.device):
-        rc = lib.spear_phalanx_mix_forward(
-            a_logit.data_ptr(), b_logit.data_ptr(), c.data_ptr(), v.data_ptr(), out.data_ptr(),
+        rc = lib.spear_phalanx_mix_prefill(
+            a_logit.data_ptr(), b_logit.data_ptr(), c.data_ptr(), v.data_ptr(), out.data_ptr(), _ptr(c_prev_tail),
             B, L, heads, kv_heads, _tag(v.dtype),
             (FLAG_MIX_QKV_GATE if qkv_gate else 0) | (FLAG_MIX_F32_RESULTS if f32 else 0), _stream_ptr(v.device),
         )

@@ -45,7 +45,7 @@ int check_common(const char* who, int B, int H, int L, int k, int in_dtype, int 
 
 extern "C" {
 
-int spear_btp_abi_version(void) { return 13; }
+int spear_btp_abi_version(void) { return 14; }
 
 const char* spear_btp_last_error(void) { return g_error; }
 
@@ -130,8 +130,14 @@ int spear_btp_backward_loggate(const float* gate, const void* x, const void* dy,
 
 int spear_phalanx_mix_forward(const void* a_logit, const void* b_logit, const void* c, const void* v, void* out, int B,
                               int L, int H, int kv_heads, int dtype, unsigned flags, void* stream) {
+  return spear_phalanx_mix_prefill(a_logit, b_logit, c, v, out, nullptr, B, L, H, kv_heads, dtype, flags, stream);
+}
+
+int spear_phalanx_mix_prefill(const void* a_logit, const void* b_logit, const void* c, const void* v, void* out,
+                              float* c_prev_tail, int B, int L, int H, int kv_heads, int dtype, unsigned flags,
+                              void* stream) {
   g_error[0] = '\0';
-  const char* who = "spear_phalanx_mix_forward";
+  const char* who = c_prev_tail ? "spear_phalanx_mix_prefill" : "spear_phalanx_mix_forward";
   if (B < 0 || L < 0 || H < 0) return fail(SPEAR_BTP_EINVAL, "%s: negative dimension (B=%d L=%d H=%d)", who, B, L, H);
   if (L % 16 != 0) return fail(SPEAR_BTP_EINVAL, "%s: Length L must be multiple of 16 (got %d)", who, L);
   if (H % 4 != 0) return fail(SPEAR_BTP_EINVAL, "%s: heads must be a multiple of 4 (got %d)", who, H);
@@ -149,7 +155,11 @@ int spear_phalanx_mix_forward(const void* a_logit, const void* b_logit, const vo
   if (!a_logit || !b_logit || !c || !v || !out) return fail(SPEAR_BTP_ENULL, "%s: NULL tensor pointer", who);
   if (!aligned16(a_logit) || !aligned16(b_logit) || !aligned16(c) || !aligned16(v) || !aligned16(out))
     return fail(SPEAR_BTP_EINVAL, "%s: tensor pointers must be 16-byte aligned", who);
-  spear_btp::MixArgs a{a_logit, b_logit, c, v, out, B, L, H, H / kv_heads, dtype, (flags & SPEAR_MIX_QKV_GATE) != 0, f32};
+  if (c_prev_tail && !aligned16(c_prev_tail)) return fail(SPEAR_BTP_EINVAL, "%s: tensor pointers must be 16-byte aligned", who);
+  if (c_prev_tail && (flags & SPEAR_MIX_QKV_GATE))
+    return fail(SPEAR_BTP_EINVAL, "%s: the hand-over state belongs to the layer form, not SPEAR_MIX_QKV_GATE", who);
+  spear_btp::MixArgs a{a_logit, b_logit, c, v, out, B, L, H, H / kv_heads, dtype, (flags & SPEAR_MIX_QKV_GATE) != 0, f32,
+                       c_prev_tail};
   const hipError_t err = spear_btp::fused_mix_forward(a, static_cast<hipStream_t>(stream));
   if (err != hipSuccess) return fail(SPEAR_BTP_ELAUNCH, "%s: launch failed: %s", who, hipGetErrorString(err));
   return 0;

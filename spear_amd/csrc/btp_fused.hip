@@ -93,8 +93,8 @@ typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
 template <class E, int kFwdWaves, bool kQkv, bool kF32>
 __global__ __launch_bounds__(64 * kFwdWaves) void phalanx_mix_fwd_kernel(
     const uint16_t* __restrict__ a_logit, const uint16_t* __restrict__ b_logit, const uint16_t* __restrict__ c_in,
-    const uint16_t* __restrict__ v_in, uint16_t* __restrict__ out, int L, int H, int kv_groups, int chunk_steps,
-    int chunks, long total_waves) {
+    const uint16_t* __restrict__ v_in, uint16_t* __restrict__ out, float* __restrict__ c_prev_tail, int L, int H,
+    int kv_groups, int chunk_steps, int chunks, long total_waves) {
   __shared__ __align__(16) float a_tile[kFwdWaves][kHeadsPerWave * kGateRow];  // [head][step] decay, fp32
 
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
@@ -252,6 +252,10 @@ __global__ __launch_bounds__(64 * kFwdWaves) void phalanx_mix_fwd_kernel(
     }
     __builtin_amdgcn_sched_barrier(0);
   }
+  // Hand-over for token-by-token decoding after this prompt: the terminal local state of the row's last block is
+  // what the next block's steps need as c_prev (the block-local state restarts at 0 and the gate product at 1).
+  if (c_prev_tail != nullptr && t_end == L && real)
+    *reinterpret_cast<float2*>(c_prev_tail + (brow * H + head) * kChan + d0) = make_float2(carry0, carry1);
 }
 
 
@@ -1046,7 +1050,7 @@ void launch_mix_fwd(const MixArgs& p, const MixPlan& m, hipStream_t s) {
   hipLaunchKernelGGL((phalanx_mix_fwd_kernel<E, kW, kQkv, kF32>), dim3(blocks), dim3(64 * kW), 0, s,
                      static_cast<const uint16_t*>(p.a_logit), static_cast<const uint16_t*>(p.b_logit),
                      static_cast<const uint16_t*>(p.c), static_cast<const uint16_t*>(p.v), static_cast<uint16_t*>(p.out),
-                     p.L, p.H, p.kv_groups, m.chunk_blocks * kTile, m.chunks, total);
+                     p.c_prev_tail, p.L, p.H, p.kv_groups, m.chunk_blocks * kTile, m.chunks, total);
 }
 
 }  // namespace

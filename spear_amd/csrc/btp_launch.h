@@ -51,6 +51,9 @@ struct MixArgs {
   // q/k/v/gate form: a_logit is an fp32 log-decay gate (a = exp(gate)), b_logit is k (used as it is), c is q
   bool qkv = false;
   bool f32_out = false;  // check mode: `out` is fp32
+  // null, or fp32 [B, H, 16]: receives the terminal local state of every row's last block (the c_prev of the
+  // streaming state after this prompt)
+  float* c_prev_tail = nullptr;
 };
 hipError_t fused_mix_forward(const MixArgs& p, hipStream_t s);
 

@@ -28,7 +28,7 @@ gated, kv-expanded ``[B, H, D]`` operands): ``phalanx_step(layer, x_t, state)`` 
 ``Phalanx`` layer -- four projections, ONE kernel for gates + recurrence step + ``* C + V`` on the projections'
 ``[B, features]`` outputs (``spear_phalanx_mix_step``), output projection -- with the block position kept on the
 device, so that the step records into one HIP graph that serves every token; ``phalanx_prefill`` runs a prompt
-through the layer and hands over the state to continue from.
+through the layer (fused forward kernel, which also leaves the hand-over state) and returns the state to continue from.
 
 The state ``parallel_jagged`` returns for a prompt whose length is a multiple of ``block_len``
 follows the reference as written (inference.py:327-341): ``h_loc`` is the last block's terminal
@@ -328,21 +328,30 @@ def phalanx_step(layer, x_t: torch.Tensor, state: PhalanxStepState, out: torch.T
 
 @torch.no_grad()
 def phalanx_prefill(layer, x: torch.Tensor) -> tuple[torch.Tensor, PhalanxStepState]:
-    """A prompt ``x`` [B, L, dim] (any L >= 1) through ``layer``: returns ``layer``'s output for it and the
-    state after its last token, from which :func:`phalanx_step` continues. The output of the whole blocks comes
-    from the layer's own forward; the state depends only on the last completed block and the partial block
-    after it (the carry is one hop), so it is rebuilt by stepping through those at most 31 tokens from the zero
-    state; a partial last block's outputs are taken from those steps."""
+    """A prompt ``x`` [B, L, dim] (any L >= 1) through ``layer``: returns the layer's output for it and the state
+    after its last token, from which :func:`phalanx_step` continues. The whole blocks go through the fused
+    forward kernel, which also leaves the hand-over state (``spear_phalanx_mix_prefill``: after a whole number of
+    blocks the state is the last block's terminal local state, a zero block-local state and a gate product of
+    one); the at most 15 tokens of a partial last block are projected together and stepped one kernel each."""
     _need_gpu(x)
     B, L, _ = x.shape
-    bl = 16
+    p, bl = layer.param, 16
+    if layer.heads % 4 != 0 or layer.k != 2:
+        raise RuntimeError("phalanx_prefill needs a layer the fused kernels serve: heads divisible by 4, k == 2")
     full = (L // bl) * bl
-    start = max(0, full - bl) if L > full else max(0, L - bl)  # a block boundary: stepping from zero there is exact
     state = PhalanxStepState.zeros(B, layer.heads, x.device, bl)
-    tail = torch.empty(B, L - start, layer.dim, device=x.device, dtype=layer.proj_out.weight.dtype)
-    for t in range(start, L):
-        phalanx_step(layer, x[:, t], state, out=tail[:, t - start])
-    if full == 0:
-        return tail, state
-    y_full = layer(x[:, :full])
-    return (y_full if L == full else torch.cat([y_full, tail[:, full - start:]], dim=1)), state
+    xc = x.to(p.compute_dtype)
+    parts = []
+    if full > 0:
+        a, b, c, v = (proj(xc[:, :full]) for proj in (p.proj_a, p.proj_b, p.proj_c, p.proj_v))
+        mixed = torch.empty_like(v)
+        _btp.mix_forward(a, b, c, v, mixed, layer.heads, layer.kv_heads, c_prev_tail=state.c_prev_loc)
+        parts.append(mixed)
+    if L > full:
+        a, b, c, v = (proj(xc[:, full:]).transpose(0, 1).contiguous() for proj in (p.proj_a, p.proj_b, p.proj_c, p.proj_v))
+        tail = torch.empty_like(v)  # [tokens, B, dim]
+        for t in range(L - full):
+            _btp.mix_step(a[t], b[t], c[t], v[t], tail[t], state.h_loc, state.r_pref, state.c_prev_loc, state.pos, False,
+                          bl, layer.heads, layer.kv_heads)
+        parts.append(tail.transpose(0, 1))
+    return layer.proj_out(parts[0] if len(parts) == 1 else torch.cat(parts, dim=1)), state

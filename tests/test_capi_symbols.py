@@ -34,6 +34,7 @@ def test_header_declares_the_expected_entry_points():
         "spear_phalanx_mix_backward_ex",
         "spear_phalanx_mix_backward_sum_rows",
         "spear_phalanx_mix_forward",
+        "spear_phalanx_mix_prefill",
         "spear_phalanx_mix_step",
     ]
 
