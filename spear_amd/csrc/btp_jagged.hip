@@ -80,7 +80,7 @@ __global__ __launch_bounds__(64 * kWaves) void jagged_prefill_kernel(
   __shared__ float left_state[kHandOver ? kWaves : 1][kChan];
 
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
-  const long span = first_span_of_workgroup() + wave;
+  const long span = first_span_of_workgroup<(SPEAR_BTP_XCD_REMAP == 2) || (SPEAR_BTP_XCD_REMAP == 1 && !kStreamIn)>() + wave;
   if (span >= total_spans) {  // wave-uniform
     if constexpr (kHandOver) __syncthreads();  // keep the barrier count equal for every wavefront
     return;

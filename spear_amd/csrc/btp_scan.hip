@@ -246,7 +246,7 @@ __device__ __forceinline__ void btp_bwd_scan_body(
 
   SPEAR_BTP_PRIO(3);
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
-  const long span = first_span_of_workgroup(kW) + wave;
+  const long span = first_span_of_workgroup<(SPEAR_BTP_XCD_REMAP == 2) || (SPEAR_BTP_XCD_REMAP == 1 && !kStreamIn)>(kW) + wave;
   if (span >= total_spans) {  // wave-uniform
     if constexpr (kHandOver) __syncthreads();  // keep the barrier count equal for every wavefront
     return;

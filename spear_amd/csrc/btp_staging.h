@@ -433,19 +433,33 @@ __device__ __forceinline__ SpanCoord span_coord(long span, int spans_per_row, in
 }
 
 // Workgroup index -> first span. Workgroups are dealt round-robin to the 8 XCDs, each with its own L2. With
-// kRemap each XCD instead walks one contiguous eighth of the tensor, so that the workgroup that reads a halo
-// and the one that streams the same lines run on the same L2. Measured: the forward kernel on rows of several
-// spans gains 1.8 % (B=16 H=64 L=8192) and 0.5 % (B=64 H=128 L=2048); the backward kernel loses 2 %, and on
-// rows of one span, where nothing is shared, both lose 12 %. So only that one case uses it.
-#ifndef SPEAR_BTP_XCD_REMAP  // 0: never, 1: forward kernel on rows of several spans, 2: every kernel
+// kRemap an XCD instead gets runs of SPEAR_BTP_XCD_GROUP neighbouring workgroups (windows of 8 such runs sweep
+// the tensor, so the chip as a whole still walks memory front to back): the workgroup that reads a halo and the
+// one that streams the same lines then run on the same L2 close in time, and the halo's 128-byte lines are
+// fetched once. Measured on rows of several spans (B=16 H=64 L=8192 / B=64 H=128 L=2048), against plain
+// round-robin: runs of 32 gain 1.3 % / 3.6 % in forward and 1.5 % / 1.6 % in backward; runs of 2-8 gain nothing,
+// runs of 128 and more lose again in backward, and one contiguous eighth of the tensor per XCD (group 0) gains
+// 1.8 % / 0.5 % in forward and loses 2 % in backward. On rows of one span nothing is shared and any dealing
+// other than round-robin loses 12 %, so those keep the plain order.
+#ifndef SPEAR_BTP_XCD_REMAP  // 0: never, 1: kernels on rows of several spans, 2: every kernel
 #define SPEAR_BTP_XCD_REMAP 1
+#endif
+#ifndef SPEAR_BTP_XCD_GROUP  // 0: one contiguous eighth per XCD; G > 0: runs of G neighbouring workgroups per XCD
+#define SPEAR_BTP_XCD_GROUP 32
 #endif
 template <bool kRemap = (SPEAR_BTP_XCD_REMAP == 2)>
 __device__ __forceinline__ long first_span_of_workgroup(int waves = kWaves) {
   if constexpr (kRemap) {
     const unsigned n = gridDim.x, b = blockIdx.x;
-    const unsigned per = n >> 3;
-    const unsigned mapped = (b < (per << 3)) ? (b & 7u) * per + (b >> 3) : b;
+    unsigned mapped = b;
+    if constexpr (SPEAR_BTP_XCD_GROUP > 0) {
+      constexpr unsigned kWin = 8u * SPEAR_BTP_XCD_GROUP;
+      const unsigned win = b / kWin, in = b - win * kWin;
+      if ((win + 1) * kWin <= n) mapped = win * kWin + (in & 7u) * SPEAR_BTP_XCD_GROUP + (in >> 3);
+    } else {
+      const unsigned per = n >> 3;
+      if (b < (per << 3)) mapped = (b & 7u) * per + (b >> 3);
+    }
     return (long)mapped * waves;
   } else {
     return (long)blockIdx.x * waves;
