@@ -169,16 +169,26 @@ __device__ __forceinline__ uint4 load16(const void* p) {
   return *reinterpret_cast<const uint4*>(p);
 }
 
+// Lanes past the row's end read the row's first chunk instead (always there) and drop it afterwards, so the
+// loads are unconditional straight-line code. With one branch per load ("valid ? load : 0") the compiler placed
+// waits for earlier loads inside the branches, and a wavefront made two or three serial trips to memory.
+// `plain` (wave-uniform) turns a streaming slab read into a plain (cached) one for this wavefront: the kernels
+// let part of a workgroup's wavefronts read that way (the masks are in btp_scan.hip).
 template <bool kStream>
 __device__ __forceinline__ void slab16_global_to_regs(const uint16_t* slab, long L, int nvalid,
-                                                      int lane, uint4 (&q)[4]) {
+                                                      int lane, uint4 (&q)[4], bool plain = false) {
   const int lr = lane >> 4, lp = lane & 15;
   const bool ok = (lp << 3) < nvalid;
+  const uint16_t* src = slab + (long)lr * L + (ok ? (lp << 3) : 0);
+  if (kStream && !plain) {
 #pragma unroll
-  for (int it = 0; it < 4; ++it) {
-    const int r = it * 4 + lr;
-    q[it] = ok ? load16<kStream>(slab + (long)r * L + (lp << 3)) : zero4();
+    for (int it = 0; it < 4; ++it) q[it] = load16<true>(src + (long)(it * 4) * L);
+  } else {
+#pragma unroll
+    for (int it = 0; it < 4; ++it) q[it] = load16<false>(src + (long)(it * 4) * L);
   }
+#pragma unroll
+  for (int it = 0; it < 4; ++it) q[it] = ok ? q[it] : zero4();
 }
 
 __device__ __forceinline__ void slab16_regs_to_lds(unsigned char* img, int lane, const uint4 (&q)[4]) {
@@ -196,6 +206,7 @@ __device__ __forceinline__ void store16(void* p, const uint4& q) {
   else *reinterpret_cast<uint4*>(p) = q;
 }
 
+// Stores stay non-temporal in every wavefront: plain stores measured 5-10 % slower in any share.
 template <bool kStream>
 __device__ __forceinline__ void slab16_lds_to_global(const unsigned char* img, uint16_t* slab, long L,
                                                      int nvalid, int lane) {
@@ -320,11 +331,11 @@ __device__ __forceinline__ void slab32_global_to_regs(const float* slab, long L,
                                                       uint4 (&q)[8]) {
   const int lr = lane >> 5, lp = lane & 31;
   const bool ok = (lp << 2) < nvalid;
+  const float* src = slab + (long)lr * L + (ok ? (lp << 2) : 0);  // see slab16_global_to_regs
 #pragma unroll
-  for (int it = 0; it < 8; ++it) {
-    const int r = it * 2 + lr;
-    q[it] = ok ? load16<kStream>(slab + (long)r * L + (lp << 2)) : zero4();
-  }
+  for (int it = 0; it < 8; ++it) q[it] = load16<kStream>(src + (long)(it * 2) * L);
+#pragma unroll
+  for (int it = 0; it < 8; ++it) q[it] = ok ? q[it] : zero4();
 }
 
 __device__ __forceinline__ void slab32_regs_to_lds(unsigned char* img, int lane, const uint4 (&q)[8]) {
@@ -385,7 +396,9 @@ __device__ __forceinline__ void lane_write32(unsigned char* img, int j, int d, c
 // reads back the 32 of its own two blocks (a broadcast read for the 16 lanes of a group).
 template <class C>
 __device__ __forceinline__ typename C::pair_t coeff_global_to_reg(const typename C::elem* arow, int nvalid, int lane) {
-  return ((lane << 1) < nvalid) ? C::load_pair(arow + (lane << 1)) : C::zero_pair();
+  const bool ok = (lane << 1) < nvalid;  // unconditional load, as in slab16_global_to_regs
+  const typename C::pair_t w = C::load_pair(arow + (ok ? (lane << 1) : 0));
+  return ok ? w : C::zero_pair();
 }
 
 // rows of any length: element-aligned address, and the last pair may hold a single coefficient
