@@ -106,7 +106,7 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--config", choices=sorted(CONFIGS), default="c3")
-    ap.add_argument("--sets", type=int, default=4, help="independent buffer sets to rotate over")
+    ap.add_argument("--sets", type=int, default=8, help="independent buffer sets to rotate over")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-fused", action="store_true", help="skip the fused layer-layout forward leg")
     ap.add_argument("--no-streaming", action="store_true", help="skip the prefill / decode-step leg")
@@ -311,7 +311,7 @@ def main() -> int:
         F = H * 16
         g = torch.Generator(device="cpu").manual_seed(seed + 7)
         msets = []
-        for _ in range(min(len(sets), 3)):
+        for _ in range(min(len(sets), 4)):
             msets.append({
                 "a": torch.randn(B, L, H, generator=g).to(torch.bfloat16).to(dev),
                 "b": torch.randn(B, L, F, generator=g).to(torch.bfloat16).to(dev),

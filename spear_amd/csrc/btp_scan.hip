@@ -61,27 +61,6 @@
 #ifndef SPEAR_BTP_HANDOVER  // 1: carries between the spans of a workgroup go through LDS; 0: every span reads its halo
 #define SPEAR_BTP_HANDOVER 1
 #endif
-// Which wavefronts of a workgroup read their x slab with plain (cached) loads instead of non-temporal ones: bit w
-// = wavefront w. *_SHORT: rows of one span (4-wavefront workgroups); *_LONG: rows of several spans. Measured at
-// B*H = 32768 rows of L = 128: every x load non-temporal 43.4 / 67.9 us (forward / backward), one wavefront in
-// four plain 40.8 / 65.0, two or three of four (any of them) 40.3 / 63.3, all four 45.1 / 68.9; plain dy loads
-// and plain stores lose in any share, and rows of several spans are fastest with every load non-temporal.
-#ifndef SPEAR_BTP_PLAIN_X_FWD_SHORT
-#define SPEAR_BTP_PLAIN_X_FWD_SHORT 0x3
-#endif
-#ifndef SPEAR_BTP_PLAIN_X_FWD_LONG
-#define SPEAR_BTP_PLAIN_X_FWD_LONG 0
-#endif
-#ifndef SPEAR_BTP_PLAIN_X_BWD_SHORT
-#define SPEAR_BTP_PLAIN_X_BWD_SHORT 0x3
-#endif
-#ifndef SPEAR_BTP_PLAIN_X_BWD_LONG
-#define SPEAR_BTP_PLAIN_X_BWD_LONG 0
-#endif
-template <bool kSingleSpan>
-__device__ __forceinline__ bool plain_wave(unsigned mask_short, unsigned mask_long, int wave) {
-  return (((kSingleSpan ? mask_short : mask_long) >> wave) & 1u) != 0;  // wave-uniform
-}
 #ifndef SPEAR_BTP_SETPRIO  // 1: wavefronts run at raised priority while they issue their global loads / stores
 #define SPEAR_BTP_SETPRIO 0
 #endif
@@ -143,8 +122,7 @@ __global__ __launch_bounds__(64 * kWaves) SPEAR_BTP_FWD_OCC void btp_fwd_scan_ke
   // the wavefronts of a workgroup (below); only a workgroup's first span re-reads 16 steps.
   constexpr bool kStreamOut = SPEAR_BTP_STREAM_STORES == 1;
   uint4 xin[4];
-  slab16_global_to_regs<nt_loads(kStreamIn)>(xslab, L, sc.nvalid, lane, xin,
-      plain_wave<kStreamIn>(SPEAR_BTP_PLAIN_X_FWD_SHORT, SPEAR_BTP_PLAIN_X_FWD_LONG, wave));
+  slab16_global_to_regs<nt_loads(kStreamIn)>(xslab, L, sc.nvalid, lane, xin);
   const typename C::pair_t ain = coeff_global_to_reg<C>(arow, sc.nvalid, lane);
 
   const bool needs_left = (k == 2) && (sc.sp > 0);            // wave-uniform
@@ -287,8 +265,7 @@ __device__ __forceinline__ void btp_bwd_scan_body(
   constexpr bool kStreamOut = SPEAR_BTP_STREAM_STORES == 1;  // see the forward kernel
   uint4 xin[4];
   uint4 gin[kGradF32 ? 8 : 4];
-  slab16_global_to_regs<nt_loads(kStreamIn)>(xslab, L, sc.nvalid, lane, xin,
-      plain_wave<kStreamIn>(SPEAR_BTP_PLAIN_X_BWD_SHORT, SPEAR_BTP_PLAIN_X_BWD_LONG, wave));
+  slab16_global_to_regs<nt_loads(kStreamIn)>(xslab, L, sc.nvalid, lane, xin);
   if constexpr (kGradF32) {
     slab32_global_to_regs<nt_loads(kStreamIn)>(reinterpret_cast<const float*>(dy) + slab_off, L, sc.nvalid, lane, gin);
   } else {

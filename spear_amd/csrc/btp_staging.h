@@ -172,21 +172,14 @@ __device__ __forceinline__ uint4 load16(const void* p) {
 // Lanes past the row's end read the row's first chunk instead (always there) and drop it afterwards, so the
 // loads are unconditional straight-line code. With one branch per load ("valid ? load : 0") the compiler placed
 // waits for earlier loads inside the branches, and a wavefront made two or three serial trips to memory.
-// `plain` (wave-uniform) turns a streaming slab read into a plain (cached) one for this wavefront: the kernels
-// let part of a workgroup's wavefronts read that way (the masks are in btp_scan.hip).
 template <bool kStream>
 __device__ __forceinline__ void slab16_global_to_regs(const uint16_t* slab, long L, int nvalid,
-                                                      int lane, uint4 (&q)[4], bool plain = false) {
+                                                      int lane, uint4 (&q)[4]) {
   const int lr = lane >> 4, lp = lane & 15;
   const bool ok = (lp << 3) < nvalid;
   const uint16_t* src = slab + (long)lr * L + (ok ? (lp << 3) : 0);
-  if (kStream && !plain) {
 #pragma unroll
-    for (int it = 0; it < 4; ++it) q[it] = load16<true>(src + (long)(it * 4) * L);
-  } else {
-#pragma unroll
-    for (int it = 0; it < 4; ++it) q[it] = load16<false>(src + (long)(it * 4) * L);
-  }
+  for (int it = 0; it < 4; ++it) q[it] = load16<kStream>(src + (long)(it * 4) * L);
 #pragma unroll
   for (int it = 0; it < 4; ++it) q[it] = ok ? q[it] : zero4();
 }
@@ -206,7 +199,6 @@ __device__ __forceinline__ void store16(void* p, const uint4& q) {
   else *reinterpret_cast<uint4*>(p) = q;
 }
 
-// Stores stay non-temporal in every wavefront: plain stores measured 5-10 % slower in any share.
 template <bool kStream>
 __device__ __forceinline__ void slab16_lds_to_global(const unsigned char* img, uint16_t* slab, long L,
                                                      int nvalid, int lane) {
