@@ -398,6 +398,20 @@ def main() -> int:
         mix_ms, unfused_ms = kernel_ms_over(mix, msets), kernel_ms_over(mix_unfused, msets)
         mix_bwd_ms, unfused_train_ms = kernel_ms_over(mix_bwd, msets), kernel_ms_over(mix_unfused_train, msets)
         mix_bwd_tile_ms = kernel_ms_over(mix_bwd_tile, msets)
+
+        # what the memory system gives these stream counts in its best shape (contiguous 4 KiB pieces, short-lived
+        # wavefronts, nothing shared): 3 inputs -> 1 output (forward) and 4 inputs -> 3 outputs (backward), without
+        # and with a compute phase between the loads and the stores
+        big = B * L * F * 2
+        def mix_probe(n_src, n_dst, compute):
+            def fn(s):
+                src = (ctypes.c_void_p * n_src)(*[s[k].data_ptr() for k in ("b", "c", "v", "dout")[:n_src]])
+                dst = (ctypes.c_void_p * n_dst)(*[s[k].data_ptr() for k in ("db", "dc", "dv")[:n_dst]])
+                rc = lib.spear_btp_stream_probe_mix(src, n_src, dst, n_dst, ctypes.c_ulonglong(big), compute, sp)
+                assert rc == 0, lib.spear_btp_last_error()
+            return (n_src + n_dst) * big / (kernel_ms_over(fn, msets) * 1e-3) / 1e9
+        ceil_fwd, ceil_fwd_c = mix_probe(3, 1, 0), mix_probe(3, 1, 1)
+        ceil_bwd, ceil_bwd_c = mix_probe(4, 3, 0), mix_probe(4, 3, 1)
         mix_bytes = B * L * H * (2 + 3 * 32 + 32)          # a, b, c, v read; out written
         mix_bwd_bytes = B * L * H * (2 + 4 * 32 + 2 + 3 * 32)  # a, b, c, v, dout read; da, db, dc, dv written
         fused = {
@@ -410,6 +424,11 @@ def main() -> int:
                 "frac": mix_bwd_bytes / (mix_bwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
                 "tile_split_avg_launch_ms": mix_bwd_tile_ms,
                 "tile_split_frac": mix_bwd_bytes / (mix_bwd_tile_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+            },
+            "ceilings_GBps": {
+                "what": "spear_btp_stream_probe_mix on the same buffers: no arithmetic / with a chain of dependent FMAs (640 forward, 1280 backward)",
+                "forward_3_inputs_1_output": [ceil_fwd, ceil_fwd_c],
+                "backward_4_inputs_3_outputs": [ceil_bwd, ceil_bwd_c],
             },
             "fwd_plus_bwd_ms": mix_ms + mix_bwd_ms,
             "same_stage_fwd_plus_bwd_from_pytorch_ops_plus_btp_kernels_ms": unfused_train_ms,

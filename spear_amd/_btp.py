@@ -84,6 +84,8 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.spear_btp_stream_probe.restype = ci
     lib.spear_btp_stream_probe_shape.argtypes = [vp, vp, vp, ctypes.c_ulonglong, ci, vp]
     lib.spear_btp_stream_probe_shape.restype = ci
+    lib.spear_btp_stream_probe_mix.argtypes = [ctypes.POINTER(vp), ci, ctypes.POINTER(vp), ci, ctypes.c_ulonglong, ci, vp]
+    lib.spear_btp_stream_probe_mix.restype = ci
 
 
 def load_library() -> ctypes.CDLL:

@@ -402,4 +402,21 @@ int spear_btp_stream_probe_shape(const void* src_a, const void* src_b, void* dst
   return 0;
 }
 
+int spear_btp_stream_probe_mix(const void* const* src, int n_src, void* const* dst, int n_dst, unsigned long long bytes,
+                               int compute, void* stream) {
+  g_error[0] = '\0';
+  const char* who = "spear_btp_stream_probe_mix";
+  if (!src || !dst) return fail(SPEAR_BTP_ENULL, "%s: NULL pointer", who);
+  if (!((n_src == 3 && n_dst == 1) || (n_src == 4 && n_dst == 3)))
+    return fail(SPEAR_BTP_EINVAL, "%s: (n_src, n_dst) must be (3, 1) or (4, 3) (got %d, %d)", who, n_src, n_dst);
+  if (bytes % 4096 != 0) return fail(SPEAR_BTP_EINVAL, "%s: size must be a multiple of 4096", who);
+  for (int i = 0; i < n_src; ++i)
+    if (!src[i] || !aligned16(src[i])) return fail(SPEAR_BTP_EINVAL, "%s: every tensor pointer must be set and 16-byte aligned", who);
+  for (int i = 0; i < n_dst; ++i)
+    if (!dst[i] || !aligned16(dst[i])) return fail(SPEAR_BTP_EINVAL, "%s: every tensor pointer must be set and 16-byte aligned", who);
+  const hipError_t err = spear_btp::stream_probe_mix(src, n_src, dst, n_dst, bytes, compute != 0, static_cast<hipStream_t>(stream));
+  if (err != hipSuccess) return fail(SPEAR_BTP_ELAUNCH, "%s: launch failed: %s", who, hipGetErrorString(err));
+  return 0;
+}
+
 }  // extern "C"

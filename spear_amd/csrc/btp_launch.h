@@ -129,5 +129,8 @@ hipError_t device_copy(const void* src, void* dst, unsigned long long bytes, hip
 hipError_t stream_probe(const void* a, const void* b, void* dst, unsigned long long bytes, hipStream_t s);
 // The same traffic in other launch shapes (0 = the one above, 1..4 see stream_probe_shape_kernel).
 hipError_t stream_probe_shape(const void* a, const void* b, void* dst, unsigned long long bytes, int shape, hipStream_t s);
+// The probe with the fused kernels' stream counts: (n_src, n_dst) = (3, 1) or (4, 3); `compute` adds a compute phase.
+hipError_t stream_probe_mix(const void* const* src, int n_src, void* const* dst, int n_dst, unsigned long long bytes,
+                            bool compute, hipStream_t s);
 
 }  // namespace spear_btp

@@ -599,6 +599,42 @@ __global__ __launch_bounds__(64 * kWaves) void stream_probe_shape_kernel(const u
   }
 }
 
+// The probe for kernels with more streams: kIn inputs combined into kOut identical outputs, every tensor `slabs`
+// pieces of 4 KiB, one piece per wavefront and tensor, non-temporal 16-byte accesses (the fused layer kernels read
+// 3 or 4 big tensors and write 1 or 3). kSpin > 0 puts 8 * kSpin dependent FMAs between the loads and the stores;
+// their result flips the lowest bit of every output's last word.
+struct ProbeMixPtrs {
+  const uint4* in[4];
+  uint4* out[3];
+};
+template <int kIn, int kOut, int kSpin>
+__global__ __launch_bounds__(64 * kWaves) void stream_probe_mix_kernel(ProbeMixPtrs p, unsigned long long slabs) {
+  const unsigned long long slab = (unsigned long long)blockIdx.x * kWaves + (threadIdx.x >> 6);
+  if (slab >= slabs) return;
+  const unsigned long long base = slab * 256 + (threadIdx.x & 63);
+  uint4 q[kIn][4];
+#pragma unroll
+  for (int t = 0; t < kIn; ++t) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) q[t][i] = stream_load16(p.in[t] + base + 64 * i);
+  }
+  float acc = __uint_as_float(q[0][0].x & 0x3fffffffu);
+#pragma unroll 1
+  for (int s = 0; s < kSpin; ++s) {
+#pragma unroll
+    for (int u = 0; u < 8; ++u) acc = __builtin_fmaf(acc, 0.999f, 0.001f);
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    uint4 o = q[0][i];
+#pragma unroll
+    for (int t = 1; t < kIn; ++t) o = make_uint4(o.x ^ q[t][i].x, o.y ^ q[t][i].y, o.z ^ q[t][i].z, o.w ^ q[t][i].w);
+    if (kSpin > 0 && i == 3) o.w ^= __float_as_uint(acc) & 1u;
+#pragma unroll
+    for (int t = 0; t < kOut; ++t) stream_store16(p.out[t] + base + 64 * i, o);
+  }
+}
+
 template <class E, class C, class OutT, bool kCheckpoint, bool kStreamIn>
 void launch_fwd_as(const FwdArgs& p, const Grid& g, hipStream_t s) {
   hipLaunchKernelGGL((btp_fwd_scan_kernel<E, C, OutT, kCheckpoint, kStreamIn>), dim3(g.blocks), dim3(64 * g.waves), 0,
@@ -719,6 +755,26 @@ hipError_t stream_probe_shape(const void* a, const void* b, void* dst, unsigned 
   if (slabs == 0) return hipSuccess;
   if (b == nullptr) launch_probe_shape<1>(a, b, dst, slabs, shape, s);
   else launch_probe_shape<2>(a, b, dst, slabs, shape, s);
+  return hipGetLastError();
+}
+
+hipError_t stream_probe_mix(const void* const* src, int n_src, void* const* dst, int n_dst, unsigned long long bytes,
+                            bool compute, hipStream_t s) {
+  const unsigned long long slabs = bytes / 4096;
+  if (slabs == 0) return hipSuccess;
+  ProbeMixPtrs p{};
+  for (int i = 0; i < n_src; ++i) p.in[i] = static_cast<const uint4*>(src[i]);
+  for (int i = 0; i < n_dst; ++i) p.out[i] = static_cast<uint4*>(dst[i]);
+  const dim3 grid((unsigned)((slabs + kWaves - 1) / kWaves)), wg(64 * kWaves);
+  if (n_src == 4 && n_dst == 3) {
+    if (compute) hipLaunchKernelGGL((stream_probe_mix_kernel<4, 3, 160>), grid, wg, 0, s, p, slabs);
+    else hipLaunchKernelGGL((stream_probe_mix_kernel<4, 3, 0>), grid, wg, 0, s, p, slabs);
+  } else if (n_src == 3 && n_dst == 1) {
+    if (compute) hipLaunchKernelGGL((stream_probe_mix_kernel<3, 1, 80>), grid, wg, 0, s, p, slabs);
+    else hipLaunchKernelGGL((stream_probe_mix_kernel<3, 1, 0>), grid, wg, 0, s, p, slabs);
+  } else {
+    return hipErrorInvalidValue;  // the caller has checked
+  }
   return hipGetLastError();
 }
 

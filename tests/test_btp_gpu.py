@@ -335,6 +335,28 @@ def test_measurement_aids_move_the_bytes_they_are_timed_for(slabs):
     diff = (out[:n] ^ (a ^ b)).view(torch.int32)
     assert bool(((diff & ~1) == 0).all()) and bool((out[n:] == 0xA5).all())
     assert lib.spear_btp_stream_probe_shape(a.data_ptr(), None, out.data_ptr(), ctypes.c_ulonglong(n), 8, sp) == -1
+    # the probe with several inputs and outputs: every output is the combination of all inputs, nothing beyond
+    ins = [a, b, a.flip(0).contiguous(), b.flip(0).contiguous()]
+    outs = [torch.full((n + guard,), 0xA5, dtype=torch.uint8, device=DEV) for _ in range(3)]
+    for n_src, n_dst in ((3, 1), (4, 3)):
+        want = ins[0]
+        for t in ins[1:n_src]:
+            want = want ^ t
+        for compute in (0, 1):
+            for o in outs:
+                o.fill_(0xA5)
+            src = (ctypes.c_void_p * n_src)(*[t.data_ptr() for t in ins[:n_src]])
+            dst = (ctypes.c_void_p * n_dst)(*[t.data_ptr() for t in outs[:n_dst]])
+            assert lib.spear_btp_stream_probe_mix(src, n_src, dst, n_dst, ctypes.c_ulonglong(n), compute, sp) == 0
+            torch.cuda.synchronize()
+            for o in outs[:n_dst]:
+                diff = (o[:n] ^ want).view(torch.int32)
+                assert bool(((diff & ~compute) == 0).all()) and bool((o[n:] == 0xA5).all()), (n_src, n_dst, compute)
+            for o in outs[n_dst:]:
+                assert bool((o == 0xA5).all())
+    src2 = (ctypes.c_void_p * 2)(a.data_ptr(), b.data_ptr())
+    dst1 = (ctypes.c_void_p * 1)(outs[0].data_ptr())
+    assert lib.spear_btp_stream_probe_mix(src2, 2, dst1, 1, ctypes.c_ulonglong(n), 0, sp) == -1
     out.fill_(0xA5)
     assert lib.spear_btp_copy(a.data_ptr(), out.data_ptr(), ctypes.c_ulonglong(n), sp) == 0
     torch.cuda.synchronize()

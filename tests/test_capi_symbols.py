@@ -26,6 +26,7 @@ def test_header_declares_the_expected_entry_points():
         "spear_btp_forward_loggate",
         "spear_btp_last_error",
         "spear_btp_stream_probe",
+        "spear_btp_stream_probe_mix",
         "spear_btp_stream_probe_shape",
         "spear_jagged_prefill",
         "spear_jagged_step",
