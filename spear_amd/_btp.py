@@ -31,7 +31,7 @@ FLAG_MIX_QKV_GATE = 0x1
 FLAG_MIX_F32_RESULTS = 0x2
 FLAG_MIX_TILE_SPLIT = 0x4
 FLAG_DX_F32 = 0x10
-_ABI_VERSION = 14
+_ABI_VERSION = 15
 _SUPPORTED_WPB = (4, 8, 16, 32)
 
 _lock = threading.Lock()

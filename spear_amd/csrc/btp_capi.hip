@@ -45,7 +45,7 @@ int check_common(const char* who, int B, int H, int L, int k, int in_dtype, int 
 
 extern "C" {
 
-int spear_btp_abi_version(void) { return 14; }
+int spear_btp_abi_version(void) { return 15; }
 
 const char* spear_btp_last_error(void) { return g_error; }
 
