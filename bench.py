@@ -33,7 +33,7 @@ FWD_BYTES, BWD_BYTES = 66, 102  # per (token, head), bf16 y / dy
 # WRITE_SIZE and scaled by what the same counters read for the copy kernel (x1.9997 / x1.0000);
 # figures and commands are in profiles/btp_kernels_c3_B1024_H32_L128.txt (and the c4 / c5 files beside it). Counters cannot be read
 # from inside this script, so the value is recorded here; it is null for shapes never profiled.
-MEASURED_BWD_TRAFFIC_BYTES = {"c3": 429.2e6, "c4": 879.0e6, "c5": 1743.9e6}
+MEASURED_BWD_TRAFFIC_BYTES = {"c3": 429.0e6, "c4": 873.6e6, "c5": 1736.3e6}
 
 CONFIGS = {
     # name: (B, H, L, seed, x_std, gate)
