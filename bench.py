@@ -226,7 +226,12 @@ def main() -> int:
                                    B, H, L, 2, 0, 0, 2, sp)
         assert rc == 0, lib.spear_btp_last_error()
 
-    fwd_mfma_ms = kernel_ms(fwd_mfma)
+    def bwd_mfma(s):  # the backward on the matrix cores (three 16x16x32 products per block)
+        rc = lib.spear_btp_backward(s["coeff"].data_ptr(), s["x"].data_ptr(), s["dy"].data_ptr(), None,
+                                    s["dx"].data_ptr(), s["dA"].data_ptr(), B, H, L, 2, 0, 0, 2, sp)
+        assert rc == 0, lib.spear_btp_last_error()
+
+    fwd_mfma_ms, bwd_mfma_ms = kernel_ms(fwd_mfma), kernel_ms(bwd_mfma)
 
     # copy kernel of the same footprint as a practical ceiling (reads n, writes n)
     nbytes = sets[0]["x"].numel() * 2
@@ -767,6 +772,9 @@ def main() -> int:
         "forward_kernel_mfma_path": {"avg_launch_ms": fwd_mfma_ms,
                                      "achieved": units * FWD_BYTES / (fwd_mfma_ms * 1e-3) / 1e9,
                                      "frac": units * FWD_BYTES / (fwd_mfma_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS},
+        "backward_kernel_mfma_path": {"avg_launch_ms": bwd_mfma_ms,
+                                      "achieved": units * BWD_BYTES / (bwd_mfma_ms * 1e-3) / 1e9,
+                                      "frac": units * BWD_BYTES / (bwd_mfma_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS},
         "log_gate_entry_points": {"forward_ms": fwd_log_ms, "backward_ms": bwd_log_ms,
                                   "achieved": units * (68 + 108) / ((fwd_log_ms + bwd_log_ms) * 1e-3) / 1e9,
                                   "algorithmic_bytes_per_unit": {"forward": 68, "backward": 108}},

@@ -47,8 +47,10 @@ extern "C" {
 
 /* flags */
 #define SPEAR_BTP_WRITE_CHECKPOINT 0x1u /* forward: also store the carry checkpoint            */
-#define SPEAR_BTP_PATH_MFMA 0x2u        /* forward: use the MFMA tile kernel (decay matrix rounded */
-                                        /* to the input dtype) instead of the exact-fp32 recurrence */
+#define SPEAR_BTP_PATH_MFMA 0x2u        /* forward and backward: use the MFMA tile kernels (decay matrices rounded */
+                                        /* to the input dtype and multiplied on the matrix cores, the reference's   */
+                                        /* formulation) instead of the exact-fp32 recurrences; the backward then    */
+                                        /* takes dy in the inputs' dtype and has no SPEAR_BTP_DX_F32                */
 
 #define SPEAR_BTP_DX_F32 0x10u          /* backward: check mode, `dx` is fp32 [B, H, 16, L] and receives the    */
                                         /* kernel's fp32 values instead of their rounding to in_dtype           */

@@ -83,11 +83,15 @@ int spear_btp_backward(const void* coeff, const void* x, const void* dy, const f
   if (!coeff || !x || !dy || !dx || !dA) return fail(SPEAR_BTP_ENULL, "spear_btp_backward: NULL tensor pointer");
   if (!aligned16(coeff) || !aligned16(x) || !aligned16(dy) || !aligned16(dx) || !aligned16(dA))
     return fail(SPEAR_BTP_EINVAL, "spear_btp_backward: tensor pointers must be 16-byte aligned");
-  if (flags & SPEAR_BTP_PATH_MFMA)
-    return fail(SPEAR_BTP_EINVAL, "spear_btp_backward: there is no MFMA variant of the backward kernel");
+  const bool mfma = (flags & SPEAR_BTP_PATH_MFMA) != 0;
+  if (mfma && dy_dtype != in_dtype)
+    return fail(SPEAR_BTP_EINVAL, "spear_btp_backward: the MFMA path takes dy in the inputs' dtype");
+  if (mfma && (flags & SPEAR_BTP_DX_F32))
+    return fail(SPEAR_BTP_EINVAL, "spear_btp_backward: the MFMA path has no fp32 dx (SPEAR_BTP_DX_F32)");
 
   spear_btp::BwdArgs a{coeff, x, dy, dx, dA, B, H, L, k, in_dtype, dy_dtype, false, (flags & SPEAR_BTP_DX_F32) != 0};
-  const hipError_t err = spear_btp::scan_backward(a, static_cast<hipStream_t>(stream));
+  const hipStream_t hs = static_cast<hipStream_t>(stream);
+  const hipError_t err = mfma ? spear_btp::mfma_backward(a, hs) : spear_btp::scan_backward(a, hs);
   if (err != hipSuccess) return fail(SPEAR_BTP_ELAUNCH, "spear_btp_backward: launch failed: %s", hipGetErrorString(err));
   return 0;
 }

@@ -36,8 +36,10 @@ struct BwdArgs {
 hipError_t scan_forward(const FwdArgs& p, hipStream_t s);
 hipError_t scan_backward(const BwdArgs& p, hipStream_t s);
 
-// MFMA tile kernel (btp_mfma.hip), forward only, bf16 or fp16 inputs; it stores no checkpoint.
+// MFMA tile kernels (btp_mfma.hip), bf16 or fp16 inputs; the forward stores no checkpoint, the backward takes
+// dy in the inputs' type and has neither log-space gates nor the fp32-dx check mode.
 hipError_t mfma_forward(const FwdArgs& p, hipStream_t s);
+hipError_t mfma_backward(const BwdArgs& p, hipStream_t s);
 
 // Fused layer-layout forward (btp_fused.hip): all operands [B, L, features], 16-bit.
 struct MixArgs {

@@ -192,6 +192,244 @@ __global__ __launch_bounds__(64 * kWaves) void btp_fwd_mfma_kernel(const uint16_
   }
 }
 
+// ==========================================================================================
+// Backward on the matrix cores. Where the reference multiplies dC by the transposed decay matrix
+// (csrc/btp/btp-backwards.cu:519-608, "dX^T = A^T dC^T") and assembles dA from shuffled partial sums
+// (:372-413, :637-796), this kernel runs three 16x16x32 products per block i, all with K = 32:
+//     V_i   = [ 0     | L_i ] * [ X_{i-1} ; X_i  ]      local forward states (zero-started)
+//     dX_i  = [ L_i^T | D_i ] * [ dY_i ; dY_{i+1} ]     the gradient of x: own block and the one-hop carry
+//     dXl_i = [ L_i^T | 0   ] * [ dY_i ; dY_{i+1} ]     its block-local part
+//     L_i^T[s][t] = prod_{j=s+1..t} a_j (t >= s),   D_i[s][t'] = (prod_{j=s+1..15} a_j) (prod_{j=0..t'} a^{next}_j)
+// and then, with c = V_{i-1}[15] (the carry into the block) and P_{r-1} = prod_{j<r} a_j,
+//     dA_r = sum over channels of  dX_i[r] V_i[r-1]  +  P_{r-1} dXl_i[r] c          (V_i[-1] = 0, P_{-1} = 1)
+// which counts every (source step, sink step) pair whose decay product contains a_r exactly once and leaves
+// out the two-hop pairs (block i-1 to block i+1) that the operator does not have. The decay operands are
+// rounded to 16 bits for the matrix instruction, as in the reference; the default backward (btp_scan.hip)
+// keeps everything in fp32.
+// A lane's 8 entries of a transposed row run left to right, entry(s, t+1) = entry(s, t) a_{t+1}, started from
+// suffix products that come from a 3-step DPP scan inside 8-lane halves plus v_readlane broadcasts.
+// ==========================================================================================
+// v from lane (n + Shift) of the same 16-lane row; lanes without a source get `fill`.
+template <int Shift>
+__device__ __forceinline__ float row_shift_left(float v, float fill) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(fill), __float_as_int(v), 0x100 + Shift, 0xF, 0xF,
+                                                    false));
+}
+
+// W[n] = prod of a over the lanes of n's 8-lane half from n (included) to the end of the half.
+__device__ __forceinline__ float half_row_suffix_product(float a_n, int n) {
+  const int n8 = n & 7;
+  float w = a_n;
+  float t = row_shift_left<1>(w, 1.0f);
+  w = (n8 <= 6) ? w * t : w;
+  t = row_shift_left<2>(w, 1.0f);
+  w = (n8 <= 5) ? w * t : w;
+  t = row_shift_left<4>(w, 1.0f);
+  w = (n8 <= 3) ? w * t : w;
+  return w;
+}
+
+template <class E, bool kStreamIn>
+__global__ __launch_bounds__(64 * kWaves) void btp_bwd_mfma_kernel(const uint16_t* __restrict__ coeff,
+                                                                   const uint16_t* __restrict__ x,
+                                                                   const uint16_t* __restrict__ dy,
+                                                                   uint16_t* __restrict__ dx, float* __restrict__ dA,
+                                                                   int L, int spans_per_row, long total_spans, int k) {
+  constexpr bool kStreamOut = SPEAR_BTP_STREAM_STORES == 1;
+  // per wavefront: x image, which dx overwrites block by block (a block's x is read by that block's V product
+  // only, before its dx is written) | dy image | x of the block before the span | dy of the block after it
+  // (16 rows x 32 B each; the span's dA takes the first one's place once the carry into the span is known) |
+  // coefficients (16 before + 128 + 16 after) | prefix products of a block. 9920 bytes: four workgroups per CU.
+  constexpr int kCoeffs = kTile + kSpan + kTile;
+  constexpr int kWaveBytes = 2 * 4096 + 2 * 512 + kCoeffs * 4 + kTile * 4;
+  __shared__ __align__(16) unsigned char lds[kWaves][kWaveBytes];
+
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+  const long span = first_span_of_workgroup() + wave;
+  if (span >= total_spans) return;
+  const SpanCoord sc = span_coord(span, spans_per_row, L);
+
+  unsigned char* img_x = lds[wave];
+  unsigned char* img_g = img_x + 4096;
+  unsigned char* img_dx = img_x;
+  unsigned char* halo_x = img_g + 4096;
+  unsigned char* halo_g = halo_x + 512;
+  float* a_ext = reinterpret_cast<float*>(halo_g + 512);  // a_ext[16 + t] = a at span step t
+  float* dA_lds = reinterpret_cast<float*>(halo_x);  // 128 floats; halo_x is read before the block loop only
+  float* pfx = a_ext + kCoeffs;
+
+  const long slab_off = (sc.row * kChan) * (long)L + sc.s0;
+  const uint16_t* xslab = x + slab_off;
+  const uint16_t* gslab = dy + slab_off;
+  const uint16_t* arow = coeff + sc.row * (long)L + sc.s0;
+  const int q = lane >> 4, n = lane & 15;
+
+  // ---- global -> LDS
+  uint4 xin[4], gin[4];
+  slab16_global_to_regs<kStreamIn>(xslab, L, sc.nvalid, lane, xin);
+  slab16_global_to_regs<kStreamIn>(gslab, L, sc.nvalid, lane, gin);
+  const uint32_t ain = coeff_global_to_reg<LinCoeff<E>>(arow, sc.nvalid, lane);
+  const bool left = (k == 2) && (sc.sp > 0);            // wave-uniform: a block before the span feeds its first block
+  const bool right = (k == 2) && (sc.s0 + kSpan < L);   // wave-uniform: the span's last block feeds a block after it
+  uint4 hx = zero4(), hg = zero4();
+  uint32_t ha = 0u, hb = 0u;
+  if (left) {
+    if (lane < 32) hx = *reinterpret_cast<const uint4*>(xslab + (long)(lane >> 1) * L - kTile + ((lane & 1) << 3));
+    if (lane < 8) ha = *reinterpret_cast<const uint32_t*>(arow - kTile + (lane << 1));
+  }
+  if (right) {
+    if (lane < 32) hg = *reinterpret_cast<const uint4*>(gslab + (long)(lane >> 1) * L + kSpan + ((lane & 1) << 3));
+    if (lane < 8) hb = *reinterpret_cast<const uint32_t*>(arow + kSpan + (lane << 1));
+  }
+  slab16_regs_to_lds(img_x, lane, xin);
+  slab16_regs_to_lds(img_g, lane, gin);
+  if (lane < 32) {
+    *reinterpret_cast<uint4*>(halo_x + (lane >> 1) * 32 + ((lane & 1) << 4)) = hx;
+    *reinterpret_cast<uint4*>(halo_g + (lane >> 1) * 32 + ((lane & 1) << 4)) = hg;
+  }
+  {
+    float2 f;
+    f.x = clamp_coeff<E>(E::lo(ain));
+    f.y = clamp_coeff<E>(E::hi(ain));
+    *reinterpret_cast<float2*>(a_ext + kTile + (lane << 1)) = f;
+    if (lane < 8) {
+      f.x = clamp_coeff<E>(E::lo(ha));
+      f.y = clamp_coeff<E>(E::hi(ha));
+      *reinterpret_cast<float2*>(a_ext + (lane << 1)) = f;
+      f.x = clamp_coeff<E>(E::lo(hb));
+      f.y = clamp_coeff<E>(E::hi(hb));
+      *reinterpret_cast<float2*>(a_ext + kTile + kSpan + (lane << 1)) = f;
+    }
+  }
+  wave_lds_handover();
+
+  const floatx4_t zero_acc = {0.0f, 0.0f, 0.0f, 0.0f};
+  // V of one block: rows 4q..4q+3 of channel n. `blk` = -1 is the block before the span.
+  auto local_states = [&](int blk, float w_pre) -> floatx4_t {
+    // A = [0 | L]: the forward kernel's operand without its carry half
+    float val = (q == 2) ? ((n >= 8) ? w_pre : 1.0f) : 1.0f;
+    const float4 a_lo = *reinterpret_cast<const float4*>(a_ext + kTile * blk + 8 * q);
+    const float4 a_hi = *reinterpret_cast<const float4*>(a_ext + kTile * blk + 8 * q + 4);
+    const float av[8] = {a_lo.x, a_lo.y, a_lo.z, a_lo.w, a_hi.x, a_hi.y, a_hi.z, a_hi.w};
+    float e[8];
+#pragma unroll
+    for (int jj = 7; jj >= 0; --jj) {
+      const bool above = (8 * q - 16 + jj) > n;
+      e[jj] = (above || q < 2) ? 0.0f : val;
+      val *= above ? 1.0f : av[jj];
+    }
+    uint4 braw = zero4();
+    if (q >= 2) {
+      braw = (blk < 0) ? *reinterpret_cast<const uint4*>(halo_x + n * 32 + ((q - 2) << 4))
+                       : *reinterpret_cast<const uint4*>(img_x + swz<256>(n, 2 * blk + q - 2));
+    }
+    return mfma_16x16x32<E>(pack8<E>(e), braw, zero_acc);
+  };
+
+  // carry into the span's first block: terminal local state of the block before it, channel n
+  float cin = 0.0f;
+  if (left) {
+    const float w = half_row_prefix_product(a_ext[n], n);
+    const floatx4_t v = local_states(-1, w);
+    cin = __int_as_float(__builtin_amdgcn_ds_bpermute((48 + n) << 2, __float_as_int(v[3])));
+  }
+
+  // scans of the first block; every iteration prepares those of the block after it
+  float w_pre = half_row_prefix_product(a_ext[kTile + n], n);
+  float w_suf = half_row_suffix_product(a_ext[kTile + n], n);
+
+#pragma unroll
+  for (int i = 0; i < kSpan / kTile; ++i) {
+    const float a_next_n = a_ext[kTile + kTile * (i + 1) + n];
+    const float w_pre_next = half_row_prefix_product(a_next_n, n);
+    const float w_suf_next = half_row_suffix_product(a_next_n, n);
+    const bool has_next = (k == 2) && (i + 1 < kSpan / kTile || right);  // wave-uniform
+
+    // prefix products of this block: p = prod_{j=0..n} a_j, parked for the dA factors P_{r-1}
+    const float s7 = lane_broadcast(w_pre, 7);
+    const float p = (n >= 8) ? w_pre * s7 : w_pre;
+    if (q == 0) pfx[n] = p;
+
+    // ---- V_i
+    const floatx4_t vloc = local_states(i, w_pre);
+
+    // ---- the transposed operand: row s = n, columns kk = 8q .. 8q+7 over [block i | block i+1]
+    const float t8 = lane_broadcast(w_suf, 8);            // prod of the block's second half
+    const float t0_next = lane_broadcast(w_suf_next, 0);  // prod of the next block's first half
+    float excl = row_shift_left<1>(w_suf, 1.0f);          // prod_{j=n+1..end of n's half}
+    excl = ((n & 7) == 7) ? 1.0f : excl;
+    const float s_full = (n < 8) ? excl * t8 : excl;      // prod_{j=n+1..15}
+    float val;
+    if (q == 0) val = 0.0f;
+    else if (q == 1) val = (n < 8) ? excl : 0.0f;
+    else if (q == 2) val = s_full;
+    else val = s_full * t0_next;
+    const float4 c_lo = *reinterpret_cast<const float4*>(a_ext + kTile + kTile * i + 8 * q);
+    const float4 c_hi = *reinterpret_cast<const float4*>(a_ext + kTile + kTile * i + 8 * q + 4);
+    const float cv[8] = {c_lo.x, c_lo.y, c_lo.z, c_lo.w, c_hi.x, c_hi.y, c_hi.z, c_hi.w};
+    float e2[8];
+#pragma unroll
+    for (int jj = 0; jj < 8; ++jj) {
+      const int kk = 8 * q + jj;
+      if (kk < n) {
+        e2[jj] = 0.0f;
+      } else if (kk == n) {
+        val = 1.0f;
+        e2[jj] = 1.0f;
+      } else {
+        val *= cv[jj];
+        e2[jj] = val;
+      }
+      if (q >= 2 && !has_next) e2[jj] = 0.0f;
+    }
+    // B: dy[channel n][steps 16 i + 8 q .. + 7], the last two chunks of the span's last block from the halo
+    const int cidx = 2 * i + q;
+    const uint4 graw = (cidx < 16) ? *reinterpret_cast<const uint4*>(img_g + swz<256>(n, cidx))
+                                   : *reinterpret_cast<const uint4*>(halo_g + n * 32 + ((cidx - 16) << 4));
+    const uint4 a2 = pack8<E>(e2);
+    const floatx4_t dxf = mfma_16x16x32<E>(a2, graw, zero_acc);
+    // the block-local part: the same operand against dy with the next block's half blanked
+    const floatx4_t dxl = mfma_16x16x32<E>(a2, (q < 2) ? graw : zero4(), zero_acc);
+
+    // ---- dx[channel n][16 i + 4 q .. + 3]
+    {
+      uint2 o;
+      o.x = E::pack2(dxf[0], dxf[1]);
+      o.y = E::pack2(dxf[2], dxf[3]);
+      *reinterpret_cast<uint2*>(img_dx + swz<256>(n, 2 * i + (q >> 1)) + ((q & 1) << 3)) = o;
+    }
+
+    // ---- dA of rows r = 4 q + j: sum over the 16 channels (lanes of a row) of dX V[r-1] + P_{r-1} dXl c
+    wave_lds_handover();
+    const float v_up = lane_rotate(vloc[3], lane, -16);  // V[4q - 1] from the lane group above
+    const float vprev[4] = {q > 0 ? v_up : 0.0f, vloc[0], vloc[1], vloc[2]};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int r = 4 * q + j;
+      const float pm1 = (r == 0) ? 1.0f : pfx[r > 0 ? r - 1 : 0];
+      float sum = fmaf(dxf[j], vprev[j], pm1 * dxl[j] * cin);
+      sum += row_xor<1>(sum);
+      sum += row_xor<2>(sum);
+      sum += row_xor<4>(sum);
+      sum += row_xor<8>(sum);
+      if (n == j) dA_lds[kTile * i + r] = sum;
+    }
+    wave_lds_handover();  // pfx is rewritten by the next block
+
+    cin = (k == 2) ? __int_as_float(__builtin_amdgcn_ds_bpermute((48 + n) << 2, __float_as_int(vloc[3]))) : 0.0f;
+    w_pre = w_pre_next;
+    w_suf = w_suf_next;
+  }
+
+  wave_lds_handover();
+  slab16_lds_to_global<kStreamOut>(img_dx, dx + slab_off, L, sc.nvalid, lane);
+  if (lane < 32 && (lane << 2) < sc.nvalid) {
+    const float4 g4 = *reinterpret_cast<const float4*>(dA_lds + (lane << 2));
+    stream_store16(dA + sc.row * (long)L + sc.s0 + (lane << 2),
+                   make_uint4(__float_as_uint(g4.x), __float_as_uint(g4.y), __float_as_uint(g4.z), __float_as_uint(g4.w)));
+  }
+}
+
 template <class E, class OutT, bool kStreamIn>
 void launch_fwd_mfma(const FwdArgs& p, const Grid& g, hipStream_t s) {
   hipLaunchKernelGGL((btp_fwd_mfma_kernel<E, OutT, kStreamIn>), dim3(g.blocks), dim3(64 * kWaves), 0, s,
@@ -200,6 +438,27 @@ void launch_fwd_mfma(const FwdArgs& p, const Grid& g, hipStream_t s) {
 }
 
 }  // namespace
+
+hipError_t mfma_backward(const BwdArgs& p, hipStream_t s) {
+  if (p.dy_dtype != p.in_dtype || p.log_gate || p.dx_f32) return hipErrorInvalidValue;  // the caller has checked
+  const Grid g = make_grid((long)p.B * p.H, p.L);
+  auto launch = [&](auto e, auto stream_in) {
+    using E = decltype(e);
+    hipLaunchKernelGGL((btp_bwd_mfma_kernel<E, decltype(stream_in)::value>), dim3(g.blocks), dim3(64 * kWaves), 0, s,
+                       static_cast<const uint16_t*>(p.coeff), static_cast<const uint16_t*>(p.x),
+                       static_cast<const uint16_t*>(p.dy), static_cast<uint16_t*>(p.dx), p.dA, p.L, g.spans_per_row,
+                       g.total_spans, p.k);
+  };
+  const bool st = stream_inputs(g);
+  if (p.in_dtype == kBf16) {
+    if (st) launch(Bf16{}, std::true_type{});
+    else launch(Bf16{}, std::false_type{});
+  } else {
+    if (st) launch(Fp16{}, std::true_type{});
+    else launch(Fp16{}, std::false_type{});
+  }
+  return hipGetLastError();
+}
 
 hipError_t mfma_forward(const FwdArgs& p, hipStream_t s) {
   const Grid g = make_grid((long)p.B * p.H, p.L);

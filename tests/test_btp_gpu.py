@@ -29,7 +29,7 @@ def run_forward(coeff, x, k=2, out_dtype=torch.bfloat16, checkpoint=False, mfma=
     return (y.cpu(), ck.cpu()) if checkpoint else y.cpu()
 
 
-def run_backward(coeff, x, dy, k=2):
+def run_backward(coeff, x, dy, k=2, mfma=False):
     from spear_amd import _btp
 
     c, xx, g = coeff.to(DEV), x.to(DEV), dy.to(DEV)
@@ -37,7 +37,7 @@ def run_backward(coeff, x, dy, k=2):
     dx = torch.full((B, H, 16, L), float("nan"), device=DEV, dtype=x.dtype)
     dA = torch.full((B, H, L), float("nan"), device=DEV, dtype=torch.float32)
     ck = torch.empty((B, H, L // 16, 16), device=DEV, dtype=torch.float32)
-    _btp.backward(c, xx, g, ck, dx, dA, k, 32)
+    _btp.backward(c, xx, g, ck, dx, dA, k, 32, flags=_btp.FLAG_PATH_MFMA if mfma else 0)
     torch.cuda.synchronize()
     return dx.cpu(), dA.cpu()
 
@@ -104,8 +104,58 @@ def test_mfma_path_rejects_what_it_does_not_do():
     ck = torch.empty(1, 2, 2, 16, device=DEV)
     with pytest.raises(RuntimeError, match="does not store the carry checkpoint"):
         _btp.forward(c, xx, y, ck, 2, 32, flags=_btp.FLAG_PATH_MFMA | _btp.FLAG_WRITE_CHECKPOINT)
-    with pytest.raises(RuntimeError, match="no MFMA variant"):
-        _btp.backward(c, xx, dy.to(DEV), ck, torch.empty_like(xx), torch.empty(1, 2, 32, device=DEV), 2, 32, flags=_btp.FLAG_PATH_MFMA)
+    dA = torch.empty(1, 2, 32, device=DEV)
+    with pytest.raises(RuntimeError, match="takes dy in the inputs' dtype"):
+        _btp.backward(c, xx, dy.float().to(DEV), ck, torch.empty_like(xx), dA, 2, 32, flags=_btp.FLAG_PATH_MFMA)
+    with pytest.raises(RuntimeError, match="no fp32 dx"):
+        _btp.backward(c, xx, dy.to(DEV), ck, torch.empty_like(xx, dtype=torch.float32), dA, 2, 32,
+                      flags=_btp.FLAG_PATH_MFMA | _btp.FLAG_DX_F32)
+
+
+# The matrix-core backward rounds its decay operands to 16 bits (as the reference's kernel does), so dA is not held
+# to the fp32 bound of the default kernel. dA_r is a sum over channels and (source, sink) pairs of products
+# decay * x * dy in which two rounded decay entries meet, so its error is at most about 2 * 2^-9 of the sum of the
+# terms' magnitudes -- which the oracle gives exactly when it is run on |x| and |dy| (the decays are not negative).
+def assert_dA_from_rounded_decays(dA, coeff, x, dy, k, what, eps=2.0 ** -8):
+    rdA = orc.backward(f64(coeff), f64(x), f64(dy), k=k)[1]
+    magnitude = orc.backward(f64(coeff), np.abs(f64(x)), np.abs(f64(dy)), k=k)[1]
+    err = np.abs(f64(dA) - rdA)
+    bound = 1e-3 + eps * magnitude
+    worst = np.argmax(err - bound)
+    assert (err <= bound).all(), f"{what}: max |err|={err.max():.3e}; worst at {worst}: err {err.flat[worst]:.3e} bound {bound.flat[worst]:.3e}"
+    # and the bound is not vacuous: it stays a small fraction of the gradient's own scale
+    assert np.median(bound) < 0.05 * max(np.abs(rdA).max(), 1.0), what
+
+
+@pytest.mark.parametrize("k", [2, 1])
+@pytest.mark.parametrize("B,H,L", SHAPES)
+def test_backward_mfma_path_matches_oracle(B, H, L, k):
+    coeff, x, dy = make_inputs(B, H, L, seed=350 + L + k)
+    print(f"bwd mfma B={B} H={H} L={L} k={k}", flush=True)
+    dx, dA = run_backward(coeff, x, dy, k=k, mfma=True)
+    rdx, rdA = orc.backward(f64(coeff), f64(x), f64(dy), k=k)
+    assert_close(f64(dx), rdx, BF16_ATOL, BF16_RTOL, "dx mfma")
+    assert_dA_from_rounded_decays(dA, coeff, x, dy, k, "dA mfma")
+
+
+def test_backward_mfma_path_fp16_stress_and_zero_coefficients():
+    coeff, x, dy = make_inputs(2, 3, 272, seed=351, dtype=torch.float16)
+    dx, dA = run_backward(coeff, x, dy, mfma=True)
+    rdx, rdA = orc.backward(f64(coeff), f64(x), f64(dy))
+    assert_close(f64(dx), rdx, 4e-3, 4e-3, "dx mfma fp16")
+    assert_dA_from_rounded_decays(dA, coeff, x, dy, 2, "dA mfma fp16", eps=2.0 ** -11)
+    coeff, x, dy = make_inputs(2, 8, 2048, seed=1236, gate="mixed")
+    dx, dA = run_backward(coeff, x, dy, mfma=True)
+    rdx, rdA = orc.backward(f64(coeff), f64(x), f64(dy))
+    assert_close(f64(dx), rdx, BF16_ATOL, BF16_RTOL, "dx mixed gates")
+    assert_dA_from_rounded_decays(dA, coeff, x, dy, 2, "dA mixed gates")
+    coeff, x, dy = make_inputs(1, 2, 160, seed=7)
+    coeff[0, 0, [0, 5, 16, 33, 127, 128]] = 0.0
+    dx, dA = run_backward(coeff, x, dy, mfma=True)
+    rdx, rdA = orc.backward(f64(coeff), f64(x), f64(dy))
+    assert torch.isfinite(dx.float()).all() and torch.isfinite(dA).all()
+    assert_close(f64(dx), rdx, BF16_ATOL, BF16_RTOL, "dx zero coefficients")
+    assert_dA_from_rounded_decays(dA, coeff, x, dy, 2, "dA zero coefficients")
 
 
 @pytest.mark.parametrize("k", [2, 1])
@@ -233,6 +283,9 @@ def test_kernels_match_committed_closed_form_vectors(case, k):
     assert_close(f64(dx), v[f"k{k}.dx"], BF16_ATOL, BF16_RTOL, "dx")
     assert_close(f64(dA), v[f"k{k}.dA"], BF16_ATOL, BF16_RTOL, "dA")
     assert_close(f64(run_forward(coeff, x, k=k, mfma=True)), v[f"k{k}.y"], BF16_ATOL, BF16_RTOL, "y mfma")
+    dx, dA = run_backward(coeff, x, dy, k=k, mfma=True)
+    assert_close(f64(dx), v[f"k{k}.dx"], BF16_ATOL, BF16_RTOL, "dx mfma")
+    assert_close(f64(dA), v[f"k{k}.dA"], 4 * BF16_ATOL, BF16_RTOL, "dA mfma")
 
 
 # ---- seeded sweep over odd launch shapes ---------------------------------------------------------
@@ -270,6 +323,10 @@ def test_forward_and_backward_on_odd_launch_shapes(B, H, L, k, f32, seed):
     rdx, rdA = orc.backward(f64(coeff), f64(x), f64(dy), k=k)
     assert_close(f64(dx), rdx, BF16_ATOL, BF16_RTOL, "dx")
     assert_close(f64(dA), rdA, F32_ATOL, F32_RTOL, "dA")
+    if not f32:  # the matrix-core backward on the same launch geometries (it takes dy in the inputs' type)
+        dxm, dAm = run_backward(coeff, x, dy, k=k, mfma=True)
+        assert_close(f64(dxm), rdx, BF16_ATOL, BF16_RTOL, "dx mfma")
+        assert_dA_from_rounded_decays(dAm, coeff, x, dy, k, "dA mfma")
 
 
 def test_kernels_match_the_reference_float64_path_vectors():

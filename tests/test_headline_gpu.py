@@ -22,14 +22,14 @@ def _fwd(c, x, k=2, out_dtype=torch.bfloat16):
     return y
 
 
-def _bwd(c, x, g, k=2):
+def _bwd(c, x, g, k=2, mfma=False):
     from spear_amd import _btp
 
     B, H, _, L = x.shape
     dx = torch.empty_like(x)
     dA = torch.empty(B, H, L, device=DEV, dtype=torch.float32)
     ck = torch.empty(B, H, L // 16, 16, device=DEV, dtype=torch.float32)
-    _btp.backward(c, x, g, ck, dx, dA, k, 32)
+    _btp.backward(c, x, g, ck, dx, dA, k, 32, flags=_btp.FLAG_PATH_MFMA if mfma else 0)
     return dx, dA
 
 
@@ -52,8 +52,10 @@ def test_full_size_properties(name):
     y32 = _fwd(c, xx, out_dtype=torch.float32)
     y16 = _fwd(c, xx)
     dx, dA = _bwd(c, xx, g)
+    dxm, dAm = _bwd(c, xx, g, mfma=True)  # the matrix-core backward at full size
     torch.cuda.synchronize()
     assert torch.isfinite(y32).all() and torch.isfinite(dx.float()).all() and torch.isfinite(dA).all()
+    assert torch.isfinite(dxm.float()).all() and torch.isfinite(dAm).all()
 
     # bf16 output is the rounding of the fp32 output
     assert torch.equal(y16, y32.to(torch.bfloat16))
@@ -97,6 +99,11 @@ def test_full_size_properties(name):
         rdx, rdA = orc.backward(a_, x_, g_)
         assert_close(f64(dx[b : b + 1, h : h + 1]), rdx, BF16_ATOL, BF16_RTOL, f"dx[{b},{h}]")
         assert_close(f64(dA[b : b + 1, h : h + 1]), rdA, F32_ATOL, F32_RTOL, f"dA[{b},{h}]")
+        # decay operands rounded to 16 bits: 2 * 2^-9 of the sum of the terms' magnitudes (the oracle on |x|, |dy|)
+        assert_close(f64(dxm[b : b + 1, h : h + 1]), rdx, BF16_ATOL, BF16_RTOL, f"dx mfma[{b},{h}]")
+        magnitude = orc.backward(a_, np.abs(x_), np.abs(g_))[1]
+        err = np.abs(f64(dAm[b : b + 1, h : h + 1]) - rdA)
+        assert (err <= 1e-3 + 2.0 ** -8 * magnitude).all(), f"dA mfma[{b},{h}]: {err.max():.3e}"
 
 
 def _free_gib():

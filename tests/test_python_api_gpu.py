@@ -40,6 +40,40 @@ def test_autograd_through_btp_matches_oracle():
     assert_close(f64(c.grad), rdA, BF16_ATOL, BF16_RTOL, "dA (rounded to the bf16 leaf dtype by autograd)")
 
 
+def test_the_op_runs_on_the_matrix_core_kernels_on_request(monkeypatch):
+    """SPEAR_BTP_PATH=mfma (read when the module is imported; set on the module here) sends btp() through the
+    matrix-core forward and, for dy in the inputs' dtype, the matrix-core backward."""
+    from spear_amd import _btp, btp
+    from spear_amd.ops.btp import interface
+
+    monkeypatch.setattr(interface, "_PATH_MFMA", True)
+    monkeypatch.setattr(interface, "_FORWARD_FLAGS", _btp.FLAG_PATH_MFMA)
+    coeff, x, dy = make_inputs(2, 4, 272, seed=43)
+    c = coeff.to(DEV).requires_grad_(True)
+    xx = x.to(DEV).requires_grad_(True)
+    y = btp(c, xx, output_dtype=torch.bfloat16)
+    y.backward(dy.to(DEV))
+    ref = orc.forward(f64(coeff), f64(x))
+    rdx, rdA = orc.backward(f64(coeff), f64(x), f64(dy))
+    assert_close(f64(y), ref, BF16_ATOL, BF16_RTOL, "y")
+    assert_close(f64(xx.grad), rdx, BF16_ATOL, BF16_RTOL, "dx")
+    magnitude = orc.backward(f64(coeff), np.abs(f64(x)), np.abs(f64(dy)))[1]
+    assert (np.abs(f64(c.grad) - rdA) <= 1e-3 + 2.0 ** -7 * magnitude + 2.0 ** -8 * np.abs(rdA)).all()
+    # these are the matrix-core kernels' values, not the default kernels': with the decay matrix rounded to 16
+    # bits the fp32 output differs from the fp32 recurrence somewhere
+    y32_mfma = btp(coeff.to(DEV), x.to(DEV))
+    monkeypatch.setattr(interface, "_PATH_MFMA", False)
+    monkeypatch.setattr(interface, "_FORWARD_FLAGS", 0)
+    assert not torch.equal(btp(coeff.to(DEV), x.to(DEV)), y32_mfma)
+    # with an fp32 dy the backward falls to the recurrence kernel, which has that input type
+    monkeypatch.setattr(interface, "_PATH_MFMA", True)
+    monkeypatch.setattr(interface, "_FORWARD_FLAGS", _btp.FLAG_PATH_MFMA)
+    c2 = coeff.to(DEV).requires_grad_(True)
+    x2 = x.to(DEV).requires_grad_(True)
+    btp(c2, x2).backward(dy.to(DEV).float())
+    assert_close(f64(x2.grad), rdx, BF16_ATOL, BF16_RTOL, "dx, fp32 dy")
+
+
 def test_non_contiguous_views_are_accepted():
     # the layer hands over transposed views (proj(x).transpose(1, 2)); btp() makes them contiguous
     from spear_amd import btp
