@@ -50,7 +50,7 @@ extern "C" {
 #define SPEAR_BTP_PATH_MFMA 0x2u        /* forward and backward: use the MFMA tile kernels (decay matrices rounded */
                                         /* to the input dtype and multiplied on the matrix cores, the reference's   */
                                         /* formulation) instead of the exact-fp32 recurrences; the backward then    */
-                                        /* takes dy in the inputs' dtype and has no SPEAR_BTP_DX_F32                */
+                                        /* rounds an fp32 dy to the inputs' dtype and has no SPEAR_BTP_DX_F32       */
 
 #define SPEAR_BTP_DX_F32 0x10u          /* backward: check mode, `dx` is fp32 [B, H, 16, L] and receives the    */
                                         /* kernel's fp32 values instead of their rounding to in_dtype           */

@@ -84,8 +84,6 @@ int spear_btp_backward(const void* coeff, const void* x, const void* dy, const f
   if (!aligned16(coeff) || !aligned16(x) || !aligned16(dy) || !aligned16(dx) || !aligned16(dA))
     return fail(SPEAR_BTP_EINVAL, "spear_btp_backward: tensor pointers must be 16-byte aligned");
   const bool mfma = (flags & SPEAR_BTP_PATH_MFMA) != 0;
-  if (mfma && dy_dtype != in_dtype)
-    return fail(SPEAR_BTP_EINVAL, "spear_btp_backward: the MFMA path takes dy in the inputs' dtype");
   if (mfma && (flags & SPEAR_BTP_DX_F32))
     return fail(SPEAR_BTP_EINVAL, "spear_btp_backward: the MFMA path has no fp32 dx (SPEAR_BTP_DX_F32)");
 

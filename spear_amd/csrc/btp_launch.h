@@ -36,8 +36,8 @@ struct BwdArgs {
 hipError_t scan_forward(const FwdArgs& p, hipStream_t s);
 hipError_t scan_backward(const BwdArgs& p, hipStream_t s);
 
-// MFMA tile kernels (btp_mfma.hip), bf16 or fp16 inputs; the forward stores no checkpoint, the backward takes
-// dy in the inputs' type and has neither log-space gates nor the fp32-dx check mode.
+// MFMA tile kernels (btp_mfma.hip), bf16 or fp16 inputs; the forward stores no checkpoint, the backward has
+// neither log-space gates nor the fp32-dx check mode (an fp32 dy is rounded to the inputs' type on load).
 hipError_t mfma_forward(const FwdArgs& p, hipStream_t s);
 hipError_t mfma_backward(const BwdArgs& p, hipStream_t s);
 

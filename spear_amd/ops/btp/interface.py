@@ -39,8 +39,8 @@ WPB_K2_DEFAULT = 32
 
 # Read once: the op sits on the hot path of every layer call.
 # SPEAR_BTP_PATH=mfma sends the op through the matrix-core kernels (the reference's formulation: decay matrices
-# rounded to 16 bits and multiplied on the matrix units) instead of the default fp32 recurrences; the backward
-# takes that path when dy arrives in the inputs' dtype and the recurrence kernel otherwise.
+# rounded to 16 bits and multiplied on the matrix units) instead of the default fp32 recurrences, forward and
+# backward.
 _PATH_MFMA = os.environ.get("SPEAR_BTP_PATH", "") == "mfma"
 _FORWARD_FLAGS = (_btp.FLAG_WRITE_CHECKPOINT if os.environ.get("SPEAR_BTP_WRITE_CHECKPOINT", "0") == "1" else 0) | (
     _btp.FLAG_PATH_MFMA if _PATH_MFMA else 0
@@ -69,7 +69,7 @@ def _backward_impl(
     k: int,
     wpb: int,
 ) -> None:
-    flags = _btp.FLAG_PATH_MFMA if (_PATH_MFMA and dy.dtype == x.dtype) else 0
+    flags = _btp.FLAG_PATH_MFMA if _PATH_MFMA else 0
     _btp.load_extension().backward(coeff, x, dy, checkpoint, dx, dA, k, wpb, flags)
 
 

@@ -42,7 +42,7 @@ def test_autograd_through_btp_matches_oracle():
 
 def test_the_op_runs_on_the_matrix_core_kernels_on_request(monkeypatch):
     """SPEAR_BTP_PATH=mfma (read when the module is imported; set on the module here) sends btp() through the
-    matrix-core forward and, for dy in the inputs' dtype, the matrix-core backward."""
+    matrix-core forward and backward."""
     from spear_amd import _btp, btp
     from spear_amd.ops.btp import interface
 
@@ -65,7 +65,7 @@ def test_the_op_runs_on_the_matrix_core_kernels_on_request(monkeypatch):
     monkeypatch.setattr(interface, "_PATH_MFMA", False)
     monkeypatch.setattr(interface, "_FORWARD_FLAGS", 0)
     assert not torch.equal(btp(coeff.to(DEV), x.to(DEV)), y32_mfma)
-    # with an fp32 dy the backward falls to the recurrence kernel, which has that input type
+    # the op's default types: fp32 y and fp32 dy
     monkeypatch.setattr(interface, "_PATH_MFMA", True)
     monkeypatch.setattr(interface, "_FORWARD_FLAGS", _btp.FLAG_PATH_MFMA)
     c2 = coeff.to(DEV).requires_grad_(True)
