@@ -61,7 +61,8 @@ __device__ __forceinline__ void local_state_at(const float (&a)[32], const float
 // ==========================================================================================
 // Prefill, tiled: 16-bit tensors, 16 channels, block length 16
 // ==========================================================================================
-// kAlign: what every channel row's start is aligned to, in bytes. 16: L is a multiple of 8 and every
+// kAlign: what every channel row's start is aligned to, in bytes (1: rows alternate between a word and an odd
+// element -- L odd, word-aligned tensors -- which is kRowsAlternate of the staging helpers). 16: L is a multiple of 8 and every
 // pointer 16-byte aligned (16-byte accesses); 4 or 2: rows of any length (see
 // slab16_global_to_regs_ragged), starting on words when L is even and the tensors are word-aligned.
 template <class E, class C, bool kEpilogue, bool kStreamIn, int kAlign>
@@ -71,6 +72,7 @@ __global__ __launch_bounds__(64 * kWaves) void jagged_prefill_kernel(
     void* __restrict__ h_tail, void* __restrict__ r_tail, void* __restrict__ c_prev_tail, int state_dtype,
     int r_dtype, int L, int spans_per_row, long total_spans) {
   constexpr bool kRagged = kAlign < 16;
+  constexpr int kRows = kAlign == 4 ? kRowsOnWords : kAlign == 1 ? kRowsAlternate : kRowsAnywhere;
   constexpr int kImages = kEpilogue ? 3 : 1;
   __shared__ __align__(16) unsigned char lds[kWaves][kImages * 4096 + kCoeffLdsBytes];
 
@@ -98,11 +100,11 @@ __global__ __launch_bounds__(64 * kWaves) void jagged_prefill_kernel(
   uint32_t xe = 0u, ce = 0u, ve = 0u;
   typename C::pair_t ain;
   if constexpr (kRagged) {
-    slab16_global_to_regs_ragged<kAlign == 4>(x + slab_off, L, sc.nvalid, lane, xw, xe);
+    slab16_global_to_regs_ragged<kRows>(x + slab_off, L, sc.nvalid, lane, xw, xe);
     ain = coeff_global_to_reg_ragged<C>(arow, sc.nvalid, lane);
     if constexpr (kEpilogue) {
-      slab16_global_to_regs_ragged<kAlign == 4>(cmul + slab_off, L, sc.nvalid, lane, cw, ce);
-      slab16_global_to_regs_ragged<kAlign == 4>(vadd + slab_off, L, sc.nvalid, lane, vw, ve);
+      slab16_global_to_regs_ragged<kRows>(cmul + slab_off, L, sc.nvalid, lane, cw, ce);
+      slab16_global_to_regs_ragged<kRows>(vadd + slab_off, L, sc.nvalid, lane, vw, ve);
     }
   } else {
     slab16_global_to_regs<nt_loads(kStreamIn)>(x + slab_off, L, sc.nvalid, lane, xin);
@@ -138,12 +140,12 @@ __global__ __launch_bounds__(64 * kWaves) void jagged_prefill_kernel(
 
   coeff_reg_to_lds<C>(a_lds, lane, ain);
   if constexpr (kRagged) {
-    slab16_regs_realign<kAlign == 4>(x + slab_off, L, sc.nvalid, lane, xw, xe);
+    slab16_regs_realign<kRows>(x + slab_off, L, sc.nvalid, lane, xw, xe);
     slab16_regs_to_lds_ragged(img, lane, xw);
     if constexpr (kEpilogue) {
-      slab16_regs_realign<kAlign == 4>(cmul + slab_off, L, sc.nvalid, lane, cw, ce);
+      slab16_regs_realign<kRows>(cmul + slab_off, L, sc.nvalid, lane, cw, ce);
       slab16_regs_to_lds_ragged(img + 4096, lane, cw);
-      slab16_regs_realign<kAlign == 4>(vadd + slab_off, L, sc.nvalid, lane, vw, ve);
+      slab16_regs_realign<kRows>(vadd + slab_off, L, sc.nvalid, lane, vw, ve);
       slab16_regs_to_lds_ragged(img + 8192, lane, vw);
     }
   } else {
@@ -219,7 +221,7 @@ __global__ __launch_bounds__(64 * kWaves) void jagged_prefill_kernel(
   wave_lds_handover();
   lane_write16<E>(img, j, d, yv);
   wave_lds_handover();
-  if constexpr (kRagged) slab16_lds_to_global_ragged<kAlign == 4>(img, y + slab_off, L, sc.nvalid, lane);
+  if constexpr (kRagged) slab16_lds_to_global_ragged<kRows>(img, y + slab_off, L, sc.nvalid, lane, sc.nvalid == L);
   else slab16_lds_to_global<true>(img, y + slab_off, L, sc.nvalid, lane);
 }
 
@@ -439,9 +441,8 @@ void launch_prefill_tiled(const JagPrefillArgs& p, hipStream_t s) {
   auto* y = static_cast<uint16_t*>(p.y);
   const bool st = stream_inputs(g);
   auto word_aligned = [](const void* q) { return (reinterpret_cast<uintptr_t>(q) & 3u) == 0; };
-  const int align = (p.L % 8 == 0 && p.aligned) ? 16
-                    : (p.L % 2 == 0 && word_aligned(p.x) && word_aligned(p.c) && word_aligned(p.v) && word_aligned(p.y)) ? 4
-                                                                                                                        : 2;
+  const bool on_words = word_aligned(p.x) && word_aligned(p.c) && word_aligned(p.v) && word_aligned(p.y);
+  const int align = (p.L % 8 == 0 && p.aligned) ? 16 : !on_words ? 2 : (p.L % 2 == 0) ? 4 : 1;
 #define SPEAR_JAG_LAUNCH(EPI, ST, AL)                                                                         \
   hipLaunchKernelGGL((jagged_prefill_kernel<E, C, EPI, ST, AL>), dim3(g.blocks), dim3(64 * kWaves), 0, s, a, x, \
                      c, v, p.carry_init, y, p.h_tail, p.r_tail, p.c_prev_tail, p.state_dtype, p.r_dtype, p.L,   \
@@ -455,6 +456,7 @@ void launch_prefill_tiled(const JagPrefillArgs& p, hipStream_t s) {
   do {                                                \
     if (align == 16) SPEAR_JAG_BY_SPAN(EPI, 16);      \
     else if (align == 4) SPEAR_JAG_BY_SPAN(EPI, 4);   \
+    else if (align == 1) SPEAR_JAG_BY_SPAN(EPI, 1);   \
     else SPEAR_JAG_BY_SPAN(EPI, 2);                   \
   } while (0)
   if (p.c != nullptr) SPEAR_JAG_BY_ALIGN(true);

@@ -222,38 +222,58 @@ __device__ __forceinline__ void slab16_lds_to_global(const unsigned char* img, u
 // the row's own 4-byte blocks is touched, and stores never write an element that is not the row's.
 __device__ __forceinline__ uint4 load16_plain_unaligned(const uint16_t* p) { return load16_plain_unaligned_fwd(p); }
 
+// Where the 16 channel rows of a slab start, which decides how much of the work below is needed:
+//   kRowsOnWords    every row starts on a 32-bit word (L even, word-aligned tensors)
+//   kRowsAlternate  row r starts on a word for even r and on an odd element for odd r (L odd, word-aligned
+//                   tensors): known when the code is generated, so even rows need no shifting at all
+//   kRowsAnywhere   found out per row at run time (tensors that start on an odd element)
+enum RowStarts : int { kRowsOnWords = 0, kRowsAlternate = 1, kRowsAnywhere = 2 };
+
+template <int kRows>
+__device__ __forceinline__ bool row_starts_odd(const uint16_t* row, int r) {  // wave-uniform
+  if constexpr (kRows == kRowsOnWords) return false;
+  else if constexpr (kRows == kRowsAlternate) return (r & 1) != 0;
+  else return ((reinterpret_cast<uintptr_t>(row) >> 1) & 1) != 0;
+}
+
 // Step 1, all loads, no dependent work between them (so that a slab's 16 loads -- and those of the
 // other slabs -- are in flight together): q[r] = the aligned word `lane` of channel row r, i.e.
 // elements (2*lane, 2*lane+1) of the span if the row starts on a word and (2*lane-1, 2*lane) if it
 // starts on an odd element. `edge` (lanes 0..15, lane = row) is word 64 of the row, which only rows on
-// an odd element need. kWordRows: every row starts on a word (L even, word-aligned tensors).
-template <bool kWordRows>
+// an odd element need.
+template <int kRows>
 __device__ __forceinline__ void slab16_global_to_regs_ragged(const uint16_t* slab, long L, int nvalid, int lane,
                                                              uint32_t (&q)[16], uint32_t& edge) {
   // (pointer arithmetic, not an integer round trip: the compiler must keep seeing global memory)
-  auto words_of = [&](int r, int& last) {
+  auto words_of = [&](int r, bool odd, int& last) {
     const uint16_t* row = slab + (long)r * L;
-    const int odd = (int)((reinterpret_cast<uintptr_t>(row) >> 1) & 1);
     last = odd ? (nvalid >> 1) : ((nvalid - 1) >> 1);  // last word that holds an element of the row
-    return reinterpret_cast<const uint32_t*>(row - odd);
+    return reinterpret_cast<const uint32_t*>(row - (odd ? 1 : 0));
   };
 #pragma unroll
   for (int r = 0; r < 16; ++r) {
     int last;
-    const uint32_t* words = words_of(r, last);
+    const uint32_t* words = words_of(r, row_starts_odd<kRows>(slab + (long)r * L, r), last);
     q[r] = __builtin_nontemporal_load(words + min(lane, last));
   }
   edge = 0u;
-  if constexpr (!kWordRows) {
-    int last;
-    const uint32_t* words = words_of(lane & 15, last);
-    edge = words[min(64, last)];
+  // word 64 exists only for a row on an odd element whose span is full (its step 127 sits there): one gather,
+  // lane i for row i (kRowsAnywhere) or for the i-th odd row (kRowsAlternate)
+  if (kRows != kRowsOnWords && nvalid == kSpan) {  // wave-uniform
+    constexpr int kEdgeLanes = kRows == kRowsAlternate ? 8 : 16;
+    if (lane < kEdgeLanes) {
+      int last;
+      const int r = kRows == kRowsAlternate ? 2 * lane + 1 : lane;
+      const bool odd = kRows == kRowsAlternate ? true : row_starts_odd<kRowsAnywhere>(slab + (long)r * L, r);
+      const uint32_t* words = words_of(r, odd, last);
+      edge = words[min(64, last)];
+    }
   }
 }
 
 // Step 2, in registers: shift the rows that start on an odd element by 16 bits (the upper neighbour
 // word comes from the next lane, for lane 63 from `edge`), and zero what lies beyond the row's end.
-template <bool kWordRows>
+template <int kRows>
 __device__ __forceinline__ void slab16_regs_realign(const uint16_t* slab, long L, int nvalid, int lane,
                                                     uint32_t (&q)[16], uint32_t edge) {
   const int e = lane << 1;
@@ -261,11 +281,11 @@ __device__ __forceinline__ void slab16_regs_realign(const uint16_t* slab, long L
 #pragma unroll
   for (int r = 0; r < 16; ++r) {
     uint32_t w = q[r];
-    if constexpr (!kWordRows) {
-      const bool odd = (reinterpret_cast<uintptr_t>(slab + (long)r * L) >> 1) & 1;  // wave-uniform
+    if (kRows == kRowsAnywhere || (kRows == kRowsAlternate && (r & 1))) {
+      const bool odd = row_starts_odd<kRows>(slab + (long)r * L, r);
       // the word held by lane + 1: a whole-wavefront DPP shift (wave_shl:1), no LDS traffic
       const uint32_t up = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)w, 0x130, 0xF, 0xF, false);
-      const uint32_t w64 = (uint32_t)__builtin_amdgcn_readlane((int)edge, r);
+      const uint32_t w64 = (uint32_t)__builtin_amdgcn_readlane((int)edge, kRows == kRowsAlternate ? (r >> 1) : r);
       const uint32_t w1 = lane == 63 ? w64 : up;
       w = odd ? (w >> 16) | (w1 << 16) : w;
     }
@@ -282,28 +302,42 @@ __device__ __forceinline__ void slab16_regs_to_lds_ragged(unsigned char* img, in
 // Image -> global. Whole aligned words first (for a row on an odd element, memory word i holds the
 // high half of lane i-1's image word and the low half of lane i's); the one or two elements per row
 // that no whole word covers are then written by lanes 0..31 acting as per-row workers.
-template <bool kWordRows>
+// `chained` (wave-uniform; kRowsAlternate only): every row ends where the next one starts (the slab is the whole
+// of its rows, nvalid == L). The word that holds a row's last element and the next row's first one is then this
+// wavefront's alone and lane 0 of the odd row writes it whole: no 2-byte stores are left (each of them costs a
+// 32-byte memory transaction: +27 % bytes written at L = 127).
+template <int kRows>
 __device__ __forceinline__ void slab16_lds_to_global_ragged(const unsigned char* img, uint16_t* slab, long L,
-                                                            int nvalid, int lane) {
+                                                            int nvalid, int lane, bool chained = false) {
   const int e = lane << 1;
   auto image_word = [&](int r, int i) {
     return *reinterpret_cast<const uint32_t*>(img + swz<256>(r, i >> 2) + ((i & 3) << 2));
   };
+  const bool link = kRows == kRowsAlternate && chained;
 #pragma unroll
   for (int r = 0; r < 16; ++r) {
     uint16_t* row = slab + (long)r * L;
-    const bool odd = !kWordRows && ((reinterpret_cast<uintptr_t>(row) >> 1) & 1);  // wave-uniform
+    const bool odd = row_starts_odd<kRows>(row, r);  // wave-uniform
     const uint32_t w = image_word(r, lane);
-    const uint32_t below = image_word(r, (lane + 63) & 63);
-    const uint32_t mw = odd ? (below >> 16) | (w << 16) : w;
-    // row on a word: lane covers (e, e+1); on an odd element: (e-1, e), lane 0 has no whole word
-    const bool whole = odd ? (lane > 0 && e < nvalid) : (e + 1 < nvalid);
+    uint32_t mw = w;
+    bool whole = e + 1 < nvalid;  // row on a word: lane covers (e, e+1)
+    if (kRows == kRowsAnywhere || (kRows == kRowsAlternate && (r & 1))) {
+      // on an odd element: lane covers (e-1, e); lane 0 has no whole word unless the rows are chained, in
+      // which case its lower half is the previous row's last element (an even index, L being odd)
+      uint32_t below = image_word(r, (lane + 63) & 63);
+      if (kRows == kRowsAlternate && r > 0) {
+        const uint32_t prev_last = image_word(r - 1, (nvalid - 1) >> 1);
+        below = (link && lane == 0) ? (prev_last << 16) : below;
+      }
+      mw = odd ? (below >> 16) | (w << 16) : w;
+      whole = odd ? ((lane > 0 || link) && e < nvalid) : whole;
+    }
     if (whole) __builtin_nontemporal_store(mw, reinterpret_cast<uint32_t*>(row + e - (odd ? 1 : 0)));
   }
-  if (lane < 32) {
+  if (lane < 32 && !link) {
     const int r = lane & 15;
     uint16_t* row = slab + (long)r * L;
-    const bool odd = !kWordRows && ((reinterpret_cast<uintptr_t>(row) >> 1) & 1);
+    const bool odd = kRows == kRowsAlternate ? (r & 1) != 0 : row_starts_odd<kRowsAnywhere>(row, r);
     // lanes 0..15: first element of a row on an odd element; lanes 16..31: the last element when no
     // whole word reaches it (even count on an odd start, odd count on a word start)
     const bool first = lane < 16;
