@@ -119,12 +119,15 @@ int spear_phalanx_mix_forward(const void* a_logit, const void* b_logit, const vo
  * elements). Inputs keep their types. Not combinable with the column sums of _backward_ex. */
 #define SPEAR_MIX_F32_RESULTS 0x2u
 
-/* Flag for spear_phalanx_mix_backward / _backward_ex: the other work split of the same backward -- one
- * wavefront per 16-step block with the two carries handed between neighbouring blocks through LDS, instead of
- * wavefronts that walk through time. Same results up to fp32 rounding; 3 % faster at B=1024 L=128 H=32, within
- * 1 % elsewhere, so it is not the default (SPEAR_BTP_FUSED_BWD=tile in the environment makes it the default for
- * calls it can serve). Not combinable with column sums or SPEAR_MIX_F32_RESULTS. */
+/* Flags for spear_phalanx_mix_backward / _backward_ex: which work split of the backward runs. TILE: one
+ * wavefront per 16-step block, the two carries handed between neighbouring blocks through LDS; it has no
+ * column sums. WALK: wavefronts that walk through time (every option). Same results up to fp32 rounding.
+ * With neither flag the tile split serves every call without column sums (it measured 181-184 us against
+ * 185-196 us at B=1024 L=128 H=32, 1 % slower at B=16 L=8192 H=64, 5 % faster at B=64 L=2048 H=128) and the
+ * walking kernel those with sums; SPEAR_BTP_FUSED_BWD=walk or =tile in the environment changes that default.
+ * The two flags exclude each other. */
 #define SPEAR_MIX_TILE_SPLIT 0x4u
+#define SPEAR_MIX_WALK_SPLIT 0x8u
 
 /* Backward of spear_phalanx_mix_forward: reads a_logit, b_logit, c, v and the upstream gradient
  * dout [B, L, H * 16]; writes da_logit [B, L, H], db_logit and dc [B, L, kv_heads * 16] (summed over

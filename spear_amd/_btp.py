@@ -30,8 +30,9 @@ FLAG_JAGGED_LOG_R = 0x8
 FLAG_MIX_QKV_GATE = 0x1
 FLAG_MIX_F32_RESULTS = 0x2
 FLAG_MIX_TILE_SPLIT = 0x4
+FLAG_MIX_WALK_SPLIT = 0x8
 FLAG_DX_F32 = 0x10
-_ABI_VERSION = 15
+_ABI_VERSION = 16
 _SUPPORTED_WPB = (4, 8, 16, 32)
 
 _lock = threading.Lock()
@@ -405,7 +406,7 @@ def mix_backward(
     kv_heads: int,
     sums: tuple[torch.Tensor, torch.Tensor, torch.Tensor] | None = None,
     qkv_gate: bool = False,
-    tile_split: bool = False,
+    tile_split: bool | None = None,
 ) -> None:
     """Gradients of :func:`mix_forward`, written in place; ``heads // kv_heads`` must be 1, 2, 4 or 8
     (see ``spear_phalanx_mix_backward`` in the C header). ``sums``: three fp32 tensors
@@ -413,8 +414,9 @@ def mix_backward(
     column sums of ``da_logit``, ``db_logit`` and ``dc``. The four gradient tensors may be column blocks of one
     wider ``[B, L, ld]`` buffer (``spear_phalanx_mix_backward_ex``). ``qkv_gate`` as in :func:`mix_forward`;
     ``da_logit`` is then the fp32 gradient of the gate. Float32 ``db_logit, dc, dv`` (and ``da_logit``) select
-    the fp32 check mode (``SPEAR_MIX_F32_RESULTS``). ``tile_split`` selects the kernel with one wavefront per
-    16-step block (``SPEAR_MIX_TILE_SPLIT``)."""
+    the fp32 check mode (``SPEAR_MIX_F32_RESULTS``). ``tile_split``: True selects the kernel with one wavefront per
+    16-step block (``SPEAR_MIX_TILE_SPLIT``; no column sums), False the one whose wavefronts walk through time
+    (``SPEAR_MIX_WALK_SPLIT``), None leaves the choice to the library."""
     tensors = (a_logit, b_logit, c, v, dout, da_logit, db_logit, dc, dv)
     _check(all(t.is_cuda for t in tensors), "All tensors must be CUDA.")
     _check(v.dim() == 3, "v must be [B, L, heads * 16].")
@@ -459,7 +461,8 @@ def mix_backward(
             *sum_ptrs, rows,
             B, L, heads, kv_heads, _tag(v.dtype),
             (FLAG_MIX_QKV_GATE if qkv_gate else 0) | (FLAG_MIX_F32_RESULTS if f32 else 0)
-            | (FLAG_MIX_TILE_SPLIT if tile_split else 0), _stream_ptr(v.device),
+            | (0 if tile_split is None else FLAG_MIX_TILE_SPLIT if tile_split else FLAG_MIX_WALK_SPLIT),
+            _stream_ptr(v.device),
         )
     if rc != 0:
         _raise_native(lib, rc)

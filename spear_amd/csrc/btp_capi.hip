@@ -45,7 +45,7 @@ int check_common(const char* who, int B, int H, int L, int k, int in_dtype, int 
 
 extern "C" {
 
-int spear_btp_abi_version(void) { return 15; }
+int spear_btp_abi_version(void) { return 16; }
 
 const char* spear_btp_last_error(void) { return g_error; }
 
@@ -225,21 +225,24 @@ int spear_phalanx_mix_backward_ex(const void* a_logit, const void* b_logit, cons
   const void* const ptrs[9] = {a_logit, b_logit, c, v, dout, da_logit, db_logit, dc, dv};
   const int lds[4] = {ld_da, ld_db, ld_dc, ld_dv};
   if (int rc = check_mix_backward(who, ptrs, lds, B, L, H, kv_heads, dtype, flags,
-                                  SPEAR_MIX_QKV_GATE | SPEAR_MIX_F32_RESULTS | SPEAR_MIX_TILE_SPLIT))
+                                  SPEAR_MIX_QKV_GATE | SPEAR_MIX_F32_RESULTS | SPEAR_MIX_TILE_SPLIT | SPEAR_MIX_WALK_SPLIT))
     return rc < 0 ? rc : 0;
   const bool qkv = (flags & SPEAR_MIX_QKV_GATE) != 0, f32 = (flags & SPEAR_MIX_F32_RESULTS) != 0;
-  // the tile split is a flag, or the process-wide default when SPEAR_BTP_FUSED_BWD=tile is set (read once)
+  // the work split is a flag, or the process-wide default: the tile split wherever it can serve the call,
+  // unless SPEAR_BTP_FUSED_BWD=walk is set (read once)
   static const bool tile_default = [] {
     const char* e = getenv("SPEAR_BTP_FUSED_BWD");
-    return e != nullptr && e[0] == 't';
+    return e == nullptr || e[0] != 'w';
   }();
-  const bool tile_asked = (flags & SPEAR_MIX_TILE_SPLIT) != 0;
+  const bool tile_asked = (flags & SPEAR_MIX_TILE_SPLIT) != 0, walk_asked = (flags & SPEAR_MIX_WALK_SPLIT) != 0;
+  if (tile_asked && walk_asked)
+    return fail(SPEAR_BTP_EINVAL, "%s: SPEAR_MIX_TILE_SPLIT and SPEAR_MIX_WALK_SPLIT exclude each other", who);
   const bool sums = sum_da || sum_db || sum_dc;
   if (sums && qkv) return fail(SPEAR_BTP_EINVAL, "%s: column sums are for the layer form, not SPEAR_MIX_QKV_GATE", who);
   if (sums && f32) return fail(SPEAR_BTP_EINVAL, "%s: column sums are not available with SPEAR_MIX_F32_RESULTS", who);
-  if (tile_asked && (sums || f32))
-    return fail(SPEAR_BTP_EINVAL, "%s: SPEAR_MIX_TILE_SPLIT has neither column sums nor fp32 results", who);
-  const bool tile = (tile_asked || (tile_default && !sums && !f32)) &&
+  if (tile_asked && sums)
+    return fail(SPEAR_BTP_EINVAL, "%s: SPEAR_MIX_TILE_SPLIT has no column sums", who);
+  const bool tile = (tile_asked || (tile_default && !walk_asked && !sums)) &&
                     (long long)B * ((L / 16 + 3) / 4) * ((H + 7) / 8) < (1ll << 31);
   if (sums) {
     if (!sum_da || !sum_db || !sum_dc) return fail(SPEAR_BTP_ENULL, "%s: the three sum arrays must be given together", who);

@@ -562,10 +562,10 @@ __global__ __launch_bounds__(64 * kWaves) void phalanx_mix_bwd_kernel(
 
 
 // ==========================================================================================
-// Backward of the fused mixing stage, tile form (SPEAR_MIX_TILE_SPLIT; not the default): the same
-// mathematics with a different work split. Measured against the walking kernel above at B=1024 L=128 H=32 it is
-// 3 % faster (180.6 against 186 us), at B=16 L=8192 H=64 1 % slower, at B=64 L=2048 H=128 1 % faster; it stays in
-// the library as the measured alternative. One
+// Backward of the fused mixing stage, tile form (SPEAR_MIX_TILE_SPLIT; what a call without a split flag runs
+// unless it asks for column sums): the same mathematics with a different work split. Measured against the walking
+// kernel above at B=1024 L=128 H=32 it takes 181-184 us against 185-196 us, at B=16 L=8192 H=64 it is 1 % slower, at
+// B=64 L=2048 H=128 5 % faster. One
 // wavefront owns ONE 16-step block of 128 features and runs no loop: every load is issued at the start, every
 // store at the end, and a workgroup (8 wavefronts = octs_w head groups x nb_w consecutive blocks of one batch
 // row) lives for a few microseconds. Copy loops with this kernel's traffic show why: wavefronts that walk
@@ -610,7 +610,8 @@ __device__ __forceinline__ float product_of_the_others(float a) {
 #ifndef SPEAR_FUSED_TILE_WAVES_PER_EU  // 4 waves per SIMD (two workgroups per CU) need <= 128 VGPRs
 #define SPEAR_FUSED_TILE_WAVES_PER_EU 4
 #endif
-template <class E, bool kQkv>
+// kF32: check mode, the four gradients leave as fp32 (the kernel's own values, not rounded to 16 bits).
+template <class E, bool kQkv, bool kF32>
 __global__ __launch_bounds__(64 * kTileWaves) __attribute__((amdgpu_waves_per_eu(SPEAR_FUSED_TILE_WAVES_PER_EU)))
 void phalanx_mix_bwd_tile_kernel(
     const uint16_t* __restrict__ a_logit, const uint16_t* __restrict__ b_logit, const uint16_t* __restrict__ c_in,
@@ -644,8 +645,8 @@ void phalanx_mix_bwd_tile_kernel(
   const int stride = 2 * F, kv_stride = 2 * Fkv;
   constexpr int kRsrcFlags = 0x00020000;
   constexpr int kGateBytes = kQkv ? 4 : 2;
-  constexpr int kDaBytes = kQkv ? 4 : 2;
-  constexpr int kGradBytes = 2;
+  constexpr int kDaBytes = (kQkv || kF32) ? 4 : 2;
+  constexpr int kGradBytes = kF32 ? 4 : 2;
   const long big = brow * L * F, kvbig = brow * L * Fkv, small = brow * L * H;
   auto rsrc = [&](const uint16_t* p, long off, int bytes) {
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(p + off), 0, bytes, kRsrcFlags);
@@ -881,9 +882,17 @@ void phalanx_mix_bwd_tile_kernel(
         }
       }
       const float dv0 = fmaf(dX0, G0, go0), dv1 = fmaf(dX1, G1, go1);
-      __builtin_amdgcn_raw_buffer_store_b32(E::pack2(dc0, dc1), rdc, okv_lane, (t0 + r) * 2 * ld_dc, kNt);
-      __builtin_amdgcn_raw_buffer_store_b32(E::pack2(dv0, dv1), rdv, o_lane, (t0 + r) * 2 * ld_dv, kNt);
-      __builtin_amdgcn_raw_buffer_store_b32(E::pack2(db0, db1), rdb, okv_lane, (t0 + r) * 2 * ld_db, kNt);
+      if constexpr (kF32) {
+        const u32x2_t wdc = {__float_as_uint(dc0), __float_as_uint(dc1)}, wdv = {__float_as_uint(dv0), __float_as_uint(dv1)},
+                      wdb = {__float_as_uint(db0), __float_as_uint(db1)};
+        __builtin_amdgcn_raw_buffer_store_b64(wdc, rdc, okv_lane, (t0 + r) * 4 * ld_dc, kNt);
+        __builtin_amdgcn_raw_buffer_store_b64(wdv, rdv, o_lane, (t0 + r) * 4 * ld_dv, kNt);
+        __builtin_amdgcn_raw_buffer_store_b64(wdb, rdb, okv_lane, (t0 + r) * 4 * ld_db, kNt);
+      } else {
+        __builtin_amdgcn_raw_buffer_store_b32(E::pack2(dc0, dc1), rdc, okv_lane, (t0 + r) * 2 * ld_dc, kNt);
+        __builtin_amdgcn_raw_buffer_store_b32(E::pack2(dv0, dv1), rdv, o_lane, (t0 + r) * 2 * ld_dv, kNt);
+        __builtin_amdgcn_raw_buffer_store_b32(E::pack2(db0, db1), rdb, okv_lane, (t0 + r) * 2 * ld_db, kNt);
+      }
     }
     asm volatile("" ::: "memory");
   }
@@ -1106,7 +1115,7 @@ void launch_mix_bwd(const MixBwdArgs& p, const MixPlan& m, hipStream_t s) {
                      p.ld_dv ? p.ld_dv : p.H * kChan, p.L, p.H, p.kv_groups, m.chunk_blocks * kTile, m.chunks, total);
 }
 
-template <class E, bool kQkv>
+template <class E, bool kQkv, bool kF32 = false>
 void launch_mix_bwd_tile(const MixBwdArgs& p, hipStream_t s) {
   const int octs = (p.H + 7) / 8, nb = p.L / kTile;
   const int octs_w = octs % 2 == 0 ? 2 : 1;  // measured with copy loops: 2 head groups x 4 blocks moves the most
@@ -1116,7 +1125,7 @@ void launch_mix_bwd_tile(const MixBwdArgs& p, hipStream_t s) {
   auto u = [](const void* q) { return static_cast<const uint16_t*>(q); };
   auto w = [](void* q) { return static_cast<uint16_t*>(q); };
   const int Fkv = (p.H / p.kv_groups) * kChan;
-  hipLaunchKernelGGL((phalanx_mix_bwd_tile_kernel<E, kQkv>), dim3((unsigned)wgs), dim3(64 * kTileWaves), 0, s,
+  hipLaunchKernelGGL((phalanx_mix_bwd_tile_kernel<E, kQkv, kF32>), dim3((unsigned)wgs), dim3(64 * kTileWaves), 0, s,
                      u(p.a_logit), u(p.b_logit), u(p.c), u(p.v), u(p.dout), w(p.da_logit), w(p.db_logit), w(p.dc), w(p.dv),
                      p.ld_da ? p.ld_da : p.H, p.ld_db ? p.ld_db : Fkv, p.ld_dc ? p.ld_dc : Fkv,
                      p.ld_dv ? p.ld_dv : p.H * kChan, p.L, p.H, p.kv_groups, octs_w, nb_w, tiles, oct_groups);
@@ -1133,14 +1142,24 @@ hipError_t fused_mix_backward(const MixBwdArgs& p, hipStream_t s) {
   const MixPlan m = plan_mix_bwd(p.B, p.H, p.L);
   const bool sums = p.sum_da != nullptr;
   if (sums && (p.qkv || p.f32_grads)) return hipErrorInvalidValue;  // the caller has checked: layer form, 16-bit results
-  if (p.tile_split) {  // the caller has checked: no sums, 16-bit results, a grid that fits
-    if (sums || p.f32_grads) return hipErrorInvalidValue;
+  if (p.tile_split) {  // the caller has checked: no sums, a grid that fits
+    if (sums) return hipErrorInvalidValue;
     if (p.dtype == kBf16) {
-      if (p.qkv) launch_mix_bwd_tile<Bf16, true>(p, s);
-      else launch_mix_bwd_tile<Bf16, false>(p, s);
+      if (p.f32_grads) {
+        if (p.qkv) launch_mix_bwd_tile<Bf16, true, true>(p, s);
+        else launch_mix_bwd_tile<Bf16, false, true>(p, s);
+      } else {
+        if (p.qkv) launch_mix_bwd_tile<Bf16, true>(p, s);
+        else launch_mix_bwd_tile<Bf16, false>(p, s);
+      }
     } else {
-      if (p.qkv) launch_mix_bwd_tile<Fp16, true>(p, s);
-      else launch_mix_bwd_tile<Fp16, false>(p, s);
+      if (p.f32_grads) {
+        if (p.qkv) launch_mix_bwd_tile<Fp16, true, true>(p, s);
+        else launch_mix_bwd_tile<Fp16, false, true>(p, s);
+      } else {
+        if (p.qkv) launch_mix_bwd_tile<Fp16, true>(p, s);
+        else launch_mix_bwd_tile<Fp16, false>(p, s);
+      }
     }
     return hipGetLastError();
   }

@@ -52,7 +52,7 @@ def test_fused_forward_fp16_and_steep_gates():
     assert_close(f64(out), ref, 4e-3, 4e-3, "out fp16")
 
 
-def run_mix_backward(a, b, c, v, dout, H, Hkv=None, tile_split=False):
+def run_mix_backward(a, b, c, v, dout, H, Hkv=None, tile_split=None):
     from spear_amd import _btp
 
     dev = [t.to(DEV) for t in (a, b, c, v, dout)]
@@ -62,8 +62,9 @@ def run_mix_backward(a, b, c, v, dout, H, Hkv=None, tile_split=False):
     return [t.cpu() for t in outs]
 
 
-# the backward kernel comes in two work splits: wavefronts that walk through time (default) and one wavefront
-# per 16-step block (SPEAR_MIX_TILE_SPLIT); both are held to the same oracle
+# the backward kernel comes in two work splits: wavefronts that walk through time (SPEAR_MIX_WALK_SPLIT) and one
+# wavefront per 16-step block (SPEAR_MIX_TILE_SPLIT, the library's own choice for calls without column sums); both
+# are held to the same oracle
 SPLITS = pytest.mark.parametrize("tile_split", [False, True], ids=["walk", "tile"])
 
 
@@ -107,7 +108,7 @@ def test_fused_backward_column_sums_match_oracle(B, L, H, Hkv):
     a, b, c, v = make_mix_inputs(B, L, H, Hkv, seed=5000 + L + H)
     dout = torch.randn(B, L, H * 16, generator=torch.Generator().manual_seed(L + 2)).bfloat16()
     print(f"fused bwd sums B={B} L={L} H={H} Hkv={Hkv}", flush=True)
-    plain = run_mix_backward(a, b, c, v, dout, H, Hkv)
+    plain = run_mix_backward(a, b, c, v, dout, H, Hkv, tile_split=False)  # sums come from the walking kernel
     dev = [t.to(DEV) for t in (a, b, c, v, dout)]
     outs = [torch.full(t.shape, float("nan"), device=DEV, dtype=t.dtype) for t in (a, b, c, v)]
     rows = _btp.mix_backward_sum_rows(B, L, H)
@@ -295,7 +296,16 @@ def test_tile_split_strided_outputs_qkv_form_and_what_it_refuses():
     rows = _btp.mix_backward_sum_rows(B, L, H)
     sums = tuple(torch.empty(rows, w, device=DEV) for w in widths[:3])
     grads = [torch.empty_like(t) for t in dev[:4]]
-    with pytest.raises(RuntimeError, match="neither column sums nor fp32 results"):
+    with pytest.raises(RuntimeError, match="has no column sums"):
         _btp.mix_backward(*dev, *grads, H, Hkv, sums=sums, tile_split=True)
-    with pytest.raises(RuntimeError, match="neither column sums nor fp32 results"):
-        _btp.mix_backward(*dev, *[torch.empty(t.shape, device=DEV) for t in dev[:4]], H, Hkv, tile_split=True)
+    # left to the library, a call runs the tile split, and the walking kernel when it asks for column sums
+    auto = [torch.full(t.shape, float("nan"), device=DEV, dtype=t.dtype) for t in (a, b, c, v)]
+    _btp.mix_backward(*dev, *auto, H, Hkv)
+    torch.cuda.synchronize()
+    for got, want in zip(auto, dense):
+        assert torch.equal(got.cpu(), want)
+    _btp.mix_backward(*dev, *grads, H, Hkv, sums=sums)
+    torch.cuda.synchronize()
+    walked = run_mix_backward(a, b, c, v, dout, H, Hkv, tile_split=False)
+    for got, want in zip(grads, walked):
+        assert torch.equal(got.cpu(), want)
