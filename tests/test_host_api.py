@@ -324,6 +324,23 @@ def test_default_method_can_be_sent_to_the_fused_kernels_by_environment(monkeypa
     assert layer._forward_fn == layer._forward_pytorch
 
 
+def test_the_kernel_path_switch_is_read_from_the_environment():
+    """SPEAR_BTP_PATH=mfma (read once, when the op module is imported) puts the matrix-core flag on both custom ops;
+    anything else leaves the default recurrence kernels."""
+    import os
+    import subprocess
+    import sys
+
+    probe = ("from spear_amd.ops.btp import interface as i; from spear_amd import _btp; "
+             "print(int(i._PATH_MFMA), int(bool(i._FORWARD_FLAGS & _btp.FLAG_PATH_MFMA)))")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    for value, want in (("mfma", "1 1"), ("", "0 0"), ("scan", "0 0")):
+        env = dict(os.environ, SPEAR_BTP_PATH=value, PYTHONPATH=root)
+        out = subprocess.run([sys.executable, "-c", probe], env=env, capture_output=True, text=True, cwd=root, timeout=300)
+        assert out.returncode == 0, out.stderr
+        assert out.stdout.strip().splitlines()[-1] == want, (value, out.stdout)
+
+
 def test_streaming_module_surface_and_state_dataclass():
     from spear_amd.nn.phalanx import inference as inf
 
