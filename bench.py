@@ -300,6 +300,25 @@ def main() -> int:
 
     fwd_log_ms, bwd_log_ms = kernel_ms(fwd_log), kernel_ms(bwd_log)
 
+    # the op's default types: btp(coeff, x) returns fp32 y and autograd hands back an fp32 dy (98 + 134 B per unit)
+    for s_ in sets:
+        s_["y32"] = torch.empty(B, H, 16, L, device=dev, dtype=torch.float32)
+
+    def fwd_f32(s):
+        rc = lib.spear_btp_forward(s["coeff"].data_ptr(), s["x"].data_ptr(), s["y32"].data_ptr(), None,
+                                   B, H, L, 2, 0, 2, 0, sp)
+        assert rc == 0, lib.spear_btp_last_error()
+
+    def bwd_f32(s):  # y32 stands in for an fp32 dy: same bytes moved, values do not matter for the time
+        rc = lib.spear_btp_backward(s["coeff"].data_ptr(), s["x"].data_ptr(), s["y32"].data_ptr(), None,
+                                    s["dx"].data_ptr(), s["dA"].data_ptr(), B, H, L, 2, 0, 2, 0, sp)
+        assert rc == 0, lib.spear_btp_last_error()
+
+    fwd_f32_ms = kernel_ms(fwd_f32)
+    bwd_f32_ms = kernel_ms(bwd_f32)
+    for s_ in sets:
+        del s_["y32"]
+
     # fused layer-layout forward (gates + recurrence + y*C+V on [B, L, features] tensors) against the
     # same stage built from PyTorch ops around the stand-alone kernel
     def guarded(leg):
@@ -775,6 +794,12 @@ def main() -> int:
         "backward_kernel_mfma_path": {"avg_launch_ms": bwd_mfma_ms,
                                       "achieved": units * BWD_BYTES / (bwd_mfma_ms * 1e-3) / 1e9,
                                       "frac": units * BWD_BYTES / (bwd_mfma_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS},
+        "op_default_dtypes_fp32_y_fp32_dy": {
+            "forward_ms": fwd_f32_ms, "backward_ms": bwd_f32_ms,
+            "algorithmic_bytes_per_unit": {"forward": 98, "backward": 134},
+            "forward_frac": units * 98 / (fwd_f32_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+            "backward_frac": units * 134 / (bwd_f32_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+        },
         "log_gate_entry_points": {"forward_ms": fwd_log_ms, "backward_ms": bwd_log_ms,
                                   "achieved": units * (68 + 108) / ((fwd_log_ms + bwd_log_ms) * 1e-3) / 1e9,
                                   "algorithmic_bytes_per_unit": {"forward": 68, "backward": 108}},
