@@ -47,9 +47,10 @@ extern "C" {
 
 /* flags */
 #define SPEAR_BTP_WRITE_CHECKPOINT 0x1u /* forward: also store the carry checkpoint            */
-#define SPEAR_BTP_PATH_MFMA 0x2u        /* forward and backward: use the MFMA tile kernels (decay matrices rounded */
-                                        /* to the input dtype and multiplied on the matrix cores, the reference's   */
-                                        /* formulation) instead of the exact-fp32 recurrences; the backward then    */
+#define SPEAR_BTP_PATH_MFMA 0x2u        /* forward and backward: use the MFMA tile kernels (decay matrices built   */
+                                        /* per block and multiplied on the matrix cores, the reference's            */
+                                        /* formulation; each entry goes in as two 16-bit pieces, so fp32 results    */
+                                        /* keep the 1e-4 bound) instead of the fp32 recurrences; the backward then  */
                                         /* rounds an fp32 dy to the inputs' dtype and has no SPEAR_BTP_DX_F32       */
 
 #define SPEAR_BTP_DX_F32 0x10u          /* backward: check mode, `dx` is fp32 [B, H, 16, L] and receives the    */

@@ -2,8 +2,9 @@
 // reference uses on sm90 -- materialise the block's decay matrix, multiply it with the activation
 // tile on the matrix cores (csrc/btp/btp-forward.cu:214-274, WarpMma in csrc/btp/btp_common.h:35-45)
 // -- rebuilt around v_mfma_f32_16x16x32_bf16 / _f16. Selected with SPEAR_BTP_PATH_MFMA; the default path
-// is the exact-fp32 recurrence (btp_scan.hip), which is at least as fast (both are HBM-bound) and
-// does not round the decay matrix to bf16.
+// is the exact-fp32 recurrence (btp_scan.hip), which is faster. Where the reference rounds its decay
+// matrix to bf16, this kernel feeds it to the matrix cores as two 16-bit pieces (split_decay below), so
+// its fp32 results meet the bound of the recurrence kernels.
 //
 // One MFMA per 16-step block i covers BOTH passes of the reference algorithm. With K = 32 running
 // over the previous block's 16 steps and the block's own 16 steps,
@@ -74,6 +75,43 @@ __device__ __forceinline__ floatx4_t mfma_16x16x32(uint4 a, uint4 b, floatx4_t a
   else
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(halfx8_t, a), __builtin_bit_cast(halfx8_t, b), acc,
                                                   0, 0, 0);
+}
+
+// A decay operand (8 fp32 entries per lane) against a 16-bit B operand, accumulated in fp32. The matrix
+// instruction takes 16-bit operands; the reference rounds its decay matrix to bf16 once and lives with 2^-9
+// relative error per entry (csrc/btp/btp-forward.cu:232-244). Here the entries go in as two 16-bit pieces,
+// e = hi + lo with hi = round16(e) and lo = round16(e - hi), i.e. two instructions on a matrix pipe that is
+// otherwise 95 % idle: about 2^-17 per entry, which keeps fp32 outputs of this path inside the 1e-4 bound of
+// the recurrence kernels. SPEAR_BTP_MFMA_SPLIT_DECAY=0 builds the single-piece form.
+#ifndef SPEAR_BTP_MFMA_SPLIT_DECAY
+#define SPEAR_BTP_MFMA_SPLIT_DECAY 1
+#endif
+struct DecayOperand {
+  uint4 hi, lo;
+};
+
+template <class E>
+__device__ __forceinline__ DecayOperand split_decay(const float (&e)[8]) {
+  DecayOperand d;
+  d.hi = pack8<E>(e);
+  d.lo = zero4();
+#if SPEAR_BTP_MFMA_SPLIT_DECAY
+  float h[8], r[8];
+  unpack8<E>(d.hi, h);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) r[i] = e[i] - h[i];
+  d.lo = pack8<E>(r);
+#endif
+  return d;
+}
+
+template <class E>
+__device__ __forceinline__ floatx4_t mfma_decay(const DecayOperand& a, uint4 b, floatx4_t acc) {
+  acc = mfma_16x16x32<E>(a.hi, b, acc);
+#if SPEAR_BTP_MFMA_SPLIT_DECAY
+  acc = mfma_16x16x32<E>(a.lo, b, acc);
+#endif
+  return acc;
 }
 
 template <class E, class OutT, bool kStreamIn>
@@ -156,7 +194,7 @@ __global__ __launch_bounds__(64 * kWaves) void btp_fwd_mfma_kernel(const uint16_
       e[jj] = above ? 0.0f : val;
       val *= above ? 1.0f : av[jj];
     }
-    const uint4 A = pack8<E>(e);
+    const DecayOperand A = split_decay<E>(e);
 
     // B: steps 16(i-1) + 8q .. +7 of channel n
     const int cidx = 2 * i - 2 + q;
@@ -168,7 +206,7 @@ __global__ __launch_bounds__(64 * kWaves) void btp_fwd_mfma_kernel(const uint16_
       braw = *reinterpret_cast<const uint4*>(img_x + swz<256>(n, cidx));
     }
     floatx4_t acc = {0.0f, 0.0f, 0.0f, 0.0f};
-    acc = mfma_16x16x32<E>(A, braw, acc);
+    acc = mfma_decay<E>(A, braw, acc);
 
     // D: y[channel n][16 i + 4 q .. + 3]
     if constexpr (kOutF32) {
@@ -203,9 +241,9 @@ __global__ __launch_bounds__(64 * kWaves) void btp_fwd_mfma_kernel(const uint16_
 // and then, with c = V_{i-1}[15] (the carry into the block) and P_{r-1} = prod_{j<r} a_j,
 //     dA_r = sum over channels of  dX_i[r] V_i[r-1]  +  P_{r-1} dXl_i[r] c          (V_i[-1] = 0, P_{-1} = 1)
 // which counts every (source step, sink step) pair whose decay product contains a_r exactly once and leaves
-// out the two-hop pairs (block i-1 to block i+1) that the operator does not have. The decay operands are
-// rounded to 16 bits for the matrix instruction, as in the reference; the default backward (btp_scan.hip)
-// keeps everything in fp32.
+// out the two-hop pairs (block i-1 to block i+1) that the operator does not have. The decay operands go
+// in as two 16-bit pieces (split_decay above); x and dy enter in 16 bits, as in the reference. The default
+// backward (btp_scan.hip) keeps everything in fp32.
 // A lane's 8 entries of a transposed row run left to right, entry(s, t+1) = entry(s, t) a_{t+1}, started from
 // suffix products that come from a 3-step DPP scan inside 8-lane halves plus v_readlane broadcasts.
 // ==========================================================================================
@@ -349,7 +387,7 @@ __global__ __launch_bounds__(64 * kWaves) void btp_bwd_mfma_kernel(const uint16_
       braw = (blk < 0) ? *reinterpret_cast<const uint4*>(halo_x + n * 32 + ((q - 2) << 4))
                        : *reinterpret_cast<const uint4*>(img_x + swz<256>(n, 2 * blk + q - 2));
     }
-    return mfma_16x16x32<E>(pack8<E>(e), braw, zero_acc);
+    return mfma_decay<E>(split_decay<E>(e), braw, zero_acc);
   };
 
   // carry into the span's first block: terminal local state of the block before it, channel n
@@ -412,10 +450,10 @@ __global__ __launch_bounds__(64 * kWaves) void btp_bwd_mfma_kernel(const uint16_
     const int cidx = 2 * i + q;
     const uint4 graw = (cidx < 16) ? *reinterpret_cast<const uint4*>(img_g + swz<256>(n, cidx))
                                    : *reinterpret_cast<const uint4*>(halo_g + n * 32 + ((cidx - 16) << 4));
-    const uint4 a2 = pack8<E>(e2);
-    const floatx4_t dxf = mfma_16x16x32<E>(a2, graw, zero_acc);
+    const DecayOperand a2 = split_decay<E>(e2);
+    const floatx4_t dxf = mfma_decay<E>(a2, graw, zero_acc);
     // the block-local part: the same operand against dy with the next block's half blanked
-    const floatx4_t dxl = mfma_16x16x32<E>(a2, (q < 2) ? graw : zero4(), zero_acc);
+    const floatx4_t dxl = mfma_decay<E>(a2, (q < 2) ? graw : zero4(), zero_acc);
 
     // ---- dx[channel n][16 i + 4 q .. + 3]
     {

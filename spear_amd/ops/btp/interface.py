@@ -38,9 +38,8 @@ WPB_K2_DEFAULT = 32
 
 
 # Read once: the op sits on the hot path of every layer call.
-# SPEAR_BTP_PATH=mfma sends the op through the matrix-core kernels (the reference's formulation: decay matrices
-# rounded to 16 bits and multiplied on the matrix units) instead of the default fp32 recurrences, forward and
-# backward.
+# SPEAR_BTP_PATH=mfma sends the op through the matrix-core kernels (the reference's formulation: a decay matrix
+# per block, multiplied on the matrix units) instead of the default fp32 recurrences, forward and backward.
 _PATH_MFMA = os.environ.get("SPEAR_BTP_PATH", "") == "mfma"
 _FORWARD_FLAGS = (_btp.FLAG_WRITE_CHECKPOINT if os.environ.get("SPEAR_BTP_WRITE_CHECKPOINT", "0") == "1" else 0) | (
     _btp.FLAG_PATH_MFMA if _PATH_MFMA else 0

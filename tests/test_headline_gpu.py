@@ -99,11 +99,11 @@ def test_full_size_properties(name):
         rdx, rdA = orc.backward(a_, x_, g_)
         assert_close(f64(dx[b : b + 1, h : h + 1]), rdx, BF16_ATOL, BF16_RTOL, f"dx[{b},{h}]")
         assert_close(f64(dA[b : b + 1, h : h + 1]), rdA, F32_ATOL, F32_RTOL, f"dA[{b},{h}]")
-        # decay operands rounded to 16 bits: 2 * 2^-9 of the sum of the terms' magnitudes (the oracle on |x|, |dy|)
+        # decay operands in two 16-bit pieces: 2^-15 of the sum of the terms' magnitudes (the oracle on |x|, |dy|)
         assert_close(f64(dxm[b : b + 1, h : h + 1]), rdx, BF16_ATOL, BF16_RTOL, f"dx mfma[{b},{h}]")
         magnitude = orc.backward(a_, np.abs(x_), np.abs(g_))[1]
         err = np.abs(f64(dAm[b : b + 1, h : h + 1]) - rdA)
-        assert (err <= 1e-3 + 2.0 ** -8 * magnitude).all(), f"dA mfma[{b},{h}]: {err.max():.3e}"
+        assert (err <= 1e-4 + 2.0 ** -15 * magnitude).all(), f"dA mfma[{b},{h}]: {err.max():.3e}"
 
 
 def _free_gib():

@@ -58,7 +58,8 @@ def test_the_op_runs_on_the_matrix_core_kernels_on_request(monkeypatch):
     assert_close(f64(y), ref, BF16_ATOL, BF16_RTOL, "y")
     assert_close(f64(xx.grad), rdx, BF16_ATOL, BF16_RTOL, "dx")
     magnitude = orc.backward(f64(coeff), np.abs(f64(x)), np.abs(f64(dy)))[1]
-    assert (np.abs(f64(c.grad) - rdA) <= 1e-3 + 2.0 ** -7 * magnitude + 2.0 ** -8 * np.abs(rdA)).all()
+    # (c.grad is rounded to the bf16 leaf dtype by autograd: 2^-8 of its own value)
+    assert (np.abs(f64(c.grad) - rdA) <= 1e-3 + 2.0 ** -14 * magnitude + 2.0 ** -8 * np.abs(rdA)).all()
     # these are the matrix-core kernels' values, not the default kernels': with the decay matrix rounded to 16
     # bits the fp32 output differs from the fp32 recurrence somewhere
     y32_mfma = btp(coeff.to(DEV), x.to(DEV))
@@ -100,8 +101,21 @@ def test_raw_custom_ops_mutate_in_place():
     assert_close(f64(dA), rdA, F32_ATOL, F32_RTOL, "dA")
 
 
+@pytest.fixture(params=["recurrence", "mfma"])
+def kernel_path(request, monkeypatch):
+    """The reference's numerics cases run on both kernel families: the default fp32 recurrences and the
+    matrix-core kernels that SPEAR_BTP_PATH=mfma selects (set on the op module here)."""
+    from spear_amd import _btp
+    from spear_amd.ops.btp import interface
+
+    if request.param == "mfma":
+        monkeypatch.setattr(interface, "_PATH_MFMA", True)
+        monkeypatch.setattr(interface, "_FORWARD_FLAGS", _btp.FLAG_PATH_MFMA)
+    return request.param
+
+
 @pytest.mark.parametrize("B,H,L,stress,seed", [(2, 8, 512, 1.0, 123), (1, 1, 64, 3.0, 321), (2, 4, 256, 2.0, 321), (4, 8, 512, 3.5, 321), (4, 16, 1024, 4.0, 321)])
-def test_reference_forward_cases(B, H, L, stress, seed):
+def test_reference_forward_cases(B, H, L, stress, seed, kernel_path):
     from spear_amd.ops.btp.runners import run_kernel_forward, run_reference, run_reference_logbtp, sample_inputs
     from spear_amd.testing.numerics import compute_error_metrics
 
@@ -112,11 +126,16 @@ def test_reference_forward_cases(B, H, L, stress, seed):
 
 
 @pytest.mark.parametrize("B,H,L,stress,seed", [(2, 8, 512, 1.0, 456), (2, 8, 256, 2.5, 789), (2, 8, 512, 3.0, 789), (4, 8, 512, 3.5, 789), (4, 8, 8192, 4.0, 789)])
-def test_reference_backward_cases(B, H, L, stress, seed):
+def test_reference_backward_cases(B, H, L, stress, seed, kernel_path):
     from spear_amd.ops.btp.runners import compare_backward_gradients, sample_inputs
 
     coeff, x = sample_inputs(B, H, L, seed=seed, stress_scale=stress, device=DEV)
-    for name, m in compare_backward_gradients(coeff, x).items():
+    # The matrix-core backward takes dy in 16 bits (an fp32 dy is rounded on load, as the reference packs dC), so it
+    # runs the op with a bf16 output, whose dy arrives in bf16 exactly; with the fp32 default the rounding of dy alone
+    # puts mean_rel of the coefficient gradient (dominated by elements whose reference is next to zero) at 1.7e2
+    # against the table's 1.5e2 in the first case.
+    out_dtype = torch.bfloat16 if kernel_path == "mfma" else torch.float32
+    for name, m in compare_backward_gradients(coeff, x, output_dtype=out_dtype).items():
         _within(m, BACKWARD_LIMITS, f"grad_{name} dims=({B},{H},{L})")
 
 
