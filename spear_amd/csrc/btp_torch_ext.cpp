@@ -165,6 +165,47 @@ void backward_log(const at::Tensor& gate, const at::Tensor& x, const at::Tensor&
   if (rc != 0) raise_native(rc);
 }
 
+// The autograd node of btp(), compiled: forward allocates y (and the checkpoint, a zero-element placeholder
+// unless the store is on), backward allocates dx and dA, both call the functions above. It does what
+// _BTPFunction of the reference does (spear/ops/btp/interface.py:126-161) without the Python frames of
+// torch.autograd.Function and of the custom-op dispatch, which at small batches cost several times the
+// kernels' time. The Python side uses it for plain eager tensors only; under torch.compile and dispatch modes
+// the Python node over the traceable custom ops runs instead.
+struct BtpNode : public torch::autograd::Function<BtpNode> {
+  static at::Tensor forward(torch::autograd::AutogradContext* ctx, const at::Tensor& coeff, const at::Tensor& x, int64_t k,
+                            int64_t wpb, bool y_f32, int64_t forward_flags, int64_t backward_flags) {
+    TORCH_CHECK(x.dim() == 4, "x must be [B, H, 16, L].");
+    at::Tensor y = at::empty(x.sizes(), x.options().dtype(y_f32 ? at::kFloat : x.scalar_type()));
+    at::Tensor checkpoint =
+        (forward_flags & SPEAR_BTP_WRITE_CHECKPOINT)
+            ? at::empty({x.size(0), x.size(1), x.size(3) / 16, 16}, x.options().dtype(at::kFloat))
+            : at::empty({0}, x.options().dtype(at::kFloat));
+    ::forward(coeff, x, y, checkpoint, k, wpb, forward_flags);
+    ctx->save_for_backward({coeff, x, checkpoint});
+    ctx->saved_data["k"] = k;
+    ctx->saved_data["wpb"] = wpb;
+    ctx->saved_data["flags"] = backward_flags;
+    return y;
+  }
+
+  static torch::autograd::variable_list backward(torch::autograd::AutogradContext* ctx,
+                                                 torch::autograd::variable_list grad_outputs) {
+    const auto saved = ctx->get_saved_variables();
+    const at::Tensor &coeff = saved[0], &x = saved[1], &checkpoint = saved[2];
+    const at::Tensor dy = grad_outputs[0].contiguous();
+    at::Tensor dx = at::empty(x.sizes(), x.options());
+    at::Tensor dA = at::empty(coeff.sizes(), coeff.options().dtype(at::kFloat));
+    ::backward(coeff, x, dy, checkpoint, dx, dA, ctx->saved_data["k"].toInt(), ctx->saved_data["wpb"].toInt(),
+               ctx->saved_data["flags"].toInt());
+    return {dA, dx, at::Tensor(), at::Tensor(), at::Tensor(), at::Tensor(), at::Tensor()};
+  }
+};
+
+at::Tensor btp_autograd(const at::Tensor& coeff, const at::Tensor& x, int64_t k, int64_t wpb, bool y_f32,
+                        int64_t forward_flags, int64_t backward_flags) {
+  return BtpNode::apply(coeff, x, k, wpb, y_f32, forward_flags, backward_flags);
+}
+
 struct MixShape {
   int64_t B, L, F, Fkv;
 };
@@ -276,6 +317,9 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         py::arg("flags") = (int64_t)SPEAR_BTP_WRITE_CHECKPOINT, "BTP Forward (HIP, gfx950)");
   m.def("backward", &backward, py::arg("coeff"), py::arg("x"), py::arg("dy"), py::arg("checkpoint"), py::arg("dx"),
         py::arg("dA"), py::arg("k"), py::arg("wpb"), py::arg("flags") = (int64_t)0, "BTP Backward (HIP, gfx950)");
+  m.def("btp_autograd", &btp_autograd, py::arg("coeff"), py::arg("x"), py::arg("k"), py::arg("wpb"), py::arg("y_f32"),
+        py::arg("forward_flags"), py::arg("backward_flags"),
+        "y = btp(coeff, x) with its autograd node (contiguous plain tensors; gradients: dA float32, dx in x's dtype)");
   m.def("forward_log", &forward_log, py::arg("gate"), py::arg("x"), py::arg("y"), py::arg("k"));
   m.def("backward_log", &backward_log, py::arg("gate"), py::arg("x"), py::arg("dy"), py::arg("dx"), py::arg("dgate"), py::arg("k"));
   m.def("mix_forward", &mix_forward, py::arg("a_logit"), py::arg("b_logit"), py::arg("c"), py::arg("v"), py::arg("out"),

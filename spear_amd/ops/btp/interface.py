@@ -165,6 +165,18 @@ class _BTPFunction(torch.autograd.Function):
         return dA, dx, None, None, None
 
 
+def _plain_eager(*tensors: torch.Tensor) -> bool:
+    """True where nothing needs to see the custom ops: ordinary tensors, no torch.compile trace, no dispatch or
+    function mode, no functorch transform. Only then may the compiled autograd node stand in for _BTPFunction."""
+    return (
+        all(type(t) is torch.Tensor or type(t) is torch.nn.Parameter for t in tensors)
+        and not torch.compiler.is_compiling()
+        and torch._C._len_torch_dispatch_stack() == 0
+        and torch._C._len_torch_function_stack() == 0
+        and torch._C._functorch.peek_interpreter_stack() is None
+    )
+
+
 def btp(
     coeff: torch.Tensor,
     x: torch.Tensor,
@@ -195,6 +207,15 @@ def btp(
         y = torch.empty_like(x, dtype=out_dtype)
         torch.ops.spear_btp.forward(coeff, x, y, _no_checkpoint(x), int(k), int(wpb_val))
         return y
+    if _plain_eager(coeff, x):
+        # the same node, compiled (spear_amd/csrc/btp_torch_ext.cpp): no Python frames between autograd and the kernels
+        assert x.dim() == 4 and x.shape[2] == DH, f"Channel dimension must be {DH}"
+        assert x.shape[3] % BLK == 0, f"Length L must be multiple of {BLK}"
+        assert wpb_val in SUPPORTED_WPB, f"WPB must be one of {SUPPORTED_WPB}"
+        return _btp.load_extension().btp_autograd(
+            coeff, x, int(k), int(wpb_val), out_dtype == torch.float32, _FORWARD_FLAGS,
+            _btp.FLAG_PATH_MFMA if _PATH_MFMA else 0,
+        )
     return _BTPFunction.apply(coeff, x, k, out_dtype, wpb_val)
 
 

@@ -47,7 +47,7 @@ def test_the_compiled_binding_is_what_spear_btp_names():
 
     assert ext is _btp.load_extension()
     assert ext.abi_version() == _btp._ABI_VERSION == _btp.load_library().spear_btp_abi_version()
-    for name in ("forward", "backward", "forward_log", "backward_log", "mix_forward", "mix_backward"):
+    for name in ("forward", "backward", "btp_autograd", "forward_log", "backward_log", "mix_forward", "mix_backward"):
         assert callable(getattr(ext, name))
     # the reference's positional signatures (csrc/btp/_bindings.cu:76-77, 152-153)
     assert ext.forward.__doc__.startswith("forward(coeff: torch.Tensor, x: torch.Tensor, y: torch.Tensor, checkpoint: torch.Tensor, k:")

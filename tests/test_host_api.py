@@ -341,6 +341,36 @@ def test_the_kernel_path_switch_is_read_from_the_environment():
         assert out.stdout.strip().splitlines()[-1] == want, (value, out.stdout)
 
 
+def test_the_compiled_autograd_node_is_for_plain_eager_tensors_only():
+    """btp() hands a call to the node compiled into the binding only when nothing has to see the custom ops:
+    tensor subclasses, dispatch / function modes and functorch transforms get the Python node."""
+    from torch._subclasses.fake_tensor import FakeTensorMode
+    from torch.utils._python_dispatch import TorchDispatchMode
+
+    from spear_amd.ops.btp.interface import _plain_eager
+
+    t = torch.ones(2, 2)
+    assert _plain_eager(t, t)
+    assert _plain_eager(t, torch.nn.Parameter(t))
+    with FakeTensorMode() as mode:
+        assert not _plain_eager(t, t)
+        assert not _plain_eager(mode.from_tensor(t))
+    assert not _plain_eager(mode.from_tensor(t))
+
+    class Passthrough(TorchDispatchMode):
+        def __torch_dispatch__(self, func, types, args=(), kwargs=None):
+            return func(*args, **(kwargs or {}))
+
+    with Passthrough():
+        assert not _plain_eager(t)
+    with torch.device("cpu"):  # a function mode
+        assert not _plain_eager(t)
+    seen = []
+    torch.func.vmap(lambda row: seen.append(_plain_eager(row)) or row)(t)
+    assert seen == [False]
+    assert _plain_eager(t)
+
+
 def test_streaming_module_surface_and_state_dataclass():
     from spear_amd.nn.phalanx import inference as inf
 

@@ -40,6 +40,48 @@ def test_autograd_through_btp_matches_oracle():
     assert_close(f64(c.grad), rdA, BF16_ATOL, BF16_RTOL, "dA (rounded to the bf16 leaf dtype by autograd)")
 
 
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+def test_eager_calls_run_the_compiled_autograd_node_with_the_results_of_the_python_node(out_dtype):
+    """A plain eager call goes through the node compiled into the binding; torch.compile, dispatch modes and tensor
+    subclasses get the Python node over the custom ops. Same kernels either way: identical bits."""
+    from spear_amd import btp
+    from spear_amd.ops.btp import interface
+
+    coeff, x, dy = make_inputs(3, 4, 272, seed=46)
+    leaves = [(coeff.to(DEV).requires_grad_(True), x.to(DEV).requires_grad_(True)) for _ in range(2)]
+    g = dy.to(DEV).to(out_dtype)
+    y_node = btp(*leaves[0], output_dtype=out_dtype)
+    assert "BtpNode" in y_node.grad_fn.name()
+    y_py = interface._BTPFunction.apply(*leaves[1], 2, out_dtype, 32)
+    assert "_BTPFunction" in y_py.grad_fn.name()
+    assert y_node.dtype == y_py.dtype == out_dtype and torch.equal(y_node, y_py)
+    # an upstream gradient that is not contiguous, as a transpose after the op produces
+    g_view = g.transpose(2, 3).contiguous().transpose(2, 3)
+    assert not g_view.is_contiguous()
+    y_node.backward(g_view)
+    y_py.backward(g_view)
+    for node_leaf, py_leaf in zip(*leaves):
+        assert node_leaf.grad.dtype == py_leaf.grad.dtype == torch.bfloat16
+        assert torch.equal(node_leaf.grad, py_leaf.grad)
+    rdx, _ = orc.backward(f64(coeff), f64(x), f64(g.float().cpu() if out_dtype == torch.float32 else dy))
+    assert_close(f64(leaves[0][1].grad), rdx, BF16_ATOL, BF16_RTOL, "dx")
+    # only one of the two inputs needs a gradient; the other's slot stays empty
+    c_only = coeff.to(DEV).requires_grad_(True)
+    x_plain = x.to(DEV)
+    btp(c_only, x_plain, output_dtype=out_dtype).backward(g)
+    assert torch.equal(c_only.grad, leaves[0][0].grad) and x_plain.grad is None
+    # a dispatch mode in force: the Python node
+    from torch.utils._python_dispatch import TorchDispatchMode
+
+    class Passthrough(TorchDispatchMode):
+        def __torch_dispatch__(self, func, types, args=(), kwargs=None):
+            return func(*args, **(kwargs or {}))
+
+    with Passthrough():
+        y_mode = btp(*leaves[1], output_dtype=out_dtype)
+    assert "_BTPFunction" in y_mode.grad_fn.name() and torch.equal(y_mode, y_node)
+
+
 def test_the_op_runs_on_the_matrix_core_kernels_on_request(monkeypatch):
     """SPEAR_BTP_PATH=mfma (read when the module is imported; set on the module here) sends btp() through the
     matrix-core forward and backward."""
