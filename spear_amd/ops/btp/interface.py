@@ -10,6 +10,9 @@ Differences that do not change results:
   * the compiled binding (``spear_amd._btp_ext``, the counterpart of ``spear._btp``) is imported on
     first use, so importing this module works before anything is built (the reference imports its
     extension unconditionally, interface.py:16); a call without it raises, there is no fallback;
+  * a plain eager call (ordinary tensors, no trace, mode or transform in force) runs the same autograd node
+    compiled into the binding (``btp_autograd``) instead of ``_BTPFunction``: same kernels, same results,
+    less host time per call;
   * ``dA`` is allocated uninitialised, because the kernel writes every element
     (the reference zero-fills it, interface.py:158);
   * the carry checkpoint is not stored by default, because this backward recomputes the carries:
