@@ -564,10 +564,10 @@ __global__ __launch_bounds__(64 * kWaves) void phalanx_mix_bwd_kernel(
 // ==========================================================================================
 // Backward of the fused mixing stage, tile form (SPEAR_MIX_TILE_SPLIT; what a call without a split flag runs
 // unless it asks for column sums): the same mathematics with a different work split. Measured against the walking
-// kernel above at B=1024 L=128 H=32 it takes 181-184 us against 185-196 us, at B=16 L=8192 H=64 it is 1 % slower, at
-// B=64 L=2048 H=128 5 % faster. One
+// kernel above at B=1024 L=128 H=32 it takes 166-167 us against 185-196 us, at B=16 L=8192 H=64 342 against 367 us,
+// at B=64 L=2048 H=128 705 against 757 us. One
 // wavefront owns ONE 16-step block of 128 features and runs no loop: every load is issued at the start, every
-// store at the end, and a workgroup (8 wavefronts = octs_w head groups x nb_w consecutive blocks of one batch
+// store at the end, and a workgroup (4 wavefronts = octs_w head groups x nb_w consecutive blocks of one batch
 // row) lives for a few microseconds. Copy loops with this kernel's traffic show why: wavefronts that walk
 // through time with two register sets reach 0.65 of the HBM peak whatever the chunking, short-lived tiles
 // 0.71-0.74 (reads and writes do not overlap on the memory bus, so what counts is how quickly a wavefront
@@ -588,8 +588,11 @@ __global__ __launch_bounds__(64 * kWaves) void phalanx_mix_bwd_kernel(
 //   dA_r = sum over the head's channels of dX_r h_{r-1}  -  (prod_{j != r} a_j) sum over channels of dC c_in
 // (the second term takes out the two-hop path c_in -> dC that h carries but the operator does not have).
 // ==========================================================================================
+// Wavefronts per workgroup and per SIMD. 4 and 3 (168 registers: nothing spills, 12 wavefronts per CU) beat 8 and 4
+// (128 registers, three or four spilled values per lane that show up as 2.5 % more HBM writes, 16 wavefronts per
+// CU) by 1 % at B=1024 L=128 H=32, 3 % at B=16 L=8192 H=64 and 5 % at B=64 L=2048 H=128.
 #ifndef SPEAR_FUSED_TILE_WAVES
-#define SPEAR_FUSED_TILE_WAVES 8
+#define SPEAR_FUSED_TILE_WAVES 4
 #endif
 constexpr int kTileWaves = SPEAR_FUSED_TILE_WAVES;
 
@@ -607,8 +610,11 @@ __device__ __forceinline__ float product_of_the_others(float a) {
   return dpp_or_one<0x111>(p) * dpp_or_one<0x101>(q);
 }
 
-#ifndef SPEAR_FUSED_TILE_WAVES_PER_EU  // 4 waves per SIMD (two workgroups per CU) need <= 128 VGPRs
-#define SPEAR_FUSED_TILE_WAVES_PER_EU 4
+#ifndef SPEAR_FUSED_TILE_XCD_GROUP  // neighbouring workgroups per XCD; 0: launch order (round-robin)
+#define SPEAR_FUSED_TILE_XCD_GROUP 128
+#endif
+#ifndef SPEAR_FUSED_TILE_WAVES_PER_EU
+#define SPEAR_FUSED_TILE_WAVES_PER_EU 3
 #endif
 // kF32: check mode, the four gradients leave as fp32 (the kernel's own values, not rounded to 16 bits).
 template <class E, bool kQkv, bool kF32>
@@ -625,7 +631,18 @@ void phalanx_mix_bwd_tile_kernel(
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   // workgroup -> (batch row, time tile, group of octs_w head groups); head groups fastest, so that workgroups
   // next to each other in launch order read neighbouring features of the same time steps
-  const unsigned wg = blockIdx.x;
+  // Launch order deals workgroups round-robin to the 8 XCDs, each with its own L2. An XCD gets runs of
+  // SPEAR_FUSED_TILE_XCD_GROUP neighbouring workgroups instead (windows of 8 runs sweep the tensors front to back):
+  // the workgroup that owns an edge block and the neighbour that reads it as its halo then share an L2 close in
+  // time. Against plain round-robin (0), runs of 128 four-wavefront workgroups: 184 -> 166-167 us at B=1024 L=128
+  // H=32, 371 -> 344 us at B=16 L=8192 H=64, 733 -> 718 us at B=64 L=2048 H=128 (all three as 1 head group x 4
+  // blocks); runs of 64 gain a little less, runs of 256 lose most of it again. The tail of the grid that does not fill a window keeps the launch order.
+  unsigned wg = blockIdx.x;
+  if constexpr (SPEAR_FUSED_TILE_XCD_GROUP > 0) {
+    constexpr unsigned kWin = 8u * SPEAR_FUSED_TILE_XCD_GROUP;
+    const unsigned win = wg / kWin, in = wg - win * kWin;
+    if ((win + 1) * kWin <= gridDim.x) wg = win * kWin + (in & 7u) * SPEAR_FUSED_TILE_XCD_GROUP + (in >> 3);
+  }
   const int og = (int)(wg % (unsigned)oct_groups);
   const unsigned tt = wg / (unsigned)oct_groups;
   const int tile = (int)(tt % (unsigned)tiles);
@@ -683,7 +700,7 @@ void phalanx_mix_bwd_tile_kernel(
   };
   // Wavefronts at a workgroup edge read the block beyond the edge first and their own b, v only once those 32
   // registers are free again (b and v are not needed before the local forward recurrence); the other
-  // wavefronts issue everything at once. That keeps the kernel within 128 registers = two workgroups per CU.
+  // wavefronts issue everything at once (with every load up front the kernel is no faster: 168 against 166 us).
   const bool halo = halo_prev || halo_next;
   auto load_bv = [&]() {
 #pragma unroll
@@ -1118,7 +1135,9 @@ void launch_mix_bwd(const MixBwdArgs& p, const MixPlan& m, hipStream_t s) {
 template <class E, bool kQkv, bool kF32 = false>
 void launch_mix_bwd_tile(const MixBwdArgs& p, hipStream_t s) {
   const int octs = (p.H + 7) / 8, nb = p.L / kTile;
-  const int octs_w = octs % 2 == 0 ? 2 : 1;  // measured with copy loops: 2 head groups x 4 blocks moves the most
+  // 1 head group x 4 blocks (two of four wavefronts read a halo) or 2 x 2 (all four do, but a workgroup reads
+  // 512-byte runs): over 14 shapes the first is 1.5-3.5 % faster up to 64 heads, the second 0.5-1.5 % from 128 on
+  const int octs_w = (octs % 2 == 0 && p.H >= 128) ? 2 : 1;
   const int nb_w = kTileWaves / octs_w;
   const int oct_groups = octs / octs_w, tiles = (nb + nb_w - 1) / nb_w;
   const long wgs = (long)p.B * tiles * oct_groups;

@@ -70,7 +70,10 @@ SPLITS = pytest.mark.parametrize("tile_split", [False, True], ids=["walk", "tile
 
 @SPLITS
 @pytest.mark.parametrize("B,L,H", [(1, 16, 4), (2, 32, 4), (2, 48, 8), (1, 80, 12), (3, 128, 8), (2, 144, 16), (1, 512, 32), (1, 1040, 4), (1, 4096, 8), (2, 2064, 16),
-                                   (5, 64, 32), (2, 112, 24), (3, 272, 64)])
+                                   (5, 64, 32), (2, 112, 24), (3, 272, 64),
+                                   # grids beyond one window of the tile split's dealing of workgroups to XCDs (512
+                                   # workgroups), with a tail that keeps the launch order: 548 and 900 workgroups
+                                   (137, 128, 32), (100, 272, 24)])
 def test_fused_backward_matches_oracle(B, L, H, tile_split):
     a, b, c, v = make_mix_inputs(B, L, H, H, seed=2000 + L + H)
     dout = torch.randn(B, L, H * 16, generator=torch.Generator().manual_seed(L)).bfloat16()
