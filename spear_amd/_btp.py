@@ -344,13 +344,16 @@ def mix_forward(
     kv_heads: int,
     qkv_gate: bool = False,
     c_prev_tail: torch.Tensor | None = None,
+    tile_split: bool | None = None,
 ) -> None:
     """``out <- btp(sigmoid(a_logit), sigmoid(b_logit) * v) * c + v`` with every operand in the
     layer's ``[B, L, features]`` layout (see ``spear_phalanx_mix_forward`` in the C header).
     ``qkv_gate``: ``a_logit`` is an fp32 log-decay gate, ``b_logit`` is k, ``c`` is q:
     ``out <- c * btp(exp(a_logit), b_logit * v) + v`` (``SPEAR_MIX_QKV_GATE``). ``c_prev_tail``: fp32
     ``[B, heads, 16]`` that receives the terminal local state of every row's last block, the hand-over state
-    for decoding after this prompt (``spear_phalanx_mix_prefill``)."""
+    for decoding after this prompt (``spear_phalanx_mix_prefill``). ``tile_split``: True selects the kernel with one
+    wavefront per 16-step block (``SPEAR_MIX_TILE_SPLIT``; no ``c_prev_tail``), False the one whose wavefronts walk
+    through time (``SPEAR_MIX_WALK_SPLIT``), None leaves the choice to the library; the results are the same bits."""
     _check(all(t.is_cuda for t in (a_logit, b_logit, c, v, out)), "All tensors must be CUDA.")
     _check(v.dim() == 3, "v must be [B, L, heads * 16].")
     B, L, F = v.shape
@@ -381,7 +384,9 @@ def mix_forward(
         rc = lib.spear_phalanx_mix_prefill(
             a_logit.data_ptr(), b_logit.data_ptr(), c.data_ptr(), v.data_ptr(), out.data_ptr(), _ptr(c_prev_tail),
             B, L, heads, kv_heads, _tag(v.dtype),
-            (FLAG_MIX_QKV_GATE if qkv_gate else 0) | (FLAG_MIX_F32_RESULTS if f32 else 0), _stream_ptr(v.device),
+            (FLAG_MIX_QKV_GATE if qkv_gate else 0) | (FLAG_MIX_F32_RESULTS if f32 else 0)
+            | (0 if tile_split is None else FLAG_MIX_TILE_SPLIT if tile_split else FLAG_MIX_WALK_SPLIT),
+            _stream_ptr(v.device),
         )
     if rc != 0:
         _raise_native(lib, rc)

@@ -616,6 +616,26 @@ __device__ __forceinline__ float product_of_the_others(float a) {
 #ifndef SPEAR_FUSED_TILE_WAVES_PER_EU
 #define SPEAR_FUSED_TILE_WAVES_PER_EU 3
 #endif
+#ifndef SPEAR_FUSED_FWD_TILE_WIDE_FROM  // heads from which the forward tile workgroup is 2 head groups x 2 blocks
+#define SPEAR_FUSED_FWD_TILE_WIDE_FROM 128
+#endif
+// Which tile workgroup this is. Launch order deals workgroups round-robin to the 8 XCDs, each with its own L2. An
+// XCD gets runs of SPEAR_FUSED_TILE_XCD_GROUP neighbouring workgroups instead (windows of 8 runs sweep the tensors
+// front to back): the workgroup that owns an edge block and the neighbour that reads it as its halo then share an
+// L2 close in time. Backward, against plain round-robin (0), runs of 128 four-wavefront workgroups: 184 -> 166-167
+// us at B=1024 L=128 H=32, 371 -> 344 us at B=16 L=8192 H=64, 733 -> 718 us at B=64 L=2048 H=128 (all three as 1
+// head group x 4 blocks); runs of 64 gain a little less, runs of 256 lose most of it again. The tail of the grid
+// that does not fill a window keeps the launch order.
+__device__ __forceinline__ unsigned tile_workgroup() {
+  unsigned wg = blockIdx.x;
+  if constexpr (SPEAR_FUSED_TILE_XCD_GROUP > 0) {
+    constexpr unsigned kWin = 8u * SPEAR_FUSED_TILE_XCD_GROUP;
+    const unsigned win = wg / kWin, in = wg - win * kWin;
+    if ((win + 1) * kWin <= gridDim.x) wg = win * kWin + (in & 7u) * SPEAR_FUSED_TILE_XCD_GROUP + (in >> 3);
+  }
+  return wg;
+}
+
 // kF32: check mode, the four gradients leave as fp32 (the kernel's own values, not rounded to 16 bits).
 template <class E, bool kQkv, bool kF32>
 __global__ __launch_bounds__(64 * kTileWaves) __attribute__((amdgpu_waves_per_eu(SPEAR_FUSED_TILE_WAVES_PER_EU)))
@@ -631,18 +651,7 @@ void phalanx_mix_bwd_tile_kernel(
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   // workgroup -> (batch row, time tile, group of octs_w head groups); head groups fastest, so that workgroups
   // next to each other in launch order read neighbouring features of the same time steps
-  // Launch order deals workgroups round-robin to the 8 XCDs, each with its own L2. An XCD gets runs of
-  // SPEAR_FUSED_TILE_XCD_GROUP neighbouring workgroups instead (windows of 8 runs sweep the tensors front to back):
-  // the workgroup that owns an edge block and the neighbour that reads it as its halo then share an L2 close in
-  // time. Against plain round-robin (0), runs of 128 four-wavefront workgroups: 184 -> 166-167 us at B=1024 L=128
-  // H=32, 371 -> 344 us at B=16 L=8192 H=64, 733 -> 718 us at B=64 L=2048 H=128 (all three as 1 head group x 4
-  // blocks); runs of 64 gain a little less, runs of 256 lose most of it again. The tail of the grid that does not fill a window keeps the launch order.
-  unsigned wg = blockIdx.x;
-  if constexpr (SPEAR_FUSED_TILE_XCD_GROUP > 0) {
-    constexpr unsigned kWin = 8u * SPEAR_FUSED_TILE_XCD_GROUP;
-    const unsigned win = wg / kWin, in = wg - win * kWin;
-    if ((win + 1) * kWin <= gridDim.x) wg = win * kWin + (in & 7u) * SPEAR_FUSED_TILE_XCD_GROUP + (in >> 3);
-  }
+  const unsigned wg = tile_workgroup();
   const int og = (int)(wg % (unsigned)oct_groups);
   const unsigned tt = wg / (unsigned)oct_groups;
   const int tile = (int)(tt % (unsigned)tiles);
@@ -964,6 +973,164 @@ void phalanx_mix_bwd_tile_kernel(
 
 
 // ==========================================================================================
+// Forward of the fused mixing stage, tile form: the work split of the tile backward above (one wavefront per
+// 16-step block of 128 features, no loop, one workgroup barrier, workgroups dealt to the XCDs in runs of
+// neighbours) with the arithmetic of phalanx_mix_fwd_kernel, operation for operation, so both splits give the
+// same bits. A block needs one neighbour quantity, the terminal value of the zero-started recurrence over the block
+// before it: every wavefront computes its own block's and leaves it in LDS for the next wavefront; the
+// first block of a workgroup reads b and v of the block before the edge (cacheable loads: the neighbouring
+// workgroup streams the same lines on the same L2) and runs that recurrence itself.
+// Serves every call that does not ask for the streaming state of the row's end (prefill), which the walking
+// kernel hands over from its registers.
+// ==========================================================================================
+template <class E, bool kQkv, bool kF32>
+__global__ __launch_bounds__(64 * kTileWaves) __attribute__((amdgpu_waves_per_eu(SPEAR_FUSED_TILE_WAVES_PER_EU)))
+void phalanx_mix_fwd_tile_kernel(const uint16_t* __restrict__ a_logit, const uint16_t* __restrict__ b_logit,
+                                 const uint16_t* __restrict__ c_in, const uint16_t* __restrict__ v_in,
+                                 uint16_t* __restrict__ out, int L, int H, int kv_groups, int octs_w, int nb_w,
+                                 int tiles, int oct_groups) {
+  __shared__ __align__(16) float gate_tiles[kTileWaves][2][kHeadsPerWave * kGateRow];  // own block, block before the edge
+  __shared__ float2 carry_out[kTileWaves][64];  // terminal local state of the wavefront's block, per lane
+
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+  const unsigned wg = tile_workgroup();
+  const int og = (int)(wg % (unsigned)oct_groups);
+  const unsigned tt = wg / (unsigned)oct_groups;
+  const int tile = (int)(tt % (unsigned)tiles);
+  const long brow = tt / (unsigned)tiles;
+  const int o = wave % octs_w, bl = wave / octs_w;  // octs_w * nb_w == kTileWaves
+  const int ho = (og * octs_w + o) * kHeadsPerWave;
+  const int t0 = (tile * nb_w + bl) * kTile;
+  const bool valid = ho < H && t0 < L;  // wave-uniform; a wavefront without a block only joins the barrier
+
+  const int head_local = lane >> 3;
+  const bool real = ho + head_local < H;
+  const int head = real ? ho + head_local : H - 1;
+  const int d0 = (lane & 7) << 1;
+  const int F = H * kChan, Fkv = (H / kv_groups) * kChan;
+  const int stride = 2 * F, kv_stride = 2 * Fkv;
+  constexpr int kRsrcFlags = 0x00020000;
+  constexpr int kGateBytes = kQkv ? 4 : 2;
+  constexpr int kOutScale = kF32 ? 2 : 1;
+  const long big = brow * L * F, kvbig = brow * L * Fkv, small = brow * L * H;
+  auto rsrc = [&](const uint16_t* p, long off, int bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(p + off), 0, bytes, kRsrcFlags);
+  };
+  const __amdgpu_buffer_rsrc_t rb = rsrc(b_logit, kvbig, L * kv_stride), rc = rsrc(c_in, kvbig, L * kv_stride),
+                               rv = rsrc(v_in, big, L * stride),
+                               ra = rsrc(a_logit, small * (kGateBytes / 2), L * H * kGateBytes),
+                               ro = rsrc(out, big * kOutScale, L * stride * kOutScale);
+  const int f_lane = 2 * (head * kChan + d0);
+  const int kv_lane = 2 * ((head / kv_groups) * kChan + d0);
+  const int o_lane = real ? f_lane * kOutScale : 0x7ffffff0;  // lanes without a head store nowhere
+  const int gt = lane & 15, ghead = min(ho + 2 * (lane >> 4), H - 2);
+  const int a_lane = kGateBytes * (gt * H + ghead);
+  constexpr int kNt = 2;
+
+  const bool halo = valid && bl == 0 && t0 > 0;  // needs the terminal local state of block t0 - 16
+  const int th = t0 - kTile;
+
+  // ---- every global read, before anything waits
+  uint32_t b[16], c[16], v[16], hb[16], hv[16];
+  GateWords araw = {0u, 0u}, haraw = {0u, 0u};
+  auto load_gate = [&](int t) {
+    GateWords w;
+    w.lo = __builtin_amdgcn_raw_buffer_load_b32(ra, a_lane, t * H * kGateBytes, 0);
+    w.hi = kQkv ? __builtin_amdgcn_raw_buffer_load_b32(ra, a_lane + 4, t * H * kGateBytes, 0) : 0u;
+    return w;
+  };
+  if (valid) {
+    araw = load_gate(t0);
+    if (halo) {
+      haraw = load_gate(th);
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        hb[r] = __builtin_amdgcn_raw_buffer_load_b32(rb, kv_lane, (th + r) * kv_stride, 0);
+        hv[r] = __builtin_amdgcn_raw_buffer_load_b32(rv, f_lane, (th + r) * stride, 0);
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      b[r] = __builtin_amdgcn_raw_buffer_load_b32(rb, kv_lane, (t0 + r) * kv_stride, kNt);
+      v[r] = __builtin_amdgcn_raw_buffer_load_b32(rv, f_lane, (t0 + r) * stride, kNt);
+    }
+#pragma unroll
+    for (int r = 0; r < 16; ++r) c[r] = __builtin_amdgcn_raw_buffer_load_b32(rc, kv_lane, (t0 + r) * kv_stride, kNt);
+  }
+  __builtin_amdgcn_sched_barrier(0);
+
+  float* ta = gate_tiles[wave][0];
+  float* tn = gate_tiles[wave][1];
+  auto write_tile = [&](float* tile_, float x0, float x1) {
+    tile_[(2 * (lane >> 4)) * kGateRow + gt] = x0;
+    tile_[(2 * (lane >> 4) + 1) * kGateRow + gt] = x1;
+  };
+  auto read_decays = [&](const float* tile_, float (&a)[16]) {
+#pragma unroll
+    for (int c4 = 0; c4 < 4; ++c4) {
+      const float4 q = *reinterpret_cast<const float4*>(tile_ + head_local * kGateRow + 4 * c4);
+      a[4 * c4 + 0] = q.x; a[4 * c4 + 1] = q.y; a[4 * c4 + 2] = q.z; a[4 * c4 + 3] = q.w;
+    }
+  };
+
+  float a[16], x0[16], x1[16];
+  float cin0 = 0.0f, cin1 = 0.0f;
+  if (valid) {
+    const float2 a01 = decay_pair<E, kQkv>(araw);
+    write_tile(ta, a01.x, a01.y);
+    if (halo) {
+      const float2 n01 = decay_pair<E, kQkv>(haraw);
+      write_tile(tn, n01.x, n01.y);
+    }
+    wave_lds_handover();
+    if (halo) {  // the zero-started recurrence over the block before the edge
+      float an[16];
+      read_decays(tn, an);
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        cin0 = fmaf(an[r], cin0, input_gate<kQkv>(E::lo(hb[r])) * E::lo(hv[r]));
+        cin1 = fmaf(an[r], cin1, input_gate<kQkv>(E::hi(hb[r])) * E::hi(hv[r]));
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    read_decays(ta, a);
+    // gated inputs and the zero-started recurrence: its terminal value is the next block's carry
+    float l0 = 0.0f, l1 = 0.0f;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      x0[r] = input_gate<kQkv>(E::lo(b[r])) * E::lo(v[r]);
+      x1[r] = input_gate<kQkv>(E::hi(b[r])) * E::hi(v[r]);
+      l0 = fmaf(a[r], l0, x0[r]);
+      l1 = fmaf(a[r], l1, x1[r]);
+    }
+    carry_out[wave][lane] = make_float2(l0, l1);
+  }
+  __syncthreads();  // the kernel's only workgroup barrier; wavefronts without a block arrive here directly
+  if (!valid) return;
+
+  if (bl > 0) {  // the block before this one belongs to the wavefront octs_w places down
+    const float2 q = carry_out[wave - octs_w][lane];
+    cin0 = q.x;
+    cin1 = q.y;
+  }
+  // the carry-started recurrence and the output mix
+  float y0 = cin0, y1 = cin1;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    y0 = fmaf(a[r], y0, x0[r]);
+    y1 = fmaf(a[r], y1, x1[r]);
+    const float o0 = fmaf(y0, E::lo(c[r]), E::lo(v[r])), o1 = fmaf(y1, E::hi(c[r]), E::hi(v[r]));
+    if constexpr (kF32) {
+      const u32x2_t ow = {__float_as_uint(o0), __float_as_uint(o1)};
+      __builtin_amdgcn_raw_buffer_store_b64(ow, ro, o_lane, (t0 + r) * stride * 2, kNt);
+    } else {
+      __builtin_amdgcn_raw_buffer_store_b32(E::pack2(o0, o1), ro, o_lane, (t0 + r) * stride, kNt);
+    }
+  }
+}
+
+
+// ==========================================================================================
 // One decode token of the mixing stage in the layer's own layout: the projections' outputs for ONE time step,
 // [B, features], and the streaming state of every (batch row, head). It is step_jagged of the reference
 // (spear/nn/phalanx/inference.py:178-278) with the gates of the layer (spear/nn/phalanx/swr.py:196-221) applied
@@ -1079,9 +1246,51 @@ void launch_mix_fwd(const MixArgs& p, const MixPlan& m, hipStream_t s) {
                      p.c_prev_tail, p.L, p.H, p.kv_groups, m.chunk_blocks * kTile, m.chunks, total);
 }
 
+// Tile geometry shared by the tile kernels: head groups x consecutive blocks per workgroup, and the grid.
+struct TileGrid {
+  int octs_w, nb_w, oct_groups, tiles;
+  long wgs;
+};
+TileGrid tile_grid(long B, int H, int L, int octs_w) {
+  const int octs = (H + 7) / 8, nb = L / kTile;
+  TileGrid g;
+  g.octs_w = octs_w;
+  g.nb_w = kTileWaves / octs_w;
+  g.oct_groups = octs / octs_w;
+  g.tiles = (nb + g.nb_w - 1) / g.nb_w;
+  g.wgs = B * g.tiles * g.oct_groups;
+  return g;
+}
+
+template <class E, bool kQkv, bool kF32 = false>
+void launch_mix_fwd_tile(const MixArgs& p, hipStream_t s) {
+  const int octs = (p.H + 7) / 8;
+  const int octs_w = (octs % 2 == 0 && p.H >= SPEAR_FUSED_FWD_TILE_WIDE_FROM) ? 2 : 1;
+  const TileGrid g = tile_grid(p.B, p.H, p.L, octs_w);
+  hipLaunchKernelGGL((phalanx_mix_fwd_tile_kernel<E, kQkv, kF32>), dim3((unsigned)g.wgs), dim3(64 * kTileWaves), 0, s,
+                     static_cast<const uint16_t*>(p.a_logit), static_cast<const uint16_t*>(p.b_logit),
+                     static_cast<const uint16_t*>(p.c), static_cast<const uint16_t*>(p.v), static_cast<uint16_t*>(p.out),
+                     p.L, p.H, p.kv_groups, g.octs_w, g.nb_w, g.tiles, g.oct_groups);
+}
+
 }  // namespace
 
 hipError_t fused_mix_forward(const MixArgs& p, hipStream_t s) {
+  if (p.tile_split) {  // the caller has checked: no streaming state asked for, a grid that fits
+    auto by_form = [&](auto e, auto q) {
+      using E = decltype(e);
+      if (p.f32_out) launch_mix_fwd_tile<E, decltype(q)::value, true>(p, s);
+      else launch_mix_fwd_tile<E, decltype(q)::value>(p, s);
+    };
+    if (p.dtype == kBf16) {
+      if (p.qkv) by_form(Bf16{}, std::true_type{});
+      else by_form(Bf16{}, std::false_type{});
+    } else {
+      if (p.qkv) by_form(Fp16{}, std::true_type{});
+      else by_form(Fp16{}, std::false_type{});
+    }
+    return hipGetLastError();
+  }
   const MixPlan m = plan_mix(p.B, p.H, p.L);
   auto by_waves = [&](auto e, auto q) {
     using E = decltype(e);

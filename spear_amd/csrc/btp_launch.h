@@ -56,6 +56,7 @@ struct MixArgs {
   // null, or fp32 [B, H, 16]: receives the terminal local state of every row's last block (the c_prev of the
   // streaming state after this prompt)
   float* c_prev_tail = nullptr;
+  bool tile_split = false;  // one wavefront per 16-step block instead of wavefronts walking through time
 };
 hipError_t fused_mix_forward(const MixArgs& p, hipStream_t s);
 

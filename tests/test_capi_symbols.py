@@ -105,10 +105,15 @@ def test_host_side_validation_needs_no_gpu():
     # fused layer kernels: a batch row must fit one 32-bit buffer resource
     assert lib.spear_phalanx_mix_forward(p, p, p, p, p, 1, 1 << 20, 128, 128, 0, 0, None) == -1
     assert b"below 2 GiB" in lib.spear_btp_last_error()
-    # SPEAR_MIX_QKV_GATE (0x1), SPEAR_MIX_F32_RESULTS (0x2) and, backward only, SPEAR_MIX_TILE_SPLIT (0x4) and
-    # SPEAR_MIX_WALK_SPLIT (0x8), which exclude each other, are the flags of the fused entry points
-    assert lib.spear_phalanx_mix_forward(p, p, p, p, p, 1, 32, 4, 4, 0, 0x4, None) == -1
+    # SPEAR_MIX_QKV_GATE (0x1), SPEAR_MIX_F32_RESULTS (0x2), SPEAR_MIX_TILE_SPLIT (0x4) and SPEAR_MIX_WALK_SPLIT
+    # (0x8), which exclude each other, are the flags of the fused entry points
+    assert lib.spear_phalanx_mix_forward(p, p, p, p, p, 1, 32, 4, 4, 0, 0x10, None) == -1
     assert b"unknown flag" in lib.spear_btp_last_error()
+    assert lib.spear_phalanx_mix_forward(p, p, p, p, p, 1, 32, 4, 4, 0, 0xc, None) == -1
+    assert b"exclude each other" in lib.spear_btp_last_error()
+    lib.spear_phalanx_mix_prefill.restype = ctypes.c_int
+    assert lib.spear_phalanx_mix_prefill(p, p, p, p, p, p, 1, 32, 4, 4, 0, 0x4, None) == -1
+    assert b"does not hand over the streaming state" in lib.spear_btp_last_error()
     assert lib.spear_phalanx_mix_backward(p, p, p, p, p, p, p, p, p, 1, 32, 4, 4, 0, 0x10, None) == -1
     assert b"unknown flag" in lib.spear_btp_last_error()
     assert lib.spear_phalanx_mix_backward(p, p, p, p, p, p, p, p, p, 1, 32, 4, 4, 0, 0xc, None) == -1

@@ -128,7 +128,7 @@ def _mix_run(ins, H, Hkv, qkv, f32, tile_split=None):
     a, b, c, v, dout = (t.to(DEV) for t in ins)
     rt = torch.float32 if f32 else v.dtype
     out = torch.full(v.shape, float("nan"), device=DEV, dtype=rt)
-    _btp.mix_forward(a, b, c, v, out, H, Hkv, qkv_gate=qkv)
+    _btp.mix_forward(a, b, c, v, out, H, Hkv, qkv_gate=qkv, tile_split=tile_split)
     grads = [torch.full(t.shape, float("nan"), device=DEV, dtype=torch.float32 if (f32 or t.dtype == torch.float32) else t.dtype)
              for t in (a, b, c, v)]
     _btp.mix_backward(a, b, c, v, dout, *grads, H, Hkv, qkv_gate=qkv, tile_split=tile_split)

@@ -22,32 +22,47 @@ def make_mix_inputs(B, L, H, Hkv, seed, dtype=torch.bfloat16, scale=1.0):
     return a, b, c, v
 
 
-def run_mix(a, b, c, v, H, Hkv):
+def run_mix(a, b, c, v, H, Hkv, tile_split=None):
     from spear_amd import _btp
 
     out = torch.full(v.shape, float("nan"), device=DEV, dtype=v.dtype)
-    _btp.mix_forward(a.to(DEV), b.to(DEV), c.to(DEV), v.to(DEV), out, H, Hkv)
+    _btp.mix_forward(a.to(DEV), b.to(DEV), c.to(DEV), v.to(DEV), out, H, Hkv, tile_split=tile_split)
     torch.cuda.synchronize()
     return out.cpu()
 
 
+# every fused kernel comes in two work splits: wavefronts that walk through time (SPEAR_MIX_WALK_SPLIT) and one
+# wavefront per 16-step block (SPEAR_MIX_TILE_SPLIT, the library's own choice wherever it can serve the call); both
+# are held to the same oracle
+SPLITS = pytest.mark.parametrize("tile_split", [False, True], ids=["walk", "tile"])
+
+
+@SPLITS
 @pytest.mark.parametrize("B,L,H,Hkv", [
     (1, 16, 4, 4), (2, 32, 4, 4), (2, 48, 8, 8), (1, 80, 4, 2), (3, 128, 8, 2), (2, 144, 16, 4),
     (1, 512, 32, 32), (2, 272, 12, 3), (1, 1040, 4, 1), (1, 4096, 8, 8), (2, 2064, 16, 2),
+    (5, 64, 32, 8), (3, 272, 128, 16),
+    # grids beyond one window of the tile split's dealing of workgroups to XCDs (1024 workgroups), with a tail
+    # that keeps the launch order: 1096 and 1500 workgroups
+    (137, 128, 32, 32), (100, 272, 24, 8),
 ])
-def test_fused_forward_matches_oracle(B, L, H, Hkv):
+def test_fused_forward_matches_oracle(B, L, H, Hkv, tile_split):
     a, b, c, v = make_mix_inputs(B, L, H, Hkv, seed=1000 + L + H)
-    print(f"fused B={B} L={L} H={H} Hkv={Hkv}", flush=True)
-    out = run_mix(a, b, c, v, H, Hkv)
+    print(f"fused B={B} L={L} H={H} Hkv={Hkv} tile={tile_split}", flush=True)
+    out = run_mix(a, b, c, v, H, Hkv, tile_split)
     ref = orc.phalanx_mix_forward(f64(a), f64(b), f64(c), f64(v), H, Hkv)
     assert_close(f64(out), ref, BF16_ATOL, BF16_RTOL, "out")
+    if tile_split:  # the two splits run the same arithmetic in the same order
+        assert torch.equal(out, run_mix(a, b, c, v, H, Hkv, False)), "tile and walking forward differ"
+        assert torch.equal(out, run_mix(a, b, c, v, H, Hkv, None)), "the library's own choice differs"
 
 
-def test_fused_forward_fp16_and_steep_gates():
+@SPLITS
+def test_fused_forward_fp16_and_steep_gates(tile_split):
     a, b, c, v = make_mix_inputs(2, 96, 8, 4, seed=5, dtype=torch.float16, scale=4.0)
     a[0, :10, :] = -30.0  # decay ~ 1e-13: counts as zero
     a[1, 20:40, 3] = 30.0  # decay -> 1
-    out = run_mix(a, b, c, v, 8, 4)
+    out = run_mix(a, b, c, v, 8, 4, tile_split)
     ref = orc.phalanx_mix_forward(f64(a), f64(b), f64(c), f64(v), 8, 4)
     assert_close(f64(out), ref, 4e-3, 4e-3, "out fp16")
 
@@ -62,17 +77,11 @@ def run_mix_backward(a, b, c, v, dout, H, Hkv=None, tile_split=None):
     return [t.cpu() for t in outs]
 
 
-# the backward kernel comes in two work splits: wavefronts that walk through time (SPEAR_MIX_WALK_SPLIT) and one
-# wavefront per 16-step block (SPEAR_MIX_TILE_SPLIT, the library's own choice for calls without column sums); both
-# are held to the same oracle
-SPLITS = pytest.mark.parametrize("tile_split", [False, True], ids=["walk", "tile"])
-
-
 @SPLITS
 @pytest.mark.parametrize("B,L,H", [(1, 16, 4), (2, 32, 4), (2, 48, 8), (1, 80, 12), (3, 128, 8), (2, 144, 16), (1, 512, 32), (1, 1040, 4), (1, 4096, 8), (2, 2064, 16),
                                    (5, 64, 32), (2, 112, 24), (3, 272, 64),
-                                   # grids beyond one window of the tile split's dealing of workgroups to XCDs (512
-                                   # workgroups), with a tail that keeps the launch order: 548 and 900 workgroups
+                                   # grids beyond one window of the tile split's dealing of workgroups to XCDs (1024
+                                   # workgroups), with a tail that keeps the launch order: 1096 and 1500 workgroups
                                    (137, 128, 32), (100, 272, 24)])
 def test_fused_backward_matches_oracle(B, L, H, tile_split):
     a, b, c, v = make_mix_inputs(B, L, H, H, seed=2000 + L + H)
