@@ -122,8 +122,7 @@ int spear_phalanx_mix_forward(const void* a_logit, const void* b_logit, const vo
 
 /* Flags for spear_phalanx_mix_forward / _backward / _backward_ex: which work split runs. TILE: one wavefront
  * per 16-step block, the carries handed between neighbouring blocks through LDS; the backward then has no
- * column sums and the forward no streaming state (spear_phalanx_mix_prefill). WALK: wavefronts that walk
- * through time (every option). Forward: the same bits from both. Backward: the same results up to fp32
+ * column sums. WALK: wavefronts that walk through time (every option). Forward: the same bits from both. Backward: the same results up to fp32
  * rounding. With neither flag the tile split serves every call it can (backward: 166-167 us against 185-196 us
  * at B=1024 L=128 H=32, 342 against 367 us at B=16 L=8192 H=64, 705 against 757 us at B=64 L=2048 H=128) and
  * the walking kernels the rest; SPEAR_BTP_FUSED_FWD / SPEAR_BTP_FUSED_BWD = walk or tile in the environment

@@ -352,7 +352,7 @@ def mix_forward(
     ``out <- c * btp(exp(a_logit), b_logit * v) + v`` (``SPEAR_MIX_QKV_GATE``). ``c_prev_tail``: fp32
     ``[B, heads, 16]`` that receives the terminal local state of every row's last block, the hand-over state
     for decoding after this prompt (``spear_phalanx_mix_prefill``). ``tile_split``: True selects the kernel with one
-    wavefront per 16-step block (``SPEAR_MIX_TILE_SPLIT``; no ``c_prev_tail``), False the one whose wavefronts walk
+    wavefront per 16-step block (``SPEAR_MIX_TILE_SPLIT``), False the one whose wavefronts walk
     through time (``SPEAR_MIX_WALK_SPLIT``), None leaves the choice to the library; the results are the same bits."""
     _check(all(t.is_cuda for t in (a_logit, b_logit, c, v, out)), "All tensors must be CUDA.")
     _check(v.dim() == 3, "v must be [B, L, heads * 16].")

@@ -150,8 +150,8 @@ int spear_phalanx_mix_prefill(const void* a_logit, const void* b_logit, const vo
   const unsigned known = SPEAR_MIX_QKV_GATE | SPEAR_MIX_F32_RESULTS | SPEAR_MIX_TILE_SPLIT | SPEAR_MIX_WALK_SPLIT;
   if (flags & ~known) return fail(SPEAR_BTP_EINVAL, "%s: unknown flag bits 0x%x", who, flags & ~known);
   const bool f32 = (flags & SPEAR_MIX_F32_RESULTS) != 0;
-  // the work split is a flag, or the process-wide default: the tile split wherever it can serve the call (it does
-  // not hand over the streaming state), unless SPEAR_BTP_FUSED_FWD=walk is set (read once)
+  // the work split is a flag, or the process-wide default: the tile split, unless SPEAR_BTP_FUSED_FWD=walk is set
+  // (read once)
   static const bool tile_default = [] {
     const char* e = getenv("SPEAR_BTP_FUSED_FWD");
     return e == nullptr || e[0] != 'w';
@@ -159,9 +159,7 @@ int spear_phalanx_mix_prefill(const void* a_logit, const void* b_logit, const vo
   const bool tile_asked = (flags & SPEAR_MIX_TILE_SPLIT) != 0, walk_asked = (flags & SPEAR_MIX_WALK_SPLIT) != 0;
   if (tile_asked && walk_asked)
     return fail(SPEAR_BTP_EINVAL, "%s: SPEAR_MIX_TILE_SPLIT and SPEAR_MIX_WALK_SPLIT exclude each other", who);
-  if (tile_asked && c_prev_tail)
-    return fail(SPEAR_BTP_EINVAL, "%s: SPEAR_MIX_TILE_SPLIT does not hand over the streaming state", who);
-  const bool tile = (tile_asked || (tile_default && !walk_asked && !c_prev_tail)) &&
+  const bool tile = (tile_asked || (tile_default && !walk_asked)) &&
                     (long long)B * ((L / 16 + 3) / 4) * ((H + 7) / 8) < (1ll << 31);
   if ((long long)B * L * H * 16ll >= (1ll << 40)) return fail(SPEAR_BTP_EINVAL, "%s: tensor too large", who);
   if ((long long)L * H * (f32 ? 64ll : 32ll) >= (1ll << 31))  // a batch row is addressed through one 32-bit buffer resource

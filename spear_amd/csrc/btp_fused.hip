@@ -616,9 +616,6 @@ __device__ __forceinline__ float product_of_the_others(float a) {
 #ifndef SPEAR_FUSED_TILE_WAVES_PER_EU
 #define SPEAR_FUSED_TILE_WAVES_PER_EU 3
 #endif
-#ifndef SPEAR_FUSED_FWD_TILE_WIDE_FROM  // heads from which the forward tile workgroup is 2 head groups x 2 blocks
-#define SPEAR_FUSED_FWD_TILE_WIDE_FROM 128
-#endif
 // Which tile workgroup this is. Launch order deals workgroups round-robin to the 8 XCDs, each with its own L2. An
 // XCD gets runs of SPEAR_FUSED_TILE_XCD_GROUP neighbouring workgroups instead (windows of 8 runs sweep the tensors
 // front to back): the workgroup that owns an edge block and the neighbour that reads it as its halo then share an
@@ -626,12 +623,13 @@ __device__ __forceinline__ float product_of_the_others(float a) {
 // us at B=1024 L=128 H=32, 371 -> 344 us at B=16 L=8192 H=64, 733 -> 718 us at B=64 L=2048 H=128 (all three as 1
 // head group x 4 blocks); runs of 64 gain a little less, runs of 256 lose most of it again. The tail of the grid
 // that does not fill a window keeps the launch order.
+template <int kRun = SPEAR_FUSED_TILE_XCD_GROUP>
 __device__ __forceinline__ unsigned tile_workgroup() {
   unsigned wg = blockIdx.x;
-  if constexpr (SPEAR_FUSED_TILE_XCD_GROUP > 0) {
-    constexpr unsigned kWin = 8u * SPEAR_FUSED_TILE_XCD_GROUP;
+  if constexpr (kRun > 0) {
+    constexpr unsigned kWin = 8u * kRun;
     const unsigned win = wg / kWin, in = wg - win * kWin;
-    if ((win + 1) * kWin <= gridDim.x) wg = win * kWin + (in & 7u) * SPEAR_FUSED_TILE_XCD_GROUP + (in >> 3);
+    if ((win + 1) * kWin <= gridDim.x) wg = win * kWin + (in & 7u) * kRun + (in >> 3);
   }
   return wg;
 }
@@ -980,25 +978,29 @@ void phalanx_mix_bwd_tile_kernel(
 // before it: every wavefront computes its own block's and leaves it in LDS for the next wavefront; the
 // first block of a workgroup reads b and v of the block before the edge (cacheable loads: the neighbouring
 // workgroup streams the same lines on the same L2) and runs that recurrence itself.
-// Serves every call that does not ask for the streaming state of the row's end (prefill), which the walking
-// kernel hands over from its registers.
+// The wavefront of a row's last block also stores the streaming state for decoding after this prompt, when asked.
+// kW wavefronts per workgroup, one head group x kW consecutive blocks (2 head groups x kW / 2 blocks measured
+// slower at every shape): 4 or 8. Microseconds for 4 / 8 / the walking kernel, B L H:
+//   1024 128 32: 87.0 / 90.8 / 96.2     256 512 32: 90.7 / 88.6 / 101.1    16 8192 32: 91.1 / 90.4 / 99.9
+//   512 128 64: 89.9 / 90.7 / 95.2      16 8192 64: 181.6 / 178.1 / 181.5  64 2048 128: 357.4 / 347.9 / 370.4
+//   256 128 128: 89.8 / 89.8 / 114.2    4096 128 8: 93.5 / 87.6 / 90.1     1024 128 48: 131.5 / 125.6 / 146.8
 // ==========================================================================================
-template <class E, bool kQkv, bool kF32>
-__global__ __launch_bounds__(64 * kTileWaves) __attribute__((amdgpu_waves_per_eu(SPEAR_FUSED_TILE_WAVES_PER_EU)))
+template <class E, int kW, bool kQkv, bool kF32>
+__global__ __launch_bounds__(64 * kW) __attribute__((amdgpu_waves_per_eu(SPEAR_FUSED_TILE_WAVES_PER_EU)))
 void phalanx_mix_fwd_tile_kernel(const uint16_t* __restrict__ a_logit, const uint16_t* __restrict__ b_logit,
                                  const uint16_t* __restrict__ c_in, const uint16_t* __restrict__ v_in,
-                                 uint16_t* __restrict__ out, int L, int H, int kv_groups, int octs_w, int nb_w,
-                                 int tiles, int oct_groups) {
-  __shared__ __align__(16) float gate_tiles[kTileWaves][2][kHeadsPerWave * kGateRow];  // own block, block before the edge
-  __shared__ float2 carry_out[kTileWaves][64];  // terminal local state of the wavefront's block, per lane
+                                 uint16_t* __restrict__ out, float* __restrict__ c_prev_tail, int L, int H,
+                                 int kv_groups, int octs_w, int nb_w, int tiles, int oct_groups) {
+  __shared__ __align__(16) float gate_tiles[kW][2][kHeadsPerWave * kGateRow];  // own block, block before the edge
+  __shared__ float2 carry_out[kW][64];  // terminal local state of the wavefront's block, per lane
 
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
-  const unsigned wg = tile_workgroup();
+  const unsigned wg = tile_workgroup<SPEAR_FUSED_TILE_XCD_GROUP * 4 / kW>();
   const int og = (int)(wg % (unsigned)oct_groups);
   const unsigned tt = wg / (unsigned)oct_groups;
   const int tile = (int)(tt % (unsigned)tiles);
   const long brow = tt / (unsigned)tiles;
-  const int o = wave % octs_w, bl = wave / octs_w;  // octs_w * nb_w == kTileWaves
+  const int o = wave % octs_w, bl = wave / octs_w;  // octs_w * nb_w == kW
   const int ho = (og * octs_w + o) * kHeadsPerWave;
   const int t0 = (tile * nb_w + bl) * kTile;
   const bool valid = ho < H && t0 < L;  // wave-uniform; a wavefront without a block only joins the barrier
@@ -1104,6 +1106,10 @@ void phalanx_mix_fwd_tile_kernel(const uint16_t* __restrict__ a_logit, const uin
       l1 = fmaf(a[r], l1, x1[r]);
     }
     carry_out[wave][lane] = make_float2(l0, l1);
+    // Hand-over for token-by-token decoding after this prompt: the terminal local state of the row's last block is
+    // what the next block's steps need as c_prev (the block-local state restarts at 0 and the gate product at 1).
+    if (c_prev_tail != nullptr && t0 + kTile == L && real)
+      *reinterpret_cast<float2*>(c_prev_tail + (brow * H + head) * kChan + d0) = make_float2(l0, l1);
   }
   __syncthreads();  // the kernel's only workgroup barrier; wavefronts without a block arrive here directly
   if (!valid) return;
@@ -1251,36 +1257,38 @@ struct TileGrid {
   int octs_w, nb_w, oct_groups, tiles;
   long wgs;
 };
-TileGrid tile_grid(long B, int H, int L, int octs_w) {
+TileGrid tile_grid(long B, int H, int L, int octs_w, int waves) {
   const int octs = (H + 7) / 8, nb = L / kTile;
   TileGrid g;
   g.octs_w = octs_w;
-  g.nb_w = kTileWaves / octs_w;
+  g.nb_w = waves / octs_w;
   g.oct_groups = octs / octs_w;
   g.tiles = (nb + g.nb_w - 1) / g.nb_w;
   g.wgs = B * g.tiles * g.oct_groups;
   return g;
 }
 
-template <class E, bool kQkv, bool kF32 = false>
+template <class E, int kW, bool kQkv, bool kF32 = false>
 void launch_mix_fwd_tile(const MixArgs& p, hipStream_t s) {
-  const int octs = (p.H + 7) / 8;
-  const int octs_w = (octs % 2 == 0 && p.H >= SPEAR_FUSED_FWD_TILE_WIDE_FROM) ? 2 : 1;
-  const TileGrid g = tile_grid(p.B, p.H, p.L, octs_w);
-  hipLaunchKernelGGL((phalanx_mix_fwd_tile_kernel<E, kQkv, kF32>), dim3((unsigned)g.wgs), dim3(64 * kTileWaves), 0, s,
+  const TileGrid g = tile_grid(p.B, p.H, p.L, 1, kW);
+  hipLaunchKernelGGL((phalanx_mix_fwd_tile_kernel<E, kW, kQkv, kF32>), dim3((unsigned)g.wgs), dim3(64 * kW), 0, s,
                      static_cast<const uint16_t*>(p.a_logit), static_cast<const uint16_t*>(p.b_logit),
                      static_cast<const uint16_t*>(p.c), static_cast<const uint16_t*>(p.v), static_cast<uint16_t*>(p.out),
-                     p.L, p.H, p.kv_groups, g.octs_w, g.nb_w, g.tiles, g.oct_groups);
+                     p.c_prev_tail, p.L, p.H, p.kv_groups, g.octs_w, g.nb_w, g.tiles, g.oct_groups);
 }
 
 }  // namespace
 
 hipError_t fused_mix_forward(const MixArgs& p, hipStream_t s) {
-  if (p.tile_split) {  // the caller has checked: no streaming state asked for, a grid that fits
+  if (p.tile_split) {  // the caller has checked: a grid that fits
+    // workgroups of 8 wavefronts on long rows and on rows of one head group, of 4 otherwise (table at the kernel)
+    static const int waves_override = env_override("SPEAR_BTP_FUSED_FWD_TILE_WAVES");
+    const bool eight = waves_override ? waves_override == 8 : (p.L >= 512 || p.H < 16);
     auto by_form = [&](auto e, auto q) {
       using E = decltype(e);
-      if (p.f32_out) launch_mix_fwd_tile<E, decltype(q)::value, true>(p, s);
-      else launch_mix_fwd_tile<E, decltype(q)::value>(p, s);
+      if (p.f32_out) launch_mix_fwd_tile<E, 4, decltype(q)::value, true>(p, s);  // check mode: one instance per form
+      else if (eight) launch_mix_fwd_tile<E, 8, decltype(q)::value>(p, s);
+      else launch_mix_fwd_tile<E, 4, decltype(q)::value>(p, s);
     };
     if (p.dtype == kBf16) {
       if (p.qkv) by_form(Bf16{}, std::true_type{});

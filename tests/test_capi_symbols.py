@@ -111,9 +111,6 @@ def test_host_side_validation_needs_no_gpu():
     assert b"unknown flag" in lib.spear_btp_last_error()
     assert lib.spear_phalanx_mix_forward(p, p, p, p, p, 1, 32, 4, 4, 0, 0xc, None) == -1
     assert b"exclude each other" in lib.spear_btp_last_error()
-    lib.spear_phalanx_mix_prefill.restype = ctypes.c_int
-    assert lib.spear_phalanx_mix_prefill(p, p, p, p, p, p, 1, 32, 4, 4, 0, 0x4, None) == -1
-    assert b"does not hand over the streaming state" in lib.spear_btp_last_error()
     assert lib.spear_phalanx_mix_backward(p, p, p, p, p, p, p, p, p, 1, 32, 4, 4, 0, 0x10, None) == -1
     assert b"unknown flag" in lib.spear_btp_last_error()
     assert lib.spear_phalanx_mix_backward(p, p, p, p, p, p, p, p, p, 1, 32, 4, 4, 0, 0xc, None) == -1
