@@ -354,6 +354,11 @@ def main() -> int:
                                                s["v"].data_ptr(), s["out"].data_ptr(), B, L, H, H, 0, 0, sp)
             assert rc == 0, lib.spear_btp_last_error()
 
+        def mix_walk(s):  # the forward whose wavefronts walk through time (SPEAR_MIX_WALK_SPLIT)
+            rc = lib.spear_phalanx_mix_forward(s["a"].data_ptr(), s["b"].data_ptr(), s["c"].data_ptr(),
+                                               s["v"].data_ptr(), s["out"].data_ptr(), B, L, H, H, 0, 0x8, sp)
+            assert rc == 0, lib.spear_btp_last_error()
+
         def mix_bwd(s):  # the work split whose wavefronts walk through time (SPEAR_MIX_WALK_SPLIT)
             rc = lib.spear_phalanx_mix_backward(s["a"].data_ptr(), s["b"].data_ptr(), s["c"].data_ptr(),
                                                 s["v"].data_ptr(), s["dout"].data_ptr(), s["da"].data_ptr(),
@@ -422,6 +427,7 @@ def main() -> int:
         mix_ms, unfused_ms = kernel_ms_over(mix, msets), kernel_ms_over(mix_unfused, msets)
         mix_bwd_ms, unfused_train_ms = kernel_ms_over(mix_bwd, msets), kernel_ms_over(mix_unfused_train, msets)
         mix_bwd_tile_ms = kernel_ms_over(mix_bwd_tile, msets)
+        mix_walk_ms = kernel_ms_over(mix_walk, msets)
 
         # what the memory system gives these stream counts in its best shape (contiguous 4 KiB pieces, short-lived
         # wavefronts, nothing shared): 3 inputs -> 1 output (forward) and 4 inputs -> 3 outputs (backward), without
@@ -441,6 +447,9 @@ def main() -> int:
         fused = {
             "avg_launch_ms": mix_ms, "algorithmic_bytes_per_launch": mix_bytes,
             "achieved": mix_bytes / (mix_ms * 1e-3) / 1e9, "frac": mix_bytes / (mix_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+            # (the library's default work split, one wavefront per 16-step block; the walking kernel beside it)
+            "walking_split_avg_launch_ms": mix_walk_ms,
+            "walking_split_frac": mix_bytes / (mix_walk_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
             "same_stage_from_pytorch_ops_plus_btp_kernel_ms": unfused_ms, "speedup": unfused_ms / mix_ms,
             "backward": {  # the library's default work split (one wavefront per 16-step block)
                 "avg_launch_ms": mix_bwd_tile_ms, "algorithmic_bytes_per_launch": mix_bwd_bytes,
