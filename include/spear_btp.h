@@ -120,13 +120,14 @@ int spear_phalanx_mix_forward(const void* a_logit, const void* b_logit, const vo
  * elements). Inputs keep their types. Not combinable with the column sums of _backward_ex. */
 #define SPEAR_MIX_F32_RESULTS 0x2u
 
-/* Flags for spear_phalanx_mix_forward / _backward / _backward_ex: which work split runs. TILE: one wavefront
- * per 16-step block, the carries handed between neighbouring blocks through LDS; the backward then has no
- * column sums. WALK: wavefronts that walk through time (every option). Forward: the same bits from both. Backward: the same results up to fp32
- * rounding. With neither flag the tile split serves every call it can (backward: 166-167 us against 185-196 us
- * at B=1024 L=128 H=32, 342 against 367 us at B=16 L=8192 H=64, 705 against 757 us at B=64 L=2048 H=128) and
- * the walking kernels the rest; SPEAR_BTP_FUSED_FWD / SPEAR_BTP_FUSED_BWD = walk or tile in the environment
- * change that default. The two flags exclude each other. */
+/* Flags for spear_phalanx_mix_forward / _prefill / _backward / _backward_ex: which work split runs. TILE: one
+ * wavefront per 16-step block, the carries handed between neighbouring blocks through LDS. WALK: wavefronts
+ * that walk through time. Forward: the same bits from both. Backward: the same results up to fp32 rounding.
+ * With neither flag the tile split serves every call except a backward with column sums, whose arrays the
+ * caller has sized for the walking kernel (backward: 166-167 us against 185-196 us at B=1024 L=128 H=32, 342
+ * against 367 us at B=16 L=8192 H=64, 705 against 757 us at B=64 L=2048 H=128);
+ * SPEAR_BTP_FUSED_FWD / SPEAR_BTP_FUSED_BWD = walk or tile in the environment change that default. The two
+ * flags exclude each other. */
 #define SPEAR_MIX_TILE_SPLIT 0x4u
 #define SPEAR_MIX_WALK_SPLIT 0x8u
 
@@ -153,11 +154,14 @@ int spear_phalanx_mix_backward(const void* a_logit, const void* b_logit, const v
  * sum them. The kernel cannot finish the sums without a second pass, so it leaves partial sums in fp32:
  *     sum_da [sum_rows, H],  sum_db [sum_rows, kv_heads * 16],  sum_dc [sum_rows, kv_heads * 16]
  * where row r sums the time steps of one (batch row, time chunk) and the caller adds the rows up
- * (sum_rows is a few per batch row at most). sum_rows must equal
- * spear_phalanx_mix_backward_sum_rows(B, L, H); every element of the three arrays is written; the sums
- * are taken before the gradients are rounded to `dtype`. All three NULL: no sums. With neither option it is
- * exactly spear_phalanx_mix_backward. */
+ * (a few rows per batch row with the walking kernel, one per 32 or 64 time steps with the tile split).
+ * sum_rows must equal spear_phalanx_mix_backward_sum_rows(B, L, H), or, in a call that asks for the tile
+ * split with SPEAR_MIX_TILE_SPLIT (the faster of the two), spear_phalanx_mix_backward_sum_rows_tile(B, L, H);
+ * a call with sums and no split flag runs the walking kernel. Every element of the three arrays is written;
+ * the sums are taken before the gradients are rounded to `dtype`. All three NULL: no sums. With neither
+ * option it is exactly spear_phalanx_mix_backward. */
 long long spear_phalanx_mix_backward_sum_rows(int B, int L, int H);
+long long spear_phalanx_mix_backward_sum_rows_tile(int B, int L, int H);
 int spear_phalanx_mix_backward_ex(const void* a_logit, const void* b_logit, const void* c, const void* v,
                                   const void* dout, void* da_logit, void* db_logit, void* dc, void* dv, int ld_da,
                                   int ld_db, int ld_dc, int ld_dv, float* sum_da, float* sum_db, float* sum_dc,

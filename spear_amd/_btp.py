@@ -32,7 +32,7 @@ FLAG_MIX_F32_RESULTS = 0x2
 FLAG_MIX_TILE_SPLIT = 0x4
 FLAG_MIX_WALK_SPLIT = 0x8
 FLAG_DX_F32 = 0x10
-_ABI_VERSION = 16
+_ABI_VERSION = 17
 _SUPPORTED_WPB = (4, 8, 16, 32)
 
 _lock = threading.Lock()
@@ -67,6 +67,8 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.spear_phalanx_mix_backward_bias.restype = ci
     lib.spear_phalanx_mix_backward_sum_rows.argtypes = [ci, ci, ci]
     lib.spear_phalanx_mix_backward_sum_rows.restype = ctypes.c_longlong
+    lib.spear_phalanx_mix_backward_sum_rows_tile.argtypes = [ci, ci, ci]
+    lib.spear_phalanx_mix_backward_sum_rows_tile.restype = ctypes.c_longlong
     lib.spear_phalanx_mix_prefill.argtypes = [vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, cu, vp]
     lib.spear_phalanx_mix_prefill.restype = ci
     lib.spear_phalanx_mix_step.argtypes = [vp] * 9 + [ci] * 6 + [cu, vp]
@@ -392,9 +394,14 @@ def mix_forward(
         _raise_native(lib, rc)
 
 
-def mix_backward_sum_rows(B: int, L: int, heads: int) -> int:
-    """Rows of the partial-sum arrays :func:`mix_backward` fills for this shape."""
-    return int(load_library().spear_phalanx_mix_backward_sum_rows(B, L, heads))
+def mix_backward_sum_rows(B: int, L: int, heads: int, tile_split: bool | None = None) -> int:
+    """Rows of the partial-sum arrays :func:`mix_backward` fills for this shape: with ``tile_split=True`` those
+    of the tile split (``SPEAR_MIX_TILE_SPLIT``), otherwise those of the walking kernel, which also serves a call
+    that names no split."""
+    lib = load_library()
+    if tile_split:
+        return int(lib.spear_phalanx_mix_backward_sum_rows_tile(B, L, heads))
+    return int(lib.spear_phalanx_mix_backward_sum_rows(B, L, heads))
 
 
 def mix_backward(
@@ -420,8 +427,9 @@ def mix_backward(
     wider ``[B, L, ld]`` buffer (``spear_phalanx_mix_backward_ex``). ``qkv_gate`` as in :func:`mix_forward`;
     ``da_logit`` is then the fp32 gradient of the gate. Float32 ``db_logit, dc, dv`` (and ``da_logit``) select
     the fp32 check mode (``SPEAR_MIX_F32_RESULTS``). ``tile_split``: True selects the kernel with one wavefront per
-    16-step block (``SPEAR_MIX_TILE_SPLIT``; no column sums), False the one whose wavefronts walk through time
-    (``SPEAR_MIX_WALK_SPLIT``), None leaves the choice to the library."""
+    16-step block (``SPEAR_MIX_TILE_SPLIT``; its sum arrays have ``mix_backward_sum_rows(B, L, heads, True)`` rows),
+    False the one whose wavefronts walk through time (``SPEAR_MIX_WALK_SPLIT``), None leaves the choice to the library
+    (the tile split, or with ``sums`` the walking kernel)."""
     tensors = (a_logit, b_logit, c, v, dout, da_logit, db_logit, dc, dv)
     _check(all(t.is_cuda for t in tensors), "All tensors must be CUDA.")
     _check(v.dim() == 3, "v must be [B, L, heads * 16].")
@@ -454,7 +462,7 @@ def mix_backward(
     lib = load_library()
     rows = 0
     if sums is not None:
-        rows = int(lib.spear_phalanx_mix_backward_sum_rows(B, L, heads))
+        rows = mix_backward_sum_rows(B, L, heads, tile_split)
         for name, t, width in (("sum_da", sums[0], heads), ("sum_db", sums[1], Fkv), ("sum_dc", sums[2], Fkv)):
             _check(t.is_cuda and t.device == v.device and t.dtype == torch.float32, f"{name} must be float32 on v's device.")
             _check_layout(name, t, (rows, width))

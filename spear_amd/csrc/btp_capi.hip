@@ -45,7 +45,7 @@ int check_common(const char* who, int B, int H, int L, int k, int in_dtype, int 
 
 extern "C" {
 
-int spear_btp_abi_version(void) { return 16; }
+int spear_btp_abi_version(void) { return 17; }
 
 const char* spear_btp_last_error(void) { return g_error; }
 
@@ -183,6 +183,11 @@ long long spear_phalanx_mix_backward_sum_rows(int B, int L, int H) {
   return spear_btp::fused_mix_backward_sum_rows(B, H, L);
 }
 
+long long spear_phalanx_mix_backward_sum_rows_tile(int B, int L, int H) {
+  if (B <= 0 || L <= 0 || H <= 0 || L % 16 != 0) return 0;
+  return spear_btp::fused_mix_backward_sum_rows(B, H, L, true);
+}
+
 int spear_phalanx_mix_backward(const void* a_logit, const void* b_logit, const void* c, const void* v, const void* dout,
                                void* da_logit, void* db_logit, void* dc, void* dv, int B, int L, int H, int kv_heads,
                                int dtype, unsigned flags, void* stream) {
@@ -251,15 +256,16 @@ int spear_phalanx_mix_backward_ex(const void* a_logit, const void* b_logit, cons
   const bool sums = sum_da || sum_db || sum_dc;
   if (sums && qkv) return fail(SPEAR_BTP_EINVAL, "%s: column sums are for the layer form, not SPEAR_MIX_QKV_GATE", who);
   if (sums && f32) return fail(SPEAR_BTP_EINVAL, "%s: column sums are not available with SPEAR_MIX_F32_RESULTS", who);
-  if (tile_asked && sums)
-    return fail(SPEAR_BTP_EINVAL, "%s: SPEAR_MIX_TILE_SPLIT has no column sums", who);
-  const bool tile = (tile_asked || (tile_default && !walk_asked && !sums)) &&
-                    (long long)B * ((L / 16 + 3) / 4) * ((H + 7) / 8) < (1ll << 31);
+  // (column sums come from the tile split only when the flag asks for it: the arrays' row count differs between
+  // the splits, and a caller without the flag has sized them with spear_phalanx_mix_backward_sum_rows)
+  const bool fits = (long long)B * ((L / 16 + 3) / 4) * ((H + 7) / 8) < (1ll << 31);
+  if (tile_asked && sums && !fits) return fail(SPEAR_BTP_EINVAL, "%s: too many tiles for SPEAR_MIX_TILE_SPLIT", who);
+  const bool tile = (tile_asked || (tile_default && !walk_asked && !sums)) && fits;
   if (sums) {
     if (!sum_da || !sum_db || !sum_dc) return fail(SPEAR_BTP_ENULL, "%s: the three sum arrays must be given together", who);
     if (!aligned16(sum_da) || !aligned16(sum_db) || !aligned16(sum_dc))
       return fail(SPEAR_BTP_EINVAL, "%s: sum arrays must be 16-byte aligned", who);
-    const long long want = spear_btp::fused_mix_backward_sum_rows(B, H, L);
+    const long long want = spear_btp::fused_mix_backward_sum_rows(B, H, L, tile);
     if (sum_rows != want)
       return fail(SPEAR_BTP_EINVAL, "%s: sum arrays must have %lld rows for this shape (got %lld)", who, want, sum_rows);
   }

@@ -635,16 +635,22 @@ __device__ __forceinline__ unsigned tile_workgroup() {
 }
 
 // kF32: check mode, the four gradients leave as fp32 (the kernel's own values, not rounded to 16 bits).
-template <class E, bool kQkv, bool kF32>
+// kSums: also leave, per workgroup (batch row, time tile), the sums over the tile's time steps of da_logit, db_logit
+// and dc in fp32 (before their rounding to 16 bits), as the walking kernel does per (batch row, chunk): every
+// wavefront sums its block's 16 steps, the workgroup's blocks are added in block order behind a second barrier
+// (a fixed order: the same bits in every run), and row `batch row * tiles + tile` of the three arrays is written.
+template <class E, bool kQkv, bool kF32, bool kSums = false>
 __global__ __launch_bounds__(64 * kTileWaves) __attribute__((amdgpu_waves_per_eu(SPEAR_FUSED_TILE_WAVES_PER_EU)))
 void phalanx_mix_bwd_tile_kernel(
     const uint16_t* __restrict__ a_logit, const uint16_t* __restrict__ b_logit, const uint16_t* __restrict__ c_in,
     const uint16_t* __restrict__ v_in, const uint16_t* __restrict__ dout, uint16_t* __restrict__ da_logit,
-    uint16_t* __restrict__ db_logit, uint16_t* __restrict__ dc, uint16_t* __restrict__ dv, int ld_da, int ld_db, int ld_dc,
-    int ld_dv, int L, int H, int kv_groups, int octs_w, int nb_w, int tiles, int oct_groups) {
+    uint16_t* __restrict__ db_logit, uint16_t* __restrict__ dc, uint16_t* __restrict__ dv, float* __restrict__ sum_da,
+    float* __restrict__ sum_db, float* __restrict__ sum_dc, int ld_da, int ld_db, int ld_dc, int ld_dv, int L, int H,
+    int kv_groups, int octs_w, int nb_w, int tiles, int oct_groups) {
   // per wavefront: decay of its block, product of the block's other decays per step, decay of the block beyond the edge
   __shared__ __align__(16) float gate_tiles[kTileWaves][3][kHeadsPerWave * kGateRow];
   __shared__ float2 carry_out[kTileWaves][2][64];  // [0] dC_out, [1] c_out of the wavefront's block, per lane
+  __shared__ float block_sums[kSums ? kTileWaves : 1][5][64];  // kSums: db (2), dc (2), da of the wavefront's block
 
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   // workgroup -> (batch row, time tile, group of octs_w head groups); head groups fastest, so that workgroups
@@ -838,8 +844,11 @@ void phalanx_mix_bwd_tile_kernel(
       carry_out[wave][1][lane] = make_float2(l0, l1);
     }
   }
-  __syncthreads();  // the kernel's only workgroup barrier; wavefronts without a block arrive here directly
-  if (!valid) return;
+  __syncthreads();  // the workgroup barrier of the carries; wavefronts without a block arrive here directly
+  if (!valid) {
+    if constexpr (kSums) __syncthreads();  // the barrier of the sums counts every wavefront of the workgroup
+    return;
+  }
 
   if (bl > 0) {  // the block before this one belongs to the wavefront octs_w places down
     const float2 q = carry_out[wave - octs_w][1][lane];
@@ -873,6 +882,7 @@ void phalanx_mix_bwd_tile_kernel(
 
   // ---- forward pass: state, gradients, per-step partial sums of dA
   float e[16];
+  float acc_b0 = 0.0f, acc_b1 = 0.0f, acc_c0 = 0.0f, acc_c1 = 0.0f;  // kSums only
   float hs0 = cin0, hs1 = cin1;  // h_{r-1}
 #pragma unroll
   for (int c4 = 0; c4 < 4; ++c4) {
@@ -904,6 +914,9 @@ void phalanx_mix_bwd_tile_kernel(
           dc0 += lane_xor(dc0, lane, 32); dc1 += lane_xor(dc1, lane, 32);
           db0 += lane_xor(db0, lane, 32); db1 += lane_xor(db1, lane, 32);
         }
+      }
+      if constexpr (kSums) {
+        acc_b0 += db0; acc_b1 += db1; acc_c0 += dc0; acc_c1 += dc1;
       }
       const float dv0 = fmaf(dX0, G0, go0), dv1 = fmaf(dX1, G1, go1);
       if constexpr (kF32) {
@@ -966,6 +979,33 @@ void phalanx_mix_bwd_tile_kernel(
     const uint32_t dap = E::pack2(da0, da1);
     __builtin_amdgcn_raw_buffer_store_b16((unsigned short)(dap & 0xffffu), rda, da_lane, t0 * ld_da * 2, 0);
     __builtin_amdgcn_raw_buffer_store_b16((unsigned short)(dap >> 16), rda, da_lane + 2 * ld_da, t0 * ld_da * 2, 0);
+  }
+
+  if constexpr (kSums) {
+    float acc_a = da0 + da1;  // lane k of a head holds steps 2k, 2k+1
+    acc_a += row_xor<1>(acc_a);
+    acc_a += row_xor<2>(acc_a);
+    acc_a += row_xor<4>(acc_a);  // now every lane of the head has the block's sum
+    block_sums[wave][0][lane] = acc_b0;
+    block_sums[wave][1][lane] = acc_b1;
+    block_sums[wave][2][lane] = acc_c0;
+    block_sums[wave][3][lane] = acc_c1;
+    block_sums[wave][4][lane] = acc_a;
+    __syncthreads();
+    if (bl == 0) {  // the first block's wavefront of each head group adds the tile's blocks, in block order
+      float t[5] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+      for (int j = 0; j < nb_w && t0 + j * kTile < L; ++j) {
+#pragma unroll
+        for (int q = 0; q < 5; ++q) t[q] += block_sums[wave + j * octs_w][q][lane];
+      }
+      const long row = brow * tiles + tile;
+      if (real && (lane & 7) == 0) sum_da[row * H + head] = t[4];
+      if (real && (head % kv_groups) == 0) {  // the group's sum is in every lane of the group
+        const long col = row * Fkv + (head / kv_groups) * kChan + d0;
+        *reinterpret_cast<float2*>(sum_db + col) = make_float2(t[0], t[1]);
+        *reinterpret_cast<float2*>(sum_dc + col) = make_float2(t[2], t[3]);
+      }
+    }
   }
 }
 
@@ -1349,37 +1389,43 @@ void launch_mix_bwd(const MixBwdArgs& p, const MixPlan& m, hipStream_t s) {
                      p.ld_dv ? p.ld_dv : p.H * kChan, p.L, p.H, p.kv_groups, m.chunk_blocks * kTile, m.chunks, total);
 }
 
-template <class E, bool kQkv, bool kF32 = false>
+// 1 head group x 4 blocks (two of four wavefronts read a halo) or 2 x 2 (all four do, but a workgroup reads
+// 512-byte runs): over 14 shapes the first is 1.5-3.5 % faster up to 64 heads, the second 0.5-1.5 % from 128 on
+TileGrid bwd_tile_grid(long B, int H, int L) {
+  const int octs = (H + 7) / 8;
+  return tile_grid(B, H, L, (octs % 2 == 0 && H >= 128) ? 2 : 1, kTileWaves);
+}
+
+template <class E, bool kQkv, bool kF32 = false, bool kSums = false>
 void launch_mix_bwd_tile(const MixBwdArgs& p, hipStream_t s) {
-  const int octs = (p.H + 7) / 8, nb = p.L / kTile;
-  // 1 head group x 4 blocks (two of four wavefronts read a halo) or 2 x 2 (all four do, but a workgroup reads
-  // 512-byte runs): over 14 shapes the first is 1.5-3.5 % faster up to 64 heads, the second 0.5-1.5 % from 128 on
-  const int octs_w = (octs % 2 == 0 && p.H >= 128) ? 2 : 1;
-  const int nb_w = kTileWaves / octs_w;
-  const int oct_groups = octs / octs_w, tiles = (nb + nb_w - 1) / nb_w;
-  const long wgs = (long)p.B * tiles * oct_groups;
+  const TileGrid g = bwd_tile_grid(p.B, p.H, p.L);
   auto u = [](const void* q) { return static_cast<const uint16_t*>(q); };
   auto w = [](void* q) { return static_cast<uint16_t*>(q); };
   const int Fkv = (p.H / p.kv_groups) * kChan;
-  hipLaunchKernelGGL((phalanx_mix_bwd_tile_kernel<E, kQkv, kF32>), dim3((unsigned)wgs), dim3(64 * kTileWaves), 0, s,
-                     u(p.a_logit), u(p.b_logit), u(p.c), u(p.v), u(p.dout), w(p.da_logit), w(p.db_logit), w(p.dc), w(p.dv),
-                     p.ld_da ? p.ld_da : p.H, p.ld_db ? p.ld_db : Fkv, p.ld_dc ? p.ld_dc : Fkv,
-                     p.ld_dv ? p.ld_dv : p.H * kChan, p.L, p.H, p.kv_groups, octs_w, nb_w, tiles, oct_groups);
+  hipLaunchKernelGGL((phalanx_mix_bwd_tile_kernel<E, kQkv, kF32, kSums>), dim3((unsigned)g.wgs), dim3(64 * kTileWaves), 0,
+                     s, u(p.a_logit), u(p.b_logit), u(p.c), u(p.v), u(p.dout), w(p.da_logit), w(p.db_logit), w(p.dc),
+                     w(p.dv), p.sum_da, p.sum_db, p.sum_dc, p.ld_da ? p.ld_da : p.H, p.ld_db ? p.ld_db : Fkv,
+                     p.ld_dc ? p.ld_dc : Fkv, p.ld_dv ? p.ld_dv : p.H * kChan, p.L, p.H, p.kv_groups, g.octs_w, g.nb_w,
+                     g.tiles, g.oct_groups);
 }
 
 }  // namespace
 
-long fused_mix_backward_sum_rows(long B, int H, int L) {
+long fused_mix_backward_sum_rows(long B, int H, int L, bool tile_split) {
   if (B <= 0 || H <= 0 || L <= 0) return 0;
-  return B * plan_mix_bwd(B, H, L).chunks;
+  return tile_split ? B * bwd_tile_grid(B, H, L).tiles : B * plan_mix_bwd(B, H, L).chunks;
 }
 
 hipError_t fused_mix_backward(const MixBwdArgs& p, hipStream_t s) {
   const MixPlan m = plan_mix_bwd(p.B, p.H, p.L);
   const bool sums = p.sum_da != nullptr;
   if (sums && (p.qkv || p.f32_grads)) return hipErrorInvalidValue;  // the caller has checked: layer form, 16-bit results
-  if (p.tile_split) {  // the caller has checked: no sums, a grid that fits
-    if (sums) return hipErrorInvalidValue;
+  if (p.tile_split) {  // the caller has checked: a grid that fits
+    if (sums) {
+      if (p.dtype == kBf16) launch_mix_bwd_tile<Bf16, false, false, true>(p, s);
+      else launch_mix_bwd_tile<Fp16, false, false, true>(p, s);
+      return hipGetLastError();
+    }
     if (p.dtype == kBf16) {
       if (p.f32_grads) {
         if (p.qkv) launch_mix_bwd_tile<Bf16, true, true>(p, s);

@@ -66,7 +66,7 @@ struct MixBwdArgs {
   void *da_logit, *db_logit, *dc, *dv;           // same shapes as the inputs they belong to
   int B, L, H, kv_groups;
   int dtype;
-  // all three null, or fp32 [fused_mix_backward_sum_rows(B, H, L), H | Hkv*16 | Hkv*16]: per-chunk sums over time
+  // all three null, or fp32 [fused_mix_backward_sum_rows(B, H, L, tile_split), H | Hkv*16 | Hkv*16]: per-chunk sums over time
   float *sum_da = nullptr, *sum_db = nullptr, *sum_dc = nullptr;
   // elements per time step of each gradient tensor; 0 = dense (its own width)
   int ld_da = 0, ld_db = 0, ld_dc = 0, ld_dv = 0;
@@ -75,7 +75,7 @@ struct MixBwdArgs {
   bool tile_split = false;  // one wavefront per 16-step block instead of wavefronts that walk through time
 };
 hipError_t fused_mix_backward(const MixBwdArgs& p, hipStream_t s);
-long fused_mix_backward_sum_rows(long B, int H, int L);
+long fused_mix_backward_sum_rows(long B, int H, int L, bool tile_split = false);
 // The same backward with the column sums finished inside the library: the per-chunk partial sums go through
 // a static device array instead of caller memory, and bias_da [H], bias_db / bias_dc [(H / kv_groups) * 16]
 // receive the sums over batch and time. Allocates nothing. `p.sum_*` are ignored.

@@ -264,7 +264,8 @@ int64_t row_stride(const char* name, const at::Tensor& t, int64_t B, int64_t L, 
 // check mode. `sums`: none, or three fp32 [rows, width] tensors receiving per-chunk column sums.
 void mix_backward(const at::Tensor& a_logit, const at::Tensor& b_logit, const at::Tensor& c, const at::Tensor& v,
                   const at::Tensor& dout, at::Tensor da_logit, at::Tensor db_logit, at::Tensor dc, at::Tensor dv,
-                  int64_t heads, int64_t kv_heads, const std::vector<at::Tensor>& sums, bool qkv_gate) {
+                  int64_t heads, int64_t kv_heads, const std::vector<at::Tensor>& sums, bool qkv_gate,
+                  bool tile_sums) {
   const MixShape s = check_mix_inputs(a_logit, b_logit, c, v, heads, kv_heads, qkv_gate);
   TORCH_CHECK(dout.is_cuda() && da_logit.is_cuda() && db_logit.is_cuda() && dc.is_cuda() && dv.is_cuda(), "All tensors must be CUDA.");
   const int64_t groups = heads / kv_heads;
@@ -289,7 +290,8 @@ void mix_backward(const at::Tensor& a_logit, const at::Tensor& b_logit, const at
   int64_t rows = 0;
   float* sp[3] = {nullptr, nullptr, nullptr};
   if (!sums.empty()) {
-    rows = spear_phalanx_mix_backward_sum_rows((int)s.B, (int)s.L, (int)heads);
+    rows = tile_sums ? spear_phalanx_mix_backward_sum_rows_tile((int)s.B, (int)s.L, (int)heads)
+                     : spear_phalanx_mix_backward_sum_rows((int)s.B, (int)s.L, (int)heads);
     const int64_t widths[3] = {heads, s.Fkv, s.Fkv};
     const char* names[3] = {"sum_da", "sum_db", "sum_dc"};
     for (int i = 0; i < 3; ++i) {
@@ -300,7 +302,8 @@ void mix_backward(const at::Tensor& a_logit, const at::Tensor& b_logit, const at
     }
   }
   const c10::DeviceGuard guard(v.device());
-  const unsigned flags = (qkv_gate ? SPEAR_MIX_QKV_GATE : 0u) | (f32 ? SPEAR_MIX_F32_RESULTS : 0u);
+  const unsigned flags = (qkv_gate ? SPEAR_MIX_QKV_GATE : 0u) | (f32 ? SPEAR_MIX_F32_RESULTS : 0u) |
+                         ((tile_sums && !sums.empty()) ? SPEAR_MIX_TILE_SPLIT : 0u);
   const int rc = spear_phalanx_mix_backward_ex(
       a_logit.data_ptr(), b_logit.data_ptr(), c.data_ptr(), v.data_ptr(), dout.data_ptr(), da_logit.data_ptr(),
       db_logit.data_ptr(), dc.data_ptr(), dv.data_ptr(), (int)ld_da, (int)ld_db, (int)ld_dc, (int)ld_dv, sp[0], sp[1], sp[2],
@@ -326,9 +329,10 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         py::arg("heads"), py::arg("kv_heads"), py::arg("qkv_gate") = false);
   m.def("mix_backward", &mix_backward, py::arg("a_logit"), py::arg("b_logit"), py::arg("c"), py::arg("v"), py::arg("dout"),
         py::arg("da_logit"), py::arg("db_logit"), py::arg("dc"), py::arg("dv"), py::arg("heads"), py::arg("kv_heads"),
-        py::arg("sums") = std::vector<at::Tensor>(), py::arg("qkv_gate") = false);
+        py::arg("sums") = std::vector<at::Tensor>(), py::arg("qkv_gate") = false, py::arg("tile_sums") = false);
   m.def("abi_version", []() { return spear_btp_abi_version(); });
-  m.def("mix_backward_sum_rows", [](int64_t B, int64_t L, int64_t heads) {
-    return (int64_t)spear_phalanx_mix_backward_sum_rows((int)B, (int)L, (int)heads);
-  });
+  m.def("mix_backward_sum_rows", [](int64_t B, int64_t L, int64_t heads, bool tile_sums) {
+    return (int64_t)(tile_sums ? spear_phalanx_mix_backward_sum_rows_tile((int)B, (int)L, (int)heads)
+                               : spear_phalanx_mix_backward_sum_rows((int)B, (int)L, (int)heads));
+  }, py::arg("B"), py::arg("L"), py::arg("heads"), py::arg("tile_sums") = false);
 }

@@ -143,9 +143,9 @@ def _mix_backward_packed(
     if used < ld:
         packed[..., used:].zero_()
     da, db, dc, dv = (packed[..., cols[k][0]:cols[k][0] + cols[k][1]] for k in "abcv")
-    rows = _btp.mix_backward_sum_rows(B, L, heads)
+    rows = _btp.mix_backward_sum_rows(B, L, heads, tile_split=True)  # the faster of the two work splits
     sums = [torch.empty((rows, t.shape[-1]), device=v.device, dtype=torch.float32) for t in (a_logits, b_logits, c)]
-    _btp.mix_backward(a_logits, b_logits, c, v, dout, da, db, dc, dv, heads, kv_heads, sums=tuple(sums))
+    _btp.mix_backward(a_logits, b_logits, c, v, dout, da, db, dc, dv, heads, kv_heads, sums=tuple(sums), tile_split=True)
     return (packed, *(s.sum(0).to(v.dtype) for s in sums))
 
 

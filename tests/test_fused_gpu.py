@@ -110,23 +110,31 @@ def test_fused_backward_with_shared_kv_heads(B, L, H, Hkv, tile_split):
     assert_close(f64(da), rda, BF16_ATOL, BF16_RTOL, "da")
 
 
+@pytest.mark.parametrize("tile_split", [None, False, True], ids=["default", "walk", "tile"])
 @pytest.mark.parametrize("B,L,H,Hkv", [(1, 16, 4, 4), (3, 128, 8, 8), (2, 144, 16, 2), (1, 80, 12, 3), (1, 272, 32, 4),
-                                       (2, 2064, 8, 1), (40, 64, 32, 32), (1, 8192, 8, 8)])
-def test_fused_backward_column_sums_match_oracle(B, L, H, Hkv):
+                                       (2, 2064, 8, 1), (40, 64, 32, 32), (1, 8192, 8, 8), (3, 112, 128, 16),
+                                       (70, 272, 32, 32)])
+def test_fused_backward_column_sums_match_oracle(B, L, H, Hkv, tile_split):
     """The partial sums the backward kernel leaves add up to the oracle's gradients summed over batch and
-    time (the bias gradients of proj_a, proj_b, proj_c); the gradients themselves are unchanged by asking."""
+    time (the bias gradients of proj_a, proj_b, proj_c); the gradients themselves are unchanged by asking. A call
+    that names no split gets them from the walking kernel, one that asks for the tile split from that (one row
+    per workgroup, i.e. per 64 or 32 time steps, instead of one per chunk)."""
     from spear_amd import _btp
 
     a, b, c, v = make_mix_inputs(B, L, H, Hkv, seed=5000 + L + H)
     dout = torch.randn(B, L, H * 16, generator=torch.Generator().manual_seed(L + 2)).bfloat16()
-    print(f"fused bwd sums B={B} L={L} H={H} Hkv={Hkv}", flush=True)
-    plain = run_mix_backward(a, b, c, v, dout, H, Hkv, tile_split=False)  # sums come from the walking kernel
+    print(f"fused bwd sums B={B} L={L} H={H} Hkv={Hkv} tile={tile_split}", flush=True)
+    plain = run_mix_backward(a, b, c, v, dout, H, Hkv, tile_split=bool(tile_split))
     dev = [t.to(DEV) for t in (a, b, c, v, dout)]
     outs = [torch.full(t.shape, float("nan"), device=DEV, dtype=t.dtype) for t in (a, b, c, v)]
-    rows = _btp.mix_backward_sum_rows(B, L, H)
+    rows = _btp.mix_backward_sum_rows(B, L, H, tile_split)
     assert rows >= B and rows % B == 0
+    if tile_split:
+        assert rows == B * -(-(L // 16) // (2 if H >= 128 else 4))
+    else:
+        assert rows == _btp.mix_backward_sum_rows(B, L, H)
     sums = tuple(torch.full((rows, w), float("nan"), device=DEV) for w in (H, Hkv * 16, Hkv * 16))
-    _btp.mix_backward(*dev, *outs, H, Hkv, sums=sums)
+    _btp.mix_backward(*dev, *outs, H, Hkv, sums=sums, tile_split=tile_split)
     torch.cuda.synchronize()
     for got, want in zip(outs, plain):
         assert torch.equal(got.cpu(), want)
@@ -137,7 +145,8 @@ def test_fused_backward_column_sums_match_oracle(B, L, H, Hkv):
         # fp32 arithmetic on bf16 inputs; the sums are taken before any rounding to bf16
         assert np.all(np.abs(got - want) <= 2e-4 * mass + 1e-5), (name, np.abs(got - want).max(), mass.max())
     with pytest.raises(RuntimeError, match="shape"):
-        _btp.mix_backward(*dev, *outs, H, Hkv, sums=tuple(torch.empty(rows + 1, w, device=DEV) for w in (H, Hkv * 16, Hkv * 16)))
+        _btp.mix_backward(*dev, *outs, H, Hkv, tile_split=tile_split,
+                          sums=tuple(torch.empty(rows + 1, w, device=DEV) for w in (H, Hkv * 16, Hkv * 16)))
 
 
 @pytest.mark.parametrize("B,L,H,Hkv", [(1, 16, 4, 4), (3, 128, 8, 8), (2, 144, 16, 2), (1, 80, 12, 3), (2, 2064, 8, 1), (40, 64, 32, 32)])
@@ -308,8 +317,9 @@ def test_tile_split_strided_outputs_qkv_form_and_what_it_refuses():
     rows = _btp.mix_backward_sum_rows(B, L, H)
     sums = tuple(torch.empty(rows, w, device=DEV) for w in widths[:3])
     grads = [torch.empty_like(t) for t in dev[:4]]
-    with pytest.raises(RuntimeError, match="has no column sums"):
-        _btp.mix_backward(*dev, *grads, H, Hkv, sums=sums, tile_split=True)
+    if _btp.mix_backward_sum_rows(B, L, H, tile_split=True) != rows:  # arrays sized for the walking kernel
+        with pytest.raises(RuntimeError, match="shape"):
+            _btp.mix_backward(*dev, *grads, H, Hkv, sums=sums, tile_split=True)
     # left to the library, a call runs the tile split, and the walking kernel when it asks for column sums
     auto = [torch.full(t.shape, float("nan"), device=DEV, dtype=t.dtype) for t in (a, b, c, v)]
     _btp.mix_backward(*dev, *auto, H, Hkv)
