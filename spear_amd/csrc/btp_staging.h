@@ -478,8 +478,8 @@ __device__ __forceinline__ SpanCoord span_coord(long span, int spans_per_row, in
 // fetched once. Measured on rows of several spans (B=16 H=64 L=8192 / B=64 H=128 L=2048), against plain
 // round-robin: runs of 32 gain 1.3 % / 3.6 % in forward and 1.5 % / 1.6 % in backward; runs of 2-8 gain nothing,
 // runs of 128 and more lose again in backward, and one contiguous eighth of the tensor per XCD (group 0) gains
-// 1.8 % / 0.5 % in forward and loses 2 % in backward. On rows of one span nothing is shared and any dealing
-// other than round-robin loses 12 %, so those keep the plain order.
+// 1.8 % / 0.5 % in forward and loses 2 % in backward. On rows of one span nothing is shared: runs of 32 or 128
+// change nothing there (+-0.3 %) and runs of 8 lose 1 %, so those keep the plain order.
 #ifndef SPEAR_BTP_XCD_REMAP  // 0: never, 1: kernels on rows of several spans, 2: every kernel
 #define SPEAR_BTP_XCD_REMAP 1
 #endif
