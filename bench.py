@@ -316,6 +316,17 @@ def main() -> int:
 
     fwd_f32_ms = kernel_ms(fwd_f32)
     bwd_f32_ms = kernel_ms(bwd_f32)
+
+    # what the memory system gives the forward's 1 read : 2 writes (x in, an fp32 y out) in the kernels' launch shape,
+    # without and with a compute phase (spear_btp_stream_probe_mix, x -> the two halves of y32)
+    def probe_1r2w(compute):
+        def fn(s):
+            src = (ctypes.c_void_p * 1)(s["x"].data_ptr())
+            dst = (ctypes.c_void_p * 2)(s["y32"].data_ptr(), s["y32"].data_ptr() + nbytes)
+            rc = lib.spear_btp_stream_probe_mix(src, 1, dst, 2, ctypes.c_ulonglong(nbytes), compute, sp)
+            assert rc == 0, lib.spear_btp_last_error()
+        return 3 * nbytes / (kernel_ms(fn) * 1e-3) / 1e9
+    ceil_1r2w = [probe_1r2w(0), probe_1r2w(1)]
     for s_ in sets:
         del s_["y32"]
 
@@ -808,6 +819,7 @@ def main() -> int:
             "algorithmic_bytes_per_unit": {"forward": 98, "backward": 134},
             "forward_frac": units * 98 / (fwd_f32_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
             "backward_frac": units * 134 / (bwd_f32_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+            "forward_ceiling_1_read_2_writes_GBps": ceil_1r2w,  # no arithmetic / 320 dependent FMAs
         },
         "log_gate_entry_points": {"forward_ms": fwd_log_ms, "backward_ms": bwd_log_ms,
                                   "achieved": units * (68 + 108) / ((fwd_log_ms + bwd_log_ms) * 1e-3) / 1e9,

@@ -295,8 +295,10 @@ int spear_btp_stream_probe_shape(const void* src_a, const void* src_b, void* dst
 /* The probe with the stream counts of the fused layer kernels (measurement aid, no counterpart in the
  * reference): `n_src` inputs of `bytes` each are combined (xor) into `n_dst` identical outputs of `bytes` each, in
  * the shape of spear_btp_stream_probe (one 4 KiB piece per wavefront and tensor, non-temporal 16-byte accesses).
- * (n_src, n_dst) = (3, 1): the fused forward's and the prefill kernel's mix; (4, 3): the fused backward's.
- * `compute` != 0 puts a chain of dependent FMAs between loads and stores (640 for (3, 1), 1280 for (4, 3); the
+ * (n_src, n_dst) = (3, 1): the fused forward's and the prefill kernel's mix; (4, 3): the fused backward's;
+ * (1, 2): the stand-alone forward's with an fp32 result (the op's default output type).
+ * `compute` != 0 puts a chain of dependent FMAs between loads and stores (640 for (3, 1), 1280 for (4, 3), 320
+ * for (1, 2); the
  * outputs' last word may then differ in its lowest bit). `src`, `dst`: host arrays of device pointers, 16-byte
  * aligned; `bytes` a multiple of 4096. */
 int spear_btp_stream_probe_mix(const void* const* src, int n_src, void* const* dst, int n_dst, unsigned long long bytes,

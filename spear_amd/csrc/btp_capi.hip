@@ -429,8 +429,8 @@ int spear_btp_stream_probe_mix(const void* const* src, int n_src, void* const* d
   g_error[0] = '\0';
   const char* who = "spear_btp_stream_probe_mix";
   if (!src || !dst) return fail(SPEAR_BTP_ENULL, "%s: NULL pointer", who);
-  if (!((n_src == 3 && n_dst == 1) || (n_src == 4 && n_dst == 3)))
-    return fail(SPEAR_BTP_EINVAL, "%s: (n_src, n_dst) must be (3, 1) or (4, 3) (got %d, %d)", who, n_src, n_dst);
+  if (!((n_src == 3 && n_dst == 1) || (n_src == 4 && n_dst == 3) || (n_src == 1 && n_dst == 2)))
+    return fail(SPEAR_BTP_EINVAL, "%s: (n_src, n_dst) must be (3, 1), (4, 3) or (1, 2) (got %d, %d)", who, n_src, n_dst);
   if (bytes % 4096 != 0) return fail(SPEAR_BTP_EINVAL, "%s: size must be a multiple of 4096", who);
   for (int i = 0; i < n_src; ++i)
     if (!src[i] || !aligned16(src[i])) return fail(SPEAR_BTP_EINVAL, "%s: every tensor pointer must be set and 16-byte aligned", who);

@@ -772,6 +772,9 @@ hipError_t stream_probe_mix(const void* const* src, int n_src, void* const* dst,
   } else if (n_src == 3 && n_dst == 1) {
     if (compute) hipLaunchKernelGGL((stream_probe_mix_kernel<3, 1, 80>), grid, wg, 0, s, p, slabs);
     else hipLaunchKernelGGL((stream_probe_mix_kernel<3, 1, 0>), grid, wg, 0, s, p, slabs);
+  } else if (n_src == 1 && n_dst == 2) {
+    if (compute) hipLaunchKernelGGL((stream_probe_mix_kernel<1, 2, 40>), grid, wg, 0, s, p, slabs);
+    else hipLaunchKernelGGL((stream_probe_mix_kernel<1, 2, 0>), grid, wg, 0, s, p, slabs);
   } else {
     return hipErrorInvalidValue;  // the caller has checked
   }

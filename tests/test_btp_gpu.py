@@ -412,7 +412,7 @@ def test_measurement_aids_move_the_bytes_they_are_timed_for(slabs):
     # the probe with several inputs and outputs: every output is the combination of all inputs, nothing beyond
     ins = [a, b, a.flip(0).contiguous(), b.flip(0).contiguous()]
     outs = [torch.full((n + guard,), 0xA5, dtype=torch.uint8, device=DEV) for _ in range(3)]
-    for n_src, n_dst in ((3, 1), (4, 3)):
+    for n_src, n_dst in ((3, 1), (4, 3), (1, 2)):
         want = ins[0]
         for t in ins[1:n_src]:
             want = want ^ t
