@@ -171,13 +171,16 @@ class _BTPFunction(torch.autograd.Function):
 def _plain_eager(*tensors: torch.Tensor) -> bool:
     """True where nothing needs to see the custom ops: ordinary tensors, no torch.compile trace, no dispatch or
     function mode, no functorch transform. Only then may the compiled autograd node stand in for _BTPFunction."""
-    return (
-        all(type(t) is torch.Tensor or type(t) is torch.nn.Parameter for t in tensors)
-        and not torch.compiler.is_compiling()
-        and torch._C._len_torch_dispatch_stack() == 0
-        and torch._C._len_torch_function_stack() == 0
-        and torch._C._functorch.peek_interpreter_stack() is None
-    )
+    try:
+        return (
+            all(type(t) is torch.Tensor or type(t) is torch.nn.Parameter for t in tensors)
+            and not torch.compiler.is_compiling()
+            and torch._C._len_torch_dispatch_stack() == 0
+            and torch._C._len_torch_function_stack() == 0
+            and torch._C._functorch.peek_interpreter_stack() is None
+        )
+    except AttributeError:  # a PyTorch without these introspection hooks: the Python node is always right
+        return False
 
 
 def btp(
