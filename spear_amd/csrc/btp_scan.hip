@@ -444,11 +444,10 @@ __device__ __forceinline__ void btp_bwd_scan_body(
 
 // 16-bit dy and 16-bit coefficients (the reference's operands): the body fits 128 VGPRs, so four
 // waves per SIMD are requested explicitly.
-template <class E, class C, bool kStreamIn>
-__global__ __launch_bounds__((64 * bwd_waves<true, kStreamIn>())) SPEAR_BTP_BWD_OCC void btp_bwd_scan_kernel(
+template <class E, class C, bool kStreamIn, int kW = bwd_waves<true, kStreamIn>()>
+__global__ __launch_bounds__((64 * kW)) SPEAR_BTP_BWD_OCC void btp_bwd_scan_kernel(
     const typename C::elem* __restrict__ coeff, const uint16_t* __restrict__ x, const uint16_t* __restrict__ dy,
     uint16_t* __restrict__ dx, float* __restrict__ dA, int L, int spans_per_row, long total_spans, int k) {
-  constexpr int kW = bwd_waves<true, kStreamIn>();
   __shared__ __align__(16) unsigned char lds[kW][4096 + 4096 + kCoeffLdsBytes];
   btp_bwd_scan_body<E, C, uint16_t, uint16_t, kStreamIn, kW>(lds, coeff, x, dy, dx, dA, L, spans_per_row, total_spans, k);
 }
@@ -671,6 +670,11 @@ void launch_bwd_as(const BwdArgs& p, const Grid& g, hipStream_t s) {
     hipLaunchKernelGGL((btp_bwd_scan_kernel_relaxed<E, C, GradT, uint16_t, kStreamIn>), dim3(g.blocks), dim3(64 * g.waves), 0, s,
                        c, x, static_cast<const GradT*>(p.dy), dx, p.dA, p.L, g.spans_per_row, g.total_spans, p.k);
   } else {
+    if (!kStreamIn && g.waves == kWaves && kWaves != kWavesLong) {  // rows of a few spans: the smaller workgroup
+      hipLaunchKernelGGL((btp_bwd_scan_kernel<E, C, kStreamIn, kWaves>), dim3(g.blocks), dim3(64 * g.waves), 0, s, c, x,
+                         static_cast<const uint16_t*>(p.dy), dx, p.dA, p.L, g.spans_per_row, g.total_spans, p.k);
+      return;
+    }
     hipLaunchKernelGGL((btp_bwd_scan_kernel<E, C, kStreamIn>), dim3(g.blocks), dim3(64 * g.waves), 0, s, c, x,
                        static_cast<const uint16_t*>(p.dy), dx, p.dA, p.L, g.spans_per_row, g.total_spans, p.k);
   }
@@ -680,7 +684,12 @@ template <class E, class C, class GradT>
 hipError_t launch_bwd(const BwdArgs& p, hipStream_t s) {
   constexpr bool kLeanIo = !(std::is_same<GradT, float>::value || C::kLog);
   const bool lean = kLeanIo && !p.dx_f32;  // the kernel launch_bwd_as picks
-  const Grid g = lean ? make_grid((long)p.B * p.H, p.L, bwd_waves<true, false>(), bwd_waves<true, true>())
+  // Workgroups of kWavesLong wavefronts hand more carries over in LDS and read fewer halos; with the workgroups
+  // dealt to the XCDs in runs (first_span_of_workgroup) halo lines are mostly L2 hits, and on rows of up to 8 spans
+  // the smaller workgroup wins: 72.5 -> 69 us at L = 256 and 512 (B H L = 4 Mi), 135.5 -> 132.6 us at L = 1024;
+  // from 16 spans on the two are within +-2 % of each other either way.
+  const int long_row_waves = (p.L + kSpan - 1) / kSpan <= 8 ? kWaves : bwd_waves<true, false>();
+  const Grid g = lean ? make_grid((long)p.B * p.H, p.L, long_row_waves, bwd_waves<true, true>())
                       : make_grid((long)p.B * p.H, p.L, bwd_waves<false, false>(), bwd_waves<false, true>());
   if (stream_inputs(g)) launch_bwd_as<E, C, GradT, true>(p, g, s);
   else launch_bwd_as<E, C, GradT, false>(p, g, s);
