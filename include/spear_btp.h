@@ -154,7 +154,7 @@ int spear_phalanx_mix_backward(const void* a_logit, const void* b_logit, const v
  * sum them. The kernel cannot finish the sums without a second pass, so it leaves partial sums in fp32:
  *     sum_da [sum_rows, H],  sum_db [sum_rows, kv_heads * 16],  sum_dc [sum_rows, kv_heads * 16]
  * where row r sums the time steps of one (batch row, time chunk) and the caller adds the rows up
- * (a few rows per batch row with the walking kernel, one per 32 or 64 time steps with the tile split).
+ * (a few rows per batch row with the walking kernel, one per 64 time steps with the tile split).
  * sum_rows must equal spear_phalanx_mix_backward_sum_rows(B, L, H), or, in a call that asks for the tile
  * split with SPEAR_MIX_TILE_SPLIT (the faster of the two), spear_phalanx_mix_backward_sum_rows_tile(B, L, H);
  * a call with sums and no split flag runs the walking kernel. Every element of the three arrays is written;

@@ -160,7 +160,7 @@ int spear_phalanx_mix_prefill(const void* a_logit, const void* b_logit, const vo
   if (tile_asked && walk_asked)
     return fail(SPEAR_BTP_EINVAL, "%s: SPEAR_MIX_TILE_SPLIT and SPEAR_MIX_WALK_SPLIT exclude each other", who);
   const bool tile = (tile_asked || (tile_default && !walk_asked)) &&
-                    (long long)B * ((L / 16 + 3) / 4) * ((H + 7) / 8) < (1ll << 31);
+                    (long long)B * ((L / 16 + 3) / 4 + 7) * ((H + 7) / 8) < (1ll << 31);
   if ((long long)B * L * H * 16ll >= (1ll << 40)) return fail(SPEAR_BTP_EINVAL, "%s: tensor too large", who);
   if ((long long)L * H * (f32 ? 64ll : 32ll) >= (1ll << 31))  // a batch row is addressed through one 32-bit buffer resource
     return fail(SPEAR_BTP_EINVAL, "%s: one batch row (L * H * 16 elements) must stay below 2 GiB", who);
@@ -258,7 +258,7 @@ int spear_phalanx_mix_backward_ex(const void* a_logit, const void* b_logit, cons
   if (sums && f32) return fail(SPEAR_BTP_EINVAL, "%s: column sums are not available with SPEAR_MIX_F32_RESULTS", who);
   // (column sums come from the tile split only when the flag asks for it: the arrays' row count differs between
   // the splits, and a caller without the flag has sized them with spear_phalanx_mix_backward_sum_rows)
-  const bool fits = (long long)B * ((L / 16 + 3) / 4) * ((H + 7) / 8) < (1ll << 31);
+  const bool fits = (long long)B * ((L / 16 + 3) / 4 + 7) * ((H + 7) / 8) < (1ll << 31);  // (+ 7: grids are padded to groups of 8 tiles)
   if (tile_asked && sums && !fits) return fail(SPEAR_BTP_EINVAL, "%s: too many tiles for SPEAR_MIX_TILE_SPLIT", who);
   const bool tile = (tile_asked || (tile_default && !walk_asked && !sums)) && fits;
   if (sums) {

@@ -610,19 +610,49 @@ __device__ __forceinline__ float product_of_the_others(float a) {
   return dpp_or_one<0x111>(p) * dpp_or_one<0x101>(q);
 }
 
-#ifndef SPEAR_FUSED_TILE_XCD_GROUP  // neighbouring workgroups per XCD; 0: launch order (round-robin)
-#define SPEAR_FUSED_TILE_XCD_GROUP 128
+#ifndef SPEAR_FUSED_TILE_XCD_GROUP  // neighbouring 4-wavefront workgroups per XCD; 0: launch order (round-robin)
+#define SPEAR_FUSED_TILE_XCD_GROUP 64
 #endif
 #ifndef SPEAR_FUSED_TILE_WAVES_PER_EU
 #define SPEAR_FUSED_TILE_WAVES_PER_EU 3
 #endif
-// Which tile workgroup this is. Launch order deals workgroups round-robin to the 8 XCDs, each with its own L2. An
-// XCD gets runs of SPEAR_FUSED_TILE_XCD_GROUP neighbouring workgroups instead (windows of 8 runs sweep the tensors
-// front to back): the workgroup that owns an edge block and the neighbour that reads it as its halo then share an
-// L2 close in time. Backward, against plain round-robin (0), runs of 128 four-wavefront workgroups: 184 -> 166-167
-// us at B=1024 L=128 H=32, 371 -> 344 us at B=16 L=8192 H=64, 733 -> 718 us at B=64 L=2048 H=128 (all three as 1
-// head group x 4 blocks); runs of 64 gain a little less, runs of 256 lose most of it again. The tail of the grid
-// that does not fill a window keeps the launch order.
+// Which tile workgroup this is: two steps, XCD dealing (tile_workgroup) and the order of the tiles (tile_place).
+// Launch order deals workgroups round-robin to the 8 XCDs, each with its own L2. An XCD gets runs of
+// SPEAR_FUSED_TILE_XCD_GROUP neighbouring workgroups instead (windows of 8 runs sweep the tensors front to back):
+// the workgroup that owns an edge block and the neighbour that reads it as its halo then share an L2 close in
+// time. Backward with head groups fastest, against plain round-robin (0), runs of 128 four-wavefront workgroups:
+// 184 -> 166-167 us at B=1024 L=128 H=32, 371 -> 344 us at B=16 L=8192 H=64, 733 -> 718 us at B=64 L=2048 H=128
+// (all three as 1 head group x 4 blocks); with the tiles in groups of 8 (below) runs of 64 are best (32: forward
+// -3 % on long rows, 256: -5 to -15 %). The tail of the grid that does not fill a window keeps the launch order.
+//
+// Workgroup -> (batch row, time tile, group of head groups). Up to SPEAR_FUSED_TILE_TIME_GROUP consecutive time
+// tiles of one head group are neighbours in this order, then come the row's other head groups, then the next
+// tiles: the workgroup that streams an edge block and the one that reads it as its halo are dispatched back to
+// back on one XCD, while the run as a whole still covers whole feature rows. Measured (forward / backward, us):
+//   tiles in groups of   1 (head groups fastest)   2           4           8           16         all (time fastest)
+//   B=1024 L=128 H=32    86.9 / 166.4              86.9 / 162  86.9 / 162  86.9 / 162  87 / 162   87.0 / 162.2
+//   B=16 L=8192 H=64     178.9 / 344.4             173 / 336   167 / 342   172 / 327   179 / 334  191.5 / 372.4
+//   B=64 L=2048 H=128    364.2 / 707               363 / 711   372 / 681   346 / 679   356 / 689  355.8 / 698.6
+// A grid padded to whole groups: workgroups of tiles past the row's end only join the barriers.
+#ifndef SPEAR_FUSED_TILE_TIME_GROUP
+#define SPEAR_FUSED_TILE_TIME_GROUP 8
+#endif
+struct TilePlace {
+  int og, tile;
+  long brow;
+};
+__device__ __forceinline__ TilePlace tile_place(unsigned wg, int tiles, int oct_groups) {
+  const unsigned tg = min((unsigned)SPEAR_FUSED_TILE_TIME_GROUP, (unsigned)tiles);
+  const unsigned tgroups = ((unsigned)tiles + tg - 1) / tg;
+  const unsigned t_lo = wg % tg, r1 = wg / tg;
+  TilePlace p;
+  p.og = (int)(r1 % (unsigned)oct_groups);
+  const unsigned r2 = r1 / (unsigned)oct_groups;
+  p.tile = (int)((r2 % tgroups) * tg + t_lo);
+  p.brow = r2 / tgroups;
+  return p;
+}
+
 template <int kRun = SPEAR_FUSED_TILE_XCD_GROUP>
 __device__ __forceinline__ unsigned tile_workgroup() {
   unsigned wg = blockIdx.x;
@@ -653,13 +683,10 @@ void phalanx_mix_bwd_tile_kernel(
   __shared__ float block_sums[kSums ? kTileWaves : 1][5][64];  // kSums: db (2), dc (2), da of the wavefront's block
 
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
-  // workgroup -> (batch row, time tile, group of octs_w head groups); head groups fastest, so that workgroups
-  // next to each other in launch order read neighbouring features of the same time steps
   const unsigned wg = tile_workgroup();
-  const int og = (int)(wg % (unsigned)oct_groups);
-  const unsigned tt = wg / (unsigned)oct_groups;
-  const int tile = (int)(tt % (unsigned)tiles);
-  const long brow = tt / (unsigned)tiles;
+  const TilePlace at = tile_place(wg, tiles, oct_groups);
+  const int og = at.og, tile = at.tile;
+  const long brow = at.brow;
   const int o = wave % octs_w, bl = wave / octs_w;  // octs_w * nb_w == kTileWaves
   const int octs = (H + kHeadsPerWave - 1) / kHeadsPerWave;
   const int ho = (og * octs_w + o) * kHeadsPerWave;
@@ -1020,10 +1047,10 @@ void phalanx_mix_bwd_tile_kernel(
 // workgroup streams the same lines on the same L2) and runs that recurrence itself.
 // The wavefront of a row's last block also stores the streaming state for decoding after this prompt, when asked.
 // kW wavefronts per workgroup, one head group x kW consecutive blocks (2 head groups x kW / 2 blocks measured
-// slower at every shape): 4 or 8. Microseconds for 4 / 8 / the walking kernel, B L H:
-//   1024 128 32: 87.0 / 90.8 / 96.2     256 512 32: 90.7 / 88.6 / 101.1    16 8192 32: 91.1 / 90.4 / 99.9
-//   512 128 64: 89.9 / 90.7 / 95.2      16 8192 64: 181.6 / 178.1 / 181.5  64 2048 128: 357.4 / 347.9 / 370.4
-//   256 128 128: 89.8 / 89.8 / 114.2    4096 128 8: 93.5 / 87.6 / 90.1     1024 128 48: 131.5 / 125.6 / 146.8
+// slower at every shape): 4 or 8. Microseconds for 4 / 8 (the walking kernel in brackets), B L H:
+//   1024 128 32: 87.3 / 91.5 (96.2)    256 512 32: 89.8 / 86.0 (101.1)    16 8192 32: 89.4 / 87.1 (99.9)
+//   512 128 64: 91.6 / 90.2 (95.2)     16 8192 64: 167.5 / 170.6 (181.5)  64 2048 128: 336.1 / 338.3 (370.4)
+//   256 128 128: 87.7 / 90.1 (114.2)   4096 128 8: 92.9 / 88.1 (90.1)     1024 128 48: 132.9 / 125.3 (146.8)
 // ==========================================================================================
 template <class E, int kW, bool kQkv, bool kF32>
 __global__ __launch_bounds__(64 * kW) __attribute__((amdgpu_waves_per_eu(SPEAR_FUSED_TILE_WAVES_PER_EU)))
@@ -1036,10 +1063,9 @@ void phalanx_mix_fwd_tile_kernel(const uint16_t* __restrict__ a_logit, const uin
 
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const unsigned wg = tile_workgroup<SPEAR_FUSED_TILE_XCD_GROUP * 4 / kW>();
-  const int og = (int)(wg % (unsigned)oct_groups);
-  const unsigned tt = wg / (unsigned)oct_groups;
-  const int tile = (int)(tt % (unsigned)tiles);
-  const long brow = tt / (unsigned)tiles;
+  const TilePlace at = tile_place(wg, tiles, oct_groups);
+  const int og = at.og, tile = at.tile;
+  const long brow = at.brow;
   const int o = wave % octs_w, bl = wave / octs_w;  // octs_w * nb_w == kW
   const int ho = (og * octs_w + o) * kHeadsPerWave;
   const int t0 = (tile * nb_w + bl) * kTile;
@@ -1304,7 +1330,8 @@ TileGrid tile_grid(long B, int H, int L, int octs_w, int waves) {
   g.nb_w = waves / octs_w;
   g.oct_groups = octs / octs_w;
   g.tiles = (nb + g.nb_w - 1) / g.nb_w;
-  g.wgs = B * g.tiles * g.oct_groups;
+  const int tg = g.tiles < SPEAR_FUSED_TILE_TIME_GROUP ? g.tiles : SPEAR_FUSED_TILE_TIME_GROUP;  // tile_place()
+  g.wgs = B * (long)((g.tiles + tg - 1) / tg) * tg * g.oct_groups;
   return g;
 }
 
@@ -1321,9 +1348,10 @@ void launch_mix_fwd_tile(const MixArgs& p, hipStream_t s) {
 
 hipError_t fused_mix_forward(const MixArgs& p, hipStream_t s) {
   if (p.tile_split) {  // the caller has checked: a grid that fits
-    // workgroups of 8 wavefronts on long rows and on rows of one head group, of 4 otherwise (table at the kernel)
+    // workgroups of 8 wavefronts on rows of one head group and on long rows of up to 32 heads, of 4 otherwise
+    // (table at the kernel)
     static const int waves_override = env_override("SPEAR_BTP_FUSED_FWD_TILE_WAVES");
-    const bool eight = waves_override ? waves_override == 8 : (p.L >= 512 || p.H < 16);
+    const bool eight = waves_override ? waves_override == 8 : (p.H < 16 || (p.L >= 512 && p.H <= 32));
     auto by_form = [&](auto e, auto q) {
       using E = decltype(e);
       if (p.f32_out) launch_mix_fwd_tile<E, 4, decltype(q)::value, true>(p, s);  // check mode: one instance per form
@@ -1389,12 +1417,9 @@ void launch_mix_bwd(const MixBwdArgs& p, const MixPlan& m, hipStream_t s) {
                      p.ld_dv ? p.ld_dv : p.H * kChan, p.L, p.H, p.kv_groups, m.chunk_blocks * kTile, m.chunks, total);
 }
 
-// 1 head group x 4 blocks (two of four wavefronts read a halo) or 2 x 2 (all four do, but a workgroup reads
-// 512-byte runs): over 14 shapes the first is 1.5-3.5 % faster up to 64 heads, the second 0.5-1.5 % from 128 on
-TileGrid bwd_tile_grid(long B, int H, int L) {
-  const int octs = (H + 7) / 8;
-  return tile_grid(B, H, L, (octs % 2 == 0 && H >= 128) ? 2 : 1, kTileWaves);
-}
+// 1 head group x 4 blocks per workgroup (two of four wavefronts read a halo). 2 x 2 (all four do, but a workgroup
+// reads 512-byte runs) is 2-9 % slower at 12 of 14 shapes and equal at the other two.
+TileGrid bwd_tile_grid(long B, int H, int L) { return tile_grid(B, H, L, 1, kTileWaves); }
 
 template <class E, bool kQkv, bool kF32 = false, bool kSums = false>
 void launch_mix_bwd_tile(const MixBwdArgs& p, hipStream_t s) {

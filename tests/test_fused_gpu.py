@@ -118,7 +118,7 @@ def test_fused_backward_column_sums_match_oracle(B, L, H, Hkv, tile_split):
     """The partial sums the backward kernel leaves add up to the oracle's gradients summed over batch and
     time (the bias gradients of proj_a, proj_b, proj_c); the gradients themselves are unchanged by asking. A call
     that names no split gets them from the walking kernel, one that asks for the tile split from that (one row
-    per workgroup, i.e. per 64 or 32 time steps, instead of one per chunk)."""
+    per workgroup, i.e. per 64 time steps, instead of one per chunk)."""
     from spear_amd import _btp
 
     a, b, c, v = make_mix_inputs(B, L, H, Hkv, seed=5000 + L + H)
@@ -130,7 +130,7 @@ def test_fused_backward_column_sums_match_oracle(B, L, H, Hkv, tile_split):
     rows = _btp.mix_backward_sum_rows(B, L, H, tile_split)
     assert rows >= B and rows % B == 0
     if tile_split:
-        assert rows == B * -(-(L // 16) // (2 if H >= 128 else 4))
+        assert rows == B * -(-(L // 16) // 4)
     else:
         assert rows == _btp.mix_backward_sum_rows(B, L, H)
     sums = tuple(torch.full((rows, w), float("nan"), device=DEV) for w in (H, Hkv * 16, Hkv * 16))
