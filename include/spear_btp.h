@@ -124,8 +124,8 @@ int spear_phalanx_mix_forward(const void* a_logit, const void* b_logit, const vo
  * wavefront per 16-step block, the carries handed between neighbouring blocks through LDS. WALK: wavefronts
  * that walk through time. Forward: the same bits from both. Backward: the same results up to fp32 rounding.
  * With neither flag the tile split serves every call except a backward with column sums, whose arrays the
- * caller has sized for the walking kernel (backward: 166-167 us against 185-196 us at B=1024 L=128 H=32, 342
- * against 367 us at B=16 L=8192 H=64, 705 against 757 us at B=64 L=2048 H=128);
+ * caller has sized for the walking kernel (backward: 163 us against 185-196 us at B=1024 L=128 H=32, 322
+ * against 367 us at B=16 L=8192 H=64, 644-669 against 757 us at B=64 L=2048 H=128);
  * SPEAR_BTP_FUSED_FWD / SPEAR_BTP_FUSED_BWD = walk or tile in the environment change that default. The two
  * flags exclude each other. */
 #define SPEAR_MIX_TILE_SPLIT 0x4u

@@ -564,8 +564,8 @@ __global__ __launch_bounds__(64 * kWaves) void phalanx_mix_bwd_kernel(
 // ==========================================================================================
 // Backward of the fused mixing stage, tile form (SPEAR_MIX_TILE_SPLIT; what a call without a split flag runs
 // unless it asks for column sums): the same mathematics with a different work split. Measured against the walking
-// kernel above at B=1024 L=128 H=32 it takes 166-167 us against 185-196 us, at B=16 L=8192 H=64 342 against 367 us,
-// at B=64 L=2048 H=128 705 against 757 us. One
+// kernel above at B=1024 L=128 H=32 it takes 163 us against 185-196 us, at B=16 L=8192 H=64 322 against 367 us,
+// at B=64 L=2048 H=128 644-669 against 757 us. One
 // wavefront owns ONE 16-step block of 128 features and runs no loop: every load is issued at the start, every
 // store at the end, and a workgroup (4 wavefronts = octs_w head groups x nb_w consecutive blocks of one batch
 // row) lives for a few microseconds. Copy loops with this kernel's traffic show why: wavefronts that walk
