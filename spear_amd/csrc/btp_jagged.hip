@@ -363,19 +363,21 @@ __global__ __launch_bounds__(256) void jagged_step_kernel(const JagStepArgs p, l
   typedef typename Oct<S>::type st_t;
 
   const StepScalars s = step_scalars(p, row);
-  float h[8], x[8], cp[8], y[8];
+  float h[8], x[8], cp[8], y[8], c[8], v[8];
   Oct<S>::get(static_cast<const st_t*>(p.h_in), e, h);
   Oct<S>::get(static_cast<const st_t*>(p.c_prev_in), e, cp);
   Oct<T>::get(static_cast<const elt_t*>(p.x_t), e, x);
+  const bool epilogue = p.c_t != nullptr;  // its two loads go out with the others, ahead of any arithmetic
+  if (epilogue) {
+    Oct<T>::get(static_cast<const elt_t*>(p.c_t), e, c);
+    Oct<T>::get(static_cast<const elt_t*>(p.v_t), e, v);
+  }
 #pragma unroll
   for (int q = 0; q < 8; ++q) {
     h[q] = s.a * h[q] + x[q];
     y[q] = h[q] + s.r_new * cp[q];
   }
-  if (p.c_t != nullptr) {
-    float c[8], v[8];
-    Oct<T>::get(static_cast<const elt_t*>(p.c_t), e, c);
-    Oct<T>::get(static_cast<const elt_t*>(p.v_t), e, v);
+  if (epilogue) {
 #pragma unroll
     for (int q = 0; q < 8; ++q) y[q] = y[q] * c[q] + v[q];
   }
