@@ -567,7 +567,7 @@ __global__ __launch_bounds__(64 * kWaves) void phalanx_mix_bwd_kernel(
 // kernel above at B=1024 L=128 H=32 it takes 163 us against 185-196 us, at B=16 L=8192 H=64 322 against 367 us,
 // at B=64 L=2048 H=128 644-669 against 757 us. One
 // wavefront owns ONE 16-step block of 128 features and runs no loop: every load is issued at the start, every
-// store at the end, and a workgroup (4 wavefronts = octs_w head groups x nb_w consecutive blocks of one batch
+// store at the end, and a workgroup (4 wavefronts = 4 consecutive blocks of one head group of one batch
 // row) lives for a few microseconds. Copy loops with this kernel's traffic show why: wavefronts that walk
 // through time with two register sets reach 0.65 of the HBM peak whatever the chunking, short-lived tiles
 // 0.71-0.74 (reads and writes do not overlap on the memory bus, so what counts is how quickly a wavefront
@@ -641,13 +641,13 @@ struct TilePlace {
   int og, tile;
   long brow;
 };
-__device__ __forceinline__ TilePlace tile_place(unsigned wg, int tiles, int oct_groups) {
+__device__ __forceinline__ TilePlace tile_place(unsigned wg, int tiles, int octs) {
   const unsigned tg = min((unsigned)SPEAR_FUSED_TILE_TIME_GROUP, (unsigned)tiles);
   const unsigned tgroups = ((unsigned)tiles + tg - 1) / tg;
   const unsigned t_lo = wg % tg, r1 = wg / tg;
   TilePlace p;
-  p.og = (int)(r1 % (unsigned)oct_groups);
-  const unsigned r2 = r1 / (unsigned)oct_groups;
+  p.og = (int)(r1 % (unsigned)octs);
+  const unsigned r2 = r1 / (unsigned)octs;
   p.tile = (int)((r2 % tgroups) * tg + t_lo);
   p.brow = r2 / tgroups;
   return p;
@@ -676,7 +676,7 @@ void phalanx_mix_bwd_tile_kernel(
     const uint16_t* __restrict__ v_in, const uint16_t* __restrict__ dout, uint16_t* __restrict__ da_logit,
     uint16_t* __restrict__ db_logit, uint16_t* __restrict__ dc, uint16_t* __restrict__ dv, float* __restrict__ sum_da,
     float* __restrict__ sum_db, float* __restrict__ sum_dc, int ld_da, int ld_db, int ld_dc, int ld_dv, int L, int H,
-    int kv_groups, int octs_w, int nb_w, int tiles, int oct_groups) {
+    int kv_groups, int tiles) {
   // per wavefront: decay of its block, product of the block's other decays per step, decay of the block beyond the edge
   __shared__ __align__(16) float gate_tiles[kTileWaves][3][kHeadsPerWave * kGateRow];
   __shared__ float2 carry_out[kTileWaves][2][64];  // [0] dC_out, [1] c_out of the wavefront's block, per lane
@@ -684,15 +684,14 @@ void phalanx_mix_bwd_tile_kernel(
 
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const unsigned wg = tile_workgroup();
-  const TilePlace at = tile_place(wg, tiles, oct_groups);
-  const int og = at.og, tile = at.tile;
-  const long brow = at.brow;
-  const int o = wave % octs_w, bl = wave / octs_w;  // octs_w * nb_w == kTileWaves
+  constexpr int nb_w = kTileWaves;  // consecutive blocks per workgroup, one per wavefront, all of one head group
   const int octs = (H + kHeadsPerWave - 1) / kHeadsPerWave;
-  const int ho = (og * octs_w + o) * kHeadsPerWave;
+  const TilePlace at = tile_place(wg, tiles, octs);
+  const int tile = at.tile, bl = wave;
+  const long brow = at.brow;
+  const int ho = at.og * kHeadsPerWave;
   const int t0 = (tile * nb_w + bl) * kTile;
   const bool valid = ho < H && t0 < L;  // wave-uniform; a wavefront without a block only joins the barrier
-  (void)octs;
 
   const int head_local = lane >> 3;
   const bool real = ho + head_local < H;
@@ -877,13 +876,13 @@ void phalanx_mix_bwd_tile_kernel(
     return;
   }
 
-  if (bl > 0) {  // the block before this one belongs to the wavefront octs_w places down
-    const float2 q = carry_out[wave - octs_w][1][lane];
+  if (bl > 0) {  // the block before this one belongs to the wavefront before this one
+    const float2 q = carry_out[wave - 1][1][lane];
     cin0 = q.x;
     cin1 = q.y;
   }
   if (bl < nb_w - 1 && t0 + kTile < L) {
-    const float2 q = carry_out[wave + octs_w][0][lane];
+    const float2 q = carry_out[wave + 1][0][lane];
     dC0 = q.x;
     dC1 = q.y;
   }
@@ -1019,11 +1018,11 @@ void phalanx_mix_bwd_tile_kernel(
     block_sums[wave][3][lane] = acc_c1;
     block_sums[wave][4][lane] = acc_a;
     __syncthreads();
-    if (bl == 0) {  // the first block's wavefront of each head group adds the tile's blocks, in block order
+    if (bl == 0) {  // the first block's wavefront adds the tile's blocks, in block order
       float t[5] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
       for (int j = 0; j < nb_w && t0 + j * kTile < L; ++j) {
 #pragma unroll
-        for (int q = 0; q < 5; ++q) t[q] += block_sums[wave + j * octs_w][q][lane];
+        for (int q = 0; q < 5; ++q) t[q] += block_sums[j][q][lane];
       }
       const long row = brow * tiles + tile;
       if (real && (lane & 7) == 0) sum_da[row * H + head] = t[4];
@@ -1057,17 +1056,17 @@ __global__ __launch_bounds__(64 * kW) __attribute__((amdgpu_waves_per_eu(SPEAR_F
 void phalanx_mix_fwd_tile_kernel(const uint16_t* __restrict__ a_logit, const uint16_t* __restrict__ b_logit,
                                  const uint16_t* __restrict__ c_in, const uint16_t* __restrict__ v_in,
                                  uint16_t* __restrict__ out, float* __restrict__ c_prev_tail, int L, int H,
-                                 int kv_groups, int octs_w, int nb_w, int tiles, int oct_groups) {
+                                 int kv_groups, int tiles) {
   __shared__ __align__(16) float gate_tiles[kW][2][kHeadsPerWave * kGateRow];  // own block, block before the edge
   __shared__ float2 carry_out[kW][64];  // terminal local state of the wavefront's block, per lane
 
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const unsigned wg = tile_workgroup<SPEAR_FUSED_TILE_XCD_GROUP * 4 / kW>();
-  const TilePlace at = tile_place(wg, tiles, oct_groups);
-  const int og = at.og, tile = at.tile;
+  constexpr int nb_w = kW;  // consecutive blocks per workgroup, one per wavefront, all of one head group
+  const TilePlace at = tile_place(wg, tiles, (H + kHeadsPerWave - 1) / kHeadsPerWave);
+  const int tile = at.tile, bl = wave;
   const long brow = at.brow;
-  const int o = wave % octs_w, bl = wave / octs_w;  // octs_w * nb_w == kW
-  const int ho = (og * octs_w + o) * kHeadsPerWave;
+  const int ho = at.og * kHeadsPerWave;
   const int t0 = (tile * nb_w + bl) * kTile;
   const bool valid = ho < H && t0 < L;  // wave-uniform; a wavefront without a block only joins the barrier
 
@@ -1180,8 +1179,8 @@ void phalanx_mix_fwd_tile_kernel(const uint16_t* __restrict__ a_logit, const uin
   __syncthreads();  // the kernel's only workgroup barrier; wavefronts without a block arrive here directly
   if (!valid) return;
 
-  if (bl > 0) {  // the block before this one belongs to the wavefront octs_w places down
-    const float2 q = carry_out[wave - octs_w][lane];
+  if (bl > 0) {  // the block before this one belongs to the wavefront before this one
+    const float2 q = carry_out[wave - 1][lane];
     cin0 = q.x;
     cin1 = q.y;
   }
@@ -1318,30 +1317,27 @@ void launch_mix_fwd(const MixArgs& p, const MixPlan& m, hipStream_t s) {
                      p.c_prev_tail, p.L, p.H, p.kv_groups, m.chunk_blocks * kTile, m.chunks, total);
 }
 
-// Tile geometry shared by the tile kernels: head groups x consecutive blocks per workgroup, and the grid.
+// Tile geometry shared by the tile kernels: a workgroup is `waves` consecutive blocks of one head group.
 struct TileGrid {
-  int octs_w, nb_w, oct_groups, tiles;
+  int tiles;  // time tiles per row: one workgroup each per head group
   long wgs;
 };
-TileGrid tile_grid(long B, int H, int L, int octs_w, int waves) {
+TileGrid tile_grid(long B, int H, int L, int waves) {
   const int octs = (H + 7) / 8, nb = L / kTile;
   TileGrid g;
-  g.octs_w = octs_w;
-  g.nb_w = waves / octs_w;
-  g.oct_groups = octs / octs_w;
-  g.tiles = (nb + g.nb_w - 1) / g.nb_w;
+  g.tiles = (nb + waves - 1) / waves;
   const int tg = g.tiles < SPEAR_FUSED_TILE_TIME_GROUP ? g.tiles : SPEAR_FUSED_TILE_TIME_GROUP;  // tile_place()
-  g.wgs = B * (long)((g.tiles + tg - 1) / tg) * tg * g.oct_groups;
+  g.wgs = B * (long)((g.tiles + tg - 1) / tg) * tg * octs;
   return g;
 }
 
 template <class E, int kW, bool kQkv, bool kF32 = false>
 void launch_mix_fwd_tile(const MixArgs& p, hipStream_t s) {
-  const TileGrid g = tile_grid(p.B, p.H, p.L, 1, kW);
+  const TileGrid g = tile_grid(p.B, p.H, p.L, kW);
   hipLaunchKernelGGL((phalanx_mix_fwd_tile_kernel<E, kW, kQkv, kF32>), dim3((unsigned)g.wgs), dim3(64 * kW), 0, s,
                      static_cast<const uint16_t*>(p.a_logit), static_cast<const uint16_t*>(p.b_logit),
                      static_cast<const uint16_t*>(p.c), static_cast<const uint16_t*>(p.v), static_cast<uint16_t*>(p.out),
-                     p.c_prev_tail, p.L, p.H, p.kv_groups, g.octs_w, g.nb_w, g.tiles, g.oct_groups);
+                     p.c_prev_tail, p.L, p.H, p.kv_groups, g.tiles);
 }
 
 }  // namespace
@@ -1419,7 +1415,7 @@ void launch_mix_bwd(const MixBwdArgs& p, const MixPlan& m, hipStream_t s) {
 
 // 1 head group x 4 blocks per workgroup (two of four wavefronts read a halo). 2 x 2 (all four do, but a workgroup
 // reads 512-byte runs) is 2-9 % slower at 12 of 14 shapes and equal at the other two.
-TileGrid bwd_tile_grid(long B, int H, int L) { return tile_grid(B, H, L, 1, kTileWaves); }
+TileGrid bwd_tile_grid(long B, int H, int L) { return tile_grid(B, H, L, kTileWaves); }
 
 template <class E, bool kQkv, bool kF32 = false, bool kSums = false>
 void launch_mix_bwd_tile(const MixBwdArgs& p, hipStream_t s) {
@@ -1430,8 +1426,7 @@ void launch_mix_bwd_tile(const MixBwdArgs& p, hipStream_t s) {
   hipLaunchKernelGGL((phalanx_mix_bwd_tile_kernel<E, kQkv, kF32, kSums>), dim3((unsigned)g.wgs), dim3(64 * kTileWaves), 0,
                      s, u(p.a_logit), u(p.b_logit), u(p.c), u(p.v), u(p.dout), w(p.da_logit), w(p.db_logit), w(p.dc),
                      w(p.dv), p.sum_da, p.sum_db, p.sum_dc, p.ld_da ? p.ld_da : p.H, p.ld_db ? p.ld_db : Fkv,
-                     p.ld_dc ? p.ld_dc : Fkv, p.ld_dv ? p.ld_dv : p.H * kChan, p.L, p.H, p.kv_groups, g.octs_w, g.nb_w,
-                     g.tiles, g.oct_groups);
+                     p.ld_dc ? p.ld_dc : Fkv, p.ld_dv ? p.ld_dv : p.H * kChan, p.L, p.H, p.kv_groups, g.tiles);
 }
 
 }  // namespace
