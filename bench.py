@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the BTP hot path: forward + backward at B=1024, L=128, dim=512 (H=32) bf16.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c3|c4|c5] [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c3|c4|c5] [--no-cpu-baseline] [--no-other-configs]
 
 A step is one forward plus one backward launch through the C ABI on one batch of synthetic
 input that is already resident in HBM. Buffers rotate over several independent sets so that a
@@ -29,11 +29,41 @@ if ROOT not in sys.path:
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
 FWD_BYTES, BWD_BYTES = 66, 102  # per (token, head), bf16 y / dy
 
-# HBM bytes per launch of the dominant (backward) kernel, measured with rocprofv3 --pmc FETCH_SIZE /
-# WRITE_SIZE and scaled by what the same counters read for the copy kernel (x1.9997 / x1.0000);
-# figures and commands are in profiles/btp_kernels_c3_B1024_H32_L128.txt (and the c4 / c5 files beside it). Counters cannot be read
-# from inside this script, so the value is recorded here; it is null for shapes never profiled.
-MEASURED_BWD_TRAFFIC_BYTES = {"c3": 429.0e6, "c4": 873.6e6, "c5": 1736.3e6}
+PROFILES = os.path.join(ROOT, "profiles")
+
+
+def profiled_traffic(config, kernel):
+    """HBM bytes per launch of `kernel` at workload `config`, as rocprofv3 counted them: the 'total MB' column of the
+    kernel's row in the 'HBM traffic per dispatch' table of profiles/btp_kernels_<config>_*.txt (FETCH_SIZE and
+    WRITE_SIZE, each scaled by what the same counter reads for the copy kernel; the commands are in that file).
+    Counters cannot be read from inside this script, so the committed summary is the source; returns
+    (bytes, source) or (None, None) when there is no such file or row."""
+    import glob
+    import re
+
+    for path in sorted(glob.glob(os.path.join(PROFILES, f"btp_kernels_{config}_*.txt"))):
+        in_table, column = False, None
+        with open(path, encoding="utf-8") as fh:
+            for line in fh:
+                if line.startswith("== "):
+                    in_table = line.startswith("== HBM traffic per dispatch")
+                    column = None
+                    continue
+                if not in_table:
+                    continue
+                if line.startswith("kernel ") and "total MB" in line:
+                    # columns after the name: read KiB, alg read, written KiB, alg written, total MB, ratio
+                    column = -2
+                    continue
+                m = re.match(r"^(\S.*?)\s{2,}([-+0-9.eE\s]+)$", line.rstrip())
+                if column is not None and m and m.group(1) == kernel:
+                    fields = m.group(2).split()
+                    if len(fields) == 6:
+                        rel = os.path.relpath(path, ROOT)
+                        return float(fields[column]) * 1e6, {"file": rel, "table": "HBM traffic per dispatch",
+                                                              "row": kernel, "column": "total MB"}
+    return None, None
+
 
 CONFIGS = {
     # name: (B, H, L, seed, x_std, gate)
@@ -111,6 +141,7 @@ def main() -> int:
     ap.add_argument("--no-fused", action="store_true", help="skip the fused layer-layout forward leg")
     ap.add_argument("--no-streaming", action="store_true", help="skip the prefill / decode-step leg")
     ap.add_argument("--no-layer", action="store_true", help="skip the whole-layer (projections + mixing) leg")
+    ap.add_argument("--no-other-configs", action="store_true", help="skip the legs at the other full-size configurations")
     ap.add_argument("--settle-seconds", type=float, default=0.3, help="untimed run-in before the warm-up steps")
     args = ap.parse_args()
 
@@ -701,6 +732,112 @@ def main() -> int:
 
     streaming = None if args.no_streaming else guarded(streaming_leg)
 
+    # The other full-size configurations (long rows: B=16 H=64 L=8192; log-space stress: B=64 H=128 L=2048), each
+    # timed in this same run: stand-alone forward, backward and forward+backward step, and the fused layer-layout
+    # forward / backward on tensors of the same size. Three rotating buffer sets (2.3-12 GiB: nothing is served
+    # from the 256 MiB memory-side cache), inputs drawn on the device with the configurations' distributions
+    # (values do not change the time), HIP events on the launch stream.
+    def other_config_leg(name, n_sets=3, n_steps=40):
+        Bc, Hc, Lc, seed_c, x_std_c, gate_c = CONFIGS[name]
+        gd = torch.Generator(device=dev).manual_seed(seed_c)
+        Fc = Hc * 16
+
+        def draw_gate():
+            if gate_c == "sigmoid":
+                return -torch.nn.functional.softplus(torch.randn(Bc, Hc, Lc, device=dev, generator=gd))
+            forget = torch.rand(Bc, Hc, 1, device=dev, generator=gd) < 0.5
+            lo = -20.0 + 15.0 * torch.rand(Bc, Hc, Lc, device=dev, generator=gd)
+            hi = -1e-4 * torch.rand(Bc, Hc, Lc, device=dev, generator=gd)
+            return torch.where(forget, lo, hi)
+
+        def timed(fn, pool):
+            for i in range(4):
+                fn(pool[i % len(pool)])
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(stream)
+            for i in range(n_steps):
+                fn(pool[i % len(pool)])
+            e1.record(stream)
+            torch.cuda.synchronize()
+            return e0.elapsed_time(e1) / n_steps
+
+        pool = []
+        for _ in range(n_sets):
+            pool.append({
+                "coeff": torch.exp(draw_gate()).to(torch.bfloat16),
+                "x": (torch.randn(Bc, Hc, 16, Lc, device=dev, generator=gd) * x_std_c).to(torch.bfloat16),
+                "dy": torch.randn(Bc, Hc, 16, Lc, device=dev, generator=gd).to(torch.bfloat16),
+                "y": torch.empty(Bc, Hc, 16, Lc, device=dev, dtype=torch.bfloat16),
+                "dx": torch.empty(Bc, Hc, 16, Lc, device=dev, dtype=torch.bfloat16),
+                "dA": torch.empty(Bc, Hc, Lc, device=dev, dtype=torch.float32),
+            })
+
+        def fwd_c(s):
+            rc = lib.spear_btp_forward(s["coeff"].data_ptr(), s["x"].data_ptr(), s["y"].data_ptr(), None,
+                                       Bc, Hc, Lc, 2, 0, 0, 0, sp)
+            assert rc == 0, lib.spear_btp_last_error()
+
+        def bwd_c(s):
+            rc = lib.spear_btp_backward(s["coeff"].data_ptr(), s["x"].data_ptr(), s["dy"].data_ptr(), None,
+                                        s["dx"].data_ptr(), s["dA"].data_ptr(), Bc, Hc, Lc, 2, 0, 0, 0, sp)
+            assert rc == 0, lib.spear_btp_last_error()
+
+        def step_c(s):
+            fwd_c(s)
+            bwd_c(s)
+
+        units_c = Bc * Hc * Lc
+        f_ms, b_ms, s_ms = timed(fwd_c, pool), timed(bwd_c, pool), timed(step_c, pool)
+        frac = lambda nbytes_, ms: nbytes_ / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS
+        res = {
+            "workload": f"B={Bc} H={Hc} L={Lc} bf16, {n_sets} buffer sets, {n_steps} timed launches each",
+            "forward_ms": f_ms, "forward_frac": frac(units_c * FWD_BYTES, f_ms),
+            "backward_ms": b_ms, "backward_frac": frac(units_c * BWD_BYTES, b_ms),
+            "step_ms": s_ms, "step_frac": frac(units_c * (FWD_BYTES + BWD_BYTES), s_ms),
+            "tokens_per_s": Bc * Lc / (s_ms * 1e-3),
+            "backward_traffic": profiled_traffic(name, "bwd_scan")[0],
+        }
+        del pool
+        torch.cuda.empty_cache()
+
+        if Hc % 4 == 0:
+            mpool = []
+            for _ in range(n_sets):
+                m = {"a": torch.randn(Bc, Lc, Hc, device=dev, generator=gd).to(torch.bfloat16)}
+                for k_ in ("b", "c", "v", "dout"):
+                    m[k_] = torch.randn(Bc, Lc, Fc, device=dev, generator=gd).to(torch.bfloat16)
+                for k_ in ("out", "db", "dc", "dv"):
+                    m[k_] = torch.empty(Bc, Lc, Fc, device=dev, dtype=torch.bfloat16)
+                m["da"] = torch.empty(Bc, Lc, Hc, device=dev, dtype=torch.bfloat16)
+                mpool.append(m)
+
+            def mix_c(s):
+                rc = lib.spear_phalanx_mix_forward(s["a"].data_ptr(), s["b"].data_ptr(), s["c"].data_ptr(),
+                                                   s["v"].data_ptr(), s["out"].data_ptr(), Bc, Lc, Hc, Hc, 0, 0, sp)
+                assert rc == 0, lib.spear_btp_last_error()
+
+            def mix_bwd_c(s):
+                rc = lib.spear_phalanx_mix_backward(s["a"].data_ptr(), s["b"].data_ptr(), s["c"].data_ptr(),
+                                                    s["v"].data_ptr(), s["dout"].data_ptr(), s["da"].data_ptr(),
+                                                    s["db"].data_ptr(), s["dc"].data_ptr(), s["dv"].data_ptr(),
+                                                    Bc, Lc, Hc, Hc, 0, 0, sp)
+                assert rc == 0, lib.spear_btp_last_error()
+
+            mf_ms, mb_ms = timed(mix_c, mpool), timed(mix_bwd_c, mpool)
+            res["fused_forward_ms"], res["fused_forward_frac"] = mf_ms, frac(units_c * 130, mf_ms)
+            res["fused_backward_ms"], res["fused_backward_frac"] = mb_ms, frac(units_c * 228, mb_ms)
+            del mpool
+            torch.cuda.empty_cache()
+        return res
+
+    other_configs = {"what": "the other full-size configurations in the same run: stand-alone kernels (66 + 102 B per "
+                             "(token, head)) and the fused layer-layout kernels (130 + 228 B); fractions of 8 TB/s"}
+    if not args.no_other_configs:
+        for name in sorted(CONFIGS):
+            if name != args.config:
+                other_configs[name] = guarded(lambda name=name: other_config_leg(name))
+
     # what a caller of the public op gets: y = btp(coeff, x); y.backward(dy) through autograd, torch.library
     # dispatch and the compiled binding, eager (host-bound on small shapes) and as a HIP-graph replay of the
     # same two ops, at this shape and at the batch of configuration 1 (B = 8)
@@ -770,6 +907,8 @@ def main() -> int:
 
     public_op = guarded(public_op_leg)
 
+    traffic_bytes, traffic_source = profiled_traffic(args.config, "bwd_scan")
+
     units = B * H * L
     tokens = B * L
     bwd_gbps = units * BWD_BYTES / (bwd_ms * 1e-3) / 1e9
@@ -802,7 +941,8 @@ def main() -> int:
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
             "frac": bwd_gbps / HBM_PEAK_GBPS,
-            "traffic": MEASURED_BWD_TRAFFIC_BYTES.get(args.config),
+            "traffic": traffic_bytes,
+            "traffic_source": traffic_source,
             "avg_launch_ms": bwd_ms,
             "algorithmic_bytes_per_launch": units * BWD_BYTES,
         },
@@ -852,6 +992,7 @@ def main() -> int:
             },
         },
         "public_op": public_op,
+        "other_configs": other_configs,
     }
     if not args.no_cpu_baseline:
         base = cpu_baseline(B, H, L, seed, x_std, gate)

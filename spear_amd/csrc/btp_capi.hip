@@ -318,11 +318,17 @@ int spear_phalanx_mix_step(const void* a_logit, const void* b_logit, const void*
   if (flags != 0u) return fail(SPEAR_BTP_EINVAL, "%s: unknown flag bits 0x%x", who, flags);
   if ((long long)B * H * 16ll >= (1ll << 40)) return fail(SPEAR_BTP_EINVAL, "%s: tensor too large", who);
   if ((long long)B * H == 0) return 0;
-  const void* ptrs[] = {a_logit, b_logit, c, v, out, h, r, c_prev};
-  for (const void* q : ptrs) {
+  // b_logit, c, v, out, h and c_prev move as 16-byte pieces; a_logit is read one 16-bit element and r one
+  // fp32 element at a time, so a row of a [tokens, B, H] tensor (any B * H) can be passed as it lies
+  const void* wide[] = {b_logit, c, v, out, h, c_prev};
+  if (!a_logit || !r) return fail(SPEAR_BTP_ENULL, "%s: NULL tensor pointer", who);
+  for (const void* q : wide) {
     if (!q) return fail(SPEAR_BTP_ENULL, "%s: NULL tensor pointer", who);
-    if (!aligned16(q)) return fail(SPEAR_BTP_EINVAL, "%s: tensor pointers must be 16-byte aligned", who);
+    if (!aligned16(q))
+      return fail(SPEAR_BTP_EINVAL, "%s: b_logit, c, v, out, h and c_prev must be 16-byte aligned", who);
   }
+  if (reinterpret_cast<uintptr_t>(a_logit) & 1u) return fail(SPEAR_BTP_EINVAL, "%s: a_logit must be 2-byte aligned", who);
+  if (reinterpret_cast<uintptr_t>(r) & 3u) return fail(SPEAR_BTP_EINVAL, "%s: r must be 4-byte aligned", who);
   if (pos && (reinterpret_cast<uintptr_t>(pos) & 3u)) return fail(SPEAR_BTP_EINVAL, "%s: pos must be 4-byte aligned", who);
   spear_btp::MixStepArgs a{a_logit, b_logit, c, v, out, h, r, c_prev, pos, boundary ? 1 : 0, block_len, B, H, H / kv_heads, dtype};
   const hipError_t err = spear_btp::fused_mix_step(a, static_cast<hipStream_t>(stream));

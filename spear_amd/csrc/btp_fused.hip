@@ -1525,29 +1525,27 @@ __global__ __launch_bounds__(64 * kSumWaves) void finish_column_sums_kernel(SumJ
   }
 }
 
-// Device address of `scratch` on the current device, looked up once per device.
+// Device address of `scratch` on the current device, looked up until it succeeds once per device. A failed
+// lookup (a first call that arrives while its stream is being captured, say) is reported and not remembered:
+// the next call on that device tries again.
 constexpr int kMaxDevices = 64;
-struct ScratchSlot {
-  std::once_flag once;
-  float* ptr = nullptr;
-  hipError_t err = hipSuccess;
-};
-ScratchSlot g_scratch[kMaxDevices];
+std::mutex g_scratch_mutex;
+float* g_scratch_ptr[kMaxDevices] = {};
 
 hipError_t scratch_of_current_device(float** out) {
   int dev = -1;
   hipError_t err = hipGetDevice(&dev);
   if (err != hipSuccess) return err;
   if (dev < 0 || dev >= kMaxDevices) return hipErrorInvalidDevice;
-  ScratchSlot& slot = g_scratch[dev];
-  std::call_once(slot.once, [&slot] {
+  std::lock_guard<std::mutex> hold(g_scratch_mutex);
+  if (g_scratch_ptr[dev] == nullptr) {
     void* p = nullptr;
-    slot.err = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
-    slot.ptr = slot.err == hipSuccess ? static_cast<float*>(p) : nullptr;
-  });
-  if (slot.err != hipSuccess) return slot.err;
-  if (slot.ptr == nullptr) return hipErrorInvalidSymbol;
-  *out = slot.ptr;
+    err = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (err != hipSuccess) return err;
+    if (p == nullptr) return hipErrorInvalidSymbol;
+    g_scratch_ptr[dev] = static_cast<float*>(p);
+  }
+  *out = g_scratch_ptr[dev];
   return hipSuccess;
 }
 

@@ -313,6 +313,8 @@ def phalanx_step(layer, x_t: torch.Tensor, state: PhalanxStepState, out: torch.T
     apart, so the call can be recorded into a HIP graph (``torch.cuda.graph``) with fixed ``x_t`` / ``out``
     buffers and replayed once per token."""
     _need_gpu(x_t, state.h_loc)
+    if layer.k != 2:  # a k = 1 layer has no carry between blocks; this step always applies the one-hop carry
+        raise RuntimeError("phalanx_step needs a layer with k == 2")
     p = layer.param
     xc = x_t.to(p.compute_dtype)
     a, b, c, v = p.proj_a(xc), p.proj_b(xc), p.proj_c(xc), p.proj_v(xc)

@@ -218,6 +218,8 @@ def btp(
         assert x.dim() == 4 and x.shape[2] == DH, f"Channel dimension must be {DH}"
         assert x.shape[3] % BLK == 0, f"Length L must be multiple of {BLK}"
         assert wpb_val in SUPPORTED_WPB, f"WPB must be one of {SUPPORTED_WPB}"
+        if out_dtype not in (torch.float32, x.dtype):  # the binding's own check (csrc/btp/_bindings.cu:33)
+            raise RuntimeError("y must be float32 or match x dtype.")
         return _btp.load_extension().btp_autograd(
             coeff, x, int(k), int(wpb_val), out_dtype == torch.float32, _FORWARD_FLAGS,
             _btp.FLAG_PATH_MFMA if _PATH_MFMA else 0,

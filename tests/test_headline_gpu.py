@@ -106,6 +106,45 @@ def test_full_size_properties(name):
         assert (err <= 1e-4 + 2.0 ** -15 * magnitude).all(), f"dA mfma[{b},{h}]: {err.max():.3e}"
 
 
+def test_every_row_of_the_headline_shape_against_the_oracle():
+    """All 32,768 (batch, head) rows of B=1024 H=32 L=128, not a sample: fp32 `y`, unrounded `dx` (check mode) and
+    `dA` within 1e-4, bf16 `y` and `dx` within 2e-2 of the float64 oracle run on the same bf16-rounded inputs
+    (the protocol of spear/ops/btp/runners.py:103-164), the oracle called on 64 batch rows at a time."""
+    from spear_amd import _btp
+
+    cfg = CONFIGS["c3_B1024_H32_L128"]
+    B, H, L = cfg["B"], cfg["H"], cfg["L"]
+    print("c3 all rows: generating inputs", flush=True)
+    coeff, x, dy = make_inputs(B, H, L, cfg["seed"], x_std=cfg["x_std"], gate=cfg["gate"])
+    c, xx, g = coeff.to(DEV), x.to(DEV), dy.to(DEV)
+    y32 = _fwd(c, xx, out_dtype=torch.float32)
+    y16 = _fwd(c, xx)
+    dx16, dA = _bwd(c, xx, g)
+    dx32 = torch.empty(B, H, 16, L, device=DEV, dtype=torch.float32)
+    dA_check = torch.empty(B, H, L, device=DEV, dtype=torch.float32)
+    ck = torch.empty(0, device=DEV, dtype=torch.float32)
+    _btp.backward(c, xx, g, ck, dx32, dA_check, 2, 32, flags=_btp.FLAG_DX_F32)
+    torch.cuda.synchronize()
+    assert torch.equal(dA_check, dA) and torch.equal(dx32.to(torch.bfloat16), dx16)
+    got = {name: t.cpu() for name, t in (("y32", y32), ("y16", y16), ("dx16", dx16), ("dx32", dx32), ("dA", dA))}
+    del y32, y16, dx16, dx32, dA, dA_check
+    worst = {name: 0.0 for name in got}
+    step = 64
+    for b0 in range(0, B, step):
+        if b0 % 256 == 0:
+            print(f"c3 all rows: oracle on batch rows {b0}..", flush=True)
+        sl = slice(b0, b0 + step)
+        a_, x_, g_ = f64(coeff[sl]), f64(x[sl]), f64(dy[sl])
+        ry = orc.forward(a_, x_)
+        rdx, rdA = orc.backward(a_, x_, g_)
+        for name, ref, atol, rtol in (("y32", ry, F32_ATOL, F32_RTOL), ("y16", ry, BF16_ATOL, BF16_RTOL),
+                                      ("dx32", rdx, F32_ATOL, F32_RTOL), ("dx16", rdx, BF16_ATOL, BF16_RTOL),
+                                      ("dA", rdA, F32_ATOL, F32_RTOL)):
+            assert_close(f64(got[name][sl]), ref, atol, rtol, f"{name}[{b0}:{b0 + step}]")
+            worst[name] = max(worst[name], float(np.abs(f64(got[name][sl]) - ref).max()))
+    print("c3 all rows: max |err| " + ", ".join(f"{k} {v:.2e}" for k, v in worst.items()), flush=True)
+
+
 def _free_gib():
     free, _ = torch.cuda.mem_get_info()
     return free / 2**30

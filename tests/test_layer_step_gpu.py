@@ -75,16 +75,19 @@ def _layer(dim=128, kv_heads=None, seed=3):
     return Phalanx(dim=dim, length=64, method="fused", dtype=torch.bfloat16, kv_heads=kv_heads).to(DEV)
 
 
-@pytest.mark.parametrize("L,kv_heads", [(48, None), (37, 2), (16, None), (5, None)])
-def test_stepping_a_layer_equals_its_forward_and_prefill_hands_over(L, kv_heads):
+# (dim 64, B 1) and (dim 192, B 3): the rows a[t] of the tail's [tokens, B, H] logits start on 8- and 2-byte
+# boundaries there (B * H * 2 bytes per token is not a multiple of 16)
+@pytest.mark.parametrize("L,kv_heads,dim,B", [(48, None, 128, 3), (37, 2, 128, 3), (16, None, 128, 3), (5, None, 128, 3),
+                                              (37, None, 64, 1), (37, None, 192, 3), (29, 6, 192, 1)])
+def test_stepping_a_layer_equals_its_forward_and_prefill_hands_over(L, kv_heads, dim, B):
     """Token t of phalanx_step equals position t of the layer's forward on the whole sequence (both run the same
     projections; the mixing stage is the fused kernel there and the step kernel here), and prefill(first part) +
     steps continues exactly like stepping from the start."""
     from spear_amd.nn.phalanx.inference import PhalanxStepState, phalanx_prefill, phalanx_step
 
-    layer = _layer(kv_heads=kv_heads)
-    B, n_more = 3, 21
-    x = torch.randn(B, L + n_more, 128, generator=torch.Generator().manual_seed(L)).bfloat16().to(DEV)
+    layer = _layer(dim=dim, kv_heads=kv_heads)
+    n_more = 21
+    x = torch.randn(B, L + n_more, dim, generator=torch.Generator().manual_seed(L)).bfloat16().to(DEV)
     Lw = ((L + n_more) // 16) * 16
     with torch.no_grad():
         whole = layer(x[:, :Lw]).float()                     # forward needs whole blocks
@@ -95,7 +98,7 @@ def test_stepping_a_layer_equals_its_forward_and_prefill_hands_over(L, kv_heads)
     assert float((stepped[:, :Lw] - whole).abs().max()) <= 2e-2 * scale
 
     y, st = phalanx_prefill(layer, x[:, :L])
-    assert y.shape == (B, L, 128)
+    assert y.shape == (B, L, dim)
     assert float((y.float() - stepped[:, :L]).abs().max()) <= 2e-2 * scale
     # the prefill projects the prompt as one matrix product and stepping projects token by token: the library may
     # sum those in another order, so the two states agree to the 16-bit rounding of the projections, not bit for bit

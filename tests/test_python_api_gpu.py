@@ -82,6 +82,19 @@ def test_eager_calls_run_the_compiled_autograd_node_with_the_results_of_the_pyth
     assert "_BTPFunction" in y_mode.grad_fn.name() and torch.equal(y_mode, y_node)
 
 
+def test_an_output_dtype_the_binding_does_not_take_raises_on_every_route():
+    """float16 results from bfloat16 inputs: the reference's binding refuses (csrc/btp/_bindings.cu:33), and so do the
+    compiled node, the Python node and the inference route."""
+    from spear_amd import btp
+
+    coeff, x, _ = make_inputs(1, 4, 32, seed=47)
+    c, xx = coeff.to(DEV), x.to(DEV)
+    with pytest.raises(RuntimeError, match="y must be float32 or match x dtype"):
+        btp(c.clone().requires_grad_(True), xx, output_dtype=torch.float16)
+    with pytest.raises(RuntimeError, match="y must be float32 or match x dtype"):
+        btp(c, xx, output_dtype=torch.float16)
+
+
 def test_the_op_runs_on_the_matrix_core_kernels_on_request(monkeypatch):
     """SPEAR_BTP_PATH=mfma (read when the module is imported; set on the module here) sends btp() through the
     matrix-core forward and backward."""

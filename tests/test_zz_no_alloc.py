@@ -39,15 +39,39 @@ def _with_caller_arrays(ins, H, Hkv):
     return grads, sums
 
 
-def _without_allocation(ins, grads, bias, H, Hkv):
-    """The call itself: every buffer it touches exists before it, and the caching allocator must not move."""
+_warmed = False
+
+
+def _warm_up_once():
+    """The process's first call loads the kernels' code object and looks the static array's address up; the
+    driver may take memory for that. One small call beforehand, so that the calls under test are steady-state."""
+    global _warmed
+    if _warmed:
+        return
     from spear_amd import _btp
 
+    ins = _inputs(1, 16, 4, 4, seed=6999)
+    grads = [torch.empty_like(t) for t in ins[:4]]
+    bias = tuple(torch.empty(w, device=DEV) for w in (4, 64, 64))
+    _btp.mix_backward_bias(*ins, *grads, bias, 4, 4)
+    torch.cuda.synchronize()
+    _warmed = True
+
+
+def _without_allocation(ins, grads, bias, H, Hkv):
+    """The call itself: every buffer it touches exists before it. Neither torch's caching allocator (which the
+    C library never uses) nor the device's free memory as the driver reports it (which a hipMalloc or hipFree
+    inside the library would move) may change across the call."""
+    from spear_amd import _btp
+
+    _warm_up_once()
     torch.cuda.synchronize()
     before = torch.cuda.memory_stats(DEV)["allocation.all.allocated"]
+    free_before = torch.cuda.mem_get_info(DEV)[0]
     _btp.mix_backward_bias(*ins, *grads, bias, H, Hkv)
     torch.cuda.synchronize()
     assert torch.cuda.memory_stats(DEV)["allocation.all.allocated"] == before
+    assert torch.cuda.mem_get_info(DEV)[0] == free_before
 
 
 @pytest.mark.parametrize("first,second", [
