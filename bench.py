@@ -396,23 +396,11 @@ def main() -> int:
                                                s["v"].data_ptr(), s["out"].data_ptr(), B, L, H, H, 0, 0, sp)
             assert rc == 0, lib.spear_btp_last_error()
 
-        def mix_walk(s):  # the forward whose wavefronts walk through time (SPEAR_MIX_WALK_SPLIT)
-            rc = lib.spear_phalanx_mix_forward(s["a"].data_ptr(), s["b"].data_ptr(), s["c"].data_ptr(),
-                                               s["v"].data_ptr(), s["out"].data_ptr(), B, L, H, H, 0, 0x8, sp)
-            assert rc == 0, lib.spear_btp_last_error()
-
-        def mix_bwd(s):  # the work split whose wavefronts walk through time (SPEAR_MIX_WALK_SPLIT)
+        def mix_bwd(s):
             rc = lib.spear_phalanx_mix_backward(s["a"].data_ptr(), s["b"].data_ptr(), s["c"].data_ptr(),
                                                 s["v"].data_ptr(), s["dout"].data_ptr(), s["da"].data_ptr(),
                                                 s["db"].data_ptr(), s["dc"].data_ptr(), s["dv"].data_ptr(),
-                                                B, L, H, H, 0, 0x8, sp)
-            assert rc == 0, lib.spear_btp_last_error()
-
-        def mix_bwd_tile(s):  # one wavefront per 16-step block (SPEAR_MIX_TILE_SPLIT), the library's default split
-            rc = lib.spear_phalanx_mix_backward(s["a"].data_ptr(), s["b"].data_ptr(), s["c"].data_ptr(),
-                                                s["v"].data_ptr(), s["dout"].data_ptr(), s["da"].data_ptr(),
-                                                s["db"].data_ptr(), s["dc"].data_ptr(), s["dv"].data_ptr(),
-                                                B, L, H, H, 0, 0x4, sp)
+                                                B, L, H, H, 0, 0, sp)
             assert rc == 0, lib.spear_btp_last_error()
 
         def unfused_stage(a, b, c, v):  # what the layer does around the stand-alone kernel (swr.py)
@@ -468,8 +456,6 @@ def main() -> int:
 
         mix_ms, unfused_ms = kernel_ms_over(mix, msets), kernel_ms_over(mix_unfused, msets)
         mix_bwd_ms, unfused_train_ms = kernel_ms_over(mix_bwd, msets), kernel_ms_over(mix_unfused_train, msets)
-        mix_bwd_tile_ms = kernel_ms_over(mix_bwd_tile, msets)
-        mix_walk_ms = kernel_ms_over(mix_walk, msets)
 
         # what the memory system gives these stream counts in its best shape (contiguous 4 KiB pieces, short-lived
         # wavefronts, nothing shared): 3 inputs -> 1 output (forward) and 4 inputs -> 3 outputs (backward), without
@@ -489,25 +475,20 @@ def main() -> int:
         fused = {
             "avg_launch_ms": mix_ms, "algorithmic_bytes_per_launch": mix_bytes,
             "achieved": mix_bytes / (mix_ms * 1e-3) / 1e9, "frac": mix_bytes / (mix_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
-            # (the library's default work split, one wavefront per 16-step block; the walking kernel beside it)
-            "walking_split_avg_launch_ms": mix_walk_ms,
-            "walking_split_frac": mix_bytes / (mix_walk_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
             "same_stage_from_pytorch_ops_plus_btp_kernel_ms": unfused_ms, "speedup": unfused_ms / mix_ms,
-            "backward": {  # the library's default work split (one wavefront per 16-step block)
-                "avg_launch_ms": mix_bwd_tile_ms, "algorithmic_bytes_per_launch": mix_bwd_bytes,
-                "achieved": mix_bwd_bytes / (mix_bwd_tile_ms * 1e-3) / 1e9,
-                "frac": mix_bwd_bytes / (mix_bwd_tile_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
-                "walking_split_avg_launch_ms": mix_bwd_ms,
-                "walking_split_frac": mix_bwd_bytes / (mix_bwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+            "backward": {
+                "avg_launch_ms": mix_bwd_ms, "algorithmic_bytes_per_launch": mix_bwd_bytes,
+                "achieved": mix_bwd_bytes / (mix_bwd_ms * 1e-3) / 1e9,
+                "frac": mix_bwd_bytes / (mix_bwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
             },
             "ceilings_GBps": {
                 "what": "spear_btp_stream_probe_mix on the same buffers: no arithmetic / with a chain of dependent FMAs (640 forward, 1280 backward)",
                 "forward_3_inputs_1_output": [ceil_fwd, ceil_fwd_c],
                 "backward_4_inputs_3_outputs": [ceil_bwd, ceil_bwd_c],
             },
-            "fwd_plus_bwd_ms": mix_ms + mix_bwd_tile_ms,
+            "fwd_plus_bwd_ms": mix_ms + mix_bwd_ms,
             "same_stage_fwd_plus_bwd_from_pytorch_ops_plus_btp_kernels_ms": unfused_train_ms,
-            "train_speedup": unfused_train_ms / (mix_ms + mix_bwd_tile_ms),
+            "train_speedup": unfused_train_ms / (mix_ms + mix_bwd_ms),
             "qkv_gate_form": {
                 "what": "out = q * btp(exp(gate), k * v) + v on [B, L, H, 16] bf16 with an fp32 log-decay gate; dq, dk, dv, dgate",
                 "forward_ms": qkv_ms, "backward_ms": qkv_bwd_ms, "tokens_per_s": B * L / ((qkv_ms + qkv_bwd_ms) * 1e-3),

@@ -98,8 +98,8 @@ int spear_btp_backward_loggate(const float* gate, const void* x, const void* dy,
  * in [B, L, features] layout (time strided, features contiguous), all in `dtype` (bf16 / fp16):
  *     a_logit [B, L, H]            b_logit, c [B, L, kv_heads * 16]        v, out [B, L, H * 16]
  *     out = btp(sigmoid(a_logit), sigmoid(b_logit) * v) * c + v      (k = 2, fp32 arithmetic)
- * Head h reads b / c of kv head h / (H / kv_heads). Requirements: L % 16 == 0, H % 4 == 0,
- * H % kv_heads == 0, 16-byte aligned pointers. */
+ * Head h reads b / c of kv head h / (H / kv_heads). Requirements: L % 16 == 0, H % kv_heads == 0 (any H >= 1, any
+ * number of heads per kv head, as spear/nn/phalanx/swr.py:37-38 accepts them), 16-byte aligned pointers. */
 int spear_phalanx_mix_forward(const void* a_logit, const void* b_logit, const void* c, const void* v, void* out,
                               int B, int L, int H, int kv_heads, int dtype, unsigned flags, void* stream);
 
@@ -120,22 +120,12 @@ int spear_phalanx_mix_forward(const void* a_logit, const void* b_logit, const vo
  * elements). Inputs keep their types. Not combinable with the column sums of _backward_ex. */
 #define SPEAR_MIX_F32_RESULTS 0x2u
 
-/* Flags for spear_phalanx_mix_forward / _prefill / _backward / _backward_ex: which work split runs. TILE: one
- * wavefront per 16-step block, the carries handed between neighbouring blocks through LDS. WALK: wavefronts
- * that walk through time. Forward: the same bits from both. Backward: the same results up to fp32 rounding.
- * With neither flag the tile split serves every call except a backward with column sums, whose arrays the
- * caller has sized for the walking kernel (backward: 163 us against 185-196 us at B=1024 L=128 H=32, 322
- * against 367 us at B=16 L=8192 H=64, 644-669 against 757 us at B=64 L=2048 H=128);
- * SPEAR_BTP_FUSED_FWD / SPEAR_BTP_FUSED_BWD = walk or tile in the environment change that default. The two
- * flags exclude each other. */
-#define SPEAR_MIX_TILE_SPLIT 0x4u
-#define SPEAR_MIX_WALK_SPLIT 0x8u
-
 /* Backward of spear_phalanx_mix_forward: reads a_logit, b_logit, c, v and the upstream gradient
  * dout [B, L, H * 16]; writes da_logit [B, L, H], db_logit and dc [B, L, kv_heads * 16] (summed over
  * the heads sharing a kv head) and dv [B, L, H * 16] -- every element, no accumulation, all in
- * `dtype`. H / kv_heads must be 1, 2, 4 or 8 (a head group has to sit inside one wavefront's 8
- * heads). It stands for the autograd chain through the ops listed at spear_phalanx_mix_forward; no
+ * `dtype`. Any number of heads per kv head: groups of 1, 2, 4 or 8 heads are summed inside a wavefront (the fast
+ * path), every other group size through LDS in a fixed order (groups of more than 8 heads are worked through 8
+ * heads at a time). It stands for the autograd chain through the ops listed at spear_phalanx_mix_forward; no
  * single counterpart in the reference. */
 int spear_phalanx_mix_backward(const void* a_logit, const void* b_logit, const void* c, const void* v,
                                const void* dout, void* da_logit, void* db_logit, void* dc, void* dv, int B, int L,
@@ -146,22 +136,18 @@ int spear_phalanx_mix_backward(const void* a_logit, const void* b_logit, const v
  * gradient tensors, 0 meaning dense (the tensor's own width). With strides the four can be column blocks of
  * one [B, L, ld] buffer (all four ld equal, the pointers offset into its first row), which is then the
  * gradient of the four projections' concatenated output: one GEMM each for the input and the weight gradient
- * instead of four. A stride is an even number of elements not below the tensor's width; elements between
- * the blocks are not touched.
+ * instead of four. A stride is a number of elements not below the tensor's width, even for db_logit, dc and dv;
+ * elements between the blocks are not touched.
  * (2) It leaves the column sums of da_logit, db_logit and dc -- the bias
  * gradients of the projections that produced a_logit, b_logit and c (spear/nn/phalanx/swr.py:157-163 gives
  * proj_a, proj_b and proj_c a bias) -- so that the caller does not read the three gradients again to
  * sum them. The kernel cannot finish the sums without a second pass, so it leaves partial sums in fp32:
  *     sum_da [sum_rows, H],  sum_db [sum_rows, kv_heads * 16],  sum_dc [sum_rows, kv_heads * 16]
- * where row r sums the time steps of one (batch row, time chunk) and the caller adds the rows up
- * (a few rows per batch row with the walking kernel, one per 64 time steps with the tile split).
- * sum_rows must equal spear_phalanx_mix_backward_sum_rows(B, L, H), or, in a call that asks for the tile
- * split with SPEAR_MIX_TILE_SPLIT (the faster of the two), spear_phalanx_mix_backward_sum_rows_tile(B, L, H);
- * a call with sums and no split flag runs the walking kernel. Every element of the three arrays is written;
- * the sums are taken before the gradients are rounded to `dtype`. All three NULL: no sums. With neither
- * option it is exactly spear_phalanx_mix_backward. */
+ * where row r sums the time steps of one (batch row, tile of 64 time steps) and the caller adds the rows up.
+ * sum_rows must equal spear_phalanx_mix_backward_sum_rows(B, L, H) = B * ceil(L / 64). Every element of the
+ * three arrays is written; the sums are taken before the gradients are rounded to `dtype`. All three NULL: no
+ * sums. With neither option it is exactly spear_phalanx_mix_backward. */
 long long spear_phalanx_mix_backward_sum_rows(int B, int L, int H);
-long long spear_phalanx_mix_backward_sum_rows_tile(int B, int L, int H);
 int spear_phalanx_mix_backward_ex(const void* a_logit, const void* b_logit, const void* c, const void* v,
                                   const void* dout, void* da_logit, void* db_logit, void* dc, void* dv, int ld_da,
                                   int ld_db, int ld_dc, int ld_dv, float* sum_da, float* sum_db, float* sum_dc,
@@ -171,7 +157,7 @@ int spear_phalanx_mix_backward_ex(const void* a_logit, const void* b_logit, cons
 /* The same backward for callers that cannot allocate device memory -- code under HIP graph capture, tight
  * serving loops, harnesses that forbid hipMalloc -- and therefore cannot bring the partial-sum arrays of
  * spear_phalanx_mix_backward_ex. It has no counterpart in the reference. The partial column sums pass through
- * a device array the library holds statically (SPEAR_MIX_BIAS_SCRATCH_FLOATS floats = 8 MiB on every GPU the
+ * a device array the library holds statically (SPEAR_MIX_BIAS_SCRATCH_FLOATS floats = 16 MiB on every GPU the
  * library is used on, until the process ends), a second kernel finishes them, and the caller receives the
  * finished bias gradients of proj_a, proj_b and proj_c (spear/nn/phalanx/swr.py:157-163):
  *     bias_da [H],  bias_db [kv_heads * 16],  bias_dc [kv_heads * 16]      fp32, sums over batch and time,
@@ -179,12 +165,12 @@ int spear_phalanx_mix_backward_ex(const void* a_logit, const void* b_logit, cons
  * else is as in spear_phalanx_mix_backward_ex (layer form only, no SPEAR_MIX_QKV_GATE). The call makes no
  * hipMalloc / hipFree and no allocating library call. Limit:
  *     spear_phalanx_mix_backward_sum_rows(B, L, H) * (H + 2 * kv_heads * 16) <= SPEAR_MIX_BIAS_SCRATCH_FLOATS
- * (B = 1024, L = 128, H = kv_heads = 32 needs 1,081,344), otherwise SPEAR_BTP_EINVAL. All calls on one GPU
+ * (B = 1024, L = 128, H = kv_heads = 32 needs 2,162,688), otherwise SPEAR_BTP_EINVAL. All calls on one GPU
  * share that GPU's array: calls that overlap in time on one GPU (two streams, two threads) race, so
  * serialise them. Nothing in the array has to be cleared between calls -- each call overwrites all it later
  * reads. The array's address is looked up on the first call on each device; make that first call outside
  * stream capture. */
-#define SPEAR_MIX_BIAS_SCRATCH_FLOATS 2097152
+#define SPEAR_MIX_BIAS_SCRATCH_FLOATS 4194304
 int spear_phalanx_mix_backward_bias(const void* a_logit, const void* b_logit, const void* c, const void* v,
                                     const void* dout, void* da_logit, void* db_logit, void* dc, void* dv, int ld_da,
                                     int ld_db, int ld_dc, int ld_dv, float* bias_da, float* bias_db, float* bias_dc,
@@ -213,7 +199,8 @@ int spear_phalanx_mix_prefill(const void* a_logit, const void* b_logit, const vo
  * block, 0 .. block_len-1) every row decides for itself (pos[b] == block_len - 1) and the call advances pos by one
  * step (wrapping to 0), so that one captured HIP graph serves every token and batch rows may be at different
  * positions; with pos == NULL the host decides for all rows through `boundary`. Calls on one state must not
- * overlap. Nothing is allocated; with `pos` the call launches two kernels. */
+ * overlap. Nothing is allocated; with `pos` the call launches two kernels. Alignment: b_logit, c, v, out, h and
+ * c_prev 16 bytes; a_logit 2 and r 4 bytes (one token's row of a [tokens, B, H] tensor can be passed as it lies). */
 int spear_phalanx_mix_step(const void* a_logit, const void* b_logit, const void* c, const void* v, void* out, float* h,
                            float* r, float* c_prev, int* pos, int boundary, int block_len, int B, int H, int kv_heads,
                            int dtype, unsigned flags, void* stream);

@@ -29,10 +29,8 @@ FLAG_JAGGED_LOG_A = 0x4
 FLAG_JAGGED_LOG_R = 0x8
 FLAG_MIX_QKV_GATE = 0x1
 FLAG_MIX_F32_RESULTS = 0x2
-FLAG_MIX_TILE_SPLIT = 0x4
-FLAG_MIX_WALK_SPLIT = 0x8
 FLAG_DX_F32 = 0x10
-_ABI_VERSION = 17
+_ABI_VERSION = 18
 _SUPPORTED_WPB = (4, 8, 16, 32)
 
 _lock = threading.Lock()
@@ -67,8 +65,6 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.spear_phalanx_mix_backward_bias.restype = ci
     lib.spear_phalanx_mix_backward_sum_rows.argtypes = [ci, ci, ci]
     lib.spear_phalanx_mix_backward_sum_rows.restype = ctypes.c_longlong
-    lib.spear_phalanx_mix_backward_sum_rows_tile.argtypes = [ci, ci, ci]
-    lib.spear_phalanx_mix_backward_sum_rows_tile.restype = ctypes.c_longlong
     lib.spear_phalanx_mix_prefill.argtypes = [vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, cu, vp]
     lib.spear_phalanx_mix_prefill.restype = ci
     lib.spear_phalanx_mix_step.argtypes = [vp] * 9 + [ci] * 6 + [cu, vp]
@@ -346,22 +342,18 @@ def mix_forward(
     kv_heads: int,
     qkv_gate: bool = False,
     c_prev_tail: torch.Tensor | None = None,
-    tile_split: bool | None = None,
 ) -> None:
     """``out <- btp(sigmoid(a_logit), sigmoid(b_logit) * v) * c + v`` with every operand in the
     layer's ``[B, L, features]`` layout (see ``spear_phalanx_mix_forward`` in the C header).
     ``qkv_gate``: ``a_logit`` is an fp32 log-decay gate, ``b_logit`` is k, ``c`` is q:
     ``out <- c * btp(exp(a_logit), b_logit * v) + v`` (``SPEAR_MIX_QKV_GATE``). ``c_prev_tail``: fp32
     ``[B, heads, 16]`` that receives the terminal local state of every row's last block, the hand-over state
-    for decoding after this prompt (``spear_phalanx_mix_prefill``). ``tile_split``: True selects the kernel with one
-    wavefront per 16-step block (``SPEAR_MIX_TILE_SPLIT``), False the one whose wavefronts walk
-    through time (``SPEAR_MIX_WALK_SPLIT``), None leaves the choice to the library; the results are the same bits."""
+    for decoding after this prompt (``spear_phalanx_mix_prefill``)."""
     _check(all(t.is_cuda for t in (a_logit, b_logit, c, v, out)), "All tensors must be CUDA.")
     _check(v.dim() == 3, "v must be [B, L, heads * 16].")
     B, L, F = v.shape
     _check(F == heads * 16, "v must be [B, L, heads * 16].")
-    _check(heads % 4 == 0, "heads must be a multiple of 4.")
-    _check(kv_heads > 0 and heads % kv_heads == 0, "heads must be divisible by kv_heads.")
+    _check(heads > 0 and kv_heads > 0 and heads % kv_heads == 0, "heads must be divisible by kv_heads.")
     _check(v.dtype in (torch.float16, torch.bfloat16), "tensors must be float16 or bfloat16.")
     _check(b_logit.dtype == c.dtype == v.dtype, "all tensors must share one dtype.")
     _check(out.dtype in (v.dtype, torch.float32), "out must be float32 (fp32 check mode) or match v dtype.")
@@ -386,22 +378,17 @@ def mix_forward(
         rc = lib.spear_phalanx_mix_prefill(
             a_logit.data_ptr(), b_logit.data_ptr(), c.data_ptr(), v.data_ptr(), out.data_ptr(), _ptr(c_prev_tail),
             B, L, heads, kv_heads, _tag(v.dtype),
-            (FLAG_MIX_QKV_GATE if qkv_gate else 0) | (FLAG_MIX_F32_RESULTS if f32 else 0)
-            | (0 if tile_split is None else FLAG_MIX_TILE_SPLIT if tile_split else FLAG_MIX_WALK_SPLIT),
+            (FLAG_MIX_QKV_GATE if qkv_gate else 0) | (FLAG_MIX_F32_RESULTS if f32 else 0),
             _stream_ptr(v.device),
         )
     if rc != 0:
         _raise_native(lib, rc)
 
 
-def mix_backward_sum_rows(B: int, L: int, heads: int, tile_split: bool | None = None) -> int:
-    """Rows of the partial-sum arrays :func:`mix_backward` fills for this shape: with ``tile_split=True`` those
-    of the tile split (``SPEAR_MIX_TILE_SPLIT``), otherwise those of the walking kernel, which also serves a call
-    that names no split."""
-    lib = load_library()
-    if tile_split:
-        return int(lib.spear_phalanx_mix_backward_sum_rows_tile(B, L, heads))
-    return int(lib.spear_phalanx_mix_backward_sum_rows(B, L, heads))
+def mix_backward_sum_rows(B: int, L: int, heads: int) -> int:
+    """Rows of the partial-sum arrays :func:`mix_backward` fills for this shape: one per (batch row, tile of 64
+    time steps)."""
+    return int(load_library().spear_phalanx_mix_backward_sum_rows(B, L, heads))
 
 
 def mix_backward(
@@ -418,26 +405,20 @@ def mix_backward(
     kv_heads: int,
     sums: tuple[torch.Tensor, torch.Tensor, torch.Tensor] | None = None,
     qkv_gate: bool = False,
-    tile_split: bool | None = None,
 ) -> None:
-    """Gradients of :func:`mix_forward`, written in place; ``heads // kv_heads`` must be 1, 2, 4 or 8
+    """Gradients of :func:`mix_forward`, written in place, for any ``heads % kv_heads == 0``
     (see ``spear_phalanx_mix_backward`` in the C header). ``sums``: three fp32 tensors
-    ``[mix_backward_sum_rows(B, L, heads), heads | kv_heads*16 | kv_heads*16]`` that receive the per-chunk
-    column sums of ``da_logit``, ``db_logit`` and ``dc``. The four gradient tensors may be column blocks of one
-    wider ``[B, L, ld]`` buffer (``spear_phalanx_mix_backward_ex``). ``qkv_gate`` as in :func:`mix_forward`;
-    ``da_logit`` is then the fp32 gradient of the gate. Float32 ``db_logit, dc, dv`` (and ``da_logit``) select
-    the fp32 check mode (``SPEAR_MIX_F32_RESULTS``). ``tile_split``: True selects the kernel with one wavefront per
-    16-step block (``SPEAR_MIX_TILE_SPLIT``; its sum arrays have ``mix_backward_sum_rows(B, L, heads, True)`` rows),
-    False the one whose wavefronts walk through time (``SPEAR_MIX_WALK_SPLIT``), None leaves the choice to the library
-    (the tile split, or with ``sums`` the walking kernel)."""
+    ``[mix_backward_sum_rows(B, L, heads), heads | kv_heads*16 | kv_heads*16]`` that receive the column sums of
+    ``da_logit``, ``db_logit`` and ``dc`` per (batch row, tile of 64 time steps). The four gradient tensors may be
+    column blocks of one wider ``[B, L, ld]`` buffer (``spear_phalanx_mix_backward_ex``). ``qkv_gate`` as in
+    :func:`mix_forward`; ``da_logit`` is then the fp32 gradient of the gate. Float32 ``db_logit, dc, dv`` (and
+    ``da_logit``) select the fp32 check mode (``SPEAR_MIX_F32_RESULTS``)."""
     tensors = (a_logit, b_logit, c, v, dout, da_logit, db_logit, dc, dv)
     _check(all(t.is_cuda for t in tensors), "All tensors must be CUDA.")
     _check(v.dim() == 3, "v must be [B, L, heads * 16].")
     B, L, F = v.shape
     _check(F == heads * 16, "v must be [B, L, heads * 16].")
-    _check(heads % 4 == 0, "heads must be a multiple of 4.")
-    _check(kv_heads > 0 and heads % kv_heads == 0, "heads must be divisible by kv_heads.")
-    _check(heads // kv_heads in (1, 2, 4, 8), "heads / kv_heads must be 1, 2, 4 or 8.")
+    _check(heads > 0 and kv_heads > 0 and heads % kv_heads == 0, "heads must be divisible by kv_heads.")
     _check(v.dtype in (torch.float16, torch.bfloat16), "tensors must be float16 or bfloat16.")
     f32 = dv.dtype == torch.float32  # fp32 check mode: the four gradients are stored unrounded
     _check(all(t.dtype == v.dtype for t in (b_logit, c, dout)), "all tensors must share one dtype.")
@@ -462,7 +443,7 @@ def mix_backward(
     lib = load_library()
     rows = 0
     if sums is not None:
-        rows = mix_backward_sum_rows(B, L, heads, tile_split)
+        rows = mix_backward_sum_rows(B, L, heads)
         for name, t, width in (("sum_da", sums[0], heads), ("sum_db", sums[1], Fkv), ("sum_dc", sums[2], Fkv)):
             _check(t.is_cuda and t.device == v.device and t.dtype == torch.float32, f"{name} must be float32 on v's device.")
             _check_layout(name, t, (rows, width))
@@ -473,8 +454,7 @@ def mix_backward(
             da_logit.data_ptr(), db_logit.data_ptr(), dc.data_ptr(), dv.data_ptr(), *lds,
             *sum_ptrs, rows,
             B, L, heads, kv_heads, _tag(v.dtype),
-            (FLAG_MIX_QKV_GATE if qkv_gate else 0) | (FLAG_MIX_F32_RESULTS if f32 else 0)
-            | (0 if tile_split is None else FLAG_MIX_TILE_SPLIT if tile_split else FLAG_MIX_WALK_SPLIT),
+            (FLAG_MIX_QKV_GATE if qkv_gate else 0) | (FLAG_MIX_F32_RESULTS if f32 else 0),
             _stream_ptr(v.device),
         )
     if rc != 0:

@@ -45,7 +45,7 @@ int check_common(const char* who, int B, int H, int L, int k, int in_dtype, int 
 
 extern "C" {
 
-int spear_btp_abi_version(void) { return 17; }
+int spear_btp_abi_version(void) { return 18; }
 
 const char* spear_btp_last_error(void) { return g_error; }
 
@@ -142,29 +142,19 @@ int spear_phalanx_mix_prefill(const void* a_logit, const void* b_logit, const vo
   const char* who = c_prev_tail ? "spear_phalanx_mix_prefill" : "spear_phalanx_mix_forward";
   if (B < 0 || L < 0 || H < 0) return fail(SPEAR_BTP_EINVAL, "%s: negative dimension (B=%d L=%d H=%d)", who, B, L, H);
   if (L % 16 != 0) return fail(SPEAR_BTP_EINVAL, "%s: Length L must be multiple of 16 (got %d)", who, L);
-  if (H % 4 != 0) return fail(SPEAR_BTP_EINVAL, "%s: heads must be a multiple of 4 (got %d)", who, H);
   if (kv_heads <= 0 || H % kv_heads != 0)
     return fail(SPEAR_BTP_EINVAL, "%s: heads (%d) must be divisible by kv_heads (%d)", who, H, kv_heads);
   if (dtype != SPEAR_BTP_BF16 && dtype != SPEAR_BTP_F16)
     return fail(SPEAR_BTP_EINVAL, "%s: tensors must be float16 or bfloat16.", who);
-  const unsigned known = SPEAR_MIX_QKV_GATE | SPEAR_MIX_F32_RESULTS | SPEAR_MIX_TILE_SPLIT | SPEAR_MIX_WALK_SPLIT;
+  const unsigned known = SPEAR_MIX_QKV_GATE | SPEAR_MIX_F32_RESULTS;
   if (flags & ~known) return fail(SPEAR_BTP_EINVAL, "%s: unknown flag bits 0x%x", who, flags & ~known);
   const bool f32 = (flags & SPEAR_MIX_F32_RESULTS) != 0;
-  // the work split is a flag, or the process-wide default: the tile split, unless SPEAR_BTP_FUSED_FWD=walk is set
-  // (read once)
-  static const bool tile_default = [] {
-    const char* e = getenv("SPEAR_BTP_FUSED_FWD");
-    return e == nullptr || e[0] != 'w';
-  }();
-  const bool tile_asked = (flags & SPEAR_MIX_TILE_SPLIT) != 0, walk_asked = (flags & SPEAR_MIX_WALK_SPLIT) != 0;
-  if (tile_asked && walk_asked)
-    return fail(SPEAR_BTP_EINVAL, "%s: SPEAR_MIX_TILE_SPLIT and SPEAR_MIX_WALK_SPLIT exclude each other", who);
-  const bool tile = (tile_asked || (tile_default && !walk_asked)) &&
-                    (long long)B * ((L / 16 + 3) / 4 + 7) * ((H + 7) / 8) < (1ll << 31);
   if ((long long)B * L * H * 16ll >= (1ll << 40)) return fail(SPEAR_BTP_EINVAL, "%s: tensor too large", who);
   if ((long long)L * H * (f32 ? 64ll : 32ll) >= (1ll << 31))  // a batch row is addressed through one 32-bit buffer resource
     return fail(SPEAR_BTP_EINVAL, "%s: one batch row (L * H * 16 elements) must stay below 2 GiB", who);
   if ((long long)B * H == 0 || L == 0) return 0;
+  if (spear_btp::fused_mix_workgroups(B, H, H / kv_heads, L, false) >= (1ll << 31))
+    return fail(SPEAR_BTP_EINVAL, "%s: too many tiles for one launch (B * L / 64 * H / 8 must stay below 2^31)", who);
   if (!a_logit || !b_logit || !c || !v || !out) return fail(SPEAR_BTP_ENULL, "%s: NULL tensor pointer", who);
   if (!aligned16(a_logit) || !aligned16(b_logit) || !aligned16(c) || !aligned16(v) || !aligned16(out))
     return fail(SPEAR_BTP_EINVAL, "%s: tensor pointers must be 16-byte aligned", who);
@@ -172,7 +162,7 @@ int spear_phalanx_mix_prefill(const void* a_logit, const void* b_logit, const vo
   if (c_prev_tail && (flags & SPEAR_MIX_QKV_GATE))
     return fail(SPEAR_BTP_EINVAL, "%s: the hand-over state belongs to the layer form, not SPEAR_MIX_QKV_GATE", who);
   spear_btp::MixArgs a{a_logit, b_logit, c, v, out, B, L, H, H / kv_heads, dtype, (flags & SPEAR_MIX_QKV_GATE) != 0, f32,
-                       c_prev_tail, tile};
+                       c_prev_tail};
   const hipError_t err = spear_btp::fused_mix_forward(a, static_cast<hipStream_t>(stream));
   if (err != hipSuccess) return fail(SPEAR_BTP_ELAUNCH, "%s: launch failed: %s", who, hipGetErrorString(err));
   return 0;
@@ -181,11 +171,6 @@ int spear_phalanx_mix_prefill(const void* a_logit, const void* b_logit, const vo
 long long spear_phalanx_mix_backward_sum_rows(int B, int L, int H) {
   if (B <= 0 || L <= 0 || H <= 0 || L % 16 != 0) return 0;
   return spear_btp::fused_mix_backward_sum_rows(B, H, L);
-}
-
-long long spear_phalanx_mix_backward_sum_rows_tile(int B, int L, int H) {
-  if (B <= 0 || L <= 0 || H <= 0 || L % 16 != 0) return 0;
-  return spear_btp::fused_mix_backward_sum_rows(B, H, L, true);
 }
 
 int spear_phalanx_mix_backward(const void* a_logit, const void* b_logit, const void* c, const void* v, const void* dout,
@@ -200,14 +185,8 @@ static int check_mix_backward(const char* who, const void* const (&ptrs)[9], con
                               int kv_heads, int dtype, unsigned flags, unsigned allowed_flags) {
   if (B < 0 || L < 0 || H < 0) return fail(SPEAR_BTP_EINVAL, "%s: negative dimension (B=%d L=%d H=%d)", who, B, L, H);
   if (L % 16 != 0) return fail(SPEAR_BTP_EINVAL, "%s: Length L must be multiple of 16 (got %d)", who, L);
-  if (H % 4 != 0) return fail(SPEAR_BTP_EINVAL, "%s: heads must be a multiple of 4 (got %d)", who, H);
   if (kv_heads <= 0 || H % kv_heads != 0)
     return fail(SPEAR_BTP_EINVAL, "%s: heads (%d) must be divisible by kv_heads (%d)", who, H, kv_heads);
-  const int groups = H / kv_heads;
-  if (groups != 1 && groups != 2 && groups != 4 && groups != 8)
-    return fail(SPEAR_BTP_EINVAL, "%s: heads / kv_heads must be 1, 2, 4 or 8 (got %d)", who, groups);
-  if (groups == 8 && H % 8 != 0)
-    return fail(SPEAR_BTP_EINVAL, "%s: groups of 8 heads need heads divisible by 8 (got %d)", who, H);
   if (dtype != SPEAR_BTP_BF16 && dtype != SPEAR_BTP_F16)
     return fail(SPEAR_BTP_EINVAL, "%s: tensors must be float16 or bfloat16.", who);
   if (flags & ~allowed_flags) return fail(SPEAR_BTP_EINVAL, "%s: unknown flag bits 0x%x", who, flags & ~allowed_flags);
@@ -216,6 +195,8 @@ static int check_mix_backward(const char* who, const void* const (&ptrs)[9], con
   if ((long long)L * H * (f32 ? 64ll : 32ll) >= (1ll << 31))  // a batch row is addressed through one 32-bit buffer resource
     return fail(SPEAR_BTP_EINVAL, "%s: one batch row (L * H * 16 elements) must stay below 2 GiB", who);
   if ((long long)B * H == 0 || L == 0) return 1;
+  if (spear_btp::fused_mix_workgroups(B, H, H / kv_heads, L, true) >= (1ll << 31))
+    return fail(SPEAR_BTP_EINVAL, "%s: too many tiles for one launch (B * L / 64 * H / 8 must stay below 2^31)", who);
   for (const void* q : ptrs) {
     if (!q) return fail(SPEAR_BTP_ENULL, "%s: NULL tensor pointer", who);
     if (!aligned16(q)) return fail(SPEAR_BTP_EINVAL, "%s: tensor pointers must be 16-byte aligned", who);
@@ -223,8 +204,10 @@ static int check_mix_backward(const char* who, const void* const (&ptrs)[9], con
   const int widths[4] = {H, kv_heads * 16, kv_heads * 16, H * 16};
   for (int i = 0; i < 4; ++i) {
     if (lds[i] == 0) continue;
-    if (lds[i] < widths[i] || lds[i] % 2 != 0)
-      return fail(SPEAR_BTP_EINVAL, "%s: a gradient's row stride must be 0 (dense) or an even number of elements not below its width (got %d for width %d)", who, lds[i], widths[i]);
+    // db, dc, dv are stored as pairs of elements (32-bit, or 64-bit in the check mode): their rows start on even
+    // elements; da_logit is stored element by element
+    if (lds[i] < widths[i] || (i != 0 && lds[i] % 2 != 0))
+      return fail(SPEAR_BTP_EINVAL, "%s: a gradient's row stride must be 0 (dense) or a number of elements not below its width, even for db_logit, dc and dv (got %d for width %d)", who, lds[i], widths[i]);
     if ((long long)L * lds[i] * ((i == 0 && qkv) || f32 ? 4ll : 2ll) >= (1ll << 31))
       return fail(SPEAR_BTP_EINVAL, "%s: one batch row (L * row stride) must stay below 2 GiB", who);
   }
@@ -240,37 +223,22 @@ int spear_phalanx_mix_backward_ex(const void* a_logit, const void* b_logit, cons
   const char* who = "spear_phalanx_mix_backward";
   const void* const ptrs[9] = {a_logit, b_logit, c, v, dout, da_logit, db_logit, dc, dv};
   const int lds[4] = {ld_da, ld_db, ld_dc, ld_dv};
-  if (int rc = check_mix_backward(who, ptrs, lds, B, L, H, kv_heads, dtype, flags,
-                                  SPEAR_MIX_QKV_GATE | SPEAR_MIX_F32_RESULTS | SPEAR_MIX_TILE_SPLIT | SPEAR_MIX_WALK_SPLIT))
+  if (int rc = check_mix_backward(who, ptrs, lds, B, L, H, kv_heads, dtype, flags, SPEAR_MIX_QKV_GATE | SPEAR_MIX_F32_RESULTS))
     return rc < 0 ? rc : 0;
   const bool qkv = (flags & SPEAR_MIX_QKV_GATE) != 0, f32 = (flags & SPEAR_MIX_F32_RESULTS) != 0;
-  // the work split is a flag, or the process-wide default: the tile split wherever it can serve the call,
-  // unless SPEAR_BTP_FUSED_BWD=walk is set (read once)
-  static const bool tile_default = [] {
-    const char* e = getenv("SPEAR_BTP_FUSED_BWD");
-    return e == nullptr || e[0] != 'w';
-  }();
-  const bool tile_asked = (flags & SPEAR_MIX_TILE_SPLIT) != 0, walk_asked = (flags & SPEAR_MIX_WALK_SPLIT) != 0;
-  if (tile_asked && walk_asked)
-    return fail(SPEAR_BTP_EINVAL, "%s: SPEAR_MIX_TILE_SPLIT and SPEAR_MIX_WALK_SPLIT exclude each other", who);
   const bool sums = sum_da || sum_db || sum_dc;
   if (sums && qkv) return fail(SPEAR_BTP_EINVAL, "%s: column sums are for the layer form, not SPEAR_MIX_QKV_GATE", who);
   if (sums && f32) return fail(SPEAR_BTP_EINVAL, "%s: column sums are not available with SPEAR_MIX_F32_RESULTS", who);
-  // (column sums come from the tile split only when the flag asks for it: the arrays' row count differs between
-  // the splits, and a caller without the flag has sized them with spear_phalanx_mix_backward_sum_rows)
-  const bool fits = (long long)B * ((L / 16 + 3) / 4 + 7) * ((H + 7) / 8) < (1ll << 31);  // (+ 7: grids are padded to groups of 8 tiles)
-  if (tile_asked && sums && !fits) return fail(SPEAR_BTP_EINVAL, "%s: too many tiles for SPEAR_MIX_TILE_SPLIT", who);
-  const bool tile = (tile_asked || (tile_default && !walk_asked && !sums)) && fits;
   if (sums) {
     if (!sum_da || !sum_db || !sum_dc) return fail(SPEAR_BTP_ENULL, "%s: the three sum arrays must be given together", who);
     if (!aligned16(sum_da) || !aligned16(sum_db) || !aligned16(sum_dc))
       return fail(SPEAR_BTP_EINVAL, "%s: sum arrays must be 16-byte aligned", who);
-    const long long want = spear_btp::fused_mix_backward_sum_rows(B, H, L, tile);
+    const long long want = spear_btp::fused_mix_backward_sum_rows(B, H, L);
     if (sum_rows != want)
       return fail(SPEAR_BTP_EINVAL, "%s: sum arrays must have %lld rows for this shape (got %lld)", who, want, sum_rows);
   }
   spear_btp::MixBwdArgs a{a_logit, b_logit, c, v, dout, da_logit, db_logit, dc, dv, B, L, H, H / kv_heads, dtype,
-                          sum_da, sum_db, sum_dc, ld_da, ld_db, ld_dc, ld_dv, qkv, f32, tile};
+                          sum_da, sum_db, sum_dc, ld_da, ld_db, ld_dc, ld_dv, qkv, f32};
   const hipError_t err = spear_btp::fused_mix_backward(a, static_cast<hipStream_t>(stream));
   if (err != hipSuccess) return fail(SPEAR_BTP_ELAUNCH, "%s: launch failed: %s", who, hipGetErrorString(err));
   return 0;

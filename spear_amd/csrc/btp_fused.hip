@@ -1,5 +1,5 @@
-// Fused Phalanx mixing kernel for gfx950 (MI355X), forward: everything the layer does between its
-// input projections and its output projection, in the projections' own [B, L, features] layout.
+// Fused Phalanx mixing kernels for gfx950 (MI355X): everything the layer does between its input
+// projections and its output projection, in the projections' own [B, L, features] layout.
 //
 //     A = sigmoid(a_logit)            [B, L, H]          decay per head and step
 //     X = sigmoid(b_logit) * v        [B, L, H*16]       gated input (b, c may have fewer, shared heads)
@@ -9,27 +9,31 @@
 // In the reference these are separate PyTorch ops around the BTP kernel
 // (spear/nn/phalanx/swr.py:166-221 for the gates, :311-327 for `y * C + V`, the permute and the
 // `.contiguous()` transposes hidden in spear/ops/btp/interface.py:186-187): about twenty passes
-// over [B, L, H*16]-sized tensors. Here each operand is read once and the result written once.
+// over [B, L, H*16]-sized tensors. Here each operand is read once and each result written once, forward
+// (phalanx_mix_fwd_tile_kernel) and backward (phalanx_mix_bwd_tile_kernel).
 //
-// Layout and work split. Features are the contiguous axis, time is strided, so a lane owns
-// features and walks through time: one wavefront owns 128 features (8 heads) of one batch row,
-// lane p the feature pair p (4 bytes), and advances one 16-step block per iteration. A wave-level
-// load or store is one contiguous 256-byte run, and the four wavefronts of a workgroup cover 512
-// consecutive features of the same time step, so a workgroup walks whole 1-KiB rows; there is no
-// LDS staging of the big operands at all. Two register sets alternate: the next block's 48 words per
-// lane are requested before the current block is processed (12 KiB per wavefront in flight). Addressing
-// uses buffer instructions: a wave-uniform resource per operand, an SGPR offset for the time step
-// and one constant per-lane byte offset, so no per-access vector address arithmetic is left.
+// Layout and work split. Features are the contiguous axis, time is strided, so a lane owns a feature
+// pair (4 bytes) of up to 8 consecutive heads' 128 features and a wavefront owns ONE 16-step block of
+// them: a wave-level load or store is one contiguous 256-byte run per time step, addressed through
+// buffer instructions (a wave-uniform resource per operand, an SGPR offset for the time step, one constant
+// per-lane byte offset). A wavefront runs no loop over time: every load is issued at the start, every store
+// at the end, and a workgroup (4 or 8 wavefronts = consecutive blocks of the same features of one batch row)
+// lives for a few microseconds. The one-hop structure makes blocks independent up to quantities that are
+// local to a block (the terminal value of its zero-started recurrence; in backward also a_0 R_0 of its
+// zero-started reverse recurrence): every wavefront computes its own block's, leaves them in LDS for its
+// neighbours behind the kernel's single barrier, and the first / last block of a workgroup recompute the
+// neighbour's from two operands of the block beyond the edge. There is no LDS staging of the big operands.
+// sigmoid(a_logit) is computed once per (step, head) -- two per lane -- and handed to the lanes that need
+// it through a 640-byte LDS tile.
 //
-// Per block a lane runs the same two fp32 recurrences as the stand-alone forward kernel: a
-// zero-started one whose terminal value is the carry for the next block, and one started from the
-// incoming carry that produces the outputs. Because a lane walks through time, the carry simply
-// stays in the lane's registers: a row of any length is processed without halo re-reads.
-// sigmoid(a_logit) is computed once per (step, head) -- two per lane -- and handed to the lanes
-// that need it through a 640-byte LDS tile.
+// Copy loops with these kernels' traffic are why the split looks like this: wavefronts that walk through
+// time with two register sets reach 0.65 of the HBM peak whatever the chunking, short-lived tiles 0.71-0.74
+// (reads and writes do not overlap on the memory bus, so what counts is how quickly a wavefront turns from
+// its read phase to its write phase and makes room for the next one). An earlier pair of kernels whose
+// wavefronts walked through time gave the same results and was slower at every shape measured (forward
+// 92-96 against 86-87 us, backward 185-196 against 163 us at B=1024 L=128 H=32).
 #include <hip/hip_runtime.h>
 #include <stdint.h>
-#include <stdlib.h>
 
 #include <mutex>
 #include <type_traits>
@@ -39,7 +43,7 @@
 #include "btp_launch.h"
 
 // Device memory owned by the library, for the one entry point that must not allocate
-// (fused_mix_backward_bias below): the per-(batch row, time chunk) partial column sums of the fused
+// (fused_mix_backward_bias below): the per-(batch row, time tile) partial column sums of the fused
 // backward kernel park here between that kernel and the kernel that finishes the sums. Every GPU the
 // library runs on holds its own copy until the process ends. In host code the name stands for the
 // symbol, not for a device address: the address is looked up once per device and only that pointer
@@ -86,511 +90,65 @@ __device__ __forceinline__ float input_gate(float b) {
 
 constexpr int kHeadsPerWave = 8;
 constexpr int kGateRow = 20;  // floats per head in the decay tile: 16 steps + 4 of padding (bank spread)
+constexpr int kNowhere = 0x7ffffff0;  // a byte offset beyond every buffer resource: the buffer unit drops the access
 
 typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
 
-// kF32: check mode, the result leaves as fp32 (the kernel's own values, not rounded to 16 bits).
-template <class E, int kFwdWaves, bool kQkv, bool kF32>
-__global__ __launch_bounds__(64 * kFwdWaves) void phalanx_mix_fwd_kernel(
-    const uint16_t* __restrict__ a_logit, const uint16_t* __restrict__ b_logit, const uint16_t* __restrict__ c_in,
-    const uint16_t* __restrict__ v_in, uint16_t* __restrict__ out, float* __restrict__ c_prev_tail, int L, int H,
-    int kv_groups, int chunk_steps, int chunks, long total_waves) {
-  __shared__ __align__(16) float a_tile[kFwdWaves][kHeadsPerWave * kGateRow];  // [head][step] decay, fp32
-
-  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
-  const long w = (long)blockIdx.x * kFwdWaves + wave;
-  if (w >= total_waves) return;
-  // wavefront -> (batch row, time chunk, group of 8 heads); heads vary fastest so that the four
-  // wavefronts of a workgroup read neighbouring features of the same time steps
-  const int octs = (H + kHeadsPerWave - 1) / kHeadsPerWave;
-  const long bc = w / octs;
-  const int ho = (int)(w - bc * octs) * kHeadsPerWave;  // first head of this wavefront
-  const long brow = bc / chunks;
-  const int t_begin = (int)(bc - brow * chunks) * chunk_steps;
-  const int t_end = min(L, t_begin + chunk_steps);
-  // A chunk that does not start the row first runs the block before it without storing, only to
-  // obtain that block's terminal state (the carry is one hop, so one block of run-in is exact).
-  const int t_first = max(t_begin - kTile, 0);
-
-  // H is a multiple of 4: the last wavefront of a row may own only 4 real heads. Lanes of heads
-  // that do not exist read a head that does and store nowhere.
-  const int head_local = lane >> 3;
-  const bool real = ho + head_local < H;
-  const int head = real ? ho + head_local : H - 1;
-  const int d0 = (lane & 7) << 1;
-  const int F = H * kChan;
-  const int Fkv = (H / kv_groups) * kChan;
-  const int v_stride = 2 * F, kv_stride = 2 * Fkv;  // bytes per time step
-  constexpr int kRsrcFlags = 0x00020000;            // raw 32-bit buffer, gfx9 encoding
-  const __amdgpu_buffer_rsrc_t rv =
-      __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(v_in + brow * L * F), 0, L * v_stride, kRsrcFlags);
-  constexpr int kOutScale = kF32 ? 2 : 1;  // bytes of an output element over bytes of an input element
-  const __amdgpu_buffer_rsrc_t ro =
-      __builtin_amdgcn_make_buffer_rsrc(out + brow * L * F * kOutScale, 0, L * v_stride * kOutScale, kRsrcFlags);
-  const __amdgpu_buffer_rsrc_t rb =
-      __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(b_logit + brow * L * Fkv), 0, L * kv_stride, kRsrcFlags);
-  const __amdgpu_buffer_rsrc_t rc =
-      __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(c_in + brow * L * Fkv), 0, L * kv_stride, kRsrcFlags);
-  constexpr int kGateBytes = kQkv ? 4 : 2;
-  const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc(
-      const_cast<char*>(reinterpret_cast<const char*>(a_logit) + brow * L * H * kGateBytes), 0, L * H * kGateBytes,
-      kRsrcFlags);
-  const int v_lane = 2 * (head * kChan + d0), kv_lane = 2 * ((head / kv_groups) * kChan + d0);
-  // A lane without a head stores at an offset beyond the resource, which the buffer unit drops.
-  const int o_lane = real ? v_lane * kOutScale : 0x7ffffff0;
-  // gate logits: lane (hg, t) = (lane / 16, lane % 16) converts heads ho + 2 hg, + 1 of step t
-  const int gt = lane & 15, ghead = min(ho + 2 * (lane >> 4), H - 2);
-  const int a_lane = kGateBytes * (gt * H + ghead);
-  float* at = a_tile[wave];
-#ifndef SPEAR_FUSED_LD_AUX
-#define SPEAR_FUSED_LD_AUX 2
-#endif
-#ifndef SPEAR_FUSED_ST_AUX
-#define SPEAR_FUSED_ST_AUX 2
-#endif
-  constexpr int kNt = SPEAR_FUSED_LD_AUX;  // non-temporal: every word is touched once
-  constexpr int kNtS = SPEAR_FUSED_ST_AUX;
-
-  // Two register sets of one block each (16 steps x {b, c, v} words per lane): while one block is
-  // being processed the next one is already in flight, so a wait only ever concerns loads that
-  // were issued a whole block earlier and never the younger stores.
-  struct Words {
-    uint32_t b[16], c[16], v[16];
-  };
-  auto issue = [&](Words& wd, int t) {
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      wd.b[r] = __builtin_amdgcn_raw_buffer_load_b32(rb, kv_lane, (t + r) * kv_stride, kNt);
-      wd.v[r] = __builtin_amdgcn_raw_buffer_load_b32(rv, v_lane, (t + r) * v_stride, kNt);
-    }
-#pragma unroll
-    for (int r = 0; r < 16; ++r) wd.c[r] = __builtin_amdgcn_raw_buffer_load_b32(rc, kv_lane, (t + r) * kv_stride, kNt);
-  };
-  // run-in block: its b and v were (or are being) read by the chunk before, so they are left
-  // cacheable; c is not needed because nothing is stored
-  auto issue_run_in = [&](Words& wd, int t) {
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      wd.b[r] = __builtin_amdgcn_raw_buffer_load_b32(rb, kv_lane, (t + r) * kv_stride, 0);
-      wd.v[r] = __builtin_amdgcn_raw_buffer_load_b32(rv, v_lane, (t + r) * v_stride, 0);
-      wd.c[r] = 0u;
-    }
-  };
-  auto issue_gate = [&](int t) -> GateWords {
-    GateWords w;
-    w.lo = __builtin_amdgcn_raw_buffer_load_b32(ra, a_lane, t * H * kGateBytes, 0);
-    w.hi = kQkv ? __builtin_amdgcn_raw_buffer_load_b32(ra, a_lane + 4, t * H * kGateBytes, 0) : 0u;
-    return w;
-  };
-
-  float carry0 = 0.0f, carry1 = 0.0f;  // terminal local state of the previous block
-
-  auto process = [&](const Words& wd, GateWords araw, int t0) {
-    const int o_off = (t0 >= t_begin) ? o_lane : 0x7ffffff0;  // run-in block: store nowhere
-    const float2 a01 = decay_pair<E, kQkv>(araw);
-    at[(2 * (lane >> 4)) * kGateRow + gt] = a01.x;
-    at[(2 * (lane >> 4) + 1) * kGateRow + gt] = a01.y;
-    wave_lds_handover();
-    float a[16];
-#pragma unroll
-    for (int c4 = 0; c4 < 4; ++c4) {
-      const float4 q = *reinterpret_cast<const float4*>(at + head_local * kGateRow + 4 * c4);
-      a[4 * c4 + 0] = q.x; a[4 * c4 + 1] = q.y; a[4 * c4 + 2] = q.z; a[4 * c4 + 3] = q.w;
-    }
-    wave_lds_handover();  // the tile may be overwritten by the next block from here on
-
-    // pass 1: gated inputs and the zero-started recurrence (its terminal value is the next carry)
-    float x0[16], x1[16];
-    float l0 = 0.0f, l1 = 0.0f;
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      x0[r] = input_gate<kQkv>(E::lo(wd.b[r])) * E::lo(wd.v[r]);
-      x1[r] = input_gate<kQkv>(E::hi(wd.b[r])) * E::hi(wd.v[r]);
-      l0 = fmaf(a[r], l0, x0[r]);
-      l1 = fmaf(a[r], l1, x1[r]);
-    }
-    // pass 2: the carry-started recurrence and the output mix
-    float y0 = carry0, y1 = carry1;
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      y0 = fmaf(a[r], y0, x0[r]);
-      y1 = fmaf(a[r], y1, x1[r]);
-      const float o0 = fmaf(y0, E::lo(wd.c[r]), E::lo(wd.v[r])), o1 = fmaf(y1, E::hi(wd.c[r]), E::hi(wd.v[r]));
-      if constexpr (kF32) {
-        const u32x2_t ow = {__float_as_uint(o0), __float_as_uint(o1)};
-        __builtin_amdgcn_raw_buffer_store_b64(ow, ro, o_off, (t0 + r) * v_stride * 2, kNtS);
-      } else {
-        __builtin_amdgcn_raw_buffer_store_b32(E::pack2(o0, o1), ro, o_off, (t0 + r) * v_stride, kNtS);
-      }
-    }
-    carry0 = l0;
-    carry1 = l1;
-  };
-
-  Words w0, w1;
-  if (t_first < t_begin) issue_run_in(w0, t_first);
-  else issue(w0, t_first);
-  GateWords g0 = issue_gate(t_first), g1 = {0u, 0u};
-  for (int t0 = t_first; t0 < t_end; t0 += 2 * kTile) {
-    // the scheduling barriers keep the look-ahead loads in front of the arithmetic (left alone,
-    // the scheduler sinks them next to their uses to save registers, which serialises the two)
-    const bool more1 = t0 + kTile < t_end, more2 = t0 + 2 * kTile < t_end;  // wave-uniform
-    if (more1) {
-      issue(w1, t0 + kTile);
-      g1 = issue_gate(t0 + kTile);
-    }
-    __builtin_amdgcn_sched_barrier(0);
-    process(w0, g0, t0);
-    if (more1) {
-      __builtin_amdgcn_sched_barrier(0);
-      if (more2) {
-        issue(w0, t0 + 2 * kTile);
-        g0 = issue_gate(t0 + 2 * kTile);
-      }
-      __builtin_amdgcn_sched_barrier(0);
-      process(w1, g1, t0 + kTile);
-    }
-    __builtin_amdgcn_sched_barrier(0);
-  }
-  // Hand-over for token-by-token decoding after this prompt: the terminal local state of the row's last block is
-  // what the next block's steps need as c_prev (the block-local state restarts at 0 and the gate product at 1).
-  if (c_prev_tail != nullptr && t_end == L && real)
-    *reinterpret_cast<float2*>(c_prev_tail + (brow * H + head) * kChan + d0) = make_float2(carry0, carry1);
-}
-
-
-// ==========================================================================================
-// Backward of the fused mixing stage, same layout and work split as the forward kernel (one
-// wavefront = 128 features of one batch row, lane = feature pair; kv head groups of 1, 2, 4 or 8
-// heads), walking
-// through time in REVERSE block order. Inputs a_logit, b_logit, c, v, dout; outputs da_logit,
-// db_logit, dc, dv -- each big tensor is read or written exactly once.
-//
-// With A = sigmoid(a), G = sigmoid(b), x = G v, g = dout * c (the recurrence's upstream gradient),
-// per block i (local index r, fwd carry c_in = local terminal state of block i-1, gradient carry
-// dC = a_0 R_0 of block i+1):
-//   pass R (r = 15..0):  R_r = g_r + a_{r+1} R_{r+1} ;  q_r = (prod_{j=r+1..15} a_j) dC ;  dX_r = R_r + q_r
-//   pass F (r = 0..15):  vloc_r = a_r vloc_{r-1} + x_r ;  z_r = (prod_{j<r} a_j) c_in ;  h_r = vloc_r + a_r z_r
-//                        dc_r = dout_r h_r ;  dv_r = dout_r + dX_r G_r ;  db_r = dX_r v_r G_r (1 - G_r)
-//                        dA_r = sum over the head's 16 channels of  dX_r vloc_{r-1} + R_r z_r
-//                        da_r = dA_r A_r (1 - A_r)
-// R and dX run against time while vloc and z run with it, so pass R parks its 16 x 4 values per
-// lane in LDS (lane-private slots, 16 KiB per wavefront) and pass F picks them up.
-// c_in needs the block before the current one: its b, v and a are loaded one iteration early (they
-// are the next iteration's operands anyway) and a short look-ahead pass runs its zero-started
-// recurrence. A time chunk that does not end the row first runs pass R alone on the block after it
-// (one block of run-in gives the exact gradient carry, the dependency being one hop).
-// ==========================================================================================
-struct MixSet {
-  uint32_t b[16], c[16], v[16], g[16];  // g: dout words
-  GateWords araw;
+// Where the gate values of a wavefront's heads come from. Lane (hg, t) = (lane / 16, lane % 16) converts the
+// head pair (first + 2 hg, first + 2 hg + 1) of step t. Heads past the last one are clamped to it (their tile
+// rows are read by lanes without a head only). 16-bit logits of a head pair are one aligned 32-bit word when
+// the row length H and the wavefront's first head are even; otherwise (`split`, wave-uniform) they are
+// fetched as two 16-bit loads.
+struct GatePlace {
+  int off0, off1;  // byte offsets of the two heads' values inside a [L, H] batch row, step t included
+  bool split;
 };
 
-// kSums: also leave, per (batch row, time chunk), the sums over the chunk's time steps of da_logit, db_logit
-// and dc in fp32 (before their rounding to 16 bits) -- the bias gradients of the projections that produced
-// a_logit, b_logit and c, up to a sum over those few rows. A lane keeps its features for the whole walk, so
-// this is five accumulators per lane and one store at the end.
-// kF32: check mode, the four gradients leave as fp32 (the kernel's own values, not rounded to 16 bits).
-template <class E, bool kSums, bool kQkv, bool kF32>
-__global__ __launch_bounds__(64 * kWaves) void phalanx_mix_bwd_kernel(
-    const uint16_t* __restrict__ a_logit, const uint16_t* __restrict__ b_logit, const uint16_t* __restrict__ c_in,
-    const uint16_t* __restrict__ v_in, const uint16_t* __restrict__ dout, uint16_t* __restrict__ da_logit,
-    uint16_t* __restrict__ db_logit, uint16_t* __restrict__ dc, uint16_t* __restrict__ dv, float* __restrict__ sum_da,
-    float* __restrict__ sum_db, float* __restrict__ sum_dc, int ld_da, int ld_db, int ld_dc, int ld_dv, int L, int H,
-    int kv_groups, int chunk_steps, int chunks, long total_waves) {
-  __shared__ __align__(16) float gate_tiles[kWaves][2][kHeadsPerWave * kGateRow];  // decay of two blocks
-  __shared__ __align__(16) float4 park[kWaves][kTile][64];                        // (R0, R1, dX0, dX1) per step, lane
-
-  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
-  const long w = (long)blockIdx.x * kWaves + wave;
-  if (w >= total_waves) return;
-  const int octs = (H + kHeadsPerWave - 1) / kHeadsPerWave;
-  const long bc = w / octs;
-  const int ho = (int)(w - bc * octs) * kHeadsPerWave;
-  const long brow = bc / chunks;
-  const int t_begin = (int)(bc - brow * chunks) * chunk_steps;
-  const int t_end = min(L, t_begin + chunk_steps);
-
-  const int head_local = lane >> 3;
-  const bool real = ho + head_local < H;
-  const int head = real ? ho + head_local : H - 1;
-  const int d0 = (lane & 7) << 1;
-  const int F = H * kChan, Fkv = (H / kv_groups) * kChan;
-  const int stride = 2 * F, kv_stride = 2 * Fkv;  // bytes per time step of the [B, L, F] / [B, L, Fkv] tensors
-  constexpr int kRsrcFlags = 0x00020000;          // raw 32-bit buffer, gfx9 encoding
-  constexpr int kGateBytes = kQkv ? 4 : 2;        // element size of the a operand
-  constexpr int kDaBytes = (kQkv || kF32) ? 4 : 2;  // element size of its gradient
-  constexpr int kGradBytes = kF32 ? 4 : 2;          // element size of db, dc, dv
-  const long big = brow * L * F, kvbig = brow * L * Fkv, small = brow * L * H;
-  auto rsrc = [&](const uint16_t* p, long off, int bytes) {
-    return __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(p + off), 0, bytes, kRsrcFlags);
-  };
-  const __amdgpu_buffer_rsrc_t rb = rsrc(b_logit, kvbig, L * kv_stride), rc = rsrc(c_in, kvbig, L * kv_stride),
-                               rv = rsrc(v_in, big, L * stride), rg = rsrc(dout, big, L * stride),
-                               ra = rsrc(a_logit, small * (kGateBytes / 2), L * H * kGateBytes),
-                               // the four gradients may sit side by side in one wider buffer: each has its
-                               // own elements-per-time-step (ld_*), equal to its width when it is dense
-                               rdb = rsrc(db_logit, brow * L * ld_db * (kGradBytes / 2), L * ld_db * kGradBytes),
-                               rdc = rsrc(dc, brow * L * ld_dc * (kGradBytes / 2), L * ld_dc * kGradBytes),
-                               rdv = rsrc(dv, brow * L * ld_dv * (kGradBytes / 2), L * ld_dv * kGradBytes),
-                               rda = rsrc(da_logit, brow * L * ld_da * (kDaBytes / 2), L * ld_da * kDaBytes);
-  const int f_lane = 2 * (head * kChan + d0);
-  const int kv_lane = 2 * ((head / kv_groups) * kChan + d0);
-  const int o_lane = real ? f_lane * (kGradBytes / 2) : 0x7ffffff0;  // lanes without a head store nowhere
-  // With shared kv heads (kv_groups = 2, 4 or 8 consecutive heads, all inside this wavefront) the
-  // gradients of b and c are summed over the group's lanes and stored by its first head only.
-  const int okv_lane = (real && (head % kv_groups) == 0) ? kv_lane * (kGradBytes / 2) : 0x7ffffff0;
-  const int gt = lane & 15, ghead = min(ho + 2 * (lane >> 4), H - 2);
-  const int a_lane = kGateBytes * (gt * H + ghead);
-  // da_logit: lane k of a head (k = lane % 8) ends up with steps 2k and 2k+1 of that head
-  const int da_lane = real ? kDaBytes * ((2 * (lane & 7)) * ld_da + head) : 0x7ffffff0;
-  constexpr int kNt = 2;
-
-  auto issue = [&](MixSet& m, int t) {
-    // b, v and the gate logits first: the look-ahead pass needs them before pass R of the next
-    // iteration needs dout and c
-    m.araw.lo = __builtin_amdgcn_raw_buffer_load_b32(ra, a_lane, t * H * kGateBytes, 0);
-    m.araw.hi = kQkv ? __builtin_amdgcn_raw_buffer_load_b32(ra, a_lane + 4, t * H * kGateBytes, 0) : 0u;
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      m.b[r] = __builtin_amdgcn_raw_buffer_load_b32(rb, kv_lane, (t + r) * kv_stride, kNt);
-      m.v[r] = __builtin_amdgcn_raw_buffer_load_b32(rv, f_lane, (t + r) * stride, kNt);
-    }
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      m.g[r] = __builtin_amdgcn_raw_buffer_load_b32(rg, f_lane, (t + r) * stride, kNt);
-      m.c[r] = __builtin_amdgcn_raw_buffer_load_b32(rc, kv_lane, (t + r) * kv_stride, kNt);
-    }
-  };
-  auto write_gate_tile = [&](float* tile, GateWords araw) {
-    const float2 a01 = decay_pair<E, kQkv>(araw);
-    tile[(2 * (lane >> 4)) * kGateRow + gt] = a01.x;
-    tile[(2 * (lane >> 4) + 1) * kGateRow + gt] = a01.y;
-  };
-  auto read_gates = [&](const float* tile, float (&a)[16]) {
-#pragma unroll
-    for (int c4 = 0; c4 < 4; ++c4) {
-      const float4 q = *reinterpret_cast<const float4*>(tile + head_local * kGateRow + 4 * c4);
-      a[4 * c4 + 0] = q.x; a[4 * c4 + 1] = q.y; a[4 * c4 + 2] = q.z; a[4 * c4 + 3] = q.w;
-    }
-  };
-
-  float dC0 = 0.0f, dC1 = 0.0f;  // gradient carry arriving from the block after the current one
-  float acc_a = 0.0f, acc_b0 = 0.0f, acc_b1 = 0.0f, acc_c0 = 0.0f, acc_c1 = 0.0f;  // kSums only
-  float4* my_park = &park[wave][0][lane];
-
-  // One iteration: `cur` holds block t0 (its decay is in tile `tc`), `nxt` receives block t0 - 16.
-  auto iterate = [&](MixSet& cur, MixSet& nxt, float* tc, float* tn, int t0) {
-    const bool has_prev = t0 > 0;        // wave-uniform
-    const bool full = t0 < t_end;        // false: run-in block after the chunk, pass R only
-    if (has_prev) issue(nxt, t0 - kTile);
-    __builtin_amdgcn_sched_barrier(0);
-
-    float a[16];
-    read_gates(tc, a);
-
-    // ---- pass R
-    float R0 = 0.0f, R1 = 0.0f, q0 = dC0, q1 = dC1;
-#pragma unroll
-    for (int r = 15; r >= 0; --r) {
-      const float g0 = E::lo(cur.g[r]) * E::lo(cur.c[r]);
-      const float g1 = E::hi(cur.g[r]) * E::hi(cur.c[r]);
-      if (r < 15) {
-        R0 = fmaf(a[r + 1], R0, g0);
-        R1 = fmaf(a[r + 1], R1, g1);
-        q0 *= a[r + 1];
-        q1 *= a[r + 1];
-      } else {
-        R0 = g0;
-        R1 = g1;
-      }
-      if (full) my_park[r * 64] = make_float4(R0, R1, R0 + q0, R1 + q1);
-    }
-    dC0 = a[0] * R0;
-    dC1 = a[0] * R1;
-    if (!full) {
-      // the tile of the block before the run-in block is still needed by the next iteration
-      if (has_prev) write_gate_tile(tn, nxt.araw);
-      wave_lds_handover();
-      return;
-    }
-
-    // ---- look-ahead: terminal zero-started state of block t0 - 16 = carry into the current block
-    float cin0 = 0.0f, cin1 = 0.0f;
-    if (has_prev) {
-      write_gate_tile(tn, nxt.araw);
-      wave_lds_handover();
-      float ap[16];
-      read_gates(tn, ap);
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        cin0 = fmaf(ap[r], cin0, input_gate<kQkv>(E::lo(nxt.b[r])) * E::lo(nxt.v[r]));
-        cin1 = fmaf(ap[r], cin1, input_gate<kQkv>(E::hi(nxt.b[r])) * E::hi(nxt.v[r]));
-      }
-    } else {
-      wave_lds_handover();
-    }
-
-    // ---- pass F
-    const int o_off = (t0 >= t_begin) ? o_lane : 0x7ffffff0;
-    const int okv_off = (t0 >= t_begin) ? okv_lane : 0x7ffffff0;
-    float vp0 = 0.0f, vp1 = 0.0f, z0 = cin0, z1 = cin1;
-    // the per-step partial sums of dA go back into the parking slot they were computed from (its
-    // first word is free once read), so that they do not occupy 16 registers during this pass
-    float* my_e = reinterpret_cast<float*>(my_park);
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const float4 pk = my_park[r * 64];  // R0, R1, dX0, dX1
-      const float G0 = input_gate<kQkv>(E::lo(cur.b[r])), G1 = input_gate<kQkv>(E::hi(cur.b[r]));
-      const float v0 = E::lo(cur.v[r]), v1 = E::hi(cur.v[r]);
-      const float go0 = E::lo(cur.g[r]), go1 = E::hi(cur.g[r]);
-      my_e[r * 256] = fmaf(pk.z, vp0, pk.x * z0) + fmaf(pk.w, vp1, pk.y * z1);
-      const float az0 = a[r] * z0, az1 = a[r] * z1;
-      vp0 = fmaf(a[r], vp0, G0 * v0);
-      vp1 = fmaf(a[r], vp1, G1 * v1);
-      float dc0 = go0 * (vp0 + az0), dc1 = go1 * (vp1 + az1);
-      float db0 = pk.z * v0, db1 = pk.w * v1;  // dX * v: the gradient of k in the q/k/v form
-      if constexpr (!kQkv) {
-        db0 *= G0 * (1.0f - G0);
-        db1 *= G1 * (1.0f - G1);
-      }
-      if (kv_groups > 1) {  // wave-uniform: sum over the heads that share this kv head
-        dc0 += row_xor<8>(dc0); dc1 += row_xor<8>(dc1); db0 += row_xor<8>(db0); db1 += row_xor<8>(db1);
-        if (kv_groups > 2) {
-          dc0 += lane_xor(dc0, lane, 16); dc1 += lane_xor(dc1, lane, 16);
-          db0 += lane_xor(db0, lane, 16); db1 += lane_xor(db1, lane, 16);
-        }
-        if (kv_groups > 4) {
-          dc0 += lane_xor(dc0, lane, 32); dc1 += lane_xor(dc1, lane, 32);
-          db0 += lane_xor(db0, lane, 32); db1 += lane_xor(db1, lane, 32);
-        }
-      }
-      if constexpr (kSums) {
-        acc_b0 += db0; acc_b1 += db1; acc_c0 += dc0; acc_c1 += dc1;
-      }
-      const float dv0 = fmaf(pk.z, G0, go0), dv1 = fmaf(pk.w, G1, go1);
-      z0 = az0;
-      z1 = az1;
-      if constexpr (kF32) {
-        const u32x2_t wdc = {__float_as_uint(dc0), __float_as_uint(dc1)}, wdv = {__float_as_uint(dv0), __float_as_uint(dv1)},
-                      wdb = {__float_as_uint(db0), __float_as_uint(db1)};
-        __builtin_amdgcn_raw_buffer_store_b64(wdc, rdc, okv_off, (t0 + r) * 4 * ld_dc, kNt);
-        __builtin_amdgcn_raw_buffer_store_b64(wdv, rdv, o_off, (t0 + r) * 4 * ld_dv, kNt);
-        __builtin_amdgcn_raw_buffer_store_b64(wdb, rdb, okv_off, (t0 + r) * 4 * ld_db, kNt);
-      } else {
-        __builtin_amdgcn_raw_buffer_store_b32(E::pack2(dc0, dc1), rdc, okv_off, (t0 + r) * 2 * ld_dc, kNt);
-        __builtin_amdgcn_raw_buffer_store_b32(E::pack2(dv0, dv1), rdv, o_off, (t0 + r) * 2 * ld_dv, kNt);
-        __builtin_amdgcn_raw_buffer_store_b32(E::pack2(db0, db1), rdb, okv_off, (t0 + r) * 2 * ld_db, kNt);
-      }
-    }
-
-    // ---- dA: sum over the 8 lanes (16 channels) of the head, transposing: lane k keeps steps 2k, 2k+1
-    const int kk = lane & 7;
-    float e[16], f8[8], f4[4];
-#pragma unroll
-    for (int r = 0; r < 16; ++r) e[r] = my_e[r * 256];
-    {
-      const bool hi = kk & 4;
-#pragma unroll
-      for (int t = 0; t < 8; ++t) {
-        const float keep = hi ? e[t + 8] : e[t], send = hi ? e[t] : e[t + 8];
-        f8[t] = keep + row_xor<4>(send);
-      }
-    }
-    {
-      const bool hi = kk & 2;
-#pragma unroll
-      for (int t = 0; t < 4; ++t) {
-        const float keep = hi ? f8[t + 4] : f8[t], send = hi ? f8[t] : f8[t + 4];
-        f4[t] = keep + row_xor<2>(send);
-      }
-    }
-    float s0, s1;
-    {
-      const bool hi = kk & 1;
-      const float k0 = hi ? f4[2] : f4[0], n0 = hi ? f4[0] : f4[2];
-      const float k1 = hi ? f4[3] : f4[1], n1 = hi ? f4[1] : f4[3];
-      s0 = k0 + row_xor<1>(n0);
-      s1 = k1 + row_xor<1>(n1);
-    }
-    const float2 aa = *reinterpret_cast<const float2*>(tc + head_local * kGateRow + 2 * kk);
-    // d/d a_logit = dA a (1 - a);  d/d gate = dA a  (gate = log a)
-    const float da0 = kQkv ? s0 * aa.x : s0 * aa.x * (1.0f - aa.x), da1 = kQkv ? s1 * aa.y : s1 * aa.y * (1.0f - aa.y);
-    if constexpr (kSums) acc_a += da0 + da1;
-    const int da_off = (t0 >= t_begin) ? da_lane : 0x7ffffff0;
-    if constexpr (kDaBytes == 4) {
-      __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(da0), rda, da_off, t0 * ld_da * 4, 0);
-      __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(da1), rda, da_off + 4 * ld_da, t0 * ld_da * 4, 0);
-    } else {
-      const uint32_t dap = E::pack2(da0, da1);
-      __builtin_amdgcn_raw_buffer_store_b16((unsigned short)(dap & 0xffffu), rda, da_off, t0 * ld_da * 2, 0);
-      __builtin_amdgcn_raw_buffer_store_b16((unsigned short)(dap >> 16), rda, da_off + 2 * ld_da, t0 * ld_da * 2, 0);
-    }
-    wave_lds_handover();  // tile `tc` and the parking slots are free for the iteration after next
-  };
-
-  // Reverse walk: start at the block after the chunk (run-in) if there is one, else at its last block.
-  const int t_start = (t_end < L) ? t_end : t_end - kTile;
-  MixSet s0, s1;
-  issue(s0, t_start);
-  float* tile0 = gate_tiles[wave][0];
-  float* tile1 = gate_tiles[wave][1];
-  __builtin_amdgcn_sched_barrier(0);
-  write_gate_tile(tile0, s0.araw);
-  wave_lds_handover();
-  // the look-ahead block before the chunk is only read, never stored: walk down to t_begin
-  for (int t0 = t_start; t0 >= t_begin; t0 -= 2 * kTile) {
-    iterate(s0, s1, tile0, tile1, t0);
-    __builtin_amdgcn_sched_barrier(0);
-    if (t0 - kTile >= t_begin) iterate(s1, s0, tile1, tile0, t0 - kTile);
-    __builtin_amdgcn_sched_barrier(0);
+template <bool kQkv>
+__device__ __forceinline__ GatePlace gate_place(int first, int H, int lane) {
+  constexpr int kGateBytes = kQkv ? 4 : 2;
+  const int gt = lane & 15, h0 = first + 2 * (lane >> 4);
+  GatePlace g;
+  g.split = !kQkv && (((H | first) & 1) != 0);
+  if (kQkv || g.split) {
+    g.off0 = kGateBytes * (gt * H + min(h0, H - 1));
+    g.off1 = kGateBytes * (gt * H + min(h0 + 1, H - 1));
+  } else {
+    g.off0 = kGateBytes * (gt * H + min(h0, H - 2));
+    g.off1 = 0;
   }
+  return g;
+}
 
-  if constexpr (kSums) {
-    // row `bc` of the sum arrays belongs to this (batch row, chunk); columns as in the tensors
-    acc_a += row_xor<1>(acc_a);
-    acc_a += row_xor<2>(acc_a);
-    acc_a += row_xor<4>(acc_a);  // lane k of a head held steps 2k, 2k+1: now every lane has the head's sum
-    if (real && (lane & 7) == 0) sum_da[bc * H + head] = acc_a;
-    if (real && (head % kv_groups) == 0) {  // the group's sum is in every lane of the group
-      const long col = bc * Fkv + (head / kv_groups) * kChan + d0;
-      *reinterpret_cast<float2*>(sum_db + col) = make_float2(acc_b0, acc_b1);
-      *reinterpret_cast<float2*>(sum_dc + col) = make_float2(acc_c0, acc_c1);
+// The gate words of the block that starts at step t (ra: the batch row's [L, H] gates).
+template <bool kQkv>
+__device__ __forceinline__ GateWords load_gate_words(__amdgpu_buffer_rsrc_t ra, const GatePlace& g, int t, int H) {
+  constexpr int kGateBytes = kQkv ? 4 : 2;
+  GateWords w;
+  if constexpr (kQkv) {
+    w.lo = __builtin_amdgcn_raw_buffer_load_b32(ra, g.off0, t * H * kGateBytes, 0);
+    w.hi = __builtin_amdgcn_raw_buffer_load_b32(ra, g.off1, t * H * kGateBytes, 0);
+  } else {
+    if (g.split) {
+      const uint32_t lo = __builtin_amdgcn_raw_buffer_load_b16(ra, g.off0, t * H * kGateBytes, 0);
+      const uint32_t hi = __builtin_amdgcn_raw_buffer_load_b16(ra, g.off1, t * H * kGateBytes, 0);
+      w.lo = lo | (hi << 16);
+    } else {
+      w.lo = __builtin_amdgcn_raw_buffer_load_b32(ra, g.off0, t * H * kGateBytes, 0);
     }
+    w.hi = 0u;
   }
+  return w;
 }
 
 
 // ==========================================================================================
-// Backward of the fused mixing stage, tile form (SPEAR_MIX_TILE_SPLIT; what a call without a split flag runs
-// unless it asks for column sums): the same mathematics with a different work split. Measured against the walking
-// kernel above at B=1024 L=128 H=32 it takes 163 us against 185-196 us, at B=16 L=8192 H=64 322 against 367 us,
-// at B=64 L=2048 H=128 644-669 against 757 us. One
-// wavefront owns ONE 16-step block of 128 features and runs no loop: every load is issued at the start, every
-// store at the end, and a workgroup (4 wavefronts = 4 consecutive blocks of one head group of one batch
-// row) lives for a few microseconds. Copy loops with this kernel's traffic show why: wavefronts that walk
-// through time with two register sets reach 0.65 of the HBM peak whatever the chunking, short-lived tiles
-// 0.71-0.74 (reads and writes do not overlap on the memory bus, so what counts is how quickly a wavefront
-// turns from its read phase to its write phase and makes room for the next one).
-//
-// The one-hop structure makes tiles independent up to two neighbour quantities, both LOCAL to a block:
-//   c_out(i)  = terminal value of the zero-started forward recurrence over block i      (carry into block i+1)
-//   dC_out(i) = a_0 R_0 of the zero-started reverse recurrence over block i             (gradient carry into block i-1)
-// Every wavefront computes both for its own block first and leaves them in LDS; after the kernel's single
-// barrier its neighbours pick them up. The first and last block of a workgroup have no neighbour inside it:
-// those wavefronts read two operands of the block beyond the edge as well (b, v for the forward carry or dout,
-// c for the gradient carry; cacheable loads, the neighbouring workgroup reads the same lines at about the
-// same time) and run the one recurrence they need on them.
-//
-// With h the state of the carry-started recurrence (h_{-1} = c_in, h_r = a_r h_{r-1} + x_r) and
-// dX_r = R_r + (prod_{j>r} a_j) dC, per step
-//   dc_r = dout_r h_r ;  dv_r = dout_r + dX_r G_r ;  db_r = dX_r v_r G_r (1 - G_r)
-//   dA_r = sum over the head's channels of dX_r h_{r-1}  -  (prod_{j != r} a_j) sum over channels of dC c_in
-// (the second term takes out the two-hop path c_in -> dC that h carries but the operator does not have).
+// Shared by the forward and the backward kernel: which tile a workgroup is.
 // ==========================================================================================
-// Wavefronts per workgroup and per SIMD. 4 and 3 (168 registers: nothing spills, 12 wavefronts per CU) beat 8 and 4
-// (128 registers, three or four spilled values per lane that show up as 2.5 % more HBM writes, 16 wavefronts per
-// CU) by 1 % at B=1024 L=128 H=32, 3 % at B=16 L=8192 H=64 and 5 % at B=64 L=2048 H=128.
+// Wavefronts per workgroup and per SIMD of the backward kernel. 4 and 3 (168 registers: nothing spills, 12
+// wavefronts per CU) beat 8 and 4 (128 registers, three or four spilled values per lane that show up as 2.5 %
+// more HBM writes, 16 wavefronts per CU) by 1 % at B=1024 L=128 H=32, 3 % at B=16 L=8192 H=64 and 5 % at B=64
+// L=2048 H=128.
 #ifndef SPEAR_FUSED_TILE_WAVES
 #define SPEAR_FUSED_TILE_WAVES 4
 #endif
@@ -620,16 +178,16 @@ __device__ __forceinline__ float product_of_the_others(float a) {
 // Launch order deals workgroups round-robin to the 8 XCDs, each with its own L2. An XCD gets runs of
 // SPEAR_FUSED_TILE_XCD_GROUP neighbouring workgroups instead (windows of 8 runs sweep the tensors front to back):
 // the workgroup that owns an edge block and the neighbour that reads it as its halo then share an L2 close in
-// time. Backward with head groups fastest, against plain round-robin (0), runs of 128 four-wavefront workgroups:
-// 184 -> 166-167 us at B=1024 L=128 H=32, 371 -> 344 us at B=16 L=8192 H=64, 733 -> 718 us at B=64 L=2048 H=128
-// (all three as 1 head group x 4 blocks); with the tiles in groups of 8 (below) runs of 64 are best (32: forward
-// -3 % on long rows, 256: -5 to -15 %). The tail of the grid that does not fill a window keeps the launch order.
+// time. Backward with head slots fastest, against plain round-robin (0), runs of 128 four-wavefront workgroups:
+// 184 -> 166-167 us at B=1024 L=128 H=32, 371 -> 344 us at B=16 L=8192 H=64, 733 -> 718 us at B=64 L=2048 H=128;
+// with the tiles in groups of 8 (below) runs of 64 are best (32: forward -3 % on long rows, 256: -5 to -15 %).
+// The tail of the grid that does not fill a window keeps the launch order.
 //
-// Workgroup -> (batch row, time tile, group of head groups). Up to SPEAR_FUSED_TILE_TIME_GROUP consecutive time
-// tiles of one head group are neighbours in this order, then come the row's other head groups, then the next
+// Workgroup -> (batch row, time tile, head slot: which 128 features). Up to SPEAR_FUSED_TILE_TIME_GROUP consecutive
+// time tiles of one head slot are neighbours in this order, then come the row's other head slots, then the next
 // tiles: the workgroup that streams an edge block and the one that reads it as its halo are dispatched back to
 // back on one XCD, while the run as a whole still covers whole feature rows. Measured (forward / backward, us):
-//   tiles in groups of   1 (head groups fastest)   2           4           8           16         all (time fastest)
+//   tiles in groups of   1 (head slots fastest)    2           4           8           16         all (time fastest)
 //   B=1024 L=128 H=32    86.9 / 166.4              86.9 / 162  86.9 / 162  86.9 / 162  87 / 162   87.0 / 162.2
 //   B=16 L=8192 H=64     178.9 / 344.4             173 / 336   167 / 342   172 / 327   179 / 334  191.5 / 372.4
 //   B=64 L=2048 H=128    364.2 / 707               363 / 711   372 / 681   346 / 679   356 / 689  355.8 / 698.6
@@ -638,16 +196,16 @@ __device__ __forceinline__ float product_of_the_others(float a) {
 #define SPEAR_FUSED_TILE_TIME_GROUP 8
 #endif
 struct TilePlace {
-  int og, tile;
+  int slot, tile;
   long brow;
 };
-__device__ __forceinline__ TilePlace tile_place(unsigned wg, int tiles, int octs) {
+__device__ __forceinline__ TilePlace tile_place(unsigned wg, int tiles, int slots) {
   const unsigned tg = min((unsigned)SPEAR_FUSED_TILE_TIME_GROUP, (unsigned)tiles);
   const unsigned tgroups = ((unsigned)tiles + tg - 1) / tg;
   const unsigned t_lo = wg % tg, r1 = wg / tg;
   TilePlace p;
-  p.og = (int)(r1 % (unsigned)octs);
-  const unsigned r2 = r1 / (unsigned)octs;
+  p.slot = (int)(r1 % (unsigned)slots);
+  const unsigned r2 = r1 / (unsigned)slots;
   p.tile = (int)((r2 % tgroups) * tg + t_lo);
   p.brow = r2 / tgroups;
   return p;
@@ -664,38 +222,98 @@ __device__ __forceinline__ unsigned tile_workgroup() {
   return wg;
 }
 
+// Which heads a wavefront of the backward kernel owns. A head slot is normally 8 consecutive heads (the last
+// slot of a row may hold fewer). The gradients of b and c are sums over the heads that share a kv head; with
+// groups of 1, 2, 4 or 8 heads a group lies inside one slot on lanes a power of two apart, and the sum is a few
+// DPP / permute exchanges. Every other grouping (kWide) gets slots cut at group borders instead:
+//   groups of 3, 5, 6, 7 heads:   a slot = as many whole groups as fit into 8 heads (2, 1, 1, 1)
+//   groups of more than 8 heads:  a slot = one kv head; the wavefront works through the group's heads 8 at a
+//                                 time (a loop around the whole tile computation) and adds up as it goes
+// and the sum over a group goes through LDS, four time steps at a time, in a fixed order.
+struct HeadSlot {
+  int first, count;        // heads [first, first + count) are this pass's, count <= 8
+  int kv_first, kv_count;  // kWide: the kv heads whose groups these are (one, if a group is worked through in passes)
+};
+template <bool kWide>
+__device__ __forceinline__ HeadSlot head_slot(int slot, int pass, int H, int group) {
+  HeadSlot s;
+  if constexpr (!kWide) {
+    s.first = slot * kHeadsPerWave;
+    s.count = min(kHeadsPerWave, H - s.first);
+    s.kv_first = s.first / group;
+    s.kv_count = 0;  // not used
+  } else if (group <= kHeadsPerWave) {
+    const int per_slot = kHeadsPerWave / group;
+    s.kv_first = slot * per_slot;
+    s.kv_count = min(per_slot, H / group - s.kv_first);
+    s.first = s.kv_first * group;
+    s.count = s.kv_count * group;
+  } else {
+    s.kv_first = slot;
+    s.kv_count = 1;
+    s.first = slot * group + pass * kHeadsPerWave;
+    s.count = min(kHeadsPerWave, group - pass * kHeadsPerWave);
+  }
+  return s;
+}
+
+// ==========================================================================================
+// Backward of the fused mixing stage. Inputs a_logit, b_logit, c, v, dout; outputs da_logit, db_logit, dc, dv --
+// each big tensor is read or written exactly once. A workgroup is kTileWaves consecutive blocks of one head slot
+// of one batch row, one wavefront each.
+//
+// The one-hop structure makes tiles independent up to two neighbour quantities, both LOCAL to a block:
+//   c_out(i)  = terminal value of the zero-started forward recurrence over block i      (carry into block i+1)
+//   dC_out(i) = a_0 R_0 of the zero-started reverse recurrence over block i             (gradient carry into block i-1)
+// Every wavefront computes both for its own block first and leaves them in LDS; after the workgroup
+// barrier its neighbours pick them up. The first and last block of a workgroup have no neighbour inside it:
+// those wavefronts read two operands of the block beyond the edge as well (b, v for the forward carry or dout,
+// c for the gradient carry; cacheable loads, the neighbouring workgroup reads the same lines at about the
+// same time) and run the one recurrence they need on them.
+//
+// With A = sigmoid(a), G = sigmoid(b), x = G v, g = dout * c (the recurrence's upstream gradient), R the
+// zero-started reverse recurrence R_r = g_r + a_{r+1} R_{r+1}, h the state of the carry-started recurrence
+// (h_{-1} = c_in, h_r = a_r h_{r-1} + x_r) and dX_r = R_r + (prod_{j>r} a_j) dC, per step
+//   dc_r = dout_r h_r ;  dv_r = dout_r + dX_r G_r ;  db_r = dX_r v_r G_r (1 - G_r)
+//   dA_r = sum over the head's channels of dX_r h_{r-1}  -  (prod_{j != r} a_j) sum over channels of dC c_in
+//   da_r = dA_r A_r (1 - A_r)
+// (the second term of dA takes out the two-hop path c_in -> dC that h carries but the operator does not have).
+//
 // kF32: check mode, the four gradients leave as fp32 (the kernel's own values, not rounded to 16 bits).
 // kSums: also leave, per workgroup (batch row, time tile), the sums over the tile's time steps of da_logit, db_logit
-// and dc in fp32 (before their rounding to 16 bits), as the walking kernel does per (batch row, chunk): every
-// wavefront sums its block's 16 steps, the workgroup's blocks are added in block order behind a second barrier
-// (a fixed order: the same bits in every run), and row `batch row * tiles + tile` of the three arrays is written.
-template <class E, bool kQkv, bool kF32, bool kSums = false>
-__global__ __launch_bounds__(64 * kTileWaves) __attribute__((amdgpu_waves_per_eu(SPEAR_FUSED_TILE_WAVES_PER_EU)))
+// and dc in fp32 (before their rounding to 16 bits): every wavefront sums its block's 16 steps, the workgroup's
+// blocks are added in block order behind a second barrier (a fixed order: the same bits in every run), and row
+// `batch row * tiles + tile` of the three arrays is written.
+// kWide: head groupings other than 1, 2, 4, 8 heads per kv head (head_slot above).
+// ==========================================================================================
+template <class E, bool kQkv, bool kF32, bool kSums = false, bool kWide = false>
+__global__ __launch_bounds__(64 * kTileWaves)
+__attribute__((amdgpu_waves_per_eu(kWide ? 2 : SPEAR_FUSED_TILE_WAVES_PER_EU)))  // kWide: room for the group's sums
 void phalanx_mix_bwd_tile_kernel(
     const uint16_t* __restrict__ a_logit, const uint16_t* __restrict__ b_logit, const uint16_t* __restrict__ c_in,
     const uint16_t* __restrict__ v_in, const uint16_t* __restrict__ dout, uint16_t* __restrict__ da_logit,
     uint16_t* __restrict__ db_logit, uint16_t* __restrict__ dc, uint16_t* __restrict__ dv, float* __restrict__ sum_da,
     float* __restrict__ sum_db, float* __restrict__ sum_dc, int ld_da, int ld_db, int ld_dc, int ld_dv, int L, int H,
-    int kv_groups, int tiles) {
+    int kv_groups, int tiles, int slots) {
   // per wavefront: decay of its block, product of the block's other decays per step, decay of the block beyond the edge
   __shared__ __align__(16) float gate_tiles[kTileWaves][3][kHeadsPerWave * kGateRow];
   __shared__ float2 carry_out[kTileWaves][2][64];  // [0] dC_out, [1] c_out of the wavefront's block, per lane
   __shared__ float block_sums[kSums ? kTileWaves : 1][5][64];  // kSums: db (2), dc (2), da of the wavefront's block
+  // kWide: (dc0, dc1, db0, db1) of four time steps per lane, before the sum over a kv head's group
+  __shared__ __align__(16) float4 group_terms[kWide ? kTileWaves : 1][4][64];
 
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const unsigned wg = tile_workgroup();
-  constexpr int nb_w = kTileWaves;  // consecutive blocks per workgroup, one per wavefront, all of one head group
-  const int octs = (H + kHeadsPerWave - 1) / kHeadsPerWave;
-  const TilePlace at = tile_place(wg, tiles, octs);
+  constexpr int nb_w = kTileWaves;  // consecutive blocks per workgroup, one per wavefront, all of one head slot
+  const TilePlace at = tile_place(wg, tiles, slots);
   const int tile = at.tile, bl = wave;
   const long brow = at.brow;
-  const int ho = at.og * kHeadsPerWave;
   const int t0 = (tile * nb_w + bl) * kTile;
-  const bool valid = ho < H && t0 < L;  // wave-uniform; a wavefront without a block only joins the barrier
+  // passes over the heads of a group that is larger than a wavefront's 8 heads (kWide only), same for the workgroup
+  const int passes = (kWide && kv_groups > kHeadsPerWave) ? (kv_groups + kHeadsPerWave - 1) / kHeadsPerWave : 1;
+  const bool valid = t0 < L;  // wave-uniform; a wavefront without a block only joins the barriers
 
   const int head_local = lane >> 3;
-  const bool real = ho + head_local < H;
-  const int head = real ? ho + head_local : H - 1;
   const int d0 = (lane & 7) << 1;
   const int F = H * kChan, Fkv = (H / kv_groups) * kChan;
   const int stride = 2 * F, kv_stride = 2 * Fkv;
@@ -710,37 +328,54 @@ void phalanx_mix_bwd_tile_kernel(
   const __amdgpu_buffer_rsrc_t rb = rsrc(b_logit, kvbig, L * kv_stride), rc = rsrc(c_in, kvbig, L * kv_stride),
                                rv = rsrc(v_in, big, L * stride), rg = rsrc(dout, big, L * stride),
                                ra = rsrc(a_logit, small * (kGateBytes / 2), L * H * kGateBytes),
+                               // the four gradients may sit side by side in one wider buffer: each has its
+                               // own elements-per-time-step (ld_*), equal to its width when it is dense
                                rdb = rsrc(db_logit, brow * L * ld_db * (kGradBytes / 2), L * ld_db * kGradBytes),
                                rdc = rsrc(dc, brow * L * ld_dc * (kGradBytes / 2), L * ld_dc * kGradBytes),
                                rdv = rsrc(dv, brow * L * ld_dv * (kGradBytes / 2), L * ld_dv * kGradBytes),
                                rda = rsrc(da_logit, brow * L * ld_da * (kDaBytes / 2), L * ld_da * kDaBytes);
-  const int f_lane = 2 * (head * kChan + d0);
-  const int kv_lane = 2 * ((head / kv_groups) * kChan + d0);
-  const int o_lane = real ? f_lane * (kGradBytes / 2) : 0x7ffffff0;
-  const int okv_lane = (real && (head % kv_groups) == 0) ? kv_lane * (kGradBytes / 2) : 0x7ffffff0;
-  const int gt = lane & 15, ghead = min(ho + 2 * (lane >> 4), H - 2);
-  const int a_lane = kGateBytes * (gt * H + ghead);
-  const int da_lane = real ? kDaBytes * ((2 * (lane & 7)) * ld_da + head) : 0x7ffffff0;
   constexpr int kNt = 2;
 
   // the block beyond the workgroup's edge that this wavefront has to look at (at most one: nb_w >= 2)
   const bool halo_prev = valid && bl == 0 && t0 > 0;                    // needs c_out of block t0 - 16
   const bool halo_next = valid && bl == nb_w - 1 && t0 + kTile < L;     // needs dC_out of block t0 + 16
+  const bool halo = halo_prev || halo_next;
   const int th = halo_prev ? t0 - kTile : t0 + kTile;
+
+  float* ta = gate_tiles[wave][0];
+  float* te = gate_tiles[wave][1];
+  float* tn = gate_tiles[wave][2];
+  const int gt = lane & 15;
+  auto write_tile = [&](float* tile_, float x0, float x1) {
+    tile_[(2 * (lane >> 4)) * kGateRow + gt] = x0;
+    tile_[(2 * (lane >> 4) + 1) * kGateRow + gt] = x1;
+  };
+
+  // kWide with passes: the sums over the group so far, for the lane's (step, feature pair) of each quarter block
+  float4 group_acc[4];
+#pragma unroll
+  for (int c4 = 0; c4 < 4; ++c4) group_acc[c4] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+
+  for (int pass = 0; pass < passes; ++pass) {
+  const HeadSlot hs = head_slot<kWide>(at.slot, pass, H, kv_groups);
+  const bool real = head_local < hs.count;
+  const int head = hs.first + (real ? head_local : hs.count - 1);  // lanes without a head read one that exists
+  const int f_lane = 2 * (head * kChan + d0);
+  const int kv_lane = 2 * ((head / kv_groups) * kChan + d0);
+  const int o_lane = real ? f_lane * (kGradBytes / 2) : kNowhere;  // and store nowhere
+  // groups of 2, 4 or 8 heads: the sums over a group end up in all its lanes; its first head stores them
+  const int okv_lane = (!kWide && real && (head % kv_groups) == 0) ? kv_lane * (kGradBytes / 2) : kNowhere;
+  const GatePlace gp = gate_place<kQkv>(hs.first, H, lane);
+  // da_logit: lane k of a head (k = lane % 8) ends up with steps 2k and 2k+1 of that head
+  const int da_lane = real ? kDaBytes * ((2 * (lane & 7)) * ld_da + head) : kNowhere;
+  const int da_lane1 = real ? da_lane + kDaBytes * ld_da : kNowhere;
 
   // ---- every global read, before anything waits
   uint32_t b[16], c[16], v[16], g[16], h0[16], h1[16];
   GateWords araw = {0u, 0u}, haraw = {0u, 0u};
-  auto load_gate = [&](int t) {
-    GateWords w;
-    w.lo = __builtin_amdgcn_raw_buffer_load_b32(ra, a_lane, t * H * kGateBytes, 0);
-    w.hi = kQkv ? __builtin_amdgcn_raw_buffer_load_b32(ra, a_lane + 4, t * H * kGateBytes, 0) : 0u;
-    return w;
-  };
   // Wavefronts at a workgroup edge read the block beyond the edge first and their own b, v only once those 32
   // registers are free again (b and v are not needed before the local forward recurrence); the other
   // wavefronts issue everything at once (with every load up front the kernel is no faster: 168 against 166 us).
-  const bool halo = halo_prev || halo_next;
   auto load_bv = [&]() {
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
@@ -749,37 +384,29 @@ void phalanx_mix_bwd_tile_kernel(
     }
   };
   if (valid) {
-    araw = load_gate(t0);
-    if (halo) haraw = load_gate(th);
-    if (halo_prev) {
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        h0[r] = __builtin_amdgcn_raw_buffer_load_b32(rb, kv_lane, (th + r) * kv_stride, 0);
-        h1[r] = __builtin_amdgcn_raw_buffer_load_b32(rv, f_lane, (th + r) * stride, 0);
-      }
-    } else if (halo_next) {
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        h0[r] = __builtin_amdgcn_raw_buffer_load_b32(rg, f_lane, (th + r) * stride, 0);
-        h1[r] = __builtin_amdgcn_raw_buffer_load_b32(rc, kv_lane, (th + r) * kv_stride, 0);
-      }
-    }
+  araw = load_gate_words<kQkv>(ra, gp, t0, H);
+  if (halo) haraw = load_gate_words<kQkv>(ra, gp, th, H);
+  if (halo_prev) {
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
-      g[r] = __builtin_amdgcn_raw_buffer_load_b32(rg, f_lane, (t0 + r) * stride, kNt);
-      c[r] = __builtin_amdgcn_raw_buffer_load_b32(rc, kv_lane, (t0 + r) * kv_stride, kNt);
+      h0[r] = __builtin_amdgcn_raw_buffer_load_b32(rb, kv_lane, (th + r) * kv_stride, 0);
+      h1[r] = __builtin_amdgcn_raw_buffer_load_b32(rv, f_lane, (th + r) * stride, 0);
     }
-    if (!halo) load_bv();
+  } else if (halo_next) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      h0[r] = __builtin_amdgcn_raw_buffer_load_b32(rg, f_lane, (th + r) * stride, 0);
+      h1[r] = __builtin_amdgcn_raw_buffer_load_b32(rc, kv_lane, (th + r) * kv_stride, 0);
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    g[r] = __builtin_amdgcn_raw_buffer_load_b32(rg, f_lane, (t0 + r) * stride, kNt);
+    c[r] = __builtin_amdgcn_raw_buffer_load_b32(rc, kv_lane, (t0 + r) * kv_stride, kNt);
+  }
+  if (!halo) load_bv();
   }
   __builtin_amdgcn_sched_barrier(0);
-
-  float* ta = gate_tiles[wave][0];
-  float* te = gate_tiles[wave][1];
-  float* tn = gate_tiles[wave][2];
-  auto write_tile = [&](float* tile_, float x0, float x1) {
-    tile_[(2 * (lane >> 4)) * kGateRow + gt] = x0;
-    tile_[(2 * (lane >> 4) + 1) * kGateRow + gt] = x1;
-  };
 
   float cin0 = 0.0f, cin1 = 0.0f, dC0 = 0.0f, dC1 = 0.0f;
   float R[32];  // local reverse states, later dX, channel pair interleaved: R[2 r], R[2 r + 1]
@@ -873,7 +500,8 @@ void phalanx_mix_bwd_tile_kernel(
   __syncthreads();  // the workgroup barrier of the carries; wavefronts without a block arrive here directly
   if (!valid) {
     if constexpr (kSums) __syncthreads();  // the barrier of the sums counts every wavefront of the workgroup
-    return;
+    if (passes > 1) __syncthreads();
+    continue;
   }
 
   if (bl > 0) {  // the block before this one belongs to the wavefront before this one
@@ -906,6 +534,17 @@ void phalanx_mix_bwd_tile_kernel(
     }
   }
 
+  // kWide: this lane's share of the sums over a group. Per quarter block (4 steps) the wavefront has 4 steps x 8
+  // feature pairs x kv_count results; lane = (kv head, feature pair, step) adds the group's heads in head order.
+  const int w_step = lane & 3, w_pair = (lane >> 2) & 7, w_kv = lane >> 5;
+  const bool w_owner = kWide && w_kv < hs.kv_count;
+  const int w_heads = kv_groups <= kHeadsPerWave ? kv_groups : hs.count;  // heads of the group in this pass
+  const int w_src = (w_kv * w_heads) * 8 + w_pair;                        // the lane of the group's first head
+  const bool w_store = w_owner && pass == passes - 1;
+  const int w_col = kGradBytes * ((hs.kv_first + w_kv) * kChan + 2 * w_pair);
+  const int w_dc = w_store ? w_col + w_step * kGradBytes * ld_dc : kNowhere;
+  const int w_db = w_store ? w_col + w_step * kGradBytes * ld_db : kNowhere;
+
   // ---- forward pass: state, gradients, per-step partial sums of dA
   float e[16];
   float acc_b0 = 0.0f, acc_b1 = 0.0f, acc_c0 = 0.0f, acc_c1 = 0.0f;  // kSums only
@@ -930,32 +569,69 @@ void phalanx_mix_bwd_tile_kernel(
         db0 *= G0 * (1.0f - G0);
         db1 *= G1 * (1.0f - G1);
       }
-      if (kv_groups > 1) {  // wave-uniform: sum over the heads that share this kv head
-        dc0 += row_xor<8>(dc0); dc1 += row_xor<8>(dc1); db0 += row_xor<8>(db0); db1 += row_xor<8>(db1);
-        if (kv_groups > 2) {
-          dc0 += lane_xor(dc0, lane, 16); dc1 += lane_xor(dc1, lane, 16);
-          db0 += lane_xor(db0, lane, 16); db1 += lane_xor(db1, lane, 16);
-        }
-        if (kv_groups > 4) {
-          dc0 += lane_xor(dc0, lane, 32); dc1 += lane_xor(dc1, lane, 32);
-          db0 += lane_xor(db0, lane, 32); db1 += lane_xor(db1, lane, 32);
-        }
-      }
-      if constexpr (kSums) {
-        acc_b0 += db0; acc_b1 += db1; acc_c0 += dc0; acc_c1 += dc1;
-      }
       const float dv0 = fmaf(dX0, G0, go0), dv1 = fmaf(dX1, G1, go1);
-      if constexpr (kF32) {
-        const u32x2_t wdc = {__float_as_uint(dc0), __float_as_uint(dc1)}, wdv = {__float_as_uint(dv0), __float_as_uint(dv1)},
-                      wdb = {__float_as_uint(db0), __float_as_uint(db1)};
-        __builtin_amdgcn_raw_buffer_store_b64(wdc, rdc, okv_lane, (t0 + r) * 4 * ld_dc, kNt);
-        __builtin_amdgcn_raw_buffer_store_b64(wdv, rdv, o_lane, (t0 + r) * 4 * ld_dv, kNt);
-        __builtin_amdgcn_raw_buffer_store_b64(wdb, rdb, okv_lane, (t0 + r) * 4 * ld_db, kNt);
+      if constexpr (kWide) {
+        group_terms[wave][i][lane] = real ? make_float4(dc0, dc1, db0, db1) : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        if constexpr (kF32) {
+          const u32x2_t wdv = {__float_as_uint(dv0), __float_as_uint(dv1)};
+          __builtin_amdgcn_raw_buffer_store_b64(wdv, rdv, o_lane, (t0 + r) * 4 * ld_dv, kNt);
+        } else {
+          __builtin_amdgcn_raw_buffer_store_b32(E::pack2(dv0, dv1), rdv, o_lane, (t0 + r) * 2 * ld_dv, kNt);
+        }
       } else {
-        __builtin_amdgcn_raw_buffer_store_b32(E::pack2(dc0, dc1), rdc, okv_lane, (t0 + r) * 2 * ld_dc, kNt);
-        __builtin_amdgcn_raw_buffer_store_b32(E::pack2(dv0, dv1), rdv, o_lane, (t0 + r) * 2 * ld_dv, kNt);
-        __builtin_amdgcn_raw_buffer_store_b32(E::pack2(db0, db1), rdb, okv_lane, (t0 + r) * 2 * ld_db, kNt);
+        if (kv_groups > 1) {  // wave-uniform: sum over the heads that share this kv head
+          dc0 += row_xor<8>(dc0); dc1 += row_xor<8>(dc1); db0 += row_xor<8>(db0); db1 += row_xor<8>(db1);
+          if (kv_groups > 2) {
+            dc0 += lane_xor(dc0, lane, 16); dc1 += lane_xor(dc1, lane, 16);
+            db0 += lane_xor(db0, lane, 16); db1 += lane_xor(db1, lane, 16);
+          }
+          if (kv_groups > 4) {
+            dc0 += lane_xor(dc0, lane, 32); dc1 += lane_xor(dc1, lane, 32);
+            db0 += lane_xor(db0, lane, 32); db1 += lane_xor(db1, lane, 32);
+          }
+        }
+        if constexpr (kSums) {
+          acc_b0 += db0; acc_b1 += db1; acc_c0 += dc0; acc_c1 += dc1;
+        }
+        if constexpr (kF32) {
+          const u32x2_t wdc = {__float_as_uint(dc0), __float_as_uint(dc1)}, wdv = {__float_as_uint(dv0), __float_as_uint(dv1)},
+                        wdb = {__float_as_uint(db0), __float_as_uint(db1)};
+          __builtin_amdgcn_raw_buffer_store_b64(wdc, rdc, okv_lane, (t0 + r) * 4 * ld_dc, kNt);
+          __builtin_amdgcn_raw_buffer_store_b64(wdv, rdv, o_lane, (t0 + r) * 4 * ld_dv, kNt);
+          __builtin_amdgcn_raw_buffer_store_b64(wdb, rdb, okv_lane, (t0 + r) * 4 * ld_db, kNt);
+        } else {
+          __builtin_amdgcn_raw_buffer_store_b32(E::pack2(dc0, dc1), rdc, okv_lane, (t0 + r) * 2 * ld_dc, kNt);
+          __builtin_amdgcn_raw_buffer_store_b32(E::pack2(dv0, dv1), rdv, o_lane, (t0 + r) * 2 * ld_dv, kNt);
+          __builtin_amdgcn_raw_buffer_store_b32(E::pack2(db0, db1), rdb, okv_lane, (t0 + r) * 2 * ld_db, kNt);
+        }
       }
+    }
+    if constexpr (kWide) {
+      wave_lds_handover();
+      float4 sum = group_acc[c4];
+      if (w_owner) {
+        for (int j = 0; j < w_heads; ++j) {  // head order: the same bits in every run
+          const float4 t = group_terms[wave][w_step][w_src + 8 * j];
+          sum.x += t.x; sum.y += t.y; sum.z += t.z; sum.w += t.w;
+        }
+      }
+      group_acc[c4] = sum;
+      if constexpr (kSums) {  // the owner's four steps are the lanes of a quad
+        float4 q = sum;
+        q.x += row_xor<1>(q.x); q.y += row_xor<1>(q.y); q.z += row_xor<1>(q.z); q.w += row_xor<1>(q.w);
+        q.x += row_xor<2>(q.x); q.y += row_xor<2>(q.y); q.z += row_xor<2>(q.z); q.w += row_xor<2>(q.w);
+        acc_c0 += q.x; acc_c1 += q.y; acc_b0 += q.z; acc_b1 += q.w;
+      }
+      const int row = t0 + 4 * c4;
+      if constexpr (kF32) {
+        const u32x2_t wdc = {__float_as_uint(sum.x), __float_as_uint(sum.y)}, wdb = {__float_as_uint(sum.z), __float_as_uint(sum.w)};
+        __builtin_amdgcn_raw_buffer_store_b64(wdc, rdc, w_dc, row * 4 * ld_dc, kNt);
+        __builtin_amdgcn_raw_buffer_store_b64(wdb, rdb, w_db, row * 4 * ld_db, kNt);
+      } else {
+        __builtin_amdgcn_raw_buffer_store_b32(E::pack2(sum.x, sum.y), rdc, w_dc, row * 2 * ld_dc, kNt);
+        __builtin_amdgcn_raw_buffer_store_b32(E::pack2(sum.z, sum.w), rdb, w_db, row * 2 * ld_db, kNt);
+      }
+      wave_lds_handover();  // the terms may be overwritten by the next quarter block from here on
     }
     asm volatile("" ::: "memory");
   }
@@ -1000,11 +676,11 @@ void phalanx_mix_bwd_tile_kernel(
   const float da0 = kQkv ? s0 * aa.x : s0 * aa.x * (1.0f - aa.x), da1 = kQkv ? s1 * aa.y : s1 * aa.y * (1.0f - aa.y);
   if constexpr (kDaBytes == 4) {
     __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(da0), rda, da_lane, t0 * ld_da * 4, 0);
-    __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(da1), rda, da_lane + 4 * ld_da, t0 * ld_da * 4, 0);
+    __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(da1), rda, da_lane1, t0 * ld_da * 4, 0);
   } else {
     const uint32_t dap = E::pack2(da0, da1);
     __builtin_amdgcn_raw_buffer_store_b16((unsigned short)(dap & 0xffffu), rda, da_lane, t0 * ld_da * 2, 0);
-    __builtin_amdgcn_raw_buffer_store_b16((unsigned short)(dap >> 16), rda, da_lane + 2 * ld_da, t0 * ld_da * 2, 0);
+    __builtin_amdgcn_raw_buffer_store_b16((unsigned short)(dap >> 16), rda, da_lane1, t0 * ld_da * 2, 0);
   }
 
   if constexpr (kSums) {
@@ -1026,30 +702,40 @@ void phalanx_mix_bwd_tile_kernel(
       }
       const long row = brow * tiles + tile;
       if (real && (lane & 7) == 0) sum_da[row * H + head] = t[4];
-      if (real && (head % kv_groups) == 0) {  // the group's sum is in every lane of the group
+      if constexpr (kWide) {  // every lane of an owner's quad has the sums of its (kv head, feature pair)
+        if (w_store && w_step == 0) {
+          const long col = row * Fkv + (hs.kv_first + w_kv) * kChan + 2 * w_pair;
+          *reinterpret_cast<float2*>(sum_dc + col) = make_float2(t[2], t[3]);
+          *reinterpret_cast<float2*>(sum_db + col) = make_float2(t[0], t[1]);
+        }
+      } else if (real && (head % kv_groups) == 0) {  // the group's sum is in every lane of the group
         const long col = row * Fkv + (head / kv_groups) * kChan + d0;
         *reinterpret_cast<float2*>(sum_db + col) = make_float2(t[0], t[1]);
         *reinterpret_cast<float2*>(sum_dc + col) = make_float2(t[2], t[3]);
       }
     }
   }
+  if (passes > 1) __syncthreads();  // carry_out and block_sums are written again by the next pass
+  }  // passes
 }
 
 
 // ==========================================================================================
-// Forward of the fused mixing stage, tile form: the work split of the tile backward above (one wavefront per
-// 16-step block of 128 features, no loop, one workgroup barrier, workgroups dealt to the XCDs in runs of
-// neighbours) with the arithmetic of phalanx_mix_fwd_kernel, operation for operation, so both splits give the
-// same bits. A block needs one neighbour quantity, the terminal value of the zero-started recurrence over the block
-// before it: every wavefront computes its own block's and leaves it in LDS for the next wavefront; the
-// first block of a workgroup reads b and v of the block before the edge (cacheable loads: the neighbouring
-// workgroup streams the same lines on the same L2) and runs that recurrence itself.
-// The wavefront of a row's last block also stores the streaming state for decoding after this prompt, when asked.
-// kW wavefronts per workgroup, one head group x kW consecutive blocks (2 head groups x kW / 2 blocks measured
-// slower at every shape): 4 or 8. Microseconds for 4 / 8 (the walking kernel in brackets), B L H:
-//   1024 128 32: 87.3 / 91.5 (96.2)    256 512 32: 89.8 / 86.0 (101.1)    16 8192 32: 89.4 / 87.1 (99.9)
-//   512 128 64: 91.6 / 90.2 (95.2)     16 8192 64: 167.5 / 170.6 (181.5)  64 2048 128: 336.1 / 338.3 (370.4)
-//   256 128 128: 87.7 / 90.1 (114.2)   4096 128 8: 92.9 / 88.1 (90.1)     1024 128 48: 132.9 / 125.3 (146.8)
+// Forward of the fused mixing stage: the work split of the backward above (one wavefront per 16-step block of
+// 128 features, no loop, one workgroup barrier, workgroups dealt to the XCDs in runs of neighbours). Per block a
+// lane runs two fp32 recurrences over its feature pair: a zero-started one whose terminal value is the carry for
+// the next block, and one started from the incoming carry that produces the outputs. A block needs one neighbour
+// quantity, the terminal value of the zero-started recurrence over the block before it: every wavefront computes
+// its own block's and leaves it in LDS for the next wavefront; the first block of a workgroup reads b and v of
+// the block before the edge (cacheable loads: the neighbouring workgroup streams the same lines on the same L2)
+// and runs that recurrence itself. A kv head shared by several heads is resolved by indexing (head h reads b, c of
+// kv head h / group), for any group size. The wavefront of a row's last block also stores the streaming state for
+// decoding after this prompt, when asked.
+// kW wavefronts per workgroup, one head slot x kW consecutive blocks (2 head slots x kW / 2 blocks measured
+// slower at every shape): 4 or 8. Microseconds for 4 / 8, B L H:
+//   1024 128 32: 87.3 / 91.5    256 512 32: 89.8 / 86.0    16 8192 32: 89.4 / 87.1
+//   512 128 64: 91.6 / 90.2     16 8192 64: 167.5 / 170.6  64 2048 128: 336.1 / 338.3
+//   256 128 128: 87.7 / 90.1    4096 128 8: 92.9 / 88.1    1024 128 48: 132.9 / 125.3
 // ==========================================================================================
 template <class E, int kW, bool kQkv, bool kF32>
 __global__ __launch_bounds__(64 * kW) __attribute__((amdgpu_waves_per_eu(SPEAR_FUSED_TILE_WAVES_PER_EU)))
@@ -1062,14 +748,16 @@ void phalanx_mix_fwd_tile_kernel(const uint16_t* __restrict__ a_logit, const uin
 
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const unsigned wg = tile_workgroup<SPEAR_FUSED_TILE_XCD_GROUP * 4 / kW>();
-  constexpr int nb_w = kW;  // consecutive blocks per workgroup, one per wavefront, all of one head group
+  constexpr int nb_w = kW;  // consecutive blocks per workgroup, one per wavefront, all of one head slot
   const TilePlace at = tile_place(wg, tiles, (H + kHeadsPerWave - 1) / kHeadsPerWave);
   const int tile = at.tile, bl = wave;
   const long brow = at.brow;
-  const int ho = at.og * kHeadsPerWave;
+  const int ho = at.slot * kHeadsPerWave;
   const int t0 = (tile * nb_w + bl) * kTile;
-  const bool valid = ho < H && t0 < L;  // wave-uniform; a wavefront without a block only joins the barrier
+  const bool valid = t0 < L;  // wave-uniform; a wavefront without a block only joins the barrier
 
+  // The last slot of a row may hold fewer than 8 heads. Lanes of heads that do not exist read a head that
+  // does and store nowhere.
   const int head_local = lane >> 3;
   const bool real = ho + head_local < H;
   const int head = real ? ho + head_local : H - 1;
@@ -1089,9 +777,9 @@ void phalanx_mix_fwd_tile_kernel(const uint16_t* __restrict__ a_logit, const uin
                                ro = rsrc(out, big * kOutScale, L * stride * kOutScale);
   const int f_lane = 2 * (head * kChan + d0);
   const int kv_lane = 2 * ((head / kv_groups) * kChan + d0);
-  const int o_lane = real ? f_lane * kOutScale : 0x7ffffff0;  // lanes without a head store nowhere
-  const int gt = lane & 15, ghead = min(ho + 2 * (lane >> 4), H - 2);
-  const int a_lane = kGateBytes * (gt * H + ghead);
+  const int o_lane = real ? f_lane * kOutScale : kNowhere;
+  const int gt = lane & 15;
+  const GatePlace gp = gate_place<kQkv>(ho, H, lane);
   constexpr int kNt = 2;
 
   const bool halo = valid && bl == 0 && t0 > 0;  // needs the terminal local state of block t0 - 16
@@ -1100,16 +788,10 @@ void phalanx_mix_fwd_tile_kernel(const uint16_t* __restrict__ a_logit, const uin
   // ---- every global read, before anything waits
   uint32_t b[16], c[16], v[16], hb[16], hv[16];
   GateWords araw = {0u, 0u}, haraw = {0u, 0u};
-  auto load_gate = [&](int t) {
-    GateWords w;
-    w.lo = __builtin_amdgcn_raw_buffer_load_b32(ra, a_lane, t * H * kGateBytes, 0);
-    w.hi = kQkv ? __builtin_amdgcn_raw_buffer_load_b32(ra, a_lane + 4, t * H * kGateBytes, 0) : 0u;
-    return w;
-  };
   if (valid) {
-    araw = load_gate(t0);
+    araw = load_gate_words<kQkv>(ra, gp, t0, H);
     if (halo) {
-      haraw = load_gate(th);
+      haraw = load_gate_words<kQkv>(ra, gp, th, H);
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         hb[r] = __builtin_amdgcn_raw_buffer_load_b32(rb, kv_lane, (th + r) * kv_stride, 0);
@@ -1263,226 +945,110 @@ __global__ __launch_bounds__(256) void advance_block_positions_kernel(int* __res
 }
 
 
-// How a row is cut into time chunks and how many wavefronts share a workgroup (measured on MI355X).
-//   * HBM serves this layout best when the wavefronts of a workgroup together read whole
-//     feature rows and the workgroups, taken in launch order, advance through memory: chunks of a
-//     few blocks whose wavefronts sit side by side (all head groups of a row, then the next chunk).
-//     Up to 4 head groups per row, "full rows x 2 chunks of 4 blocks" per workgroup measured
-//     0.75 of peak at B=1024 L=128 H=32 against 0.69 for one long walk per row.
-//   * A chunk costs one extra block of (cacheable) reads and arithmetic for its run-in, so chunks
-//     shorter than 4 blocks only pay when the GPU would otherwise be underfilled.
-//   * With 8 head groups per row (2 KiB rows) long walks measured best; chunks are then only cut to
-//     reach about one wavefront per SIMD.
-struct MixPlan {
-  int wg_waves, chunk_blocks, chunks;
-};
 
-// Tuning overrides, read once per process (0 = not set).
-int env_override(const char* name) {
-  const char* e = getenv(name);
-  const int v = e ? atoi(e) : 0;
-  return v > 0 ? v : 0;
-}
-
-MixPlan plan_mix(long B, int H, int L) {
-  const long octs = (H + 7) / 8;
-  const int nb = L / kTile;
-  MixPlan m;
-  if (octs <= 4) {
-    m.wg_waves = octs > 2 ? 8 : 4;
-    m.chunk_blocks = 4;
-    if (B * octs * ((nb + 3) / 4) < 1024) m.chunk_blocks = 2;
-  } else {
-    m.wg_waves = 4;
-    long chunks = (1024 + B * octs - 1) / (B * octs);
-    if (chunks > nb / 8) chunks = nb / 8 > 0 ? nb / 8 : 1;
-    m.chunk_blocks = (int)((nb + chunks - 1) / chunks);
-  }
-  static const int chunk_override = env_override("SPEAR_BTP_FUSED_CHUNK_BLOCKS");
-  static const int waves_override = env_override("SPEAR_BTP_FUSED_WG_WAVES");
-  if (chunk_override) m.chunk_blocks = chunk_override;
-  if (waves_override) m.wg_waves = waves_override == 8 ? 8 : 4;
-  if (m.chunk_blocks > nb) m.chunk_blocks = nb;
-  m.chunks = (nb + m.chunk_blocks - 1) / m.chunk_blocks;
-  return m;
-}
-
-template <class E, int kW, bool kQkv, bool kF32 = false>
-void launch_mix_fwd(const MixArgs& p, const MixPlan& m, hipStream_t s) {
-  const long total = (long)p.B * m.chunks * ((p.H + 7) / 8);
-  const unsigned blocks = (unsigned)((total + kW - 1) / kW);
-  hipLaunchKernelGGL((phalanx_mix_fwd_kernel<E, kW, kQkv, kF32>), dim3(blocks), dim3(64 * kW), 0, s,
-                     static_cast<const uint16_t*>(p.a_logit), static_cast<const uint16_t*>(p.b_logit),
-                     static_cast<const uint16_t*>(p.c), static_cast<const uint16_t*>(p.v), static_cast<uint16_t*>(p.out),
-                     p.c_prev_tail, p.L, p.H, p.kv_groups, m.chunk_blocks * kTile, m.chunks, total);
-}
-
-// Tile geometry shared by the tile kernels: a workgroup is `waves` consecutive blocks of one head group.
+// Tile geometry shared by the two kernels: a workgroup is `waves` consecutive blocks of one head slot.
 struct TileGrid {
-  int tiles;  // time tiles per row: one workgroup each per head group
+  int tiles;  // time tiles per row: one workgroup each per head slot
   long wgs;
 };
-TileGrid tile_grid(long B, int H, int L, int waves) {
-  const int octs = (H + 7) / 8, nb = L / kTile;
+TileGrid tile_grid(long B, int slots, int L, int waves) {
+  const int nb = L / kTile;
   TileGrid g;
   g.tiles = (nb + waves - 1) / waves;
   const int tg = g.tiles < SPEAR_FUSED_TILE_TIME_GROUP ? g.tiles : SPEAR_FUSED_TILE_TIME_GROUP;  // tile_place()
-  g.wgs = B * (long)((g.tiles + tg - 1) / tg) * tg * octs;
+  g.wgs = B * (long)((g.tiles + tg - 1) / tg) * tg * slots;
   return g;
 }
 
+// Workgroups of 8 wavefronts on rows of one head slot and on long rows of up to 32 heads, of 4 otherwise
+// (table at the forward kernel).
+bool forward_takes_eight_waves(int H, int L) { return H < 16 || (L >= 512 && H <= 32); }
+
 template <class E, int kW, bool kQkv, bool kF32 = false>
 void launch_mix_fwd_tile(const MixArgs& p, hipStream_t s) {
-  const TileGrid g = tile_grid(p.B, p.H, p.L, kW);
+  const TileGrid g = tile_grid(p.B, (p.H + kHeadsPerWave - 1) / kHeadsPerWave, p.L, kW);
   hipLaunchKernelGGL((phalanx_mix_fwd_tile_kernel<E, kW, kQkv, kF32>), dim3((unsigned)g.wgs), dim3(64 * kW), 0, s,
                      static_cast<const uint16_t*>(p.a_logit), static_cast<const uint16_t*>(p.b_logit),
                      static_cast<const uint16_t*>(p.c), static_cast<const uint16_t*>(p.v), static_cast<uint16_t*>(p.out),
                      p.c_prev_tail, p.L, p.H, p.kv_groups, g.tiles);
 }
 
+// Groups of 1, 2, 4, 8 heads per kv head are summed inside a wavefront's 8 heads; the others take slots cut at
+// group borders (head_slot).
+bool wide_grouping(int kv_groups) { return kv_groups != 1 && kv_groups != 2 && kv_groups != 4 && kv_groups != 8; }
+
+int backward_slots(int H, int kv_groups) {
+  if (!wide_grouping(kv_groups)) return (H + kHeadsPerWave - 1) / kHeadsPerWave;
+  const int kv_heads = H / kv_groups;
+  if (kv_groups > kHeadsPerWave) return kv_heads;
+  const int per_slot = kHeadsPerWave / kv_groups;
+  return (kv_heads + per_slot - 1) / per_slot;
+}
+
+template <class E, bool kQkv, bool kF32, bool kSums, bool kWide>
+void launch_mix_bwd_tile(const MixBwdArgs& p, hipStream_t s) {
+  const int slots = backward_slots(p.H, p.kv_groups);
+  const TileGrid g = tile_grid(p.B, slots, p.L, kTileWaves);
+  auto u = [](const void* q) { return static_cast<const uint16_t*>(q); };
+  auto w = [](void* q) { return static_cast<uint16_t*>(q); };
+  const int Fkv = (p.H / p.kv_groups) * kChan;
+  hipLaunchKernelGGL((phalanx_mix_bwd_tile_kernel<E, kQkv, kF32, kSums, kWide>), dim3((unsigned)g.wgs),
+                     dim3(64 * kTileWaves), 0, s, u(p.a_logit), u(p.b_logit), u(p.c), u(p.v), u(p.dout), w(p.da_logit),
+                     w(p.db_logit), w(p.dc), w(p.dv), p.sum_da, p.sum_db, p.sum_dc, p.ld_da ? p.ld_da : p.H,
+                     p.ld_db ? p.ld_db : Fkv, p.ld_dc ? p.ld_dc : Fkv, p.ld_dv ? p.ld_dv : p.H * kChan, p.L, p.H,
+                     p.kv_groups, g.tiles, slots);
+}
+
 }  // namespace
 
+long fused_mix_workgroups(long B, int H, int kv_groups, int L, bool backward) {
+  if (B <= 0 || H <= 0 || L <= 0 || kv_groups <= 0) return 0;
+  if (backward) return tile_grid(B, backward_slots(H, kv_groups), L, kTileWaves).wgs;
+  return tile_grid(B, (H + kHeadsPerWave - 1) / kHeadsPerWave, L, forward_takes_eight_waves(H, L) ? 8 : 4).wgs;
+}
+
 hipError_t fused_mix_forward(const MixArgs& p, hipStream_t s) {
-  if (p.tile_split) {  // the caller has checked: a grid that fits
-    // workgroups of 8 wavefronts on rows of one head group and on long rows of up to 32 heads, of 4 otherwise
-    // (table at the kernel)
-    static const int waves_override = env_override("SPEAR_BTP_FUSED_FWD_TILE_WAVES");
-    const bool eight = waves_override ? waves_override == 8 : (p.H < 16 || (p.L >= 512 && p.H <= 32));
-    auto by_form = [&](auto e, auto q) {
-      using E = decltype(e);
-      if (p.f32_out) launch_mix_fwd_tile<E, 4, decltype(q)::value, true>(p, s);  // check mode: one instance per form
-      else if (eight) launch_mix_fwd_tile<E, 8, decltype(q)::value>(p, s);
-      else launch_mix_fwd_tile<E, 4, decltype(q)::value>(p, s);
-    };
-    if (p.dtype == kBf16) {
-      if (p.qkv) by_form(Bf16{}, std::true_type{});
-      else by_form(Bf16{}, std::false_type{});
-    } else {
-      if (p.qkv) by_form(Fp16{}, std::true_type{});
-      else by_form(Fp16{}, std::false_type{});
-    }
-    return hipGetLastError();
-  }
-  const MixPlan m = plan_mix(p.B, p.H, p.L);
-  auto by_waves = [&](auto e, auto q) {
+  const bool eight = forward_takes_eight_waves(p.H, p.L);
+  auto by_form = [&](auto e, auto q) {
     using E = decltype(e);
-    if (p.f32_out) launch_mix_fwd<E, 4, decltype(q)::value, true>(p, m, s);  // check mode: one instance per form
-    else if (m.wg_waves == 8) launch_mix_fwd<E, 8, decltype(q)::value>(p, m, s);
-    else launch_mix_fwd<E, 4, decltype(q)::value>(p, m, s);
+    if (p.f32_out) launch_mix_fwd_tile<E, 4, decltype(q)::value, true>(p, s);  // check mode: one instance per form
+    else if (eight) launch_mix_fwd_tile<E, 8, decltype(q)::value>(p, s);
+    else launch_mix_fwd_tile<E, 4, decltype(q)::value>(p, s);
   };
   if (p.dtype == kBf16) {
-    if (p.qkv) by_waves(Bf16{}, std::true_type{});
-    else by_waves(Bf16{}, std::false_type{});
+    if (p.qkv) by_form(Bf16{}, std::true_type{});
+    else by_form(Bf16{}, std::false_type{});
   } else {
-    if (p.qkv) by_waves(Fp16{}, std::true_type{});
-    else by_waves(Fp16{}, std::false_type{});
+    if (p.qkv) by_form(Fp16{}, std::true_type{});
+    else by_form(Fp16{}, std::false_type{});
   }
   return hipGetLastError();
 }
 
-namespace {
-
-// The backward kernel holds twice the state per wavefront and measured best with long walks in
-// workgroups of 4; rows are cut (at a cost of two extra blocks of reads per chunk) only to fill the GPU.
-MixPlan plan_mix_bwd(long B, int H, int L) {
-  const long octs = (H + 7) / 8;
-  const int nb = L / kTile;
-  MixPlan m;
-  m.wg_waves = kWaves;
-  long chunks = (1024 + B * octs - 1) / (B * octs);
-  const int min_blocks = B * octs * ((nb + 7) / 8) < 512 ? 2 : 8;  // badly underfilled: shorter chunks still pay
-  if (chunks > nb / min_blocks) chunks = nb / min_blocks > 0 ? nb / min_blocks : 1;
-  m.chunk_blocks = (int)((nb + chunks - 1) / chunks);
-  static const int chunk_override = env_override("SPEAR_BTP_FUSED_BWD_CHUNK_BLOCKS");
-  if (chunk_override) m.chunk_blocks = chunk_override;
-  if (m.chunk_blocks > nb) m.chunk_blocks = nb;
-  m.chunks = (nb + m.chunk_blocks - 1) / m.chunk_blocks;
-  return m;
-}
-
-template <class E, bool kSums, bool kQkv, bool kF32 = false>
-void launch_mix_bwd(const MixBwdArgs& p, const MixPlan& m, hipStream_t s) {
-  const long total = (long)p.B * m.chunks * ((p.H + 7) / 8);
-  const unsigned blocks = (unsigned)((total + kWaves - 1) / kWaves);
-  auto u = [](const void* q) { return static_cast<const uint16_t*>(q); };
-  auto w = [](void* q) { return static_cast<uint16_t*>(q); };
-  const int Fkv = (p.H / p.kv_groups) * kChan;
-  hipLaunchKernelGGL((phalanx_mix_bwd_kernel<E, kSums, kQkv, kF32>), dim3(blocks), dim3(64 * kWaves), 0, s, u(p.a_logit),
-                     u(p.b_logit), u(p.c), u(p.v), u(p.dout), w(p.da_logit), w(p.db_logit), w(p.dc), w(p.dv), p.sum_da,
-                     p.sum_db, p.sum_dc, p.ld_da ? p.ld_da : p.H, p.ld_db ? p.ld_db : Fkv, p.ld_dc ? p.ld_dc : Fkv,
-                     p.ld_dv ? p.ld_dv : p.H * kChan, p.L, p.H, p.kv_groups, m.chunk_blocks * kTile, m.chunks, total);
-}
-
-// 1 head group x 4 blocks per workgroup (two of four wavefronts read a halo). 2 x 2 (all four do, but a workgroup
-// reads 512-byte runs) is 2-9 % slower at 12 of 14 shapes and equal at the other two.
-TileGrid bwd_tile_grid(long B, int H, int L) { return tile_grid(B, H, L, kTileWaves); }
-
-template <class E, bool kQkv, bool kF32 = false, bool kSums = false>
-void launch_mix_bwd_tile(const MixBwdArgs& p, hipStream_t s) {
-  const TileGrid g = bwd_tile_grid(p.B, p.H, p.L);
-  auto u = [](const void* q) { return static_cast<const uint16_t*>(q); };
-  auto w = [](void* q) { return static_cast<uint16_t*>(q); };
-  const int Fkv = (p.H / p.kv_groups) * kChan;
-  hipLaunchKernelGGL((phalanx_mix_bwd_tile_kernel<E, kQkv, kF32, kSums>), dim3((unsigned)g.wgs), dim3(64 * kTileWaves), 0,
-                     s, u(p.a_logit), u(p.b_logit), u(p.c), u(p.v), u(p.dout), w(p.da_logit), w(p.db_logit), w(p.dc),
-                     w(p.dv), p.sum_da, p.sum_db, p.sum_dc, p.ld_da ? p.ld_da : p.H, p.ld_db ? p.ld_db : Fkv,
-                     p.ld_dc ? p.ld_dc : Fkv, p.ld_dv ? p.ld_dv : p.H * kChan, p.L, p.H, p.kv_groups, g.tiles);
-}
-
-}  // namespace
-
-long fused_mix_backward_sum_rows(long B, int H, int L, bool tile_split) {
+long fused_mix_backward_sum_rows(long B, int H, int L) {
   if (B <= 0 || H <= 0 || L <= 0) return 0;
-  return tile_split ? B * bwd_tile_grid(B, H, L).tiles : B * plan_mix_bwd(B, H, L).chunks;
+  return B * ((L / kTile + kTileWaves - 1) / kTileWaves);
 }
 
 hipError_t fused_mix_backward(const MixBwdArgs& p, hipStream_t s) {
-  const MixPlan m = plan_mix_bwd(p.B, p.H, p.L);
   const bool sums = p.sum_da != nullptr;
   if (sums && (p.qkv || p.f32_grads)) return hipErrorInvalidValue;  // the caller has checked: layer form, 16-bit results
-  if (p.tile_split) {  // the caller has checked: a grid that fits
-    if (sums) {
-      if (p.dtype == kBf16) launch_mix_bwd_tile<Bf16, false, false, true>(p, s);
-      else launch_mix_bwd_tile<Fp16, false, false, true>(p, s);
-      return hipGetLastError();
-    }
-    if (p.dtype == kBf16) {
-      if (p.f32_grads) {
-        if (p.qkv) launch_mix_bwd_tile<Bf16, true, true>(p, s);
-        else launch_mix_bwd_tile<Bf16, false, true>(p, s);
-      } else {
-        if (p.qkv) launch_mix_bwd_tile<Bf16, true>(p, s);
-        else launch_mix_bwd_tile<Bf16, false>(p, s);
-      }
-    } else {
-      if (p.f32_grads) {
-        if (p.qkv) launch_mix_bwd_tile<Fp16, true, true>(p, s);
-        else launch_mix_bwd_tile<Fp16, false, true>(p, s);
-      } else {
-        if (p.qkv) launch_mix_bwd_tile<Fp16, true>(p, s);
-        else launch_mix_bwd_tile<Fp16, false>(p, s);
-      }
-    }
-    return hipGetLastError();
-  }
-  if (p.f32_grads) {
-    if (p.dtype == kBf16) {
-      if (p.qkv) launch_mix_bwd<Bf16, false, true, true>(p, m, s);
-      else launch_mix_bwd<Bf16, false, false, true>(p, m, s);
-    } else {
-      if (p.qkv) launch_mix_bwd<Fp16, false, true, true>(p, m, s);
-      else launch_mix_bwd<Fp16, false, false, true>(p, m, s);
-    }
-    return hipGetLastError();
-  }
+  const bool wide = wide_grouping(p.kv_groups);
+  auto by_options = [&](auto e, auto wd) {
+    using E = decltype(e);
+    constexpr bool kWide = decltype(wd)::value;
+    if (sums) launch_mix_bwd_tile<E, false, false, true, kWide>(p, s);
+    else if (p.f32_grads && p.qkv) launch_mix_bwd_tile<E, true, true, false, kWide>(p, s);
+    else if (p.f32_grads) launch_mix_bwd_tile<E, false, true, false, kWide>(p, s);
+    else if (p.qkv) launch_mix_bwd_tile<E, true, false, false, kWide>(p, s);
+    else launch_mix_bwd_tile<E, false, false, false, kWide>(p, s);
+  };
   if (p.dtype == kBf16) {
-    if (p.qkv) launch_mix_bwd<Bf16, false, true>(p, m, s);
-    else if (sums) launch_mix_bwd<Bf16, true, false>(p, m, s);
-    else launch_mix_bwd<Bf16, false, false>(p, m, s);
+    if (wide) by_options(Bf16{}, std::true_type{});
+    else by_options(Bf16{}, std::false_type{});
   } else {
-    if (p.qkv) launch_mix_bwd<Fp16, false, true>(p, m, s);
-    else if (sums) launch_mix_bwd<Fp16, true, false>(p, m, s);
-    else launch_mix_bwd<Fp16, false, false>(p, m, s);
+    if (wide) by_options(Fp16{}, std::true_type{});
+    else by_options(Fp16{}, std::false_type{});
   }
   return hipGetLastError();
 }

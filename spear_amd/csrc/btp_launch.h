@@ -56,27 +56,28 @@ struct MixArgs {
   // null, or fp32 [B, H, 16]: receives the terminal local state of every row's last block (the c_prev of the
   // streaming state after this prompt)
   float* c_prev_tail = nullptr;
-  bool tile_split = false;  // one wavefront per 16-step block instead of wavefronts walking through time
 };
 hipError_t fused_mix_forward(const MixArgs& p, hipStream_t s);
+// Workgroups the forward / backward kernel launches for a shape (must fit a 31-bit grid).
+long fused_mix_workgroups(long B, int H, int kv_groups, int L, bool backward);
 
-// Fused layer-layout backward (btp_fused.hip); kv_groups = H / kv_heads must be 1, 2, 4 or 8.
+// Fused layer-layout backward (btp_fused.hip); kv_groups = H / kv_heads, any positive integer.
 struct MixBwdArgs {
   const void *a_logit, *b_logit, *c, *v, *dout;  // [B,L,H], [B,L,Hkv*16] x 2, [B,L,H*16] x 2
   void *da_logit, *db_logit, *dc, *dv;           // same shapes as the inputs they belong to
   int B, L, H, kv_groups;
   int dtype;
-  // all three null, or fp32 [fused_mix_backward_sum_rows(B, H, L, tile_split), H | Hkv*16 | Hkv*16]: per-chunk sums over time
+  // all three null, or fp32 [fused_mix_backward_sum_rows(B, H, L), H | Hkv*16 | Hkv*16]: sums over the time steps of
+  // one (batch row, time tile) per row
   float *sum_da = nullptr, *sum_db = nullptr, *sum_dc = nullptr;
   // elements per time step of each gradient tensor; 0 = dense (its own width)
   int ld_da = 0, ld_db = 0, ld_dc = 0, ld_dv = 0;
   bool qkv = false;  // as in MixArgs; da_logit is then the fp32 gradient of the gate
   bool f32_grads = false;  // check mode: da_logit, db_logit, dc, dv are fp32
-  bool tile_split = false;  // one wavefront per 16-step block instead of wavefronts that walk through time
 };
 hipError_t fused_mix_backward(const MixBwdArgs& p, hipStream_t s);
-long fused_mix_backward_sum_rows(long B, int H, int L, bool tile_split = false);
-// The same backward with the column sums finished inside the library: the per-chunk partial sums go through
+long fused_mix_backward_sum_rows(long B, int H, int L);
+// The same backward with the column sums finished inside the library: the per-tile partial sums go through
 // a static device array instead of caller memory, and bias_da [H], bias_db / bias_dc [(H / kv_groups) * 16]
 // receive the sums over batch and time. Allocates nothing. `p.sum_*` are ignored.
 hipError_t fused_mix_backward_bias(const MixBwdArgs& p, float* bias_da, float* bias_db, float* bias_dc, hipStream_t s);

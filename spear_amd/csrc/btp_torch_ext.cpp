@@ -214,8 +214,7 @@ MixShape check_mix_inputs(const at::Tensor& a_logit, const at::Tensor& b_logit, 
                           int64_t heads, int64_t kv_heads, bool qkv_gate) {
   TORCH_CHECK(a_logit.is_cuda() && b_logit.is_cuda() && c.is_cuda() && v.is_cuda(), "All tensors must be CUDA.");
   TORCH_CHECK(v.dim() == 3 && v.size(2) == heads * 16, "v must be [B, L, heads * 16].");
-  TORCH_CHECK(heads % 4 == 0, "heads must be a multiple of 4.");
-  TORCH_CHECK(kv_heads > 0 && heads % kv_heads == 0, "heads must be divisible by kv_heads.");
+  TORCH_CHECK(heads > 0 && kv_heads > 0 && heads % kv_heads == 0, "heads must be divisible by kv_heads.");
   TORCH_CHECK(is_16bit(v), "tensors must be float16 or bfloat16.");
   TORCH_CHECK(b_logit.scalar_type() == v.scalar_type() && c.scalar_type() == v.scalar_type(), "all tensors must share one dtype.");
   if (qkv_gate) {
@@ -261,15 +260,13 @@ int64_t row_stride(const char* name, const at::Tensor& t, int64_t B, int64_t L, 
 }
 
 // Gradients of mix_forward, written in place. Float32 db_logit / dc / dv (and da_logit) select the fp32
-// check mode. `sums`: none, or three fp32 [rows, width] tensors receiving per-chunk column sums.
+// check mode. `sums`: none, or three fp32 [rows, width] tensors receiving the column sums of every (batch row,
+// tile of 64 time steps).
 void mix_backward(const at::Tensor& a_logit, const at::Tensor& b_logit, const at::Tensor& c, const at::Tensor& v,
                   const at::Tensor& dout, at::Tensor da_logit, at::Tensor db_logit, at::Tensor dc, at::Tensor dv,
-                  int64_t heads, int64_t kv_heads, const std::vector<at::Tensor>& sums, bool qkv_gate,
-                  bool tile_sums) {
+                  int64_t heads, int64_t kv_heads, const std::vector<at::Tensor>& sums, bool qkv_gate) {
   const MixShape s = check_mix_inputs(a_logit, b_logit, c, v, heads, kv_heads, qkv_gate);
   TORCH_CHECK(dout.is_cuda() && da_logit.is_cuda() && db_logit.is_cuda() && dc.is_cuda() && dv.is_cuda(), "All tensors must be CUDA.");
-  const int64_t groups = heads / kv_heads;
-  TORCH_CHECK(groups == 1 || groups == 2 || groups == 4 || groups == 8, "heads / kv_heads must be 1, 2, 4 or 8.");
   TORCH_CHECK(dout.scalar_type() == v.scalar_type(), "all tensors must share one dtype.");
   check_layout("dout", dout, {s.B, s.L, s.F});
   const bool f32 = dv.scalar_type() == at::kFloat;
@@ -290,8 +287,7 @@ void mix_backward(const at::Tensor& a_logit, const at::Tensor& b_logit, const at
   int64_t rows = 0;
   float* sp[3] = {nullptr, nullptr, nullptr};
   if (!sums.empty()) {
-    rows = tile_sums ? spear_phalanx_mix_backward_sum_rows_tile((int)s.B, (int)s.L, (int)heads)
-                     : spear_phalanx_mix_backward_sum_rows((int)s.B, (int)s.L, (int)heads);
+    rows = spear_phalanx_mix_backward_sum_rows((int)s.B, (int)s.L, (int)heads);
     const int64_t widths[3] = {heads, s.Fkv, s.Fkv};
     const char* names[3] = {"sum_da", "sum_db", "sum_dc"};
     for (int i = 0; i < 3; ++i) {
@@ -302,13 +298,72 @@ void mix_backward(const at::Tensor& a_logit, const at::Tensor& b_logit, const at
     }
   }
   const c10::DeviceGuard guard(v.device());
-  const unsigned flags = (qkv_gate ? SPEAR_MIX_QKV_GATE : 0u) | (f32 ? SPEAR_MIX_F32_RESULTS : 0u) |
-                         ((tile_sums && !sums.empty()) ? SPEAR_MIX_TILE_SPLIT : 0u);
+  const unsigned flags = (qkv_gate ? SPEAR_MIX_QKV_GATE : 0u) | (f32 ? SPEAR_MIX_F32_RESULTS : 0u);
   const int rc = spear_phalanx_mix_backward_ex(
       a_logit.data_ptr(), b_logit.data_ptr(), c.data_ptr(), v.data_ptr(), dout.data_ptr(), da_logit.data_ptr(),
       db_logit.data_ptr(), dc.data_ptr(), dv.data_ptr(), (int)ld_da, (int)ld_db, (int)ld_dc, (int)ld_dv, sp[0], sp[1], sp[2],
       rows, (int)s.B, (int)s.L, (int)heads, (int)kv_heads, tag_of(v.scalar_type()), flags, stream_of(v));
   if (rc != 0) raise_native(rc);
+}
+
+// The autograd node of btp_log(), compiled like BtpNode: forward allocates y, backward dx and dgate.
+struct BtpLogNode : public torch::autograd::Function<BtpLogNode> {
+  static at::Tensor forward(torch::autograd::AutogradContext* ctx, const at::Tensor& gate, const at::Tensor& x, int64_t k,
+                            bool y_f32) {
+    TORCH_CHECK(x.dim() == 4, "x must be [B, H, 16, L].");
+    at::Tensor y = at::empty(x.sizes(), x.options().dtype(y_f32 ? at::kFloat : x.scalar_type()));
+    forward_log(gate, x, y, k);
+    ctx->save_for_backward({gate, x});
+    ctx->saved_data["k"] = k;
+    return y;
+  }
+
+  static torch::autograd::variable_list backward(torch::autograd::AutogradContext* ctx,
+                                                 torch::autograd::variable_list grad_outputs) {
+    const auto saved = ctx->get_saved_variables();
+    const at::Tensor &gate = saved[0], &x = saved[1];
+    at::Tensor dx = at::empty(x.sizes(), x.options());
+    at::Tensor dgate = at::empty(gate.sizes(), gate.options());
+    backward_log(gate, x, grad_outputs[0].contiguous(), dx, dgate, ctx->saved_data["k"].toInt());
+    return {dgate, dx, at::Tensor(), at::Tensor()};
+  }
+};
+
+at::Tensor btp_log_autograd(const at::Tensor& gate, const at::Tensor& x, int64_t k, bool y_f32) {
+  return BtpLogNode::apply(gate, x, k, y_f32);
+}
+
+// The autograd node of phalanx_mix() and, with qkv_gate, of btp_qkv() (operands then in the kernel's order: gate,
+// k, q, v), compiled: forward allocates out, backward the four gradients (the first one in a_logit's dtype, which
+// for the q/k/v/gate form is the fp32 of the gate). What spear_amd/ops/btp/fused.py does in torch.autograd.Function
+// classes over the traceable custom ops, without their Python frames; used for plain eager tensors only.
+struct MixNode : public torch::autograd::Function<MixNode> {
+  static at::Tensor forward(torch::autograd::AutogradContext* ctx, const at::Tensor& a_logit, const at::Tensor& b_logit,
+                            const at::Tensor& c, const at::Tensor& v, int64_t heads, int64_t kv_heads, bool qkv_gate) {
+    at::Tensor out = at::empty(v.sizes(), v.options());
+    mix_forward(a_logit, b_logit, c, v, out, heads, kv_heads, qkv_gate);
+    ctx->save_for_backward({a_logit, b_logit, c, v});
+    ctx->saved_data["heads"] = heads;
+    ctx->saved_data["kv_heads"] = kv_heads;
+    ctx->saved_data["qkv_gate"] = qkv_gate;
+    return out;
+  }
+
+  static torch::autograd::variable_list backward(torch::autograd::AutogradContext* ctx,
+                                                 torch::autograd::variable_list grad_outputs) {
+    const auto saved = ctx->get_saved_variables();
+    const at::Tensor &a_logit = saved[0], &b_logit = saved[1], &c = saved[2], &v = saved[3];
+    at::Tensor da = at::empty(a_logit.sizes(), a_logit.options()), db = at::empty(b_logit.sizes(), b_logit.options()),
+               dc = at::empty(c.sizes(), c.options()), dv = at::empty(v.sizes(), v.options());
+    mix_backward(a_logit, b_logit, c, v, grad_outputs[0].contiguous(), da, db, dc, dv, ctx->saved_data["heads"].toInt(),
+                 ctx->saved_data["kv_heads"].toInt(), {}, ctx->saved_data["qkv_gate"].toBool());
+    return {da, db, dc, dv, at::Tensor(), at::Tensor(), at::Tensor()};
+  }
+};
+
+at::Tensor mix_autograd(const at::Tensor& a_logit, const at::Tensor& b_logit, const at::Tensor& c, const at::Tensor& v,
+                        int64_t heads, int64_t kv_heads, bool qkv_gate) {
+  return MixNode::apply(a_logit, b_logit, c, v, heads, kv_heads, qkv_gate);
 }
 
 }  // namespace
@@ -329,10 +384,14 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         py::arg("heads"), py::arg("kv_heads"), py::arg("qkv_gate") = false);
   m.def("mix_backward", &mix_backward, py::arg("a_logit"), py::arg("b_logit"), py::arg("c"), py::arg("v"), py::arg("dout"),
         py::arg("da_logit"), py::arg("db_logit"), py::arg("dc"), py::arg("dv"), py::arg("heads"), py::arg("kv_heads"),
-        py::arg("sums") = std::vector<at::Tensor>(), py::arg("qkv_gate") = false, py::arg("tile_sums") = false);
+        py::arg("sums") = std::vector<at::Tensor>(), py::arg("qkv_gate") = false);
+  m.def("btp_log_autograd", &btp_log_autograd, py::arg("gate"), py::arg("x"), py::arg("k"), py::arg("y_f32"),
+        "y = btp(exp(gate), x) with its autograd node (contiguous plain tensors; gradients: dgate float32, dx in x's dtype)");
+  m.def("mix_autograd", &mix_autograd, py::arg("a_logit"), py::arg("b_logit"), py::arg("c"), py::arg("v"), py::arg("heads"),
+        py::arg("kv_heads"), py::arg("qkv_gate") = false,
+        "out = phalanx_mix(...) (or the q/k/v/gate form) with its autograd node (contiguous plain tensors)");
   m.def("abi_version", []() { return spear_btp_abi_version(); });
-  m.def("mix_backward_sum_rows", [](int64_t B, int64_t L, int64_t heads, bool tile_sums) {
-    return (int64_t)(tile_sums ? spear_phalanx_mix_backward_sum_rows_tile((int)B, (int)L, (int)heads)
-                               : spear_phalanx_mix_backward_sum_rows((int)B, (int)L, (int)heads));
-  }, py::arg("B"), py::arg("L"), py::arg("heads"), py::arg("tile_sums") = false);
+  m.def("mix_backward_sum_rows", [](int64_t B, int64_t L, int64_t heads) {
+    return (int64_t)spear_phalanx_mix_backward_sum_rows((int)B, (int)L, (int)heads);
+  }, py::arg("B"), py::arg("L"), py::arg("heads"));
 }

@@ -338,8 +338,8 @@ def phalanx_prefill(layer, x: torch.Tensor) -> tuple[torch.Tensor, PhalanxStepSt
     _need_gpu(x)
     B, L, _ = x.shape
     p, bl = layer.param, 16
-    if layer.heads % 4 != 0 or layer.k != 2:
-        raise RuntimeError("phalanx_prefill needs a layer the fused kernels serve: heads divisible by 4, k == 2")
+    if layer.k != 2:
+        raise RuntimeError("phalanx_prefill needs a layer with k == 2")
     full = (L // bl) * bl
     state = PhalanxStepState.zeros(B, layer.heads, x.device, bl)
     xc = x.to(p.compute_dtype)

@@ -11,7 +11,7 @@ three additions. ``project_and_mix`` goes further for the fused mixing stage: it
 four gradients side by side into one ``[B, L, ld]`` buffer, which is the gradient of the concatenated
 projection, so input and weight gradients are one GEMM each against the stacked weights (the forward stays
 four GEMMs, which measured faster than one wide one); and the kernel leaves the column sums of the gate
-gradients (the three bias gradients) as it walks through time, so they are not read again to be summed.
+gradients (the three bias gradients) per tile of 64 time steps, so they are not read again to be summed.
 
 Short token axes gain nothing (their step is bound by launch overhead, of which this path has more), so
 the layer uses these functions from 8192 tokens on (``pays_off``).
@@ -25,8 +25,7 @@ from __future__ import annotations
 import torch
 import torch.nn.functional as F
 
-__all__ = ["weight_grad", "input_projections", "linear", "pays_off", "project_and_mix", "mix_kernel_sums_groups",
-           "packed_columns"]
+__all__ = ["weight_grad", "input_projections", "linear", "pays_off", "project_and_mix", "packed_columns"]
 
 _TILE = 128           # output tile edge the slice count is sized against
 _TARGET_TILES = 1024  # about four tiles per compute unit
@@ -110,12 +109,6 @@ class _Linear(torch.autograd.Function):
         return (d @ w if ctx.needs_input_grad[0] else None, weight_grad(d, x) if ctx.needs_input_grad[1] else None)
 
 
-def mix_kernel_sums_groups(heads: int, kv_heads: int) -> bool:
-    """Whether the fused backward kernel handles this head grouping (a group inside one wavefront)."""
-    groups = heads // kv_heads
-    return heads % 4 == 0 and heads % kv_heads == 0 and groups in (1, 2, 4, 8) and (groups < 8 or heads % 8 == 0)
-
-
 def packed_columns(heads: int, kv_heads: int) -> tuple[dict[str, tuple[int, int]], int]:
     """Column blocks ``name -> (first column, width)`` of the four projections' outputs laid side by side
     as ``[b | c | v | a | padding]``, and the padded row length (a multiple of 64 elements, so that every
@@ -143,9 +136,9 @@ def _mix_backward_packed(
     if used < ld:
         packed[..., used:].zero_()
     da, db, dc, dv = (packed[..., cols[k][0]:cols[k][0] + cols[k][1]] for k in "abcv")
-    rows = _btp.mix_backward_sum_rows(B, L, heads, tile_split=True)  # the faster of the two work splits
+    rows = _btp.mix_backward_sum_rows(B, L, heads)
     sums = [torch.empty((rows, t.shape[-1]), device=v.device, dtype=torch.float32) for t in (a_logits, b_logits, c)]
-    _btp.mix_backward(a_logits, b_logits, c, v, dout, da, db, dc, dv, heads, kv_heads, sums=tuple(sums), tile_split=True)
+    _btp.mix_backward(a_logits, b_logits, c, v, dout, da, db, dc, dv, heads, kv_heads, sums=tuple(sums))
     return (packed, *(s.sum(0).to(v.dtype) for s in sums))
 
 
@@ -194,8 +187,7 @@ class _ProjectAndMix(torch.autograd.Function):
 
 def project_and_mix(x: torch.Tensor, proj_a, proj_b, proj_c, proj_v, heads: int, kv_heads: int) -> torch.Tensor:
     """``phalanx_mix(proj_a(x), proj_b(x), proj_c(x), proj_v(x), heads, kv_heads)`` for ``x[B, L, K]`` with the
-    projections' backward of this module and the bias gradients taken from the mixing kernel. Needs a head
-    grouping the fused backward kernel handles (``mix_kernel_sums_groups``)."""
+    projections' backward of this module and the bias gradients taken from the mixing kernel."""
     import spear_amd.ops.btp.fused  # noqa: F401  (registers torch.ops.spear_btp.mix_forward)
 
     return _ProjectAndMix.apply(x.contiguous(), proj_a.weight, proj_a.bias, proj_b.weight, proj_b.bias,

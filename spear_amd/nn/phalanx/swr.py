@@ -15,10 +15,11 @@ initialises identical weights).
   ``"pytorch"``           the log-space PyTorch statement of the two-pass algorithm
   ``"pytorch_linspace"``  the linear-space PyTorch statement
   ``"fused"``             (addition) one HIP kernel for gates + recurrence + ``* C + V`` working
-                          directly on the projection outputs; needs ``heads % 4 == 0``, ``k == 2``
+                          directly on the projection outputs, for any ``heads % kv_heads == 0``;
+                          needs ``k == 2``
 The choice is explicit; ``"default"`` and ``"fused"`` never degrade to a PyTorch path. Code written
 against the reference says ``method="default"``; with ``SPEAR_PHALANX_DEFAULT=fused`` in the environment
-such a layer runs the fused kernels wherever they apply (``heads % 4 == 0``, ``k == 2``, bf16 output) and
+such a layer runs the fused kernels wherever they apply (``k == 2``, 16-bit output) and
 the stand-alone kernels elsewhere, without a change to the calling code.
 
 On a GPU, from 8192 tokens per call on, the ``"default"`` and ``"fused"`` layers run their five
@@ -34,7 +35,7 @@ import os
 import torch
 import torch.nn as nn
 
-from .projections import input_projections, linear, mix_kernel_sums_groups, pays_off, project_and_mix
+from .projections import input_projections, linear, pays_off, project_and_mix
 
 _HEAD_DIM = 16
 _METHODS = ("default", "pytorch", "pytorch_linspace", "fused")
@@ -165,8 +166,8 @@ class Phalanx(nn.Module):
                 raise ValueError(f"head_dim must be 16, got {dim // heads}. Use heads=dim//16 or leave heads=None")
         if method not in _METHODS:
             raise ValueError(f"method must be one of 'default', 'pytorch', 'pytorch_linspace', got {method}")
-        if method == "fused" and (heads % 4 != 0 or k != 2):
-            raise ValueError("method 'fused' needs heads divisible by 4 and k == 2")
+        if method == "fused" and k != 2:
+            raise ValueError("method 'fused' needs k == 2")
 
         self.dim = dim
         self.heads = heads
@@ -187,7 +188,7 @@ class Phalanx(nn.Module):
 
         runs_fused = method == "fused" or (
             method == "default" and os.environ.get("SPEAR_PHALANX_DEFAULT", "") == "fused"
-            and heads % 4 == 0 and k == 2 and self.output_dtype == self.compute_dtype
+            and k == 2 and self.output_dtype == self.compute_dtype
         )
         if method == "default" and not runs_fused:
             from spear_amd.ops.btp import btp
@@ -228,7 +229,7 @@ class Phalanx(nn.Module):
     def _forward_fused(self, x: torch.Tensor) -> torch.Tensor:
         p = self.param
         xc = x.to(p.compute_dtype)
-        if xc.dim() == 3 and pays_off(xc) and mix_kernel_sums_groups(self.heads, self.kv_heads):
+        if xc.dim() == 3 and pays_off(xc):
             mixed = project_and_mix(xc, p.proj_a, p.proj_b, p.proj_c, p.proj_v, self.heads, self.kv_heads)
         else:
             mixed = self.mix_module(*p.project(xc), self.heads, self.kv_heads)

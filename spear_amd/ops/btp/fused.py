@@ -7,11 +7,10 @@ result once (no transposing copies, no intermediate tensors). It fuses what the 
 separate PyTorch ops around its BTP kernel (spear/nn/phalanx/swr.py:166-221, 311-327 and the
 ``.contiguous()`` calls of spear/ops/btp/interface.py:186-187).
 
-Backward is a second fused kernel (reverse walk through time, every operand read once, every
-gradient written once), including the sum of the ``b`` / ``c`` gradients over the heads that share
-a kv head when a group has 2, 4 or 8 heads. Larger groups span several wavefronts; that case
-recomputes the gates with PyTorch ops in the ``[B, H, 16, L]`` layout and calls the stand-alone
-BTP kernels.
+Backward is a second fused kernel (every operand read once, every gradient written once), including
+the sum of the ``b`` / ``c`` gradients over the heads that share a kv head, for any
+``heads % kv_heads == 0``: groups of 1, 2, 4 or 8 heads are summed inside a wavefront, other group
+sizes through LDS (spear/nn/phalanx/swr.py:21-126 accepts every such grouping).
 """
 
 from __future__ import annotations
@@ -21,7 +20,7 @@ import torch.library
 
 from spear_amd import _btp
 
-from .interface import lib, register_traceable_op
+from .interface import _plain_eager, lib, register_traceable_op
 
 __all__ = ["phalanx_mix", "btp_qkv"]
 
@@ -92,18 +91,6 @@ register_traceable_op(
 )
 
 
-def _to_heads(t: torch.Tensor, heads: int) -> torch.Tensor:
-    """[B, L, heads*16] -> [B, heads, 16, L] (a view)."""
-    B, L, _ = t.shape
-    return t.view(B, L, heads, 16).permute(0, 2, 3, 1)
-
-
-def _from_heads(t: torch.Tensor) -> torch.Tensor:
-    """[B, heads, 16, L] -> [B, L, heads*16] (materialised)."""
-    B, H, D, L = t.shape
-    return t.permute(0, 3, 1, 2).reshape(B, L, H * D)
-
-
 class _PhalanxMix(torch.autograd.Function):
     @staticmethod
     def forward(ctx, a_logits, b_logits, c, v, heads: int, kv_heads: int):
@@ -117,56 +104,9 @@ class _PhalanxMix(torch.autograd.Function):
     def backward(ctx, dout):
         a_logits, b_logits, c, v = ctx.saved_tensors
         H, Hkv = ctx.heads, ctx.kv_heads
-        groups = H // Hkv
-        dout = dout.contiguous()
-        if groups in (1, 2, 4, 8) and (groups < 8 or H % 8 == 0):
-            da, db, dc, dv = (torch.empty_like(t) for t in (a_logits, b_logits, c, v))
-            torch.ops.spear_btp.mix_backward(a_logits, b_logits, c, v, dout, da, db, dc, dv, H, Hkv)
-            return da, db, dc, dv, None, None
-
-        # Head groups that span wavefronts: gates recomputed with PyTorch ops, stand-alone kernels for the
-        # recurrence. The decay and the gated input are rounded to the tensors' 16-bit type on the way (the
-        # stand-alone op takes 16-bit operands), so these gradients differ from the fused kernel's in the last
-        # bits of that rounding.
-
-        B, L, _ = v.shape
-        dt = v.dtype
-
-        def expand(t):  # [B, Hkv, 16, L] -> [B, H, 16, L]
-            return t.repeat_interleave(groups, dim=1) if groups > 1 else t
-
-        A32 = torch.sigmoid(a_logits.float()).transpose(1, 2)            # [B, H, L]
-        G32 = expand(torch.sigmoid(_to_heads(b_logits, Hkv).float()))    # [B, H, 16, L]
-        C32 = expand(_to_heads(c, Hkv).float())
-        V32 = _to_heads(v, H).float()
-        dO = _to_heads(dout, H).float()
-
-        A = A32.to(dt).contiguous()
-        X = (G32 * V32).to(dt).contiguous()
-        ck = torch.empty((B, H, L // 16, 16), device=v.device, dtype=torch.float32)
-        h = torch.empty((B, H, 16, L), device=v.device, dtype=torch.float32)
-        torch.ops.spear_btp.forward(A, X, h, ck, 2, 32)
-        dh = (dO * C32).contiguous()
-        dX = torch.empty_like(X)
-        dA = torch.empty((B, H, L), device=v.device, dtype=torch.float32)
-        torch.ops.spear_btp.backward(A, X, dh, ck, dX, dA, 2, 32)
-        dX32 = dX.float()
-
-        dC = dO * h
-        dV = dO + dX32 * G32
-        dB = dX32 * V32 * G32 * (1.0 - G32)
-        da = (dA * A32 * (1.0 - A32)).transpose(1, 2)
-        if groups > 1:
-            dC = dC.view(B, Hkv, groups, 16, L).sum(2)
-            dB = dB.view(B, Hkv, groups, 16, L).sum(2)
-        return (
-            da.to(dt).contiguous(),
-            _from_heads(dB).to(dt),
-            _from_heads(dC).to(dt),
-            _from_heads(dV).to(dt),
-            None,
-            None,
-        )
+        da, db, dc, dv = (torch.empty_like(t) for t in (a_logits, b_logits, c, v))
+        torch.ops.spear_btp.mix_backward(a_logits, b_logits, c, v, dout.contiguous(), da, db, dc, dv, H, Hkv)
+        return da, db, dc, dv, None, None
 
 
 def phalanx_mix(
@@ -184,30 +124,43 @@ def phalanx_mix(
         b_logits: ``[B, L, kv_heads*16]`` input-gate logits (``proj_b`` output).
         c: ``[B, L, kv_heads*16]`` output gate (``proj_c`` output).
         v: ``[B, L, heads*16]`` values (``proj_v`` output).
-        heads: number of heads (a multiple of 4); head_dim is 16.
+        heads: number of heads; head_dim is 16.
         kv_heads: number of shared b/c heads (default ``heads``); head ``h`` uses ``h // (heads // kv_heads)``.
 
     All tensors bf16 or fp16, ``L`` a multiple of 16. Returns ``[B, L, heads*16]`` in the same dtype.
     """
     kv = heads if kv_heads is None else kv_heads
-    return _PhalanxMix.apply(a_logits.contiguous(), b_logits.contiguous(), c.contiguous(), v.contiguous(), heads, kv)
+    operands = (a_logits.contiguous(), b_logits.contiguous(), c.contiguous(), v.contiguous())
+    return _run_node(_PhalanxMix, operands, heads, kv, False)
+
+
+def _run_node(python_node, operands, heads: int, kv_heads: int, qkv_gate: bool) -> torch.Tensor:
+    """The mixing stage on contiguous operands in the kernel's order. Plain eager tensors that need gradients go
+    through the autograd node compiled into the binding (``mix_autograd``: same kernels, same bits, no Python frames
+    between autograd and the C ABI); under torch.compile, a dispatch or function mode, a functorch transform or with
+    tensor subclasses the Python node over the traceable custom ops runs."""
+    if torch.is_grad_enabled() and any(t.requires_grad for t in operands) and _plain_eager(*operands):
+        return _btp.load_extension().mix_autograd(*operands, int(heads), int(kv_heads), qkv_gate)
+    return python_node.apply(*operands, heads, kv_heads)
 
 
 class _BtpQkv(torch.autograd.Function):
+    """Operands in the kernel's order: gate, k, q, v."""
+
     @staticmethod
-    def forward(ctx, q, k, v, gate, heads: int, kv_heads: int):
+    def forward(ctx, gate, k, q, v, heads: int, kv_heads: int):
         out = torch.empty_like(v)
         torch.ops.spear_btp.qkv_forward(gate, k, q, v, out, heads, kv_heads)
-        ctx.save_for_backward(q, k, v, gate)
+        ctx.save_for_backward(gate, k, q, v)
         ctx.heads, ctx.kv_heads = heads, kv_heads
         return out
 
     @staticmethod
     def backward(ctx, dout):
-        q, k, v, gate = ctx.saved_tensors
-        dq, dk, dv, dgate = (torch.empty_like(t) for t in (q, k, v, gate))
+        gate, k, q, v = ctx.saved_tensors
+        dgate, dk, dq, dv = (torch.empty_like(t) for t in (gate, k, q, v))
         torch.ops.spear_btp.qkv_backward(gate, k, q, v, dout.contiguous(), dgate, dk, dq, dv, ctx.heads, ctx.kv_heads)
-        return dq, dk, dv, dgate, None, None
+        return dgate, dk, dq, dv, None, None
 
 
 def btp_qkv(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, gate: torch.Tensor) -> torch.Tensor:
@@ -218,9 +171,9 @@ def btp_qkv(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, gate: torch.Tenso
     one fused kernel forward and one backward (``dq, dk, dv, dgate``), no transposes.
 
     Args:
-        q, k: ``[B, L, kv_heads, 16]`` bf16 / fp16 (``kv_heads`` divides ``heads``; ``heads // kv_heads`` in
-            1, 2, 4, 8; head ``h`` uses q/k of kv head ``h // (heads // kv_heads)``).
-        v: ``[B, L, heads, 16]``, same dtype; ``heads`` a multiple of 4, ``L`` a multiple of 16.
+        q, k: ``[B, L, kv_heads, 16]`` bf16 / fp16 (``kv_heads`` divides ``heads``; head ``h`` uses q/k of kv head
+            ``h // (heads // kv_heads)``).
+        v: ``[B, L, heads, 16]``, same dtype; ``L`` a multiple of 16.
         gate: ``[B, L, heads]`` float32 log-decay (``<= 0``, e.g. ``-softplus(logit)``); the decay
             ``exp(gate)`` is formed in fp32 inside the kernel, and the gradient is w.r.t. ``gate``.
 
@@ -232,10 +185,8 @@ def btp_qkv(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, gate: torch.Tenso
         raise RuntimeError("q, k must be [B, L, kv_heads, 16] and v [B, L, heads, 16].")
     B, L, H, _ = v.shape
     Hkv = q.shape[2]
-    if Hkv == 0 or H % Hkv != 0 or H // Hkv not in (1, 2, 4, 8) or (H // Hkv == 8 and H % 8 != 0):
-        raise RuntimeError("heads / kv_heads must be 1, 2, 4 or 8.")
-    out = _BtpQkv.apply(
-        q.reshape(B, L, Hkv * 16).contiguous(), k.reshape(B, L, Hkv * 16).contiguous(),
-        v.reshape(B, L, H * 16).contiguous(), gate.contiguous(), H, Hkv,
-    )
-    return out.view(B, L, H, 16)
+    if Hkv == 0 or H % Hkv != 0:
+        raise RuntimeError("heads must be divisible by kv_heads.")
+    operands = (gate.contiguous(), k.reshape(B, L, Hkv * 16).contiguous(), q.reshape(B, L, Hkv * 16).contiguous(),
+                v.reshape(B, L, H * 16).contiguous())
+    return _run_node(_BtpQkv, operands, H, Hkv, True).view(B, L, H, 16)

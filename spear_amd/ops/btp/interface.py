@@ -262,4 +262,13 @@ def btp_log(
     ``x``: ``[B, H, 16, L]`` bf16/fp16. Returns ``[B, H, 16, L]`` in ``output_dtype`` (default fp32);
     backward yields ``dgate`` in fp32 and ``dx`` in ``x.dtype``.
     """
-    return _BTPLogFunction.apply(gate.contiguous(), x.contiguous(), k, output_dtype or torch.float32)
+    out_dtype = output_dtype or torch.float32
+    gate, x = gate.contiguous(), x.contiguous()
+    if torch.is_grad_enabled() and (gate.requires_grad or x.requires_grad) and _plain_eager(gate, x):
+        # the same node, compiled (spear_amd/csrc/btp_torch_ext.cpp), as btp() has it
+        assert x.dim() == 4 and x.shape[2] == DH, f"Channel dimension must be {DH}"
+        assert x.shape[3] % BLK == 0, f"Length L must be multiple of {BLK}"
+        if out_dtype not in (torch.float32, x.dtype):
+            raise RuntimeError("y must be float32 or match x dtype.")
+        return _btp.load_extension().btp_log_autograd(gate, x, int(k), out_dtype == torch.float32)
+    return _BTPLogFunction.apply(gate, x, k, out_dtype)

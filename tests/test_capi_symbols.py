@@ -34,7 +34,6 @@ def test_header_declares_the_expected_entry_points():
         "spear_phalanx_mix_backward_bias",
         "spear_phalanx_mix_backward_ex",
         "spear_phalanx_mix_backward_sum_rows",
-        "spear_phalanx_mix_backward_sum_rows_tile",
         "spear_phalanx_mix_forward",
         "spear_phalanx_mix_prefill",
         "spear_phalanx_mix_step",
@@ -106,24 +105,24 @@ def test_host_side_validation_needs_no_gpu():
     # fused layer kernels: a batch row must fit one 32-bit buffer resource
     assert lib.spear_phalanx_mix_forward(p, p, p, p, p, 1, 1 << 20, 128, 128, 0, 0, None) == -1
     assert b"below 2 GiB" in lib.spear_btp_last_error()
-    # SPEAR_MIX_QKV_GATE (0x1), SPEAR_MIX_F32_RESULTS (0x2), SPEAR_MIX_TILE_SPLIT (0x4) and SPEAR_MIX_WALK_SPLIT
-    # (0x8), which exclude each other, are the flags of the fused entry points
-    assert lib.spear_phalanx_mix_forward(p, p, p, p, p, 1, 32, 4, 4, 0, 0x10, None) == -1
-    assert b"unknown flag" in lib.spear_btp_last_error()
-    assert lib.spear_phalanx_mix_forward(p, p, p, p, p, 1, 32, 4, 4, 0, 0xc, None) == -1
-    assert b"exclude each other" in lib.spear_btp_last_error()
-    assert lib.spear_phalanx_mix_backward(p, p, p, p, p, p, p, p, p, 1, 32, 4, 4, 0, 0x10, None) == -1
-    assert b"unknown flag" in lib.spear_btp_last_error()
-    assert lib.spear_phalanx_mix_backward(p, p, p, p, p, p, p, p, p, 1, 32, 4, 4, 0, 0xc, None) == -1
-    assert b"exclude each other" in lib.spear_btp_last_error()
+    # SPEAR_MIX_QKV_GATE (0x1) and SPEAR_MIX_F32_RESULTS (0x2) are the flags of the fused entry points
+    for bad in (0x4, 0x8, 0x10):
+        assert lib.spear_phalanx_mix_forward(p, p, p, p, p, 1, 32, 4, 4, 0, bad, None) == -1
+        assert b"unknown flag" in lib.spear_btp_last_error()
+        assert lib.spear_phalanx_mix_backward(p, p, p, p, p, p, p, p, p, 1, 32, 4, 4, 0, bad, None) == -1
+        assert b"unknown flag" in lib.spear_btp_last_error()
+    # heads must be a multiple of kv_heads, nothing else
+    assert lib.spear_phalanx_mix_forward(p, p, p, p, p, 1, 32, 6, 4, 0, 0, None) == -1
+    assert b"divisible by kv_heads" in lib.spear_btp_last_error()
+    assert lib.spear_phalanx_mix_backward(p, p, p, p, p, p, p, p, p, 1, 32, 6, 4, 0, 0, None) == -1
+    assert b"divisible by kv_heads" in lib.spear_btp_last_error()
     assert _btp.FLAG_MIX_QKV_GATE == int(re.search(r"#define SPEAR_MIX_QKV_GATE (0x[0-9a-f]+)u", open(HEADER).read()).group(1), 16)
     # backward with column sums: the three arrays come together and with the row count the library states
     rows = lib.spear_phalanx_mix_backward_sum_rows(2, 64, 8)
-    assert rows >= 2 and rows % 2 == 0
     assert lib.spear_phalanx_mix_backward_sum_rows(2, 60, 8) == 0 and lib.spear_phalanx_mix_backward_sum_rows(0, 64, 8) == 0
-    # the tile split leaves one row per workgroup: 4 blocks of 16 steps
-    assert lib.spear_phalanx_mix_backward_sum_rows_tile(2, 64, 8) == 2 and lib.spear_phalanx_mix_backward_sum_rows_tile(3, 80, 8) == 6
-    assert lib.spear_phalanx_mix_backward_sum_rows_tile(3, 80, 128) == 6 and lib.spear_phalanx_mix_backward_sum_rows_tile(2, 60, 8) == 0
+    # one row per workgroup: 4 blocks of 16 steps of a batch row
+    assert rows == 2 and lib.spear_phalanx_mix_backward_sum_rows(3, 80, 8) == 6
+    assert lib.spear_phalanx_mix_backward_sum_rows(3, 80, 128) == 6
     sums = lambda sa, sb, sc, n, ld=(0, 0, 0, 0): lib.spear_phalanx_mix_backward_ex(
         p, p, p, p, p, p, p, p, p, *ld, sa, sb, sc, n, 2, 64, 8, 8, 0, 0, None)
     assert sums(p, p, None, rows) == -2

@@ -216,8 +216,6 @@ def test_fused_mix_host_checks(monkeypatch):
     with pytest.raises(RuntimeError, match="All tensors must be CUDA"):
         _btp.mix_forward(a, b, c, v, out, 4, 4)
     monkeypatch.setattr(torch.Tensor, "is_cuda", property(lambda self: True))
-    with pytest.raises(RuntimeError, match="heads must be a multiple of 4"):
-        _btp.mix_forward(a[..., :2], b[..., :32], c[..., :32], v[..., :32], out[..., :32], 2, 2)
     with pytest.raises(RuntimeError, match="divisible by kv_heads"):
         _btp.mix_forward(a, b, c, v, out, 4, 3)
     with pytest.raises(RuntimeError, match="b_logit must have shape"):
@@ -229,8 +227,8 @@ def test_fused_mix_host_checks(monkeypatch):
 
 
 def test_fused_method_construction_rules():
-    with pytest.raises(ValueError, match="divisible by 4"):
-        Phalanx(dim=32, method="fused", dtype=torch.bfloat16)
+    assert Phalanx(dim=32, method="fused", dtype=torch.bfloat16).heads == 2   # any head count
+    assert Phalanx(dim=96, method="fused", dtype=torch.bfloat16, kv_heads=2).param.kv_repeat.kv_groups == 3
     with pytest.raises(ValueError, match="k == 2"):
         Phalanx(dim=128, method="fused", k=1, dtype=torch.bfloat16)
     layer = Phalanx(dim=128, method="fused", dtype=torch.bfloat16, kv_heads=2)  # builds without a GPU
@@ -315,10 +313,12 @@ def test_default_method_can_be_sent_to_the_fused_kernels_by_environment(monkeypa
     sent = Phalanx(dim=64, dtype=torch.bfloat16)
     assert sent.method == "default" and sent._forward_fn == sent._forward_fused
     assert list(sent.state_dict()) == list(plain.state_dict())
-    # where the fused kernels do not apply the stand-alone kernels stay: k = 1, heads not a multiple of 4, fp32 output
-    for kwargs in (dict(dim=64, k=1), dict(dim=32), dict(dim=64, output_dtype=torch.float32)):
+    # where the fused kernels do not apply the stand-alone kernels stay: k = 1, fp32 output; any head count is served
+    for kwargs in (dict(dim=64, k=1), dict(dim=64, output_dtype=torch.float32)):
         layer = Phalanx(dtype=torch.bfloat16, **kwargs)
         assert layer._forward_fn == layer._forward_default
+    layer = Phalanx(dim=32, dtype=torch.bfloat16)
+    assert layer._forward_fn == layer._forward_fused
     # the explicit PyTorch methods are never rerouted
     layer = Phalanx(dim=64, dtype=torch.bfloat16, method="pytorch")
     assert layer._forward_fn == layer._forward_pytorch

@@ -82,6 +82,60 @@ def test_eager_calls_run_the_compiled_autograd_node_with_the_results_of_the_pyth
     assert "_BTPFunction" in y_mode.grad_fn.name() and torch.equal(y_mode, y_node)
 
 
+@pytest.mark.parametrize("H,Hkv", [(8, 8), (8, 2), (6, 2)])
+def test_fused_ops_and_the_log_gate_op_run_compiled_autograd_nodes_with_the_python_nodes_results(H, Hkv):
+    """phalanx_mix, btp_qkv and btp_log on plain eager tensors go through nodes compiled into the binding; a dispatch
+    mode in force gets the Python nodes over the custom ops. Same kernels either way: identical bits."""
+    from torch.utils._python_dispatch import TorchDispatchMode
+
+    from spear_amd import btp_log, btp_qkv, phalanx_mix
+    from spear_amd.ops.btp import fused, interface
+
+    class Passthrough(TorchDispatchMode):
+        def __torch_dispatch__(self, func, types, args=(), kwargs=None):
+            return func(*args, **(kwargs or {}))
+
+    B, L = 2, 80
+    g = torch.Generator().manual_seed(61)
+    a = torch.randn(B, L, H, generator=g).bfloat16()
+    b, c = (torch.randn(B, L, Hkv * 16, generator=g).bfloat16() for _ in range(2))
+    v, dout = (torch.randn(B, L, H * 16, generator=g).bfloat16() for _ in range(2))
+
+    def both(fn, python_name, compiled_name, operands, upstream):
+        results = []
+        for mode in (None, Passthrough()):
+            leaves = [t.clone().to(DEV).requires_grad_(True) for t in operands]
+            if mode is None:
+                out = fn(*leaves)
+                assert compiled_name in out.grad_fn.name(), out.grad_fn.name()
+            else:
+                with mode:
+                    out = fn(*leaves)
+                # (a view of the node's output for btp_qkv: look through it)
+                names = {out.grad_fn.name()} | {f[0].name() for f in out.grad_fn.next_functions if f[0] is not None}
+                assert any(python_name in n for n in names), names
+            # an upstream gradient that is not contiguous
+            up = upstream.to(DEV)
+            out.backward(up.transpose(1, 2).contiguous().transpose(1, 2))
+            results.append((out.detach(), [t.grad for t in leaves]))
+        (o1, g1), (o2, g2) = results
+        assert torch.equal(o1, o2)
+        for x, y in zip(g1, g2):
+            assert x.dtype == y.dtype and torch.equal(x, y)
+
+    both(lambda *t: phalanx_mix(*t, heads=H, kv_heads=Hkv), "_PhalanxMix", "MixNode", (a, b, c, v), dout)
+    gate = -torch.nn.functional.softplus(a.float())
+    q, k = c.view(B, L, Hkv, 16), (0.25 * b.float()).bfloat16().view(B, L, Hkv, 16)
+    both(btp_qkv, "_BtpQkv", "MixNode", (q, k, v.view(B, L, H, 16), gate), dout.view(B, L, H, 16))
+    x = v.view(B, L, H, 16).permute(0, 2, 3, 1).contiguous()
+    both(lambda gt, xx: btp_log(gt, xx, output_dtype=torch.bfloat16), "_BTPLogFunction", "BtpLogNode",
+         (gate.transpose(1, 2).contiguous(), x), dout.view(B, L, H, 16).permute(0, 2, 3, 1).contiguous())
+    # nothing to differentiate: no node at all
+    with torch.no_grad():
+        assert phalanx_mix(*(t.to(DEV) for t in (a, b, c, v)), heads=H, kv_heads=Hkv).grad_fn is None
+    assert fused._run_node is not None and interface._plain_eager is not None
+
+
 def test_an_output_dtype_the_binding_does_not_take_raises_on_every_route():
     """float16 results from bfloat16 inputs: the reference's binding refuses (csrc/btp/_bindings.cu:33), and so do the
     compiled node, the Python node and the inference route."""

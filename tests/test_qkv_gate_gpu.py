@@ -52,14 +52,15 @@ def check(q, k, v, gate, dout, atol=BF16_ATOL, rtol=BF16_RTOL):
     assert_close(f64(flat(out)), orc.qkv_gate_forward(*args, H, Hkv), atol, rtol, "out")
     rgate, rk, rq, rv = orc.qkv_gate_backward(*args, f64(flat(dout)), H, Hkv)
     assert_close(f64(flat(dv)), rv, atol, rtol, "dv")
-    assert_close(f64(flat(dq)), rq, atol * (H // Hkv) ** 0.5, rtol, "dq")
-    assert_close(f64(flat(dk)), rk, atol * (H // Hkv) ** 0.5, rtol, "dk")
+    assert_close(f64(flat(dq)), rq, atol, rtol, "dq")  # sums over a head group: fp32, rounded once
+    assert_close(f64(flat(dk)), rk, atol, rtol, "dk")
     scale = max(1.0, float(np.abs(rgate).max()))
     assert float(np.abs(f64(dgate) - rgate).max()) <= 1e-4 * scale, ("dgate", float(np.abs(f64(dgate) - rgate).max()), scale)
 
 
 @pytest.mark.parametrize("B,L,H,Hkv", [(1, 16, 4, 4), (2, 48, 8, 8), (1, 80, 12, 3), (3, 128, 8, 2), (2, 144, 16, 16),
-                                       (1, 512, 32, 32), (1, 1040, 4, 1), (2, 2064, 16, 2), (1, 4096, 8, 8)])
+                                       (1, 512, 32, 32), (1, 1040, 4, 1), (2, 2064, 16, 2), (1, 4096, 8, 8),
+                                       (2, 64, 6, 2), (1, 80, 16, 1), (2, 48, 5, 5), (1, 112, 24, 2)])
 def test_qkv_gate_forward_and_backward_match_oracle(B, L, H, Hkv):
     print(f"qkv B={B} L={L} H={H} Hkv={Hkv}", flush=True)
     check(*make_qkv(B, L, H, Hkv, seed=7000 + L + H))
@@ -189,8 +190,8 @@ def test_log_gate_operator_at_the_log_space_stress_shape():
 def test_rejects_what_it_cannot_do():
     from spear_amd import _btp, btp_qkv
 
-    q, k, v, gate, _ = make_qkv(1, 32, 16, 1, seed=76)
-    with pytest.raises(RuntimeError, match="1, 2, 4 or 8"):
+    q, k, v, gate, _ = make_qkv(1, 32, 16, 3, seed=76)
+    with pytest.raises(RuntimeError, match="divisible by kv_heads"):
         btp_qkv(*(t.to(DEV) for t in (q, k, v, gate)))
     q, k, v, gate, _ = make_qkv(1, 32, 4, 4, seed=77)
     with pytest.raises(RuntimeError, match="float32"):

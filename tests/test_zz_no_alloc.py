@@ -75,8 +75,9 @@ def _without_allocation(ins, grads, bias, H, Hkv):
 
 
 @pytest.mark.parametrize("first,second", [
-    ((6, 256, 32, 32), (3, 64, 8, 4)),       # one chunk per row, then a smaller shape with shared kv heads
-    ((2, 4096, 8, 8), (1, 48, 4, 4)),        # rows cut into several chunks (several partial rows per batch row)
+    ((6, 256, 32, 32), (3, 64, 8, 4)),       # then a smaller shape with shared kv heads
+    ((2, 4096, 8, 8), (1, 48, 4, 4)),        # long rows: many partial rows per batch row
+    ((3, 128, 16, 1), (2, 80, 6, 2)),        # head groups that are summed through LDS (16 and 3 heads per kv head)
 ])
 def test_two_calls_in_a_row_match_the_allocating_entry_point(first, second):
     for call, (B, L, H, Hkv) in enumerate((first, second)):
@@ -124,8 +125,8 @@ def test_shapes_beyond_the_static_array_are_refused():
     from spear_amd import _btp
 
     lib = _btp.load_library()
-    B, L, H = 2048, 128, 32  # 2048 partial rows x (32 + 2 * 512) floats > 2 Mi floats
-    assert _btp.mix_backward_sum_rows(B, L, H) * (H + 2 * H * 16) > 2097152
+    B, L, H = 2048, 128, 32  # 4096 partial rows x (32 + 2 * 512) floats > 4 Mi floats
+    assert _btp.mix_backward_sum_rows(B, L, H) * (H + 2 * H * 16) > 4194304
     t = torch.zeros(64, device=DEV)
     p = t.data_ptr()
     rc = lib.spear_phalanx_mix_backward_bias(p, p, p, p, p, p, p, p, p, 0, 0, 0, 0, p, p, p, B, L, H, H, 0, 0, None)
