@@ -883,8 +883,60 @@ def main() -> int:
                     "forward_only": {"eager_no_grad_ms": eager_fwd_ms, "hip_graph_replay_ms": fwd_graph_ms,
                                      "eager_over_graph": eager_fwd_ms / fwd_graph_ms}}
 
+        def measure_fused(bs):
+            """phalanx_mix(a, b, c, v) + backward on [bs, L, features] tensors: eager through the autograd node compiled
+            into the binding, the two custom ops on preallocated outputs, and a HIP-graph replay of those two ops."""
+            from spear_amd import phalanx_mix
+            import spear_amd.ops.btp.fused  # noqa: F401  (registers the custom ops)
+
+            F = H * 16
+            gq = torch.Generator(device=dev).manual_seed(seed + 23)
+            a = torch.randn(bs, L, H, device=dev, generator=gq).to(torch.bfloat16)
+            b, c, v, dout = (torch.randn(bs, L, F, device=dev, generator=gq).to(torch.bfloat16) for _ in range(4))
+            out = torch.empty_like(v)
+            grads = [torch.empty_like(t) for t in (a, b, c, v)]
+
+            def eager():
+                leaves = [t.detach().requires_grad_(True) for t in (a, b, c, v)]
+                phalanx_mix(*leaves, heads=H, kv_heads=H).backward(dout)
+
+            def eager_python_node():  # the torch.autograd.Function over the custom ops (what torch.compile traces)
+                leaves = [t.detach().requires_grad_(True) for t in (a, b, c, v)]
+                spear_amd.ops.btp.fused._PhalanxMix.apply(*leaves, H, H).backward(dout)
+
+            def ops_only():
+                torch.ops.spear_btp.mix_forward(a, b, c, v, out, H, H)
+                torch.ops.spear_btp.mix_backward(a, b, c, v, dout, *grads, H, H)
+
+            def timed(fn, n):
+                for _ in range(5):
+                    fn()
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                for _ in range(n):
+                    fn()
+                torch.cuda.synchronize()
+                return (time.perf_counter() - t0) * 1e3 / n
+
+            n = max(20, args.steps // 2)
+            eager_ms, ops_ms, python_node_ms = timed(eager, n), timed(ops_only, n), timed(eager_python_node, n)
+            side = torch.cuda.Stream()
+            side.wait_stream(stream)
+            with torch.cuda.stream(side):
+                ops_only()
+            stream.wait_stream(side)
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=side):
+                ops_only()
+            torch.cuda.synchronize()
+            graph_ms = timed(graph.replay, n)
+            return {"B": bs, "eager_autograd_ms": eager_ms, "eager_autograd_python_node_ms": python_node_ms,
+                    "two_ops_preallocated_ms": ops_ms, "hip_graph_replay_ms": graph_ms,
+                    "eager_over_graph": eager_ms / graph_ms}
+
         return {"what": "btp(coeff, x, output_dtype=bf16) + backward through the public op (wall clock per fwd+bwd)",
-                "this_shape": measure(B), "config1_batch": measure(min(B, 8))}
+                "this_shape": measure(B), "config1_batch": measure(min(B, 8)),
+                "fused_op_config1_batch": guarded(lambda: measure_fused(min(B, 8)))}
 
     public_op = guarded(public_op_leg)
 

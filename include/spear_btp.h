@@ -51,7 +51,9 @@ extern "C" {
                                         /* per block and multiplied on the matrix cores, the reference's            */
                                         /* formulation; each entry goes in as two 16-bit pieces, so fp32 results    */
                                         /* keep the 1e-4 bound) instead of the fp32 recurrences; the backward then  */
-                                        /* rounds an fp32 dy to the inputs' dtype and has no SPEAR_BTP_DX_F32       */
+                                        /* takes dy in in_dtype only (SPEAR_BTP_EINVAL for an fp32 dy, which the    */
+                                        /* 16-bit operands of the matrix instruction cannot hold) and has no        */
+                                        /* SPEAR_BTP_DX_F32                                                          */
 
 #define SPEAR_BTP_DX_F32 0x10u          /* backward: check mode, `dx` is fp32 [B, H, 16, L] and receives the    */
                                         /* kernel's fp32 values instead of their rounding to in_dtype           */
@@ -199,7 +201,8 @@ int spear_phalanx_mix_prefill(const void* a_logit, const void* b_logit, const vo
  * block, 0 .. block_len-1) every row decides for itself (pos[b] == block_len - 1) and the call advances pos by one
  * step (wrapping to 0), so that one captured HIP graph serves every token and batch rows may be at different
  * positions; with pos == NULL the host decides for all rows through `boundary`. Calls on one state must not
- * overlap. Nothing is allocated; with `pos` the call launches two kernels. Alignment: b_logit, c, v, out, h and
+ * overlap. Nothing is allocated; with `pos` the call launches one kernel when 2 * H divides 64 (a batch row's
+ * threads then share a wavefront and advance the position themselves), two otherwise. Alignment: b_logit, c, v, out, h and
  * c_prev 16 bytes; a_logit 2 and r 4 bytes (one token's row of a [tokens, B, H] tensor can be passed as it lies). */
 int spear_phalanx_mix_step(const void* a_logit, const void* b_logit, const void* c, const void* v, void* out, float* h,
                            float* r, float* c_prev, int* pos, int boundary, int block_len, int B, int H, int kv_heads,
@@ -251,45 +254,6 @@ const char* spear_btp_last_error(void);
 
 /* ABI version of this header: bumped whenever a signature above changes. */
 int spear_btp_abi_version(void);
-
-/* Measurement aid, not part of the operator: a plain device-to-device copy kernel of known
- * traffic (reads `bytes`, writes `bytes`; `bytes` a multiple of 16), used to calibrate hardware
- * counters and to measure the copy bandwidth the BTP kernels are compared with. */
-int spear_btp_copy(const void* src, void* dst, unsigned long long bytes, void* stream);
-
-/* Measurement aid as well: the operator's own access shape and cache policy without its arithmetic.
- * Every wavefront moves one 4 KiB slab with non-temporal 16-byte loads and stores; with src_b == NULL
- * it is a copy (reads `bytes`, writes `bytes`), otherwise dst = src_a ^ src_b (reads 2 x `bytes`, writes
- * `bytes`: the backward kernel's read/write mix). `bytes` a multiple of 4096. What this reaches is what
- * the memory system gives kernels of this shape, which is the practical ceiling the BTP kernels are
- * compared with beside the 8 TB/s peak. */
-int spear_btp_stream_probe(const void* src_a, const void* src_b, void* dst, unsigned long long bytes, void* stream);
-
-/* The same traffic in other launch shapes, to show where the kernels' own shape stands among the
- * alternatives: shape 0 = spear_btp_stream_probe (one 4 KiB slab per wavefront); 1 = two slabs per
- * wavefront, all loads issued before the first store; 2 = four slabs per wavefront in a loop that issues
- * the next slab's loads before the current slab's stores; 3 = that loop as a persistent grid striding over
- * the buffer; 4 = one 16-byte element per thread; 5 = reads only (src_a, and src_b if given; `dst` is not
- * written unless every input word is all ones); 6 = writes only (`dst` is filled, nothing is read). HBM serves
- * reads and writes one after the other, so shapes 5 and 6 give the two rates from which the floor of a mixed
- * kernel follows: R bytes read and W bytes written take at least R / read rate + W / write rate; 7 = shape 0
- * with 640 dependent FMAs between loads and stores (the output's last word may differ from shape 0's in its
- * lowest bit). Same arguments and result as spear_btp_stream_probe. */
-#define SPEAR_BTP_PROBE_SHAPES 8
-int spear_btp_stream_probe_shape(const void* src_a, const void* src_b, void* dst, unsigned long long bytes, int shape,
-                                 void* stream);
-
-/* The probe with the stream counts of the fused layer kernels (measurement aid, no counterpart in the
- * reference): `n_src` inputs of `bytes` each are combined (xor) into `n_dst` identical outputs of `bytes` each, in
- * the shape of spear_btp_stream_probe (one 4 KiB piece per wavefront and tensor, non-temporal 16-byte accesses).
- * (n_src, n_dst) = (3, 1): the fused forward's and the prefill kernel's mix; (4, 3): the fused backward's;
- * (1, 2): the stand-alone forward's with an fp32 result (the op's default output type).
- * `compute` != 0 puts a chain of dependent FMAs between loads and stores (640 for (3, 1), 1280 for (4, 3), 320
- * for (1, 2); the
- * outputs' last word may then differ in its lowest bit). `src`, `dst`: host arrays of device pointers, 16-byte
- * aligned; `bytes` a multiple of 4096. */
-int spear_btp_stream_probe_mix(const void* const* src, int n_src, void* const* dst, int n_dst, unsigned long long bytes,
-                               int compute, void* stream);
 
 #ifdef __cplusplus
 }

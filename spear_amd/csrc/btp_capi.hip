@@ -23,6 +23,24 @@ int fail(int code, const char* fmt, ...) {
   return code;
 }
 
+}  // namespace
+
+namespace spear_btp {
+
+// Error reporting for the entry points that live in other files (btp_probe.hip).
+int report_error(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_error, sizeof(g_error), fmt, ap);
+  va_end(ap);
+  return code;
+}
+void clear_error() { g_error[0] = '\0'; }
+
+}  // namespace spear_btp
+
+namespace {
+
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 bool dtype_ok(int d) { return d == SPEAR_BTP_BF16 || d == SPEAR_BTP_F16 || d == SPEAR_BTP_F32; }
@@ -86,6 +104,11 @@ int spear_btp_backward(const void* coeff, const void* x, const void* dy, const f
   const bool mfma = (flags & SPEAR_BTP_PATH_MFMA) != 0;
   if (mfma && (flags & SPEAR_BTP_DX_F32))
     return fail(SPEAR_BTP_EINVAL, "spear_btp_backward: the MFMA path has no fp32 dx (SPEAR_BTP_DX_F32)");
+  if (mfma && dy_dtype == SPEAR_BTP_F32)
+    return fail(SPEAR_BTP_EINVAL,
+                "spear_btp_backward: the MFMA path takes dy in the inputs' 16-bit type (the matrix instruction's operand "
+                "width) and does not round a float32 dy silently; use the default path, or give the forward an output "
+                "in the inputs' dtype so that dy arrives in it");
 
   spear_btp::BwdArgs a{coeff, x, dy, dx, dA, B, H, L, k, in_dtype, dy_dtype, false, (flags & SPEAR_BTP_DX_F32) != 0};
   const hipStream_t hs = static_cast<hipStream_t>(stream);
@@ -359,58 +382,6 @@ int spear_jagged_step(const void* a_t, const void* x_t, const void* c_t, const v
                            boundary ? 1 : 0, a_dtype, x_dtype, state_dtype, r_dtype,
                            (flags & SPEAR_JAGGED_LOG_A) ? 1 : 0, (flags & SPEAR_JAGGED_LOG_R) ? 1 : 0, tiny, al};
   const hipError_t err = spear_btp::jagged_step(p, static_cast<hipStream_t>(stream));
-  if (err != hipSuccess) return fail(SPEAR_BTP_ELAUNCH, "%s: launch failed: %s", who, hipGetErrorString(err));
-  return 0;
-}
-
-int spear_btp_copy(const void* src, void* dst, unsigned long long bytes, void* stream) {
-  g_error[0] = '\0';
-  if (!src || !dst) return fail(SPEAR_BTP_ENULL, "spear_btp_copy: NULL pointer");
-  if (bytes % 16 != 0 || !aligned16(src) || !aligned16(dst))
-    return fail(SPEAR_BTP_EINVAL, "spear_btp_copy: size and pointers must be multiples of 16 bytes");
-  const hipError_t err = spear_btp::device_copy(src, dst, bytes, static_cast<hipStream_t>(stream));
-  if (err != hipSuccess) return fail(SPEAR_BTP_ELAUNCH, "spear_btp_copy: launch failed: %s", hipGetErrorString(err));
-  return 0;
-}
-
-int spear_btp_stream_probe(const void* src_a, const void* src_b, void* dst, unsigned long long bytes, void* stream) {
-  g_error[0] = '\0';
-  if (!src_a || !dst) return fail(SPEAR_BTP_ENULL, "spear_btp_stream_probe: NULL pointer");
-  if (bytes % 4096 != 0 || !aligned16(src_a) || !aligned16(src_b) || !aligned16(dst))
-    return fail(SPEAR_BTP_EINVAL, "spear_btp_stream_probe: size must be a multiple of 4096, pointers of 16 bytes");
-  const hipError_t err = spear_btp::stream_probe(src_a, src_b, dst, bytes, static_cast<hipStream_t>(stream));
-  if (err != hipSuccess)
-    return fail(SPEAR_BTP_ELAUNCH, "spear_btp_stream_probe: launch failed: %s", hipGetErrorString(err));
-  return 0;
-}
-
-int spear_btp_stream_probe_shape(const void* src_a, const void* src_b, void* dst, unsigned long long bytes, int shape,
-                                 void* stream) {
-  g_error[0] = '\0';
-  if (!src_a || !dst) return fail(SPEAR_BTP_ENULL, "spear_btp_stream_probe_shape: NULL pointer");
-  if (bytes % 4096 != 0 || !aligned16(src_a) || !aligned16(src_b) || !aligned16(dst))
-    return fail(SPEAR_BTP_EINVAL, "spear_btp_stream_probe_shape: size must be a multiple of 4096, pointers of 16 bytes");
-  if (shape < 0 || shape >= SPEAR_BTP_PROBE_SHAPES)
-    return fail(SPEAR_BTP_EINVAL, "spear_btp_stream_probe_shape: shape must be 0..%d (got %d)", SPEAR_BTP_PROBE_SHAPES - 1, shape);
-  const hipError_t err = spear_btp::stream_probe_shape(src_a, src_b, dst, bytes, shape, static_cast<hipStream_t>(stream));
-  if (err != hipSuccess)
-    return fail(SPEAR_BTP_ELAUNCH, "spear_btp_stream_probe_shape: launch failed: %s", hipGetErrorString(err));
-  return 0;
-}
-
-int spear_btp_stream_probe_mix(const void* const* src, int n_src, void* const* dst, int n_dst, unsigned long long bytes,
-                               int compute, void* stream) {
-  g_error[0] = '\0';
-  const char* who = "spear_btp_stream_probe_mix";
-  if (!src || !dst) return fail(SPEAR_BTP_ENULL, "%s: NULL pointer", who);
-  if (!((n_src == 3 && n_dst == 1) || (n_src == 4 && n_dst == 3) || (n_src == 1 && n_dst == 2)))
-    return fail(SPEAR_BTP_EINVAL, "%s: (n_src, n_dst) must be (3, 1), (4, 3) or (1, 2) (got %d, %d)", who, n_src, n_dst);
-  if (bytes % 4096 != 0) return fail(SPEAR_BTP_EINVAL, "%s: size must be a multiple of 4096", who);
-  for (int i = 0; i < n_src; ++i)
-    if (!src[i] || !aligned16(src[i])) return fail(SPEAR_BTP_EINVAL, "%s: every tensor pointer must be set and 16-byte aligned", who);
-  for (int i = 0; i < n_dst; ++i)
-    if (!dst[i] || !aligned16(dst[i])) return fail(SPEAR_BTP_EINVAL, "%s: every tensor pointer must be set and 16-byte aligned", who);
-  const hipError_t err = spear_btp::stream_probe_mix(src, n_src, dst, n_dst, bytes, compute != 0, static_cast<hipStream_t>(stream));
   if (err != hipSuccess) return fail(SPEAR_BTP_ELAUNCH, "%s: launch failed: %s", who, hipGetErrorString(err));
   return 0;
 }

@@ -892,12 +892,16 @@ void phalanx_mix_fwd_tile_kernel(const uint16_t* __restrict__ a_logit, const uin
 //   a token that completes a block:  c_prev = h, h = 0, r = 1
 // A thread owns 8 consecutive features (16-byte accesses); the two threads of a head sit in neighbouring lanes,
 // so the head's scalar r is read by both before one of them writes it back (in-place state).
+// kAdvance: the kernel also moves pos[b] to the next token's position. That needs every thread of a batch row to
+// have read pos[b] before one of them writes it, which holds when a row's 2 H threads lie inside one wavefront
+// (2 H divides 64: the stored value depends on the loaded one, so the wavefront's load has returned for all its
+// lanes before the store is issued); otherwise a second kernel does it.
 // ==========================================================================================
-template <class E>
+template <class E, bool kAdvance>
 __global__ __launch_bounds__(256) void phalanx_mix_step_kernel(
     const uint16_t* __restrict__ a_logit, const uint16_t* __restrict__ b_logit, const uint16_t* __restrict__ c_in,
     const uint16_t* __restrict__ v_in, uint16_t* __restrict__ out, float* __restrict__ h, float* __restrict__ r,
-    float* __restrict__ c_prev, const int* __restrict__ pos, int boundary_all, int block_len, long total, int H,
+    float* __restrict__ c_prev, int* __restrict__ pos, int boundary_all, int block_len, long total, int H,
     int kv_groups) {
   const long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
   if (idx >= total) return;
@@ -906,7 +910,8 @@ __global__ __launch_bounds__(256) void phalanx_mix_step_kernel(
   const int piece = (int)(idx - brow * per_row);
   const int head = piece >> 1, half = piece & 1;
   const long kv_piece = brow * (2 * (H / kv_groups)) + 2 * (head / kv_groups) + half;
-  const bool boundary = pos != nullptr ? (pos[brow] == block_len - 1) : (boundary_all != 0);
+  const int at = pos != nullptr ? pos[brow] : 0;
+  const bool boundary = pos != nullptr ? (at == block_len - 1) : (boundary_all != 0);
 
   const uint32_t aw = a_logit[brow * H + head];
   const float a = clamp_coeff<E>(fast_sigmoid(E::lo(aw)));
@@ -934,6 +939,9 @@ __global__ __launch_bounds__(256) void phalanx_mix_step_kernel(
   *reinterpret_cast<float4*>(h + idx * 8) = make_float4(hf[0], hf[1], hf[2], hf[3]);
   *reinterpret_cast<float4*>(h + idx * 8 + 4) = make_float4(hf[4], hf[5], hf[6], hf[7]);
   if (half == 0) r[brow * H + head] = boundary ? 1.0f : r_new;
+  if constexpr (kAdvance) {
+    if (piece == 0) pos[brow] = boundary ? 0 : at + 1;
+  }
 }
 
 // pos[b] <- position of the next token inside its block
@@ -1121,14 +1129,22 @@ hipError_t fused_mix_step(const MixStepArgs& p, hipStream_t s) {
   const long total = (long)p.B * p.H * 2;
   const unsigned blocks = (unsigned)((total + 255) / 256);
   auto u = [](const void* q) { return static_cast<const uint16_t*>(q); };
-  if (p.dtype == kBf16)
-    hipLaunchKernelGGL(phalanx_mix_step_kernel<Bf16>, dim3(blocks), dim3(256), 0, s, u(p.a_logit), u(p.b_logit), u(p.c), u(p.v),
-                       static_cast<uint16_t*>(p.out), p.h, p.r, p.c_prev, p.pos, p.boundary, p.block_len, total, p.H, p.kv_groups);
-  else
-    hipLaunchKernelGGL(phalanx_mix_step_kernel<Fp16>, dim3(blocks), dim3(256), 0, s, u(p.a_logit), u(p.b_logit), u(p.c), u(p.v),
-                       static_cast<uint16_t*>(p.out), p.h, p.r, p.c_prev, p.pos, p.boundary, p.block_len, total, p.H, p.kv_groups);
+  // a batch row's 2 H threads inside one wavefront: the step kernel advances the positions itself
+  const bool advance_inside = p.pos != nullptr && 64 % (2 * p.H) == 0;
+  auto launch = [&](auto e, auto adv) {
+    hipLaunchKernelGGL((phalanx_mix_step_kernel<decltype(e), decltype(adv)::value>), dim3(blocks), dim3(256), 0, s,
+                       u(p.a_logit), u(p.b_logit), u(p.c), u(p.v), static_cast<uint16_t*>(p.out), p.h, p.r, p.c_prev, p.pos,
+                       p.boundary, p.block_len, total, p.H, p.kv_groups);
+  };
+  if (p.dtype == kBf16) {
+    if (advance_inside) launch(Bf16{}, std::true_type{});
+    else launch(Bf16{}, std::false_type{});
+  } else {
+    if (advance_inside) launch(Fp16{}, std::true_type{});
+    else launch(Fp16{}, std::false_type{});
+  }
   if (hipError_t err = hipGetLastError(); err != hipSuccess) return err;
-  if (p.pos != nullptr) {  // stream order puts this after every read of pos above
+  if (p.pos != nullptr && !advance_inside) {  // stream order puts this after every read of pos above
     hipLaunchKernelGGL(advance_block_positions_kernel, dim3((unsigned)((p.B + 255) / 256)), dim3(256), 0, s, p.pos, p.B, p.block_len);
     return hipGetLastError();
   }

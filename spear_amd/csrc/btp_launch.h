@@ -37,7 +37,7 @@ hipError_t scan_forward(const FwdArgs& p, hipStream_t s);
 hipError_t scan_backward(const BwdArgs& p, hipStream_t s);
 
 // MFMA tile kernels (btp_mfma.hip), bf16 or fp16 inputs; the forward stores no checkpoint, the backward has
-// neither log-space gates nor the fp32-dx check mode (an fp32 dy is rounded to the inputs' type on load).
+// neither log-space gates nor the fp32-dx check mode and takes dy in the inputs' type only.
 hipError_t mfma_forward(const FwdArgs& p, hipStream_t s);
 hipError_t mfma_backward(const BwdArgs& p, hipStream_t s);
 
@@ -125,11 +125,16 @@ struct JagStepArgs {
 };
 hipError_t jagged_step(const JagStepArgs& p, hipStream_t s);
 
-// Plain copy kernel used for bandwidth / counter calibration (btp_scan.hip).
+// ---- measurement aids (btp_probe.hip), not part of the operator -------------------------------------------
+// Records / clears the calling thread's error string (btp_capi.hip) for entry points that live in other files.
+int report_error(int code, const char* fmt, ...);
+void clear_error();
+
+// Plain copy kernel used for bandwidth / counter calibration.
 hipError_t device_copy(const void* src, void* dst, unsigned long long bytes, hipStream_t s);
 
 // Slab-shaped non-temporal copy (b == nullptr) or two-input combine, for measuring what the memory
-// system gives the operator's access pattern (btp_scan.hip).
+// system gives the operator's access pattern.
 hipError_t stream_probe(const void* a, const void* b, void* dst, unsigned long long bytes, hipStream_t s);
 // The same traffic in other launch shapes (0 = the one above, 1..4 see stream_probe_shape_kernel).
 hipError_t stream_probe_shape(const void* a, const void* b, void* dst, unsigned long long bytes, int shape, hipStream_t s);

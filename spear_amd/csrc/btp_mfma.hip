@@ -267,16 +267,15 @@ __device__ __forceinline__ float half_row_suffix_product(float a_n, int n) {
   return w;
 }
 
-// GradT: uint16_t (dy in the inputs' type) or float; an fp32 dy is rounded to the inputs' type on its way into
-// the LDS image, since the matrix instruction takes 16-bit operands (the reference packs dC the same way,
-// csrc/btp/btp-backwards.cu:562-587).
-template <class E, class GradT, bool kStreamIn>
+// dy arrives in the inputs' 16-bit type: the matrix instruction takes 16-bit operands, and an fp32 dy (which the
+// reference rounds when it packs dC, csrc/btp/btp-backwards.cu:562-587) is refused by the entry point rather than
+// rounded silently.
+template <class E, bool kStreamIn>
 __global__ __launch_bounds__(64 * kWaves) void btp_bwd_mfma_kernel(const uint16_t* __restrict__ coeff,
                                                                    const uint16_t* __restrict__ x,
-                                                                   const GradT* __restrict__ dy,
+                                                                   const uint16_t* __restrict__ dy,
                                                                    uint16_t* __restrict__ dx, float* __restrict__ dA,
                                                                    int L, int spans_per_row, long total_spans, int k) {
-  constexpr bool kGradF32 = std::is_same<GradT, float>::value;
   constexpr bool kStreamOut = SPEAR_BTP_STREAM_STORES == 1;
   // per wavefront: x image, which dx overwrites block by block (a block's x is read by that block's V product
   // only, before its dx is written) | dy image | x of the block before the span | dy of the block after it
@@ -302,15 +301,14 @@ __global__ __launch_bounds__(64 * kWaves) void btp_bwd_mfma_kernel(const uint16_
 
   const long slab_off = (sc.row * kChan) * (long)L + sc.s0;
   const uint16_t* xslab = x + slab_off;
-  const GradT* gslab = dy + slab_off;
+  const uint16_t* gslab = dy + slab_off;
   const uint16_t* arow = coeff + sc.row * (long)L + sc.s0;
   const int q = lane >> 4, n = lane & 15;
 
   // ---- global -> LDS
-  uint4 xin[4], gin[kGradF32 ? 8 : 4];
+  uint4 xin[4], gin[4];
   slab16_global_to_regs<kStreamIn>(xslab, L, sc.nvalid, lane, xin);
-  if constexpr (kGradF32) slab32_global_to_regs<kStreamIn>(gslab, L, sc.nvalid, lane, gin);
-  else slab16_global_to_regs<kStreamIn>(gslab, L, sc.nvalid, lane, gin);
+  slab16_global_to_regs<kStreamIn>(gslab, L, sc.nvalid, lane, gin);
   const uint32_t ain = coeff_global_to_reg<LinCoeff<E>>(arow, sc.nvalid, lane);
   const bool left = (k == 2) && (sc.sp > 0);            // wave-uniform: a block before the span feeds its first block
   const bool right = (k == 2) && (sc.s0 + kSpan < L);   // wave-uniform: the span's last block feeds a block after it
@@ -322,31 +320,12 @@ __global__ __launch_bounds__(64 * kWaves) void btp_bwd_mfma_kernel(const uint16_
   }
   if (right) {
     if (lane < 32) {  // lane = (channel row, half): 8 steps of the block after the span
-      const GradT* hp = gslab + (long)(lane >> 1) * L + kSpan + ((lane & 1) << 3);
-      if constexpr (kGradF32) {
-        const float4 f0 = *reinterpret_cast<const float4*>(hp), f1 = *reinterpret_cast<const float4*>(hp + 4);
-        hg = make_uint4(E::pack2(f0.x, f0.y), E::pack2(f0.z, f0.w), E::pack2(f1.x, f1.y), E::pack2(f1.z, f1.w));
-      } else {
-        hg = *reinterpret_cast<const uint4*>(hp);
-      }
+      hg = *reinterpret_cast<const uint4*>(gslab + (long)(lane >> 1) * L + kSpan + ((lane & 1) << 3));
     }
     if (lane < 8) hb = *reinterpret_cast<const uint32_t*>(arow + kSpan + (lane << 1));
   }
   slab16_regs_to_lds(img_x, lane, xin);
-  if constexpr (kGradF32) {
-    // lane (row half lr, chunk lp of 4 steps) -> four 16-bit values = half of a 16-byte chunk of the 16-bit image
-    const int lr = lane >> 5, lp = lane & 31;
-#pragma unroll
-    for (int it = 0; it < 8; ++it) {
-      const int r = it * 2 + lr;
-      uint2 o;
-      o.x = E::pack2(__uint_as_float(gin[it].x), __uint_as_float(gin[it].y));
-      o.y = E::pack2(__uint_as_float(gin[it].z), __uint_as_float(gin[it].w));
-      *reinterpret_cast<uint2*>(img_g + swz<256>(r, lp >> 1) + ((lp & 1) << 3)) = o;
-    }
-  } else {
-    slab16_regs_to_lds(img_g, lane, gin);
-  }
+  slab16_regs_to_lds(img_g, lane, gin);
   if (lane < 32) {
     *reinterpret_cast<uint4*>(halo_x + (lane >> 1) * 32 + ((lane & 1) << 4)) = hx;
     *reinterpret_cast<uint4*>(halo_g + (lane >> 1) * 32 + ((lane & 1) << 4)) = hg;
@@ -504,7 +483,7 @@ void launch_fwd_mfma(const FwdArgs& p, const Grid& g, hipStream_t s) {
 }  // namespace
 
 hipError_t mfma_backward(const BwdArgs& p, hipStream_t s) {
-  if (p.log_gate || p.dx_f32) return hipErrorInvalidValue;  // the caller has checked
+  if (p.log_gate || p.dx_f32 || p.dy_dtype == kF32) return hipErrorInvalidValue;  // the caller has checked
   const Grid g = make_grid((long)p.B * p.H, p.L);
   auto launch = [&](auto e, auto stream_in) {
     using E = decltype(e);
@@ -512,12 +491,8 @@ hipError_t mfma_backward(const BwdArgs& p, hipStream_t s) {
     const auto* c = static_cast<const uint16_t*>(p.coeff);
     const auto* x = static_cast<const uint16_t*>(p.x);
     auto* dx = static_cast<uint16_t*>(p.dx);
-    if (p.dy_dtype == kF32)
-      hipLaunchKernelGGL((btp_bwd_mfma_kernel<E, float, kIn>), dim3(g.blocks), dim3(64 * kWaves), 0, s, c, x,
-                         static_cast<const float*>(p.dy), dx, p.dA, p.L, g.spans_per_row, g.total_spans, p.k);
-    else
-      hipLaunchKernelGGL((btp_bwd_mfma_kernel<E, uint16_t, kIn>), dim3(g.blocks), dim3(64 * kWaves), 0, s, c, x,
-                         static_cast<const uint16_t*>(p.dy), dx, p.dA, p.L, g.spans_per_row, g.total_spans, p.k);
+    hipLaunchKernelGGL((btp_bwd_mfma_kernel<E, kIn>), dim3(g.blocks), dim3(64 * kWaves), 0, s, c, x,
+                       static_cast<const uint16_t*>(p.dy), dx, p.dA, p.L, g.spans_per_row, g.total_spans, p.k);
   };
   const bool st = stream_inputs(g);
   if (p.in_dtype == kBf16) {

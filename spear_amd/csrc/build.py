@@ -18,8 +18,9 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 PKG = os.path.dirname(HERE)
 LIB_NAME = "libspear_btp.so"
-SOURCES = ["btp_scan.hip", "btp_mfma.hip", "btp_fused.hip", "btp_jagged.hip", "btp_capi.hip"]
-HEADERS = ["btp_device.h", "btp_launch.h", "btp_staging.h", os.path.join("..", "..", "include", "spear_btp.h")]
+SOURCES = ["btp_scan.hip", "btp_mfma.hip", "btp_fused.hip", "btp_jagged.hip", "btp_capi.hip", "btp_probe.hip"]
+HEADERS = ["btp_device.h", "btp_launch.h", "btp_staging.h", os.path.join("..", "..", "include", "spear_btp.h"),
+           os.path.join("..", "..", "include", "spear_btp_probe.h")]
 
 # -packed-fp32-ops is switched off on purpose: scalar fp32 code must not be fused into
 # v_pk_*_f32 instructions on this hardware pool.

@@ -109,13 +109,16 @@ def test_mfma_path_rejects_what_it_does_not_do():
     with pytest.raises(RuntimeError, match="no fp32 dx"):
         _btp.backward(c, xx, dy.to(DEV), ck, torch.empty_like(xx, dtype=torch.float32), dA, 2, 32,
                       flags=_btp.FLAG_PATH_MFMA | _btp.FLAG_DX_F32)
+    # an fp32 dy (the reference accepts one, csrc/btp/_bindings.cu:52-59, and rounds it for its MMA) is refused, not
+    # rounded behind the caller's back
+    with pytest.raises(RuntimeError, match="takes dy in the inputs' 16-bit type"):
+        _btp.backward(c, xx, dy.to(DEV).float(), ck, torch.empty_like(xx), dA, 2, 32, flags=_btp.FLAG_PATH_MFMA)
 
 
 # The matrix-core backward takes its decay operands as two 16-bit pieces (hi + lo: about 2^-17 per entry with bf16).
 # dA_r is a sum over channels and (source, sink) pairs of products decay * x * dy in which two rounded decay entries
 # meet, so its error is at most about 2 * 2^-17 of the sum of the terms' magnitudes -- which the oracle gives exactly
-# when it is run on |x| and |dy| (the decays are not negative). `eps` is that factor; an fp32 dy that the kernel
-# rounds to 16 bits on load brings 2^-9 of its own.
+# when it is run on |x| and |dy| (the decays are not negative). `eps` is that factor.
 def assert_dA_from_rounded_decays(dA, coeff, x, dy, k, what, eps=2.0 ** -15):
     rdA = orc.backward(f64(coeff), f64(x), f64(dy), k=k)[1]
     magnitude = orc.backward(f64(coeff), np.abs(f64(x)), np.abs(f64(dy)), k=k)[1]
@@ -136,23 +139,6 @@ def test_backward_mfma_path_matches_oracle(B, H, L, k):
     rdx, rdA = orc.backward(f64(coeff), f64(x), f64(dy), k=k)
     assert_close(f64(dx), rdx, BF16_ATOL, BF16_RTOL, "dx mfma")
     assert_dA_from_rounded_decays(dA, coeff, x, dy, k, "dA mfma")
-
-
-@pytest.mark.parametrize("B,H,L", [(2, 3, 32), (2, 2, 144), (2, 8, 512)])
-def test_backward_mfma_path_fp32_dy(B, H, L):
-    """An fp32 dy (the op's default) is rounded to the inputs' type on its way to the matrix instruction."""
-    from spear_amd import _btp
-
-    coeff, x, _ = make_inputs(B, H, L, seed=450 + L)
-    dy = torch.randn(B, H, 16, L, generator=torch.Generator().manual_seed(451 + L))
-    dx = torch.full((B, H, 16, L), float("nan"), device=DEV, dtype=x.dtype)
-    dA = torch.full((B, H, L), float("nan"), device=DEV, dtype=torch.float32)
-    _btp.backward(coeff.to(DEV), x.to(DEV), dy.to(DEV), torch.empty((B, H, L // 16, 16), device=DEV), dx, dA, 2, 32,
-                  flags=_btp.FLAG_PATH_MFMA)
-    rdx, _ = orc.backward(f64(coeff), f64(x), f64(dy))
-    assert_close(f64(dx), rdx, 3e-2, BF16_RTOL, "dx mfma, fp32 dy")
-    # dA: dy's rounding to 16 bits (2^-9) against the sum of the terms' magnitudes
-    assert_dA_from_rounded_decays(dA.cpu(), coeff, x, dy, 2, "dA mfma, fp32 dy", eps=2.0 ** -8)
 
 
 def test_backward_mfma_path_fp16_stress_and_zero_coefficients():

@@ -1,4 +1,5 @@
-"""The C-ABI library loads without a GPU and exports exactly what include/spear_btp.h declares."""
+"""The C-ABI library loads without a GPU and exports exactly what include/spear_btp.h (the operator) and
+include/spear_btp_probe.h (the measurement aids) declare."""
 
 import ctypes
 import os
@@ -8,12 +9,19 @@ import pytest
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 HEADER = os.path.join(ROOT, "include", "spear_btp.h")
+PROBE_HEADER = os.path.join(ROOT, "include", "spear_btp_probe.h")
 
 
-def declared_functions():
-    text = open(HEADER).read()
+def declared_functions(header=HEADER):
+    text = open(header).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     return sorted(set(re.findall(r"\b(spear_(?:btp|phalanx|jagged)_\w+)\s*\(", text)))
+
+
+def test_measurement_aids_are_declared_apart_from_the_operator():
+    assert declared_functions(PROBE_HEADER) == [
+        "spear_btp_copy", "spear_btp_stream_probe", "spear_btp_stream_probe_mix", "spear_btp_stream_probe_shape"]
+    assert not set(declared_functions(PROBE_HEADER)) & set(declared_functions())
 
 
 def test_header_declares_the_expected_entry_points():
@@ -21,13 +29,9 @@ def test_header_declares_the_expected_entry_points():
         "spear_btp_abi_version",
         "spear_btp_backward",
         "spear_btp_backward_loggate",
-        "spear_btp_copy",
         "spear_btp_forward",
         "spear_btp_forward_loggate",
         "spear_btp_last_error",
-        "spear_btp_stream_probe",
-        "spear_btp_stream_probe_mix",
-        "spear_btp_stream_probe_shape",
         "spear_jagged_prefill",
         "spear_jagged_step",
         "spear_phalanx_mix_backward",
@@ -47,7 +51,7 @@ def test_library_exports_every_declared_symbol():
     if not os.path.exists(path):
         pytest.fail(f"{path} is not built; run `python -m spear_amd.csrc.build`")
     lib = ctypes.CDLL(path)
-    for name in declared_functions():
+    for name in declared_functions() + declared_functions(PROBE_HEADER):
         assert hasattr(lib, name), f"{name} missing from {path}"
 
 

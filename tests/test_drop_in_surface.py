@@ -79,7 +79,7 @@ def test_the_cmake_target_builds_the_same_library(tmp_path):
     clang = "/opt/rocm/lib/llvm/bin/clang++"
     if not (cmake and ninja and os.path.exists(clang)):
         pytest.skip("needs cmake, ninja and the ROCm clang")
-    from test_capi_symbols import declared_functions
+    from test_capi_symbols import PROBE_HEADER, declared_functions
 
     from spear_amd import _btp
 
@@ -91,7 +91,7 @@ def test_the_cmake_target_builds_the_same_library(tmp_path):
     assert built.exists()
     assert not (build / "_btp_ext.so").exists()  # switched off above: the C-ABI library needs no PyTorch
     lib = ctypes.CDLL(str(built))
-    for name in declared_functions():
+    for name in declared_functions() + declared_functions(PROBE_HEADER):
         assert hasattr(lib, name), f"{name} missing from the CMake-built library"
     lib.spear_btp_abi_version.restype = ctypes.c_int
     assert lib.spear_btp_abi_version() == _btp._ABI_VERSION
