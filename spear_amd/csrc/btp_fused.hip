@@ -174,6 +174,11 @@ __device__ __forceinline__ float product_of_the_others(float a) {
 #ifndef SPEAR_FUSED_TILE_WAVES_PER_EU
 #define SPEAR_FUSED_TILE_WAVES_PER_EU 3
 #endif
+// The kWide backward (head groups summed through LDS) at 2 per SIMD: 220-250 registers, nothing spills. At 3 it
+// spills 204 bytes per lane and takes 1.8-2.3 times as long (B=1024 L=128 H=32 in groups of 16: 171 -> 301 us).
+#ifndef SPEAR_FUSED_WIDE_WAVES_PER_EU
+#define SPEAR_FUSED_WIDE_WAVES_PER_EU 2
+#endif
 // Which tile workgroup this is: two steps, XCD dealing (tile_workgroup) and the order of the tiles (tile_place).
 // Launch order deals workgroups round-robin to the 8 XCDs, each with its own L2. An XCD gets runs of
 // SPEAR_FUSED_TILE_XCD_GROUP neighbouring workgroups instead (windows of 8 runs sweep the tensors front to back):
@@ -288,7 +293,7 @@ __device__ __forceinline__ HeadSlot head_slot(int slot, int pass, int H, int gro
 // ==========================================================================================
 template <class E, bool kQkv, bool kF32, bool kSums = false, bool kWide = false>
 __global__ __launch_bounds__(64 * kTileWaves)
-__attribute__((amdgpu_waves_per_eu(kWide ? 2 : SPEAR_FUSED_TILE_WAVES_PER_EU)))  // kWide: room for the group's sums
+__attribute__((amdgpu_waves_per_eu(kWide ? SPEAR_FUSED_WIDE_WAVES_PER_EU : SPEAR_FUSED_TILE_WAVES_PER_EU)))
 void phalanx_mix_bwd_tile_kernel(
     const uint16_t* __restrict__ a_logit, const uint16_t* __restrict__ b_logit, const uint16_t* __restrict__ c_in,
     const uint16_t* __restrict__ v_in, const uint16_t* __restrict__ dout, uint16_t* __restrict__ da_logit,
