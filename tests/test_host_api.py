@@ -409,3 +409,28 @@ def test_config1_cpu_path_reproduces_the_reference_layer():
         y = layer(x)
     assert y.dtype == torch.bfloat16 and bool(v["y.dtype_is_bf16"][0])
     np.testing.assert_allclose(y[:, ::8, :].float().numpy(), v["y.every8"], rtol=2.0 ** -7, atol=2.0 ** -8)
+
+
+def test_bench_reads_the_roofline_traffic_from_the_committed_profiles(tmp_path, monkeypatch):
+    """`roofline.traffic` of the bench line is the "total MB" of the dominant kernel's row in the committed rocprofv3
+    summary, with its source named; a missing file or row gives null, never a stale constant."""
+    import os
+
+    import bench
+
+    got, src = bench.profiled_traffic("c3", "bwd_scan")
+    assert src == {"file": "profiles/btp_kernels_c3_B1024_H32_L128.txt", "table": "HBM traffic per dispatch",
+                   "row": "bwd_scan", "column": "total MB"}
+    # within a few per cent of the algorithmic bytes of that launch (102 B x 4,194,304 units), and from the file
+    assert 0.99 <= got / (102 * 1024 * 32 * 128) <= 1.05
+    text = open(os.path.join(bench.ROOT, src["file"])).read()
+    assert ("%.1f" % (got / 1e6)) in text
+    for cfg in ("c4", "c5"):
+        assert bench.profiled_traffic(cfg, "bwd_scan")[0] is not None
+    assert bench.profiled_traffic("c3", "no_such_kernel") == (None, None)
+    assert bench.profiled_traffic("c9", "bwd_scan") == (None, None)
+    # a kernel whose name has a blank in it, and a file that lacks the table
+    assert bench.profiled_traffic("c3", "fwd_scan log-gate")[0] is not None
+    monkeypatch.setattr(bench, "PROFILES", str(tmp_path))
+    (tmp_path / "btp_kernels_c3_x.txt").write_text("== kernel durations ==\nbwd_scan   1  2  3  4  5.0  1.0\n")
+    assert bench.profiled_traffic("c3", "bwd_scan") == (None, None)
