@@ -87,26 +87,42 @@ namespace {
 // ==========================================================================================
 // Forward
 // ==========================================================================================
-template <class E, class C, class OutT, bool kCheckpoint, bool kStreamIn>
-__global__ __launch_bounds__(64 * kWaves) SPEAR_BTP_FWD_OCC void btp_fwd_scan_kernel(
+#ifndef SPEAR_BTP_BWD_LINES_WAVES  // same for backward: 0 = as for rows of whole lines, else kWaves or kWavesLong
+#define SPEAR_BTP_BWD_LINES_WAVES 0
+#endif
+#ifndef SPEAR_BTP_FWD_LINES_WAVES  // wavefronts per workgroup of the forward kernel that moves whole lines
+#define SPEAR_BTP_FWD_LINES_WAVES 4
+#endif
+constexpr int kFwdLinesWaves = SPEAR_BTP_FWD_LINES_WAVES;
+
+// kLines: rows of several spans whose byte length is not a multiple of 128; x and y move as whole cache lines
+// (line_place in btp_staging.h), at the price of two more workgroup barriers.
+template <class E, class C, class OutT, bool kCheckpoint, bool kStreamIn, bool kLines = false,
+          int kW = kLines ? kFwdLinesWaves : kWaves>
+__global__ __launch_bounds__(64 * kW) SPEAR_BTP_FWD_OCC void btp_fwd_scan_kernel(
     const typename C::elem* __restrict__ coeff, const uint16_t* __restrict__ x, OutT* __restrict__ y,
     float* __restrict__ ckpt, int L, int spans_per_row, long total_spans, int k) {
   constexpr bool kOutF32 = std::is_same<OutT, float>::value;
   constexpr int kImgBytes = kOutF32 ? 8192 : 4096;
-  constexpr int kW = kWaves;  // wavefronts in this workgroup (8 measured 1-3 % slower here, unlike backward)
-  __shared__ __align__(16) unsigned char lds[kW][kImgBytes + kCoeffLdsBytes];
+  // kW: wavefronts in this workgroup (8 measured 1-3 % slower than 4 on rows of whole lines, unlike backward)
+  constexpr int kImgStride = kImgBytes + kCoeffLdsBytes;
+  __shared__ __align__(16) unsigned char lds[kW][kImgStride];
   // Rows longer than one span (kStreamIn == false): a span's first block needs the terminal local
   // state of the block before it. Inside a workgroup the neighbouring wavefront has just computed
   // it, so it is handed over through LDS with the kernel's only workgroup barrier; only the first
   // wavefront of a workgroup recomputes it from a halo read (measured: the halo reads of every span
   // added 12 % to the bytes fetched).
   constexpr bool kHandOver = SPEAR_BTP_HANDOVER && !kStreamIn && kW > 1;
+  static_assert(!kLines || (kHandOver && !kOutF32), "whole-line staging: 16-bit y, rows of several spans");
   __shared__ float left_state[kHandOver ? kW : 1][kChan];
 
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const long span = first_span_of_workgroup<(SPEAR_BTP_XCD_REMAP == 2) || (SPEAR_BTP_XCD_REMAP == 1 && !kStreamIn)>(kW) + wave;
   if (span >= total_spans) {  // wave-uniform
-    if constexpr (kHandOver) __syncthreads();  // keep the barrier count equal for every wavefront
+    // keep the barrier count equal for every wavefront
+    if constexpr (kLines) __syncthreads();
+    if constexpr (kHandOver) __syncthreads();
+    if constexpr (kLines) __syncthreads();
     return;
   }
   const SpanCoord sc = span_coord(span, spans_per_row, L);
@@ -122,7 +138,18 @@ __global__ __launch_bounds__(64 * kWaves) SPEAR_BTP_FWD_OCC void btp_fwd_scan_ke
   // the wavefronts of a workgroup (below); only a workgroup's first span re-reads 16 steps.
   constexpr bool kStreamOut = SPEAR_BTP_STREAM_STORES == 1;
   uint4 xin[4];
-  slab16_global_to_regs<nt_loads(kStreamIn)>(xslab, L, sc.nvalid, lane, xin);
+  [[maybe_unused]] uint4 xtail[2];
+  [[maybe_unused]] LinePlace px;
+  [[maybe_unused]] const uint16_t* xrows = x + (sc.row * kChan) * (long)L;
+  // whether this wavefront moves the last chunks of its rows itself (wave-uniform)
+  [[maybe_unused]] const bool tail = kLines && (wave == kW - 1 || sc.sp == spans_per_row - 1);
+  if constexpr (kLines) {
+    px = line_place(xrows, L, sc.sp, lane, wave == 0);
+    line16_global_to_regs<nt_loads(kStreamIn)>(xrows, L, sc.sp, px, lane, xin);
+    if (tail) line16_tail_global_to_regs(xrows, L, sc.sp, lane, xtail);
+  } else {
+    slab16_global_to_regs<nt_loads(kStreamIn)>(xslab, L, sc.nvalid, lane, xin);
+  }
   const typename C::pair_t ain = coeff_global_to_reg<C>(arow, sc.nvalid, lane);
 
   const bool needs_left = (k == 2) && (sc.sp > 0);            // wave-uniform
@@ -141,9 +168,16 @@ __global__ __launch_bounds__(64 * kWaves) SPEAR_BTP_FWD_OCC void btp_fwd_scan_ke
     c_halo = h;
   }
 
-  slab16_regs_to_lds(img, lane, xin);
-  coeff_reg_to_lds<C>(a_lds, lane, ain);
-  wave_lds_handover();
+  if constexpr (kLines) {
+    line16_regs_to_lds(img, kImgStride, px, lane, xin);
+    if (tail) line16_tail_regs_to_lds(img, xrows, L, lane, xtail);
+    coeff_reg_to_lds<C>(a_lds, lane, ain);
+    __syncthreads();  // the neighbouring wavefronts have written into this image too
+  } else {
+    slab16_regs_to_lds(img, lane, xin);
+    coeff_reg_to_lds<C>(a_lds, lane, ain);
+    wave_lds_handover();
+  }
 
   float xf[32], a[32];
   lane_read16<E>(img, j, d, xf);
@@ -205,9 +239,17 @@ __global__ __launch_bounds__(64 * kWaves) SPEAR_BTP_FWD_OCC void btp_fwd_scan_ke
     slab32_lds_to_global<kStreamOut>(img, yslab, L, sc.nvalid, lane);
   } else {
     lane_write16<E>(img, j, d, yv);
-    wave_lds_handover();
-    uint16_t* yslab = reinterpret_cast<uint16_t*>(y) + (sc.row * kChan) * (long)L + sc.s0;
-    slab16_lds_to_global<kStreamOut>(img, yslab, L, sc.nvalid, lane);
+    if constexpr (kLines) {
+      __syncthreads();  // the wavefront after this one stores the end of this image
+      uint16_t* yrows = reinterpret_cast<uint16_t*>(y) + (sc.row * kChan) * (long)L;
+      const LinePlace py = line_place(yrows, L, sc.sp, lane, wave == 0);
+      line16_lds_to_global<kStreamOut>(img, kImgStride, yrows, L, py, lane);
+      if (tail) line16_tail_lds_to_global(img, yrows, L, sc.sp, lane);
+    } else {
+      wave_lds_handover();
+      uint16_t* yslab = reinterpret_cast<uint16_t*>(y) + (sc.row * kChan) * (long)L + sc.s0;
+      slab16_lds_to_global<kStreamOut>(img, yslab, L, sc.nvalid, lane);
+    }
   }
 }
 
@@ -228,7 +270,7 @@ constexpr int bwd_waves() {
   return kStreamIn ? SPEAR_BTP_BWD_SHORT_ROW_WAVES : kWavesLong;
 }
 
-template <class E, class C, class GradT, class DxT, bool kStreamIn, int kW>
+template <class E, class C, class GradT, class DxT, bool kStreamIn, int kW, bool kLines = false>
 __device__ __forceinline__ void btp_bwd_scan_body(
     unsigned char (*lds)[4096 + (std::is_same<GradT, float>::value ? 8192 : 4096) + kCoeffLdsBytes],
     const typename C::elem* __restrict__ coeff, const uint16_t* __restrict__ x, const GradT* __restrict__ dy,
@@ -242,13 +284,19 @@ __device__ __forceinline__ void btp_bwd_scan_body(
   // forward state from the left neighbour, the gradient carry from the right one) are handed over
   // through LDS with one workgroup barrier; only the workgroup's outer edges read a halo.
   constexpr bool kHandOver = SPEAR_BTP_HANDOVER && !kStreamIn && kW > 1;
+  // kLines: x, dy and dx move as whole cache lines (line_place in btp_staging.h); see the forward kernel
+  static_assert(!kLines || (kHandOver && !kGradF32 && !kDxF32), "whole-line staging: 16-bit dy and dx, rows of several spans");
+  constexpr int kImgStride = 4096 + kGradBytes + kCoeffLdsBytes;
   __shared__ float edge_state[kHandOver ? kW : 1][2][kChan];
 
   SPEAR_BTP_PRIO(3);
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const long span = first_span_of_workgroup<(SPEAR_BTP_XCD_REMAP == 2) || (SPEAR_BTP_XCD_REMAP == 1 && !kStreamIn)>(kW) + wave;
   if (span >= total_spans) {  // wave-uniform
-    if constexpr (kHandOver) __syncthreads();  // keep the barrier count equal for every wavefront
+    // keep the barrier count equal for every wavefront
+    if constexpr (kLines) __syncthreads();
+    if constexpr (kHandOver) __syncthreads();
+    if constexpr (kLines) __syncthreads();
     return;
   }
   const SpanCoord sc = span_coord(span, spans_per_row, L);
@@ -265,11 +313,29 @@ __device__ __forceinline__ void btp_bwd_scan_body(
   constexpr bool kStreamOut = SPEAR_BTP_STREAM_STORES == 1;  // see the forward kernel
   uint4 xin[4];
   uint4 gin[kGradF32 ? 8 : 4];
-  slab16_global_to_regs<nt_loads(kStreamIn)>(xslab, L, sc.nvalid, lane, xin);
-  if constexpr (kGradF32) {
-    slab32_global_to_regs<nt_loads(kStreamIn)>(reinterpret_cast<const float*>(dy) + slab_off, L, sc.nvalid, lane, gin);
+  [[maybe_unused]] uint4 xtail[2], gtail[2];
+  [[maybe_unused]] LinePlace px, pg;
+  const long rows_off = (sc.row * kChan) * (long)L;
+  [[maybe_unused]] const uint16_t* xrows = x + rows_off;
+  [[maybe_unused]] const uint16_t* grows = reinterpret_cast<const uint16_t*>(dy) + rows_off;
+  // whether this wavefront moves the last chunks of its rows itself (wave-uniform)
+  [[maybe_unused]] const bool tail = kLines && (wave == kW - 1 || sc.sp == spans_per_row - 1);
+  if constexpr (kLines) {
+    px = line_place(xrows, L, sc.sp, lane, wave == 0);
+    pg = line_place(grows, L, sc.sp, lane, wave == 0);
+    line16_global_to_regs<nt_loads(kStreamIn)>(xrows, L, sc.sp, px, lane, xin);
+    line16_global_to_regs<nt_loads(kStreamIn)>(grows, L, sc.sp, pg, lane, gin);
+    if (tail) {
+      line16_tail_global_to_regs(xrows, L, sc.sp, lane, xtail);
+      line16_tail_global_to_regs(grows, L, sc.sp, lane, gtail);
+    }
   } else {
-    slab16_global_to_regs<nt_loads(kStreamIn)>(reinterpret_cast<const uint16_t*>(dy) + slab_off, L, sc.nvalid, lane, gin);
+    slab16_global_to_regs<nt_loads(kStreamIn)>(xslab, L, sc.nvalid, lane, xin);
+    if constexpr (kGradF32) {
+      slab32_global_to_regs<nt_loads(kStreamIn)>(reinterpret_cast<const float*>(dy) + slab_off, L, sc.nvalid, lane, gin);
+    } else {
+      slab16_global_to_regs<nt_loads(kStreamIn)>(reinterpret_cast<const uint16_t*>(dy) + slab_off, L, sc.nvalid, lane, gin);
+    }
   }
   const typename C::pair_t ain = coeff_global_to_reg<C>(arow, sc.nvalid, lane);
 
@@ -314,15 +380,27 @@ __device__ __forceinline__ void btp_bwd_scan_body(
   }
 
   SPEAR_BTP_PRIO(0);
-  slab16_regs_to_lds(img_x, lane, xin);
-  if constexpr (kGradF32) {
-    slab32_regs_to_lds(img_g, lane, gin);
-  } else {
+  if constexpr (kLines) {
     uint4 g4[4] = {gin[0], gin[1], gin[2], gin[3]};
-    slab16_regs_to_lds(img_g, lane, g4);
+    line16_regs_to_lds(img_x, kImgStride, px, lane, xin);
+    line16_regs_to_lds(img_g, kImgStride, pg, lane, g4);
+    if (tail) {
+      line16_tail_regs_to_lds(img_x, xrows, L, lane, xtail);
+      line16_tail_regs_to_lds(img_g, grows, L, lane, gtail);
+    }
+    coeff_reg_to_lds<C>(a_lds, lane, ain);
+    __syncthreads();  // the neighbouring wavefronts have written into these images too
+  } else {
+    slab16_regs_to_lds(img_x, lane, xin);
+    if constexpr (kGradF32) {
+      slab32_regs_to_lds(img_g, lane, gin);
+    } else {
+      uint4 g4[4] = {gin[0], gin[1], gin[2], gin[3]};
+      slab16_regs_to_lds(img_g, lane, g4);
+    }
+    coeff_reg_to_lds<C>(a_lds, lane, ain);
+    wave_lds_handover();
   }
-  coeff_reg_to_lds<C>(a_lds, lane, ain);
-  wave_lds_handover();
 
   // Register-lean ordering: x and dy are consumed by the two local recurrences and are dead
   // afterwards; dx is then formed in place from the local reverse state,
@@ -437,19 +515,27 @@ __device__ __forceinline__ void btp_bwd_scan_body(
   } else {
     // dx goes back through the x image: every lane overwrites exactly the chunks it read
     lane_write16<E>(img_x, j, d, dxv);
-    wave_lds_handover();
-    slab16_lds_to_global<kStreamOut>(img_x, dx + slab_off, L, sc.nvalid, lane);
+    if constexpr (kLines) {
+      __syncthreads();  // the wavefront after this one stores the end of this image
+      uint16_t* dxrows = dx + rows_off;
+      const LinePlace pd = line_place(dxrows, L, sc.sp, lane, wave == 0);
+      line16_lds_to_global<kStreamOut>(img_x, kImgStride, dxrows, L, pd, lane);
+      if (tail) line16_tail_lds_to_global(img_x, dxrows, L, sc.sp, lane);
+    } else {
+      wave_lds_handover();
+      slab16_lds_to_global<kStreamOut>(img_x, dx + slab_off, L, sc.nvalid, lane);
+    }
   }
 }
 
 // 16-bit dy and 16-bit coefficients (the reference's operands): the body fits 128 VGPRs, so four
 // waves per SIMD are requested explicitly.
-template <class E, class C, bool kStreamIn, int kW = bwd_waves<true, kStreamIn>()>
+template <class E, class C, bool kStreamIn, int kW = bwd_waves<true, kStreamIn>(), bool kLines = false>
 __global__ __launch_bounds__((64 * kW)) SPEAR_BTP_BWD_OCC void btp_bwd_scan_kernel(
     const typename C::elem* __restrict__ coeff, const uint16_t* __restrict__ x, const uint16_t* __restrict__ dy,
     uint16_t* __restrict__ dx, float* __restrict__ dA, int L, int spans_per_row, long total_spans, int k) {
   __shared__ __align__(16) unsigned char lds[kW][4096 + 4096 + kCoeffLdsBytes];
-  btp_bwd_scan_body<E, C, uint16_t, uint16_t, kStreamIn, kW>(lds, coeff, x, dy, dx, dA, L, spans_per_row, total_spans, k);
+  btp_bwd_scan_body<E, C, uint16_t, uint16_t, kStreamIn, kW, kLines>(lds, coeff, x, dy, dx, dA, L, spans_per_row, total_spans, k);
 }
 
 // fp32 dy (twice the staging registers and LDS), log-space gates (an exponential per coefficient)
@@ -464,17 +550,25 @@ __global__ __launch_bounds__((64 * bwd_waves<false, kStreamIn>())) void btp_bwd_
   btp_bwd_scan_body<E, C, GradT, DxT, kStreamIn, kW>(lds, coeff, x, dy, dx, dA, L, spans_per_row, total_spans, k);
 }
 
-template <class E, class C, class OutT, bool kCheckpoint, bool kStreamIn>
+template <class E, class C, class OutT, bool kCheckpoint, bool kStreamIn, bool kLines = false>
 void launch_fwd_as(const FwdArgs& p, const Grid& g, hipStream_t s) {
-  hipLaunchKernelGGL((btp_fwd_scan_kernel<E, C, OutT, kCheckpoint, kStreamIn>), dim3(g.blocks), dim3(64 * g.waves), 0,
+  hipLaunchKernelGGL((btp_fwd_scan_kernel<E, C, OutT, kCheckpoint, kStreamIn, kLines>), dim3(g.blocks), dim3(64 * g.waves), 0,
                      s, static_cast<const typename C::elem*>(p.coeff), static_cast<const uint16_t*>(p.x),
                      static_cast<OutT*>(p.y), p.checkpoint, p.L, g.spans_per_row, g.total_spans, p.k);
 }
 
 template <class E, class C, class OutT>
 hipError_t launch_fwd(const FwdArgs& p, hipStream_t s) {
-  const Grid g = make_grid((long)p.B * p.H, p.L);
+  Grid g = make_grid((long)p.B * p.H, p.L);
   const bool ck = p.checkpoint != nullptr, st = stream_inputs(g);
+  if constexpr (!std::is_same<OutT, float>::value) {
+    if (g.lines) {
+      g = make_grid((long)p.B * p.H, p.L, kFwdLinesWaves);
+      if (ck) launch_fwd_as<E, C, OutT, true, false, true>(p, g, s);
+      else launch_fwd_as<E, C, OutT, false, false, true>(p, g, s);
+      return hipGetLastError();
+    }
+  }
   if (ck) {
     if (st) launch_fwd_as<E, C, OutT, true, true>(p, g, s);
     else launch_fwd_as<E, C, OutT, true, false>(p, g, s);
@@ -500,6 +594,17 @@ void launch_bwd_as(const BwdArgs& p, const Grid& g, hipStream_t s) {
     hipLaunchKernelGGL((btp_bwd_scan_kernel_relaxed<E, C, GradT, uint16_t, kStreamIn>), dim3(g.blocks), dim3(64 * g.waves), 0, s,
                        c, x, static_cast<const GradT*>(p.dy), dx, p.dA, p.L, g.spans_per_row, g.total_spans, p.k);
   } else {
+    if constexpr (!kStreamIn) {
+      if (g.lines) {  // rows that do not end on a cache line
+        if (g.waves == kWaves)
+          hipLaunchKernelGGL((btp_bwd_scan_kernel<E, C, false, kWaves, true>), dim3(g.blocks), dim3(64 * g.waves), 0, s, c,
+                             x, static_cast<const uint16_t*>(p.dy), dx, p.dA, p.L, g.spans_per_row, g.total_spans, p.k);
+        else
+          hipLaunchKernelGGL((btp_bwd_scan_kernel<E, C, false, kWavesLong, true>), dim3(g.blocks), dim3(64 * g.waves), 0,
+                             s, c, x, static_cast<const uint16_t*>(p.dy), dx, p.dA, p.L, g.spans_per_row, g.total_spans, p.k);
+        return;
+      }
+    }
     if (!kStreamIn && g.waves == kWaves && kWaves != kWavesLong) {  // rows of a few spans: the smaller workgroup
       hipLaunchKernelGGL((btp_bwd_scan_kernel<E, C, kStreamIn, kWaves>), dim3(g.blocks), dim3(64 * g.waves), 0, s, c, x,
                          static_cast<const uint16_t*>(p.dy), dx, p.dA, p.L, g.spans_per_row, g.total_spans, p.k);
@@ -518,7 +623,8 @@ hipError_t launch_bwd(const BwdArgs& p, hipStream_t s) {
   // dealt to the XCDs in runs (first_span_of_workgroup) halo lines are mostly L2 hits, and on rows of up to 8 spans
   // the smaller workgroup wins: 72.5 -> 69 us at L = 256 and 512 (B H L = 4 Mi), 135.5 -> 132.6 us at L = 1024;
   // from 16 spans on the two are within +-2 % of each other either way.
-  const int long_row_waves = (p.L + kSpan - 1) / kSpan <= 8 ? kWaves : bwd_waves<true, false>();
+  int long_row_waves = (p.L + kSpan - 1) / kSpan <= 8 ? kWaves : bwd_waves<true, false>();
+  if (SPEAR_BTP_BWD_LINES_WAVES && (p.L % 64) != 0) long_row_waves = SPEAR_BTP_BWD_LINES_WAVES;
   const Grid g = lean ? make_grid((long)p.B * p.H, p.L, long_row_waves, bwd_waves<true, true>())
                       : make_grid((long)p.B * p.H, p.L, bwd_waves<false, false>(), bwd_waves<false, true>());
   if (stream_inputs(g)) launch_bwd_as<E, C, GradT, true>(p, g, s);

@@ -20,6 +20,9 @@
 #ifndef SPEAR_BTP_STREAM_LOADS   // 0: never, 1: always, 2: only when a row is a single span
 #define SPEAR_BTP_STREAM_LOADS 1
 #endif
+#ifndef SPEAR_BTP_WHOLE_LINES    // 1: rows of several spans that do not end on a 128-byte line move as whole lines
+#define SPEAR_BTP_WHOLE_LINES 1
+#endif
 #ifndef SPEAR_BTP_STREAM_STORES  // 0: never, 1: always
 #define SPEAR_BTP_STREAM_STORES 1
 #endif
@@ -209,6 +212,128 @@ __device__ __forceinline__ void slab16_lds_to_global(const unsigned char* img, u
     const int r = it * 4 + lr;
     const uint4 v = *reinterpret_cast<const uint4*>(img + swz<256>(r, lp));
     if (ok) store16<kStream>(slab + (long)r * L + (lp << 3), v);
+  }
+}
+
+// ---- rows that do not end on a 128-byte line (rows of several spans) --------------------------
+// A channel row of L 16-bit steps is 2 L bytes long. When that is not a multiple of 128 the rows start at
+// different offsets inside their cache lines, the 256-byte piece a span owns of each row straddles three lines,
+// and two of the three are shared with the neighbouring spans: measured, such launches move 0.60-0.69 of the
+// peak rate where rows of whole lines move 0.8, whatever the access width or cache policy. Here the wavefronts
+// of a workgroup therefore move whole lines instead: for each of its 16 rows, wavefront `sp` of a row moves the two
+// lines [16 sp - m, 16 sp + 16 - m) (in 16-byte chunks of the row; m = chunks between the line boundary and the
+// row's start, 0..7), drops the first m chunks into the image of the wavefront before it (they are the end of
+// that wavefront's span) and finds the last m chunks of its own image delivered by the wavefront after it. Where
+// there is no such neighbour in the workgroup -- its last wavefront, a row's last span -- the wavefront moves
+// that tail itself (`tail`, at most 7 chunks per row). Rows 4 apart lie 8 L bytes apart, a whole number of lines
+// because L is a multiple of 16, so a lane meets the same m in all of its four passes. Images are complete after
+// a workgroup barrier; the arithmetic then runs on block-aligned spans exactly as in the plain path, and the
+// results are bit-identical to it.
+struct LinePlace {
+  int c;      // chunk of the row that this lane moves, in each of its 4 passes; may lie outside the row
+  bool own;   // the chunk belongs to this wavefront's image (else to the image of the wavefront before it)
+  bool here;  // the chunk exists and its image is in this workgroup
+};
+
+__device__ __forceinline__ int chunks_into_line(const void* p) {
+  return (int)((reinterpret_cast<uintptr_t>(p) >> 4) & 7);
+}
+
+// `rows` = the start of channel row 0 of the span's (batch, head) row; `first_wave` = first wavefront of the workgroup
+__device__ __forceinline__ LinePlace line_place(const uint16_t* rows, long L, int sp, int lane, bool first_wave) {
+  LinePlace p;
+  p.c = 16 * sp + (lane & 15) - chunks_into_line(rows + (long)(lane >> 4) * L);
+  p.own = p.c >= 16 * sp;
+  p.here = p.c >= 0 && p.c < (int)(L >> 3) && (p.own || !first_wave);
+  return p;
+}
+
+// Lanes without a chunk read the span's first one (always there) and drop it, as in slab16_global_to_regs.
+template <bool kStream>
+__device__ __forceinline__ void line16_global_to_regs(const uint16_t* rows, long L, int sp, const LinePlace& p,
+                                                      int lane, uint4 (&q)[4]) {
+  const uint16_t* src = rows + (long)(lane >> 4) * L + ((p.here ? p.c : 16 * sp) << 3);
+#pragma unroll
+  for (int it = 0; it < 4; ++it) q[it] = load16<kStream>(src + (long)(it * 4) * L);
+#pragma unroll
+  for (int it = 0; it < 4; ++it) q[it] = p.here ? q[it] : zero4();
+}
+
+// Chunks of the wavefront's own image are always written (zeros past the row's end, which the arithmetic
+// relies on); chunks of the image before it only when they exist. `stride` = bytes between two wavefronts' images.
+__device__ __forceinline__ void line16_regs_to_lds(unsigned char* img, int stride, const LinePlace& p, int lane,
+                                                   const uint4 (&q)[4]) {
+  if (p.own || p.here) {
+    unsigned char* dst = img - (p.own ? 0 : stride);
+#pragma unroll
+    for (int it = 0; it < 4; ++it)
+      *reinterpret_cast<uint4*>(dst + swz<256>(it * 4 + (lane >> 4), p.c & 15)) = q[it];
+  }
+}
+
+template <bool kStream>
+__device__ __forceinline__ void line16_lds_to_global(const unsigned char* img, int stride, uint16_t* rows, long L,
+                                                     const LinePlace& p, int lane) {
+  if (p.here) {
+    const unsigned char* src = img - (p.own ? 0 : stride);
+#pragma unroll
+    for (int it = 0; it < 4; ++it) {
+      const int r = it * 4 + (lane >> 4);
+      const uint4 v = *reinterpret_cast<const uint4*>(src + swz<256>(r, p.c & 15));
+      store16<kStream>(rows + (long)r * L + (p.c << 3), v);
+    }
+  }
+}
+
+// The tail: the last m chunks of each row of the wavefront's own image. Lane l takes row l / 4 and, in pass u,
+// the chunk (l % 4) + 4 u of that row's tail.
+struct LineTail {
+  int m;  // of the lane's row
+  const uint16_t* row;
+};
+
+__device__ __forceinline__ LineTail line_tail(const uint16_t* rows, long L, int lane) {
+  LineTail t;
+  t.row = rows + (long)(lane >> 2) * L;
+  t.m = chunks_into_line(t.row);
+  return t;
+}
+
+// Tails are the one place where two workgroups touch the same line, so they use plain (cached) accesses: measured
+// 2-3 % of the whole launch against streaming ones.
+__device__ __forceinline__ void line16_tail_global_to_regs(const uint16_t* rows, long L, int sp, int lane,
+                                                           uint4 (&q)[2]) {
+  const LineTail t = line_tail(rows, L, lane);
+#pragma unroll
+  for (int u = 0; u < 2; ++u) {
+    const int i = (lane & 3) + 4 * u, c = 16 * sp + 16 - t.m + i;
+    // a real branch here: a lane without a chunk must not ask for some other line (a tail is 16 lines per
+    // instruction as it is, twice what a pass over the span's own lines touches)
+    q[u] = zero4();
+    if (i < t.m && c < (int)(L >> 3)) q[u] = load16<false>(t.row + (c << 3));
+  }
+}
+
+__device__ __forceinline__ void line16_tail_regs_to_lds(unsigned char* img, const uint16_t* rows, long L, int lane,
+                                                        const uint4 (&q)[2]) {
+  const LineTail t = line_tail(rows, L, lane);
+#pragma unroll
+  for (int u = 0; u < 2; ++u) {
+    const int i = (lane & 3) + 4 * u;
+    if (i < t.m) *reinterpret_cast<uint4*>(img + swz<256>(lane >> 2, 16 - t.m + i)) = q[u];
+  }
+}
+
+__device__ __forceinline__ void line16_tail_lds_to_global(const unsigned char* img, uint16_t* rows, long L, int sp,
+                                                          int lane) {
+  const LineTail t = line_tail(rows, L, lane);
+#pragma unroll
+  for (int u = 0; u < 2; ++u) {
+    const int i = (lane & 3) + 4 * u, c = 16 * sp + 16 - t.m + i;
+    if (i < t.m && c < (int)(L >> 3)) {
+      const uint4 v = *reinterpret_cast<const uint4*>(img + swz<256>(lane >> 2, 16 - t.m + i));
+      store16<false>(const_cast<uint16_t*>(t.row) + (c << 3), v);
+    }
   }
 }
 
@@ -509,6 +634,7 @@ struct Grid {
   int spans_per_row;
   long total_spans;
   bool stream;     // kStreamIn of the kernels
+  bool lines;      // rows of several spans that do not end on a 128-byte line: kLines of the kernels that have it
   int waves;       // wavefronts per workgroup
   unsigned blocks;
 };
@@ -521,6 +647,7 @@ inline Grid make_grid(long rows, int L, int waves_long = kWaves, int waves_short
   g.spans_per_row = (L + kSpan - 1) / kSpan;
   g.total_spans = rows * g.spans_per_row;
   g.stream = g.spans_per_row == 1;  // template argument kStreamIn of the kernels: rows of a single span
+  g.lines = !g.stream && (L % 64) != 0 && SPEAR_BTP_WHOLE_LINES;
   g.waves = g.stream ? waves_short : waves_long;
   g.blocks = (unsigned)((g.total_spans + g.waves - 1) / g.waves);
   return g;

@@ -332,6 +332,58 @@ def test_forward_and_backward_on_odd_launch_shapes(B, H, L, k, f32, seed):
         assert_dA_from_rounded_decays(dAm, coeff, x, dy, k, "dA mfma")
 
 
+def _carve(shape, dtype, offset, fill):
+    """A contiguous tensor of `shape` that starts `offset` elements into a larger buffer filled with `fill`."""
+    n = int(np.prod(shape))
+    buf = torch.full((n + offset + 64,), fill, device=DEV, dtype=dtype)
+    return buf, buf[offset : offset + n].view(shape)
+
+
+@pytest.mark.parametrize("offsets", [(0, 0, 0, 0), (8, 16, 24, 40), (56, 8, 0, 32)], ids=["on_lines", "offsets_a", "offsets_b"])
+@pytest.mark.parametrize("B,H,L", [(2, 3, 144), (1, 2, 272), (3, 5, 400), (2, 2, 1040), (1, 3, 2032), (5, 1, 2000), (7, 3, 272)])
+def test_rows_of_several_spans_that_do_not_end_on_a_cache_line(B, H, L, offsets):
+    """Rows of 2 L bytes with L % 64 != 0 start at different offsets inside their 128-byte lines; the 16-bit kernels then
+    move whole lines and hand the ends of the rows from wavefront to wavefront. Tensors are placed at 16-byte steps
+    off the line grid (x, dy, y and dx each at their own), so every row start 0..7 chunks into a line occurs; results
+    against the oracle, equal to the fp32-output / fp32-dx kernels (which move rows the plain way) after rounding, and
+    nothing written outside the tensors."""
+    from spear_amd import _btp
+
+    coeff, x, dy = make_inputs(B, H, L, seed=600 + L + offsets[0], stress=1.5)
+    c = coeff.to(DEV)
+    shape = (B, H, 16, L)
+    (bx, xv), (bg, gv) = _carve(shape, x.dtype, offsets[0], 0.0), _carve(shape, x.dtype, offsets[1], 0.0)
+    xv.copy_(x)
+    gv.copy_(dy)
+    ck = torch.empty(0, device=DEV, dtype=torch.float32)
+    for k in (2, 1):
+        print(f"rows off lines B={B} H={H} L={L} offsets={offsets} k={k}", flush=True)
+        (by, yv), (bd, dxv) = _carve(shape, x.dtype, offsets[2], 7.0), _carve(shape, x.dtype, offsets[3], 7.0)
+        dA = torch.full((B, H, L), float("nan"), device=DEV)
+        _btp.forward(c, xv, yv, ck, k, 32, flags=0)
+        _btp.backward(c, xv, gv, ck, dxv, dA, k, 32)
+        y32 = torch.empty(shape, device=DEV, dtype=torch.float32)
+        dx32 = torch.empty(shape, device=DEV, dtype=torch.float32)
+        dA32 = torch.empty(B, H, L, device=DEV)
+        _btp.forward(c, xv, y32, ck, k, 32, flags=0)
+        _btp.backward(c, xv, gv, ck, dx32, dA32, k, 32, flags=_btp.FLAG_DX_F32)
+        torch.cuda.synchronize()
+        n = xv.numel()
+        for name, buf, off in (("y", by, offsets[2]), ("dx", bd, offsets[3])):
+            assert bool((buf[:off] == 7).all()) and bool((buf[off + n :] == 7).all()), f"{name}: bytes outside the tensor changed"
+        assert torch.equal(yv, y32.to(x.dtype)) and torch.equal(dxv, dx32.to(x.dtype)) and torch.equal(dA, dA32)
+        assert_close(f64(yv.cpu()), orc.forward(f64(coeff), f64(x), k=k), BF16_ATOL, BF16_RTOL, "y")
+        rdx, rdA = orc.backward(f64(coeff), f64(x), f64(dy), k=k)
+        assert_close(f64(dxv.cpu()), rdx, BF16_ATOL, BF16_RTOL, "dx")
+        assert_close(f64(dA.cpu()), rdA, F32_ATOL, F32_RTOL, "dA")
+    # the carries written beside y do not depend on how y moves
+    y_ck, carries = run_forward(coeff, x, k=2, checkpoint=True)
+    assert torch.equal(y_ck, run_forward(coeff, x, k=2))
+    nb = L // 16
+    rck = orc.forward(f64(coeff), f64(x), with_checkpoint=True)[1]
+    assert_close(f64(carries)[:, :, : nb - 1], rck[:, :, : nb - 1], F32_ATOL, F32_RTOL, "checkpoint")
+
+
 def test_kernels_match_the_reference_float64_path_vectors():
     """Forward and backward kernels against y, dx, dA computed by the reference's own float64 path and
     autograd (tests/golden/make_cpu_path_vectors.py)."""

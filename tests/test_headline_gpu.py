@@ -37,6 +37,10 @@ CONFIGS = {
     "c3_B1024_H32_L128": dict(B=1024, H=32, L=128, seed=1234, x_std=0.25, gate="sigmoid"),
     "c4_B16_H64_L8192": dict(B=16, H=64, L=8192, seed=1235, x_std=0.25, gate="sigmoid"),
     "c5_B64_H128_L2048": dict(B=64, H=128, L=2048, seed=1236, x_std=1.0, gate="mixed"),
+    # not a benchmark shape: rows of 4064 bytes, which do not end on a 128-byte line. The 16-bit forward and backward
+    # move whole lines there (their wavefronts pass row ends to each other through LDS); fp32 y and the fp32-dx check
+    # mode keep the plain movement, so the bit-equality checks below compare the two.
+    "rows_off_lines_B64_H128_L2032": dict(B=64, H=128, L=2032, seed=1237, x_std=0.25, gate="sigmoid"),
 }
 
 
@@ -108,8 +112,8 @@ def test_full_size_properties(name):
 
 @pytest.mark.parametrize("name", list(CONFIGS))
 def test_every_row_of_the_benchmark_shapes_against_the_oracle(name):
-    """Every (batch, head) row of B1024·H32·L128 (32,768 rows), B16·H64·L8192 (1,024) and B64·H128·L2048 (8,192), not
-    a sample: fp32 `y`, unrounded `dx` (check mode) and `dA` within 1e-4, bf16 `y` and `dx` within 2e-2 of the float64
+    """Every (batch, head) row of B1024·H32·L128 (32,768 rows), B16·H64·L8192 (1,024), B64·H128·L2048 (8,192) and of
+    B64·H128·L2032 (rows that do not end on a cache line), not a sample: fp32 `y`, unrounded `dx` (check mode) and `dA` within 1e-4, bf16 `y` and `dx` within 2e-2 of the float64
     oracle run on the same bf16-rounded inputs (the protocol of spear/ops/btp/runners.py:103-164), the oracle called
     on about half a million (token, head) units at a time."""
     from spear_amd import _btp
