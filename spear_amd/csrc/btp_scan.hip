@@ -113,7 +113,7 @@ __global__ __launch_bounds__(64 * kW) SPEAR_BTP_FWD_OCC void btp_fwd_scan_kernel
   // wavefront of a workgroup recomputes it from a halo read (measured: the halo reads of every span
   // added 12 % to the bytes fetched).
   constexpr bool kHandOver = SPEAR_BTP_HANDOVER && !kStreamIn && kW > 1;
-  static_assert(!kLines || (kHandOver && !kOutF32), "whole-line staging: 16-bit y, rows of several spans");
+  static_assert(!kLines || kHandOver, "whole-line staging is for rows of several spans");
   __shared__ float left_state[kHandOver ? kW : 1][kChan];
 
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
@@ -145,8 +145,8 @@ __global__ __launch_bounds__(64 * kW) SPEAR_BTP_FWD_OCC void btp_fwd_scan_kernel
   [[maybe_unused]] const bool tail = kLines && (wave == kW - 1 || sc.sp == spans_per_row - 1);
   if constexpr (kLines) {
     px = line_place(xrows, L, sc.sp, lane, wave == 0);
-    line16_global_to_regs<nt_loads(kStreamIn)>(xrows, L, sc.sp, px, lane, xin);
-    if (tail) line16_tail_global_to_regs(xrows, L, sc.sp, lane, xtail);
+    line_global_to_regs<nt_loads(kStreamIn)>(xrows, L, sc.sp, px, lane, xin);
+    if (tail) line_tail_global_to_regs(xrows, L, sc.sp, lane, xtail);
   } else {
     slab16_global_to_regs<nt_loads(kStreamIn)>(xslab, L, sc.nvalid, lane, xin);
   }
@@ -169,8 +169,8 @@ __global__ __launch_bounds__(64 * kW) SPEAR_BTP_FWD_OCC void btp_fwd_scan_kernel
   }
 
   if constexpr (kLines) {
-    line16_regs_to_lds(img, kImgStride, px, lane, xin);
-    if (tail) line16_tail_regs_to_lds(img, xrows, L, lane, xtail);
+    line_regs_to_lds<uint16_t>(img, kImgStride, px, lane, xin);
+    if (tail) line_tail_regs_to_lds(img, xrows, L, lane, xtail);
     coeff_reg_to_lds<C>(a_lds, lane, ain);
     __syncthreads();  // the neighbouring wavefronts have written into this image too
   } else {
@@ -230,26 +230,22 @@ __global__ __launch_bounds__(64 * kW) SPEAR_BTP_FWD_OCC void btp_fwd_scan_kernel
     }
   }
 
-  // ---- results back through LDS so that the global writes are coalesced
+  // ---- results back through LDS so that the global writes are coalesced (whole lines: the wavefront after
+  // this one stores the end of this image, hence the workgroup barrier there)
   wave_lds_handover();
-  if constexpr (kOutF32) {
-    lane_write32(img, j, d, yv);
-    wave_lds_handover();
-    float* yslab = reinterpret_cast<float*>(y) + (sc.row * kChan) * (long)L + sc.s0;
-    slab32_lds_to_global<kStreamOut>(img, yslab, L, sc.nvalid, lane);
+  typedef typename std::conditional<kOutF32, float, uint16_t>::type Y;
+  if constexpr (kOutF32) lane_write32(img, j, d, yv);
+  else lane_write16<E>(img, j, d, yv);
+  Y* yrows = reinterpret_cast<Y*>(y) + (sc.row * kChan) * (long)L;
+  if constexpr (kLines) {
+    __syncthreads();
+    const LinePlace py = line_place(yrows, L, sc.sp, lane, wave == 0);
+    line_lds_to_global<kStreamOut>(img, kImgStride, yrows, L, py, lane);
+    if (tail) line_tail_lds_to_global(img, yrows, L, sc.sp, lane);
   } else {
-    lane_write16<E>(img, j, d, yv);
-    if constexpr (kLines) {
-      __syncthreads();  // the wavefront after this one stores the end of this image
-      uint16_t* yrows = reinterpret_cast<uint16_t*>(y) + (sc.row * kChan) * (long)L;
-      const LinePlace py = line_place(yrows, L, sc.sp, lane, wave == 0);
-      line16_lds_to_global<kStreamOut>(img, kImgStride, yrows, L, py, lane);
-      if (tail) line16_tail_lds_to_global(img, yrows, L, sc.sp, lane);
-    } else {
-      wave_lds_handover();
-      uint16_t* yslab = reinterpret_cast<uint16_t*>(y) + (sc.row * kChan) * (long)L + sc.s0;
-      slab16_lds_to_global<kStreamOut>(img, yslab, L, sc.nvalid, lane);
-    }
+    wave_lds_handover();
+    if constexpr (kOutF32) slab32_lds_to_global<kStreamOut>(img, yrows + sc.s0, L, sc.nvalid, lane);
+    else slab16_lds_to_global<kStreamOut>(img, yrows + sc.s0, L, sc.nvalid, lane);
   }
 }
 
@@ -285,7 +281,7 @@ __device__ __forceinline__ void btp_bwd_scan_body(
   // through LDS with one workgroup barrier; only the workgroup's outer edges read a halo.
   constexpr bool kHandOver = SPEAR_BTP_HANDOVER && !kStreamIn && kW > 1;
   // kLines: x, dy and dx move as whole cache lines (line_place in btp_staging.h); see the forward kernel
-  static_assert(!kLines || (kHandOver && !kGradF32 && !kDxF32), "whole-line staging: 16-bit dy and dx, rows of several spans");
+  static_assert(!kLines || (kHandOver && !kDxF32), "whole-line staging: 16-bit dx, rows of several spans");
   constexpr int kImgStride = 4096 + kGradBytes + kCoeffLdsBytes;
   __shared__ float edge_state[kHandOver ? kW : 1][2][kChan];
 
@@ -317,17 +313,17 @@ __device__ __forceinline__ void btp_bwd_scan_body(
   [[maybe_unused]] LinePlace px, pg;
   const long rows_off = (sc.row * kChan) * (long)L;
   [[maybe_unused]] const uint16_t* xrows = x + rows_off;
-  [[maybe_unused]] const uint16_t* grows = reinterpret_cast<const uint16_t*>(dy) + rows_off;
+  [[maybe_unused]] const GradT* grows = dy + rows_off;
   // whether this wavefront moves the last chunks of its rows itself (wave-uniform)
   [[maybe_unused]] const bool tail = kLines && (wave == kW - 1 || sc.sp == spans_per_row - 1);
   if constexpr (kLines) {
     px = line_place(xrows, L, sc.sp, lane, wave == 0);
     pg = line_place(grows, L, sc.sp, lane, wave == 0);
-    line16_global_to_regs<nt_loads(kStreamIn)>(xrows, L, sc.sp, px, lane, xin);
-    line16_global_to_regs<nt_loads(kStreamIn)>(grows, L, sc.sp, pg, lane, gin);
+    line_global_to_regs<nt_loads(kStreamIn)>(xrows, L, sc.sp, px, lane, xin);
+    line_global_to_regs<nt_loads(kStreamIn)>(grows, L, sc.sp, pg, lane, gin);
     if (tail) {
-      line16_tail_global_to_regs(xrows, L, sc.sp, lane, xtail);
-      line16_tail_global_to_regs(grows, L, sc.sp, lane, gtail);
+      line_tail_global_to_regs(xrows, L, sc.sp, lane, xtail);
+      line_tail_global_to_regs(grows, L, sc.sp, lane, gtail);
     }
   } else {
     slab16_global_to_regs<nt_loads(kStreamIn)>(xslab, L, sc.nvalid, lane, xin);
@@ -381,12 +377,11 @@ __device__ __forceinline__ void btp_bwd_scan_body(
 
   SPEAR_BTP_PRIO(0);
   if constexpr (kLines) {
-    uint4 g4[4] = {gin[0], gin[1], gin[2], gin[3]};
-    line16_regs_to_lds(img_x, kImgStride, px, lane, xin);
-    line16_regs_to_lds(img_g, kImgStride, pg, lane, g4);
+    line_regs_to_lds<uint16_t>(img_x, kImgStride, px, lane, xin);
+    line_regs_to_lds<GradT>(img_g, kImgStride, pg, lane, gin);
     if (tail) {
-      line16_tail_regs_to_lds(img_x, xrows, L, lane, xtail);
-      line16_tail_regs_to_lds(img_g, grows, L, lane, gtail);
+      line_tail_regs_to_lds(img_x, xrows, L, lane, xtail);
+      line_tail_regs_to_lds(img_g, grows, L, lane, gtail);
     }
     coeff_reg_to_lds<C>(a_lds, lane, ain);
     __syncthreads();  // the neighbouring wavefronts have written into these images too
@@ -519,8 +514,8 @@ __device__ __forceinline__ void btp_bwd_scan_body(
       __syncthreads();  // the wavefront after this one stores the end of this image
       uint16_t* dxrows = dx + rows_off;
       const LinePlace pd = line_place(dxrows, L, sc.sp, lane, wave == 0);
-      line16_lds_to_global<kStreamOut>(img_x, kImgStride, dxrows, L, pd, lane);
-      if (tail) line16_tail_lds_to_global(img_x, dxrows, L, sc.sp, lane);
+      line_lds_to_global<kStreamOut>(img_x, kImgStride, dxrows, L, pd, lane);
+      if (tail) line_tail_lds_to_global(img_x, dxrows, L, sc.sp, lane);
     } else {
       wave_lds_handover();
       slab16_lds_to_global<kStreamOut>(img_x, dx + slab_off, L, sc.nvalid, lane);
@@ -540,14 +535,14 @@ __global__ __launch_bounds__((64 * kW)) SPEAR_BTP_BWD_OCC void btp_bwd_scan_kern
 
 // fp32 dy (twice the staging registers and LDS), log-space gates (an exponential per coefficient)
 // and the fp32-dx check mode: occupancy is left to the compiler.
-template <class E, class C, class GradT, class DxT, bool kStreamIn>
+template <class E, class C, class GradT, class DxT, bool kStreamIn, bool kLines = false>
 __global__ __launch_bounds__((64 * bwd_waves<false, kStreamIn>())) void btp_bwd_scan_kernel_relaxed(
     const typename C::elem* __restrict__ coeff, const uint16_t* __restrict__ x, const GradT* __restrict__ dy,
     DxT* __restrict__ dx, float* __restrict__ dA, int L, int spans_per_row, long total_spans, int k) {
   constexpr int kGradBytes = std::is_same<GradT, float>::value ? 8192 : 4096;
   constexpr int kW = bwd_waves<false, kStreamIn>();
   __shared__ __align__(16) unsigned char lds[kW][4096 + kGradBytes + kCoeffLdsBytes];
-  btp_bwd_scan_body<E, C, GradT, DxT, kStreamIn, kW>(lds, coeff, x, dy, dx, dA, L, spans_per_row, total_spans, k);
+  btp_bwd_scan_body<E, C, GradT, DxT, kStreamIn, kW, kLines>(lds, coeff, x, dy, dx, dA, L, spans_per_row, total_spans, k);
 }
 
 template <class E, class C, class OutT, bool kCheckpoint, bool kStreamIn, bool kLines = false>
@@ -561,13 +556,11 @@ template <class E, class C, class OutT>
 hipError_t launch_fwd(const FwdArgs& p, hipStream_t s) {
   Grid g = make_grid((long)p.B * p.H, p.L);
   const bool ck = p.checkpoint != nullptr, st = stream_inputs(g);
-  if constexpr (!std::is_same<OutT, float>::value) {
-    if (g.lines) {
-      g = make_grid((long)p.B * p.H, p.L, kFwdLinesWaves);
-      if (ck) launch_fwd_as<E, C, OutT, true, false, true>(p, g, s);
-      else launch_fwd_as<E, C, OutT, false, false, true>(p, g, s);
-      return hipGetLastError();
-    }
+  if (g.lines) {  // rows that do not end on a cache line
+    g = make_grid((long)p.B * p.H, p.L, kFwdLinesWaves);
+    if (ck) launch_fwd_as<E, C, OutT, true, false, true>(p, g, s);
+    else launch_fwd_as<E, C, OutT, false, false, true>(p, g, s);
+    return hipGetLastError();
   }
   if (ck) {
     if (st) launch_fwd_as<E, C, OutT, true, true>(p, g, s);
@@ -591,6 +584,17 @@ void launch_bwd_as(const BwdArgs& p, const Grid& g, hipStream_t s) {
     return;
   }
   if constexpr (std::is_same<GradT, float>::value || C::kLog) {
+    // Rows that do not end on a cache line: whole lines with 16-bit dy (log-space gates: +2-3 % on rows of 8 spans
+    // and more). With an fp32 dy, whose rows are twice as long and at worst 64 bytes off the lines, it measured
+    // the same on long rows and 5 % slower at L = 272 (two more barriers at this kernel's lower occupancy).
+    if constexpr (!kStreamIn && !std::is_same<GradT, float>::value) {
+      if (g.lines) {
+        hipLaunchKernelGGL((btp_bwd_scan_kernel_relaxed<E, C, GradT, uint16_t, false, true>), dim3(g.blocks),
+                           dim3(64 * g.waves), 0, s, c, x, static_cast<const GradT*>(p.dy), dx, p.dA, p.L,
+                           g.spans_per_row, g.total_spans, p.k);
+        return;
+      }
+    }
     hipLaunchKernelGGL((btp_bwd_scan_kernel_relaxed<E, C, GradT, uint16_t, kStreamIn>), dim3(g.blocks), dim3(64 * g.waves), 0, s,
                        c, x, static_cast<const GradT*>(p.dy), dx, p.dA, p.L, g.spans_per_row, g.total_spans, p.k);
   } else {

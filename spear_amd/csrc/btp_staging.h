@@ -230,9 +230,20 @@ __device__ __forceinline__ void slab16_lds_to_global(const unsigned char* img, u
 // a workgroup barrier; the arithmetic then runs on block-aligned spans exactly as in the plain path, and the
 // results are bit-identical to it.
 struct LinePlace {
-  int c;      // chunk of the row that this lane moves, in each of its 4 passes; may lie outside the row
+  int c;      // chunk of the row that this lane moves, in each of its passes; may lie outside the row
   bool own;   // the chunk belongs to this wavefront's image (else to the image of the wavefront before it)
   bool here;  // the chunk exists and its image is in this workgroup
+};
+
+// The same movement for 16-bit rows (T = uint16_t: 16 chunks per span and row, 4 rows per pass, 4 passes) and
+// fp32 rows (T = float: 32 chunks, 2 rows per pass, 8 passes; rows 2 apart lie 8 L bytes apart again).
+template <class T>
+struct LineGeom {
+  static constexpr int kChunks = 8 * (int)sizeof(T);    // 16-byte chunks of one row in a span
+  static constexpr int kRowBytes = 16 * kChunks;         // of the LDS image
+  static constexpr int kRowsPerPass = 64 / kChunks;
+  static constexpr int kPasses = kChan / kRowsPerPass;
+  static constexpr int kStepsShift = sizeof(T) == 2 ? 3 : 2;  // log2 of the steps in a chunk
 };
 
 __device__ __forceinline__ int chunks_into_line(const void* p) {
@@ -240,99 +251,98 @@ __device__ __forceinline__ int chunks_into_line(const void* p) {
 }
 
 // `rows` = the start of channel row 0 of the span's (batch, head) row; `first_wave` = first wavefront of the workgroup
-__device__ __forceinline__ LinePlace line_place(const uint16_t* rows, long L, int sp, int lane, bool first_wave) {
+template <class T>
+__device__ __forceinline__ LinePlace line_place(const T* rows, long L, int sp, int lane, bool first_wave) {
+  typedef LineGeom<T> G;
   LinePlace p;
-  p.c = 16 * sp + (lane & 15) - chunks_into_line(rows + (long)(lane >> 4) * L);
-  p.own = p.c >= 16 * sp;
-  p.here = p.c >= 0 && p.c < (int)(L >> 3) && (p.own || !first_wave);
+  p.c = G::kChunks * sp + (lane & (G::kChunks - 1)) - chunks_into_line(rows + (long)(lane / G::kChunks) * L);
+  p.own = p.c >= G::kChunks * sp;
+  p.here = p.c >= 0 && p.c < (int)(L >> G::kStepsShift) && (p.own || !first_wave);
   return p;
 }
 
 // Lanes without a chunk read the span's first one (always there) and drop it, as in slab16_global_to_regs.
-template <bool kStream>
-__device__ __forceinline__ void line16_global_to_regs(const uint16_t* rows, long L, int sp, const LinePlace& p,
-                                                      int lane, uint4 (&q)[4]) {
-  const uint16_t* src = rows + (long)(lane >> 4) * L + ((p.here ? p.c : 16 * sp) << 3);
+template <bool kStream, class T>
+__device__ __forceinline__ void line_global_to_regs(const T* rows, long L, int sp, const LinePlace& p, int lane,
+                                                    uint4 (&q)[LineGeom<T>::kPasses]) {
+  typedef LineGeom<T> G;
+  const T* src = rows + (long)(lane / G::kChunks) * L + ((long)(p.here ? p.c : G::kChunks * sp) << G::kStepsShift);
 #pragma unroll
-  for (int it = 0; it < 4; ++it) q[it] = load16<kStream>(src + (long)(it * 4) * L);
+  for (int it = 0; it < G::kPasses; ++it) q[it] = load16<kStream>(src + (long)(it * G::kRowsPerPass) * L);
 #pragma unroll
-  for (int it = 0; it < 4; ++it) q[it] = p.here ? q[it] : zero4();
+  for (int it = 0; it < G::kPasses; ++it) q[it] = p.here ? q[it] : zero4();
 }
 
 // Chunks of the wavefront's own image are always written (zeros past the row's end, which the arithmetic
 // relies on); chunks of the image before it only when they exist. `stride` = bytes between two wavefronts' images.
-__device__ __forceinline__ void line16_regs_to_lds(unsigned char* img, int stride, const LinePlace& p, int lane,
-                                                   const uint4 (&q)[4]) {
+template <class T>
+__device__ __forceinline__ void line_regs_to_lds(unsigned char* img, int stride, const LinePlace& p, int lane,
+                                                 const uint4 (&q)[LineGeom<T>::kPasses]) {
+  typedef LineGeom<T> G;
   if (p.own || p.here) {
     unsigned char* dst = img - (p.own ? 0 : stride);
 #pragma unroll
-    for (int it = 0; it < 4; ++it)
-      *reinterpret_cast<uint4*>(dst + swz<256>(it * 4 + (lane >> 4), p.c & 15)) = q[it];
+    for (int it = 0; it < G::kPasses; ++it)
+      *reinterpret_cast<uint4*>(dst + swz<G::kRowBytes>(it * G::kRowsPerPass + lane / G::kChunks, p.c & (G::kChunks - 1))) = q[it];
   }
 }
 
-template <bool kStream>
-__device__ __forceinline__ void line16_lds_to_global(const unsigned char* img, int stride, uint16_t* rows, long L,
-                                                     const LinePlace& p, int lane) {
+template <bool kStream, class T>
+__device__ __forceinline__ void line_lds_to_global(const unsigned char* img, int stride, T* rows, long L,
+                                                   const LinePlace& p, int lane) {
+  typedef LineGeom<T> G;
   if (p.here) {
     const unsigned char* src = img - (p.own ? 0 : stride);
 #pragma unroll
-    for (int it = 0; it < 4; ++it) {
-      const int r = it * 4 + (lane >> 4);
-      const uint4 v = *reinterpret_cast<const uint4*>(src + swz<256>(r, p.c & 15));
-      store16<kStream>(rows + (long)r * L + (p.c << 3), v);
+    for (int it = 0; it < G::kPasses; ++it) {
+      const int r = it * G::kRowsPerPass + lane / G::kChunks;
+      const uint4 v = *reinterpret_cast<const uint4*>(src + swz<G::kRowBytes>(r, p.c & (G::kChunks - 1)));
+      store16<kStream>(rows + (long)r * L + ((long)p.c << G::kStepsShift), v);
     }
   }
 }
 
 // The tail: the last m chunks of each row of the wavefront's own image. Lane l takes row l / 4 and, in pass u,
-// the chunk (l % 4) + 4 u of that row's tail.
-struct LineTail {
-  int m;  // of the lane's row
-  const uint16_t* row;
-};
-
-__device__ __forceinline__ LineTail line_tail(const uint16_t* rows, long L, int lane) {
-  LineTail t;
-  t.row = rows + (long)(lane >> 2) * L;
-  t.m = chunks_into_line(t.row);
-  return t;
-}
-
-// Tails are the one place where two workgroups touch the same line, so they use plain (cached) accesses: measured
-// 2-3 % of the whole launch against streaming ones.
-__device__ __forceinline__ void line16_tail_global_to_regs(const uint16_t* rows, long L, int sp, int lane,
-                                                           uint4 (&q)[2]) {
-  const LineTail t = line_tail(rows, L, lane);
+// the chunk (l % 4) + 4 u of that row's tail. Tails are the one place where two workgroups touch the same line, so
+// they use plain (cached) accesses: measured 2-3 % of the whole launch against streaming ones. The loads sit in a
+// real branch: a lane without a chunk must not ask for some other line instead (a tail is 16 lines per instruction
+// as it is, twice what a pass over the span's own lines touches; unconditional loads cost 8 % of the launch).
+template <class T>
+__device__ __forceinline__ void line_tail_global_to_regs(const T* rows, long L, int sp, int lane, uint4 (&q)[2]) {
+  typedef LineGeom<T> G;
+  const T* row = rows + (long)(lane >> 2) * L;
+  const int m = chunks_into_line(row);
 #pragma unroll
   for (int u = 0; u < 2; ++u) {
-    const int i = (lane & 3) + 4 * u, c = 16 * sp + 16 - t.m + i;
-    // a real branch here: a lane without a chunk must not ask for some other line (a tail is 16 lines per
-    // instruction as it is, twice what a pass over the span's own lines touches)
+    const int i = (lane & 3) + 4 * u, c = G::kChunks * (sp + 1) - m + i;
     q[u] = zero4();
-    if (i < t.m && c < (int)(L >> 3)) q[u] = load16<false>(t.row + (c << 3));
+    if (i < m && c < (int)(L >> G::kStepsShift)) q[u] = load16<false>(row + ((long)c << G::kStepsShift));
   }
 }
 
-__device__ __forceinline__ void line16_tail_regs_to_lds(unsigned char* img, const uint16_t* rows, long L, int lane,
-                                                        const uint4 (&q)[2]) {
-  const LineTail t = line_tail(rows, L, lane);
+template <class T>
+__device__ __forceinline__ void line_tail_regs_to_lds(unsigned char* img, const T* rows, long L, int lane,
+                                                      const uint4 (&q)[2]) {
+  typedef LineGeom<T> G;
+  const int m = chunks_into_line(rows + (long)(lane >> 2) * L);
 #pragma unroll
   for (int u = 0; u < 2; ++u) {
     const int i = (lane & 3) + 4 * u;
-    if (i < t.m) *reinterpret_cast<uint4*>(img + swz<256>(lane >> 2, 16 - t.m + i)) = q[u];
+    if (i < m) *reinterpret_cast<uint4*>(img + swz<G::kRowBytes>(lane >> 2, G::kChunks - m + i)) = q[u];
   }
 }
 
-__device__ __forceinline__ void line16_tail_lds_to_global(const unsigned char* img, uint16_t* rows, long L, int sp,
-                                                          int lane) {
-  const LineTail t = line_tail(rows, L, lane);
+template <class T>
+__device__ __forceinline__ void line_tail_lds_to_global(const unsigned char* img, T* rows, long L, int sp, int lane) {
+  typedef LineGeom<T> G;
+  T* row = rows + (long)(lane >> 2) * L;
+  const int m = chunks_into_line(row);
 #pragma unroll
   for (int u = 0; u < 2; ++u) {
-    const int i = (lane & 3) + 4 * u, c = 16 * sp + 16 - t.m + i;
-    if (i < t.m && c < (int)(L >> 3)) {
-      const uint4 v = *reinterpret_cast<const uint4*>(img + swz<256>(lane >> 2, 16 - t.m + i));
-      store16<false>(const_cast<uint16_t*>(t.row) + (c << 3), v);
+    const int i = (lane & 3) + 4 * u, c = G::kChunks * (sp + 1) - m + i;
+    if (i < m && c < (int)(L >> G::kStepsShift)) {
+      const uint4 v = *reinterpret_cast<const uint4*>(img + swz<G::kRowBytes>(lane >> 2, G::kChunks - m + i));
+      store16<false>(row + ((long)c << G::kStepsShift), v);
     }
   }
 }

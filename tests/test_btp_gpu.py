@@ -342,40 +342,71 @@ def _carve(shape, dtype, offset, fill):
 @pytest.mark.parametrize("offsets", [(0, 0, 0, 0), (8, 16, 24, 40), (56, 8, 0, 32)], ids=["on_lines", "offsets_a", "offsets_b"])
 @pytest.mark.parametrize("B,H,L", [(2, 3, 144), (1, 2, 272), (3, 5, 400), (2, 2, 1040), (1, 3, 2032), (5, 1, 2000), (7, 3, 272)])
 def test_rows_of_several_spans_that_do_not_end_on_a_cache_line(B, H, L, offsets):
-    """Rows of 2 L bytes with L % 64 != 0 start at different offsets inside their 128-byte lines; the 16-bit kernels then
-    move whole lines and hand the ends of the rows from wavefront to wavefront. Tensors are placed at 16-byte steps
-    off the line grid (x, dy, y and dx each at their own), so every row start 0..7 chunks into a line occurs; results
-    against the oracle, equal to the fp32-output / fp32-dx kernels (which move rows the plain way) after rounding, and
-    nothing written outside the tensors."""
+    """Rows of several spans with L % 64 != 0 start at different offsets inside their 128-byte lines; forward and
+    backward then move whole lines and hand the ends of the rows from wavefront to wavefront (16-bit and fp32 y, 16-bit
+    dy, linear and log-space gates; an fp32 dy and the fp32-dx check mode keep the plain movement). Tensors are placed at
+    16-byte steps off the line grid (x, dy, y and dx each at their own), so every row start 0..7 chunks into a line
+    occurs. Results against the oracle; the 16-bit results equal the rounded fp32 ones (y: another instance of the
+    whole-line movement with rows twice as long; dx: the plain movement), the fp32-dy and log-gate instances agree
+    with the 16-bit linear one, and nothing is written outside the tensors."""
     from spear_amd import _btp
 
     coeff, x, dy = make_inputs(B, H, L, seed=600 + L + offsets[0], stress=1.5)
     c = coeff.to(DEV)
+    gate = torch.log(c.float())  # exp(gate) gives back the 16-bit decays to fp32 rounding
     shape = (B, H, 16, L)
+    n = int(np.prod(shape))
     (bx, xv), (bg, gv) = _carve(shape, x.dtype, offsets[0], 0.0), _carve(shape, x.dtype, offsets[1], 0.0)
+    bg32, gv32 = _carve(shape, torch.float32, offsets[1] // 2, 0.0)
     xv.copy_(x)
     gv.copy_(dy)
+    gv32.copy_(dy)
     ck = torch.empty(0, device=DEV, dtype=torch.float32)
+
+    def untouched(name, buf, off):
+        assert bool((buf[:off] == 7).all()) and bool((buf[off + n :] == 7).all()), f"{name}: bytes outside the tensor changed"
+
     for k in (2, 1):
         print(f"rows off lines B={B} H={H} L={L} offsets={offsets} k={k}", flush=True)
         (by, yv), (bd, dxv) = _carve(shape, x.dtype, offsets[2], 7.0), _carve(shape, x.dtype, offsets[3], 7.0)
+        by32, y32 = _carve(shape, torch.float32, offsets[2] // 2, 7.0)
         dA = torch.full((B, H, L), float("nan"), device=DEV)
         _btp.forward(c, xv, yv, ck, k, 32, flags=0)
+        _btp.forward(c, xv, y32, ck, k, 32, flags=0)
         _btp.backward(c, xv, gv, ck, dxv, dA, k, 32)
-        y32 = torch.empty(shape, device=DEV, dtype=torch.float32)
         dx32 = torch.empty(shape, device=DEV, dtype=torch.float32)
         dA32 = torch.empty(B, H, L, device=DEV)
-        _btp.forward(c, xv, y32, ck, k, 32, flags=0)
         _btp.backward(c, xv, gv, ck, dx32, dA32, k, 32, flags=_btp.FLAG_DX_F32)
         torch.cuda.synchronize()
-        n = xv.numel()
-        for name, buf, off in (("y", by, offsets[2]), ("dx", bd, offsets[3])):
-            assert bool((buf[:off] == 7).all()) and bool((buf[off + n :] == 7).all()), f"{name}: bytes outside the tensor changed"
+        untouched("y", by, offsets[2])
+        untouched("y fp32", by32, offsets[2] // 2)
+        untouched("dx", bd, offsets[3])
         assert torch.equal(yv, y32.to(x.dtype)) and torch.equal(dxv, dx32.to(x.dtype)) and torch.equal(dA, dA32)
-        assert_close(f64(yv.cpu()), orc.forward(f64(coeff), f64(x), k=k), BF16_ATOL, BF16_RTOL, "y")
+        ry = orc.forward(f64(coeff), f64(x), k=k)
         rdx, rdA = orc.backward(f64(coeff), f64(x), f64(dy), k=k)
+        assert_close(f64(y32.cpu()), ry, F32_ATOL, F32_RTOL, "y fp32")
+        assert_close(f64(yv.cpu()), ry, BF16_ATOL, BF16_RTOL, "y")
         assert_close(f64(dxv.cpu()), rdx, BF16_ATOL, BF16_RTOL, "dx")
         assert_close(f64(dA.cpu()), rdA, F32_ATOL, F32_RTOL, "dA")
+
+        # fp32 dy holding the same values: the same arithmetic, dy moved the plain way
+        (bd2, dx2), dA2 = _carve(shape, x.dtype, offsets[3], 7.0), torch.empty(B, H, L, device=DEV)
+        _btp.backward(c, xv, gv32, ck, dx2, dA2, k, 32)
+        torch.cuda.synchronize()
+        untouched("dx (fp32 dy)", bd2, offsets[3])
+        assert torch.equal(dx2, dxv) and torch.equal(dA2, dA)
+
+        # log-space gates: y and dx to the 16-bit bound, dgate = a * dA
+        (by3, y3), (bd3, dx3) = _carve(shape, x.dtype, offsets[2], 7.0), _carve(shape, x.dtype, offsets[3], 7.0)
+        dgate = torch.empty(B, H, L, device=DEV)
+        _btp.forward_log(gate, xv, y3, k)
+        _btp.backward_log(gate, xv, gv, dx3, dgate, k)
+        torch.cuda.synchronize()
+        untouched("y (log gates)", by3, offsets[2])
+        untouched("dx (log gates)", bd3, offsets[3])
+        assert_close(f64(y3.cpu()), ry, BF16_ATOL, BF16_RTOL, "y (log gates)")
+        assert_close(f64(dx3.cpu()), rdx, BF16_ATOL, BF16_RTOL, "dx (log gates)")
+        assert_close(f64(dgate.cpu()), rdA * f64(coeff), 2 * F32_ATOL, 2 * F32_RTOL, "dgate")
     # the carries written beside y do not depend on how y moves
     y_ck, carries = run_forward(coeff, x, k=2, checkpoint=True)
     assert torch.equal(y_ck, run_forward(coeff, x, k=2))

@@ -37,9 +37,9 @@ CONFIGS = {
     "c3_B1024_H32_L128": dict(B=1024, H=32, L=128, seed=1234, x_std=0.25, gate="sigmoid"),
     "c4_B16_H64_L8192": dict(B=16, H=64, L=8192, seed=1235, x_std=0.25, gate="sigmoid"),
     "c5_B64_H128_L2048": dict(B=64, H=128, L=2048, seed=1236, x_std=1.0, gate="mixed"),
-    # not a benchmark shape: rows of 4064 bytes, which do not end on a 128-byte line. The 16-bit forward and backward
-    # move whole lines there (their wavefronts pass row ends to each other through LDS); fp32 y and the fp32-dx check
-    # mode keep the plain movement, so the bit-equality checks below compare the two.
+    # not a benchmark shape: rows of 4064 bytes, which do not end on a 128-byte line. Forward and backward move whole
+    # lines there (their wavefronts pass row ends to each other through LDS); the fp32-dx check mode keeps the plain
+    # movement, so the bit-equality checks of dx and dA below compare the two.
     "rows_off_lines_B64_H128_L2032": dict(B=64, H=128, L=2032, seed=1237, x_std=0.25, gate="sigmoid"),
 }
 
