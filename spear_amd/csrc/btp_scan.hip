@@ -97,11 +97,13 @@ constexpr int kFwdLinesWaves = SPEAR_BTP_FWD_LINES_WAVES;
 
 // kLines: rows of several spans whose byte length is not a multiple of 128; x and y move as whole cache lines
 // (line_place in btp_staging.h), at the price of two more workgroup barriers.
+// kPack: rows of at most half a span, `pack` of them to a wavefront (pack_lane in btp_staging.h); `total_spans`
+// counts rows then.
 template <class E, class C, class OutT, bool kCheckpoint, bool kStreamIn, bool kLines = false,
-          int kW = kLines ? kFwdLinesWaves : kWaves>
+          int kW = kLines ? kFwdLinesWaves : kWaves, bool kPack = false>
 __global__ __launch_bounds__(64 * kW) SPEAR_BTP_FWD_OCC void btp_fwd_scan_kernel(
     const typename C::elem* __restrict__ coeff, const uint16_t* __restrict__ x, OutT* __restrict__ y,
-    float* __restrict__ ckpt, int L, int spans_per_row, long total_spans, int k) {
+    float* __restrict__ ckpt, int L, int spans_per_row, long total_spans, int k, int pack) {
   constexpr bool kOutF32 = std::is_same<OutT, float>::value;
   constexpr int kImgBytes = kOutF32 ? 8192 : 4096;
   // kW: wavefronts in this workgroup (8 measured 1-3 % slower than 4 on rows of whole lines, unlike backward)
@@ -114,18 +116,19 @@ __global__ __launch_bounds__(64 * kW) SPEAR_BTP_FWD_OCC void btp_fwd_scan_kernel
   // added 12 % to the bytes fetched).
   constexpr bool kHandOver = SPEAR_BTP_HANDOVER && !kStreamIn && kW > 1;
   static_assert(!kLines || kHandOver, "whole-line staging is for rows of several spans");
+  static_assert(!kPack || (kStreamIn && !kCheckpoint), "packing is for rows of one span, without the carry store");
   __shared__ float left_state[kHandOver ? kW : 1][kChan];
 
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const long span = first_span_of_workgroup<(SPEAR_BTP_XCD_REMAP == 2) || (SPEAR_BTP_XCD_REMAP == 1 && !kStreamIn)>(kW) + wave;
-  if (span >= total_spans) {  // wave-uniform
+  if (kPack ? span * pack >= total_spans : span >= total_spans) {  // wave-uniform
     // keep the barrier count equal for every wavefront
     if constexpr (kLines) __syncthreads();
     if constexpr (kHandOver) __syncthreads();
     if constexpr (kLines) __syncthreads();
     return;
   }
-  const SpanCoord sc = span_coord(span, spans_per_row, L);
+  const SpanCoord sc = kPack ? pack_coord(span, pack, total_spans, L) : span_coord(span, spans_per_row, L);
 
   unsigned char* img = lds[wave];
   float* a_lds = reinterpret_cast<float*>(img + kImgBytes);
@@ -147,10 +150,14 @@ __global__ __launch_bounds__(64 * kW) SPEAR_BTP_FWD_OCC void btp_fwd_scan_kernel
     px = line_place(xrows, L, sc.sp, lane, wave == 0);
     line_global_to_regs<nt_loads(kStreamIn)>(xrows, L, sc.sp, px, lane, xin);
     if (tail) line_tail_global_to_regs(xrows, L, sc.sp, lane, xtail);
+  } else if constexpr (kPack) {
+    pack_global_to_regs<nt_loads(kStreamIn)>(xslab, L, pack_lane<uint16_t>(lane, L, sc.nvalid / L), xin);
   } else {
     slab16_global_to_regs<nt_loads(kStreamIn)>(xslab, L, sc.nvalid, lane, xin);
   }
   const typename C::pair_t ain = coeff_global_to_reg<C>(arow, sc.nvalid, lane);
+  // packed rows: no carry enters a block with which a row starts (wave-uniform per lane group)
+  const bool startA = kPack && (32 * j) % L == 0, startB = kPack && (32 * j + 16) % L == 0;
 
   const bool needs_left = (k == 2) && (sc.sp > 0);            // wave-uniform
   const bool halo = needs_left && !(kHandOver && wave > 0);     // recompute from a halo read
@@ -191,7 +198,7 @@ __global__ __launch_bounds__(64 * kW) SPEAR_BTP_FWD_OCC void btp_fwd_scan_kernel
 #pragma unroll
   for (int r = 0; r < 16; ++r) h = fmaf(a[r], h, xf[r]);
   const float vA_last = h;
-  h = (k == 2) ? vA_last : 0.0f;
+  h = (k == 2 && !startB) ? vA_last : 0.0f;
 #pragma unroll
   for (int r = 16; r < 32; ++r) {
     h = fmaf(a[r], h, xf[r]);
@@ -211,7 +218,7 @@ __global__ __launch_bounds__(64 * kW) SPEAR_BTP_FWD_OCC void btp_fwd_scan_kernel
     __syncthreads();
     if (needs_left && wave > 0 && j == 0) c_halo = left_state[wave - 1][d];
   }
-  const float cA = (k == 2) ? (j == 0 ? c_halo : from_left) : 0.0f;
+  const float cA = (k == 2 && !startA) ? (j == 0 ? c_halo : from_left) : 0.0f;
   // chain 3: block A started from its carry
   h = cA;
 #pragma unroll
@@ -242,6 +249,9 @@ __global__ __launch_bounds__(64 * kW) SPEAR_BTP_FWD_OCC void btp_fwd_scan_kernel
     const LinePlace py = line_place(yrows, L, sc.sp, lane, wave == 0);
     line_lds_to_global<kStreamOut>(img, kImgStride, yrows, L, py, lane);
     if (tail) line_tail_lds_to_global(img, yrows, L, sc.sp, lane);
+  } else if constexpr (kPack) {
+    wave_lds_handover();
+    pack_lds_to_global<kStreamOut>(img, yrows, L, pack_lane<Y>(lane, L, sc.nvalid / L), lane);
   } else {
     wave_lds_handover();
     if constexpr (kOutF32) slab32_lds_to_global<kStreamOut>(img, yrows + sc.s0, L, sc.nvalid, lane);
@@ -266,12 +276,12 @@ constexpr int bwd_waves() {
   return kStreamIn ? SPEAR_BTP_BWD_SHORT_ROW_WAVES : kWavesLong;
 }
 
-template <class E, class C, class GradT, class DxT, bool kStreamIn, int kW, bool kLines = false>
+template <class E, class C, class GradT, class DxT, bool kStreamIn, int kW, bool kLines = false, bool kPack = false>
 __device__ __forceinline__ void btp_bwd_scan_body(
     unsigned char (*lds)[4096 + (std::is_same<GradT, float>::value ? 8192 : 4096) + kCoeffLdsBytes],
     const typename C::elem* __restrict__ coeff, const uint16_t* __restrict__ x, const GradT* __restrict__ dy,
     DxT* __restrict__ dx, float* __restrict__ dA, int L, int spans_per_row, long total_spans,
-    int k) {
+    int k, int pack) {
   constexpr bool kGradF32 = std::is_same<GradT, float>::value;
   constexpr bool kDxF32 = std::is_same<DxT, float>::value;  // check mode: dx leaves unrounded
   constexpr int kGradBytes = kGradF32 ? 8192 : 4096;
@@ -282,20 +292,22 @@ __device__ __forceinline__ void btp_bwd_scan_body(
   constexpr bool kHandOver = SPEAR_BTP_HANDOVER && !kStreamIn && kW > 1;
   // kLines: x, dy and dx move as whole cache lines (line_place in btp_staging.h); see the forward kernel
   static_assert(!kLines || (kHandOver && !kDxF32), "whole-line staging: 16-bit dx, rows of several spans");
+  // kPack: rows of at most half a span, `pack` of them to a wavefront; `total_spans` counts rows then
+  static_assert(!kPack || kStreamIn, "packing is for rows of one span");
   constexpr int kImgStride = 4096 + kGradBytes + kCoeffLdsBytes;
   __shared__ float edge_state[kHandOver ? kW : 1][2][kChan];
 
   SPEAR_BTP_PRIO(3);
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const long span = first_span_of_workgroup<(SPEAR_BTP_XCD_REMAP == 2) || (SPEAR_BTP_XCD_REMAP == 1 && !kStreamIn)>(kW) + wave;
-  if (span >= total_spans) {  // wave-uniform
+  if (kPack ? span * pack >= total_spans : span >= total_spans) {  // wave-uniform
     // keep the barrier count equal for every wavefront
     if constexpr (kLines) __syncthreads();
     if constexpr (kHandOver) __syncthreads();
     if constexpr (kLines) __syncthreads();
     return;
   }
-  const SpanCoord sc = span_coord(span, spans_per_row, L);
+  const SpanCoord sc = kPack ? pack_coord(span, pack, total_spans, L) : span_coord(span, spans_per_row, L);
 
   unsigned char* img_x = lds[wave];
   unsigned char* img_g = img_x + 4096;
@@ -325,6 +337,9 @@ __device__ __forceinline__ void btp_bwd_scan_body(
       line_tail_global_to_regs(xrows, L, sc.sp, lane, xtail);
       line_tail_global_to_regs(grows, L, sc.sp, lane, gtail);
     }
+  } else if constexpr (kPack) {
+    pack_global_to_regs<nt_loads(kStreamIn)>(xslab, L, pack_lane<uint16_t>(lane, L, sc.nvalid / L), xin);
+    pack_global_to_regs<nt_loads(kStreamIn)>(dy + slab_off, L, pack_lane<GradT>(lane, L, sc.nvalid / L), gin);
   } else {
     slab16_global_to_regs<nt_loads(kStreamIn)>(xslab, L, sc.nvalid, lane, xin);
     if constexpr (kGradF32) {
@@ -449,10 +464,13 @@ __device__ __forceinline__ void btp_bwd_scan_body(
     if (needs_left && wave > 0 && j == 0) c_halo = edge_state[wave - 1][0][d];
     if (needs_right && right_here && j == 3) dc_halo = edge_state[wave + 1][1][d];
   }
-  const float cA = two ? (j == 0 ? c_halo : from_left) : 0.0f;
-  const float cB = two ? v[15] : 0.0f;
-  const float dcA = two ? dcA_raw : 0.0f;
-  const float dcB = two ? (j == 3 ? dc_halo : from_right) : 0.0f;
+  // packed rows: no carry crosses from one row into the next (wave-uniform per lane group)
+  const bool startA = kPack && (32 * j) % L == 0, startB = kPack && (32 * j + 16) % L == 0;
+  const bool endB = kPack && (32 * j + 32) % L == 0;
+  const float cA = (two && !startA) ? (j == 0 ? c_halo : from_left) : 0.0f;
+  const float cB = (two && !startB) ? v[15] : 0.0f;
+  const float dcA = (two && !startB) ? dcA_raw : 0.0f;
+  const float dcB = (two && !endB) ? (j == 3 ? dc_halo : from_right) : 0.0f;
 
   float dA_A, dA_B;
 #pragma unroll
@@ -506,7 +524,8 @@ __device__ __forceinline__ void btp_bwd_scan_body(
     wave_lds_handover();
     lane_write32(img_x, j, d, dxv);
     wave_lds_handover();
-    slab32_lds_to_global<kStreamOut>(img_x, dx + slab_off, L, sc.nvalid, lane);
+    if constexpr (kPack) pack_lds_to_global<kStreamOut>(img_x, dx + slab_off, L, pack_lane<float>(lane, L, sc.nvalid / L), lane);
+    else slab32_lds_to_global<kStreamOut>(img_x, dx + slab_off, L, sc.nvalid, lane);
   } else {
     // dx goes back through the x image: every lane overwrites exactly the chunks it read
     lane_write16<E>(img_x, j, d, dxv);
@@ -516,6 +535,9 @@ __device__ __forceinline__ void btp_bwd_scan_body(
       const LinePlace pd = line_place(dxrows, L, sc.sp, lane, wave == 0);
       line_lds_to_global<kStreamOut>(img_x, kImgStride, dxrows, L, pd, lane);
       if (tail) line_tail_lds_to_global(img_x, dxrows, L, sc.sp, lane);
+    } else if constexpr (kPack) {
+      wave_lds_handover();
+      pack_lds_to_global<kStreamOut>(img_x, dx + slab_off, L, pack_lane<uint16_t>(lane, L, sc.nvalid / L), lane);
     } else {
       wave_lds_handover();
       slab16_lds_to_global<kStreamOut>(img_x, dx + slab_off, L, sc.nvalid, lane);
@@ -525,44 +547,49 @@ __device__ __forceinline__ void btp_bwd_scan_body(
 
 // 16-bit dy and 16-bit coefficients (the reference's operands): the body fits 128 VGPRs, so four
 // waves per SIMD are requested explicitly.
-template <class E, class C, bool kStreamIn, int kW = bwd_waves<true, kStreamIn>(), bool kLines = false>
+template <class E, class C, bool kStreamIn, int kW = bwd_waves<true, kStreamIn>(), bool kLines = false, bool kPack = false>
 __global__ __launch_bounds__((64 * kW)) SPEAR_BTP_BWD_OCC void btp_bwd_scan_kernel(
     const typename C::elem* __restrict__ coeff, const uint16_t* __restrict__ x, const uint16_t* __restrict__ dy,
-    uint16_t* __restrict__ dx, float* __restrict__ dA, int L, int spans_per_row, long total_spans, int k) {
+    uint16_t* __restrict__ dx, float* __restrict__ dA, int L, int spans_per_row, long total_spans, int k, int pack) {
   __shared__ __align__(16) unsigned char lds[kW][4096 + 4096 + kCoeffLdsBytes];
-  btp_bwd_scan_body<E, C, uint16_t, uint16_t, kStreamIn, kW, kLines>(lds, coeff, x, dy, dx, dA, L, spans_per_row, total_spans, k);
+  btp_bwd_scan_body<E, C, uint16_t, uint16_t, kStreamIn, kW, kLines, kPack>(lds, coeff, x, dy, dx, dA, L, spans_per_row,
+                                                                        total_spans, k, pack);
 }
 
 // fp32 dy (twice the staging registers and LDS), log-space gates (an exponential per coefficient)
 // and the fp32-dx check mode: occupancy is left to the compiler.
-template <class E, class C, class GradT, class DxT, bool kStreamIn, bool kLines = false>
+template <class E, class C, class GradT, class DxT, bool kStreamIn, bool kLines = false, bool kPack = false>
 __global__ __launch_bounds__((64 * bwd_waves<false, kStreamIn>())) void btp_bwd_scan_kernel_relaxed(
     const typename C::elem* __restrict__ coeff, const uint16_t* __restrict__ x, const GradT* __restrict__ dy,
-    DxT* __restrict__ dx, float* __restrict__ dA, int L, int spans_per_row, long total_spans, int k) {
+    DxT* __restrict__ dx, float* __restrict__ dA, int L, int spans_per_row, long total_spans, int k, int pack) {
   constexpr int kGradBytes = std::is_same<GradT, float>::value ? 8192 : 4096;
   constexpr int kW = bwd_waves<false, kStreamIn>();
   __shared__ __align__(16) unsigned char lds[kW][4096 + kGradBytes + kCoeffLdsBytes];
-  btp_bwd_scan_body<E, C, GradT, DxT, kStreamIn, kW, kLines>(lds, coeff, x, dy, dx, dA, L, spans_per_row, total_spans, k);
+  btp_bwd_scan_body<E, C, GradT, DxT, kStreamIn, kW, kLines, kPack>(lds, coeff, x, dy, dx, dA, L, spans_per_row,
+                                                                    total_spans, k, pack);
 }
 
-template <class E, class C, class OutT, bool kCheckpoint, bool kStreamIn, bool kLines = false>
+template <class E, class C, class OutT, bool kCheckpoint, bool kStreamIn, bool kLines = false, bool kPack = false>
 void launch_fwd_as(const FwdArgs& p, const Grid& g, hipStream_t s) {
-  hipLaunchKernelGGL((btp_fwd_scan_kernel<E, C, OutT, kCheckpoint, kStreamIn, kLines>), dim3(g.blocks), dim3(64 * g.waves), 0,
-                     s, static_cast<const typename C::elem*>(p.coeff), static_cast<const uint16_t*>(p.x),
-                     static_cast<OutT*>(p.y), p.checkpoint, p.L, g.spans_per_row, g.total_spans, p.k);
+  constexpr int kW = kLines ? kFwdLinesWaves : kWaves;
+  hipLaunchKernelGGL((btp_fwd_scan_kernel<E, C, OutT, kCheckpoint, kStreamIn, kLines, kW, kPack>), dim3(g.blocks),
+                     dim3(64 * g.waves), 0, s, static_cast<const typename C::elem*>(p.coeff),
+                     static_cast<const uint16_t*>(p.x), static_cast<OutT*>(p.y), p.checkpoint, p.L, g.spans_per_row,
+                     g.total_spans, p.k, g.pack);
 }
 
 template <class E, class C, class OutT>
 hipError_t launch_fwd(const FwdArgs& p, hipStream_t s) {
-  Grid g = make_grid((long)p.B * p.H, p.L);
+  const long rows = (long)p.B * p.H;
+  const Grid g = make_grid(rows, p.L);
   const bool ck = p.checkpoint != nullptr, st = stream_inputs(g);
-  if (g.lines) {  // rows that do not end on a cache line
-    g = make_grid((long)p.B * p.H, p.L, kFwdLinesWaves);
-    if (ck) launch_fwd_as<E, C, OutT, true, false, true>(p, g, s);
-    else launch_fwd_as<E, C, OutT, false, false, true>(p, g, s);
-    return hipGetLastError();
-  }
-  if (ck) {
+  if (g.lines) {  // rows of several spans that do not end on a cache line
+    const Grid gl = make_grid(rows, p.L, kFwdLinesWaves);
+    if (ck) launch_fwd_as<E, C, OutT, true, false, true>(p, gl, s);
+    else launch_fwd_as<E, C, OutT, false, false, true>(p, gl, s);
+  } else if (st && g.pack > 1 && !ck) {  // rows of at most half a span, several to a wavefront
+    launch_fwd_as<E, C, OutT, false, true, false, true>(p, packed(g, rows), s);
+  } else if (ck) {
     if (st) launch_fwd_as<E, C, OutT, true, true>(p, g, s);
     else launch_fwd_as<E, C, OutT, true, false>(p, g, s);
   } else {
@@ -572,50 +599,47 @@ hipError_t launch_fwd(const FwdArgs& p, hipStream_t s) {
   return hipGetLastError();
 }
 
+// `g` is the grid of the kernel this picks: see launch_bwd
 template <class E, class C, class GradT, bool kStreamIn>
 void launch_bwd_as(const BwdArgs& p, const Grid& g, hipStream_t s) {
+  constexpr bool kGradF32 = std::is_same<GradT, float>::value;
   const auto* c = static_cast<const typename C::elem*>(p.coeff);
   const auto* x = static_cast<const uint16_t*>(p.x);
-  auto* dx = static_cast<uint16_t*>(p.dx);
-  if (p.dx_f32) {
-    hipLaunchKernelGGL((btp_bwd_scan_kernel_relaxed<E, C, GradT, float, kStreamIn>), dim3(g.blocks), dim3(64 * g.waves),
-                       0, s, c, x, static_cast<const GradT*>(p.dy), static_cast<float*>(p.dx), p.dA, p.L,
-                       g.spans_per_row, g.total_spans, p.k);
-    return;
+  const auto* dy = static_cast<const GradT*>(p.dy);
+  auto go = [&](auto kernel, auto* dx) {
+    hipLaunchKernelGGL(kernel, dim3(g.blocks), dim3(64 * g.waves), 0, s, c, x, dy, dx, p.dA, p.L, g.spans_per_row,
+                       g.total_spans, p.k, g.pack);
+  };
+  auto* dx16 = static_cast<uint16_t*>(p.dx);
+  const bool pack = kStreamIn && g.pack > 1;  // rows of at most half a span, several to a wavefront
+  if (p.dx_f32) {                             // fp32 check mode
+    auto* dx32 = static_cast<float*>(p.dx);
+    if constexpr (kStreamIn) {
+      if (pack) return go(btp_bwd_scan_kernel_relaxed<E, C, GradT, float, true, false, true>, dx32);
+    }
+    return go(btp_bwd_scan_kernel_relaxed<E, C, GradT, float, kStreamIn>, dx32);
   }
-  if constexpr (std::is_same<GradT, float>::value || C::kLog) {
+  if constexpr (kGradF32 || C::kLog) {
+    if constexpr (kStreamIn) {
+      if (pack) return go(btp_bwd_scan_kernel_relaxed<E, C, GradT, uint16_t, true, false, true>, dx16);
+    }
     // Rows that do not end on a cache line: whole lines with 16-bit dy (log-space gates: +2-3 % on rows of 8 spans
     // and more). With an fp32 dy, whose rows are twice as long and at worst 64 bytes off the lines, it measured
     // the same on long rows and 5 % slower at L = 272 (two more barriers at this kernel's lower occupancy).
-    if constexpr (!kStreamIn && !std::is_same<GradT, float>::value) {
-      if (g.lines) {
-        hipLaunchKernelGGL((btp_bwd_scan_kernel_relaxed<E, C, GradT, uint16_t, false, true>), dim3(g.blocks),
-                           dim3(64 * g.waves), 0, s, c, x, static_cast<const GradT*>(p.dy), dx, p.dA, p.L,
-                           g.spans_per_row, g.total_spans, p.k);
-        return;
-      }
+    if constexpr (!kStreamIn && !kGradF32) {
+      if (g.lines) return go(btp_bwd_scan_kernel_relaxed<E, C, GradT, uint16_t, false, true>, dx16);
     }
-    hipLaunchKernelGGL((btp_bwd_scan_kernel_relaxed<E, C, GradT, uint16_t, kStreamIn>), dim3(g.blocks), dim3(64 * g.waves), 0, s,
-                       c, x, static_cast<const GradT*>(p.dy), dx, p.dA, p.L, g.spans_per_row, g.total_spans, p.k);
+    return go(btp_bwd_scan_kernel_relaxed<E, C, GradT, uint16_t, kStreamIn>, dx16);
+  } else if constexpr (kStreamIn) {
+    if (pack) return go(btp_bwd_scan_kernel<E, C, true, bwd_waves<true, true>(), false, true>, dx16);
+    return go(btp_bwd_scan_kernel<E, C, true>, dx16);
   } else {
-    if constexpr (!kStreamIn) {
-      if (g.lines) {  // rows that do not end on a cache line
-        if (g.waves == kWaves)
-          hipLaunchKernelGGL((btp_bwd_scan_kernel<E, C, false, kWaves, true>), dim3(g.blocks), dim3(64 * g.waves), 0, s, c,
-                             x, static_cast<const uint16_t*>(p.dy), dx, p.dA, p.L, g.spans_per_row, g.total_spans, p.k);
-        else
-          hipLaunchKernelGGL((btp_bwd_scan_kernel<E, C, false, kWavesLong, true>), dim3(g.blocks), dim3(64 * g.waves), 0,
-                             s, c, x, static_cast<const uint16_t*>(p.dy), dx, p.dA, p.L, g.spans_per_row, g.total_spans, p.k);
-        return;
-      }
+    const bool small = g.waves == kWaves;  // rows of a few spans: the smaller workgroup
+    if (g.lines) {                         // rows that do not end on a cache line
+      return small ? go(btp_bwd_scan_kernel<E, C, false, kWaves, true>, dx16)
+                   : go(btp_bwd_scan_kernel<E, C, false, kWavesLong, true>, dx16);
     }
-    if (!kStreamIn && g.waves == kWaves && kWaves != kWavesLong) {  // rows of a few spans: the smaller workgroup
-      hipLaunchKernelGGL((btp_bwd_scan_kernel<E, C, kStreamIn, kWaves>), dim3(g.blocks), dim3(64 * g.waves), 0, s, c, x,
-                         static_cast<const uint16_t*>(p.dy), dx, p.dA, p.L, g.spans_per_row, g.total_spans, p.k);
-      return;
-    }
-    hipLaunchKernelGGL((btp_bwd_scan_kernel<E, C, kStreamIn>), dim3(g.blocks), dim3(64 * g.waves), 0, s, c, x,
-                       static_cast<const uint16_t*>(p.dy), dx, p.dA, p.L, g.spans_per_row, g.total_spans, p.k);
+    return small ? go(btp_bwd_scan_kernel<E, C, false, kWaves>, dx16) : go(btp_bwd_scan_kernel<E, C, false, kWavesLong>, dx16);
   }
 }
 
@@ -623,15 +647,16 @@ template <class E, class C, class GradT>
 hipError_t launch_bwd(const BwdArgs& p, hipStream_t s) {
   constexpr bool kLeanIo = !(std::is_same<GradT, float>::value || C::kLog);
   const bool lean = kLeanIo && !p.dx_f32;  // the kernel launch_bwd_as picks
+  const long rows = (long)p.B * p.H;
   // Workgroups of kWavesLong wavefronts hand more carries over in LDS and read fewer halos; with the workgroups
   // dealt to the XCDs in runs (first_span_of_workgroup) halo lines are mostly L2 hits, and on rows of up to 8 spans
   // the smaller workgroup wins: 72.5 -> 69 us at L = 256 and 512 (B H L = 4 Mi), 135.5 -> 132.6 us at L = 1024;
   // from 16 spans on the two are within +-2 % of each other either way.
   int long_row_waves = (p.L + kSpan - 1) / kSpan <= 8 ? kWaves : bwd_waves<true, false>();
   if (SPEAR_BTP_BWD_LINES_WAVES && (p.L % 64) != 0) long_row_waves = SPEAR_BTP_BWD_LINES_WAVES;
-  const Grid g = lean ? make_grid((long)p.B * p.H, p.L, long_row_waves, bwd_waves<true, true>())
-                      : make_grid((long)p.B * p.H, p.L, bwd_waves<false, false>(), bwd_waves<false, true>());
-  if (stream_inputs(g)) launch_bwd_as<E, C, GradT, true>(p, g, s);
+  const Grid g = lean ? make_grid(rows, p.L, long_row_waves, bwd_waves<true, true>())
+                      : make_grid(rows, p.L, bwd_waves<false, false>(), bwd_waves<false, true>());
+  if (stream_inputs(g)) launch_bwd_as<E, C, GradT, true>(p, g.pack > 1 ? packed(g, rows) : g, s);
   else launch_bwd_as<E, C, GradT, false>(p, g, s);
   return hipGetLastError();
 }

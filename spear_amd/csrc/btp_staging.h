@@ -23,6 +23,9 @@
 #ifndef SPEAR_BTP_WHOLE_LINES    // 1: rows of several spans that do not end on a 128-byte line move as whole lines
 #define SPEAR_BTP_WHOLE_LINES 1
 #endif
+#ifndef SPEAR_BTP_PACK_SHORT_ROWS  // 1: rows of at most half a span are packed several to a wavefront
+#define SPEAR_BTP_PACK_SHORT_ROWS 1
+#endif
 #ifndef SPEAR_BTP_STREAM_STORES  // 0: never, 1: always
 #define SPEAR_BTP_STREAM_STORES 1
 #endif
@@ -347,6 +350,52 @@ __device__ __forceinline__ void line_tail_lds_to_global(const unsigned char* img
   }
 }
 
+// ---- rows of at most half a span ---------------------------------------------------------------
+// A wavefront works on a [16 channel x 128 step] image. A row of L <= 64 steps fills at most half of it, and with
+// one row per wavefront a launch at L = 64 / 32 / 16 moved 0.63 / 0.39 / 0.21 of the peak rate. Such rows are
+// therefore packed: a wavefront takes floor(128 / L) consecutive (batch, head) rows, whose slabs follow each other
+// in memory, and lays them side by side in its image (row q of the pack at steps [q L, (q + 1) L)). Coefficients,
+// dA and the carry arithmetic see 128 consecutive steps as before; the kernels only have to drop the carries at
+// the steps where a new row starts.
+struct PackLane {
+  long off;  // of the lane's chunk in pass 0, in elements from the slab of the pack's first row
+  bool ok;   // the chunk exists (its row is one of the pack's)
+};
+
+template <class T>
+__device__ __forceinline__ PackLane pack_lane(int lane, int L, int rows_here) {
+  typedef LineGeom<T> G;
+  const int lp = lane & (G::kChunks - 1), lr = lane / G::kChunks;
+  const int per_row = L >> G::kStepsShift;           // chunks of one row
+  const int q = lp / per_row, cw = lp - q * per_row;  // which row of the pack, which chunk of it
+  PackLane p;
+  p.ok = q < rows_here;
+  p.off = p.ok ? (long)(q * kChan + lr) * L + (cw << G::kStepsShift) : (long)lr * L;  // else: a chunk that is always there
+  return p;
+}
+
+template <bool kStream, class T>
+__device__ __forceinline__ void pack_global_to_regs(const T* first, long L, const PackLane& p,
+                                                    uint4 (&q)[LineGeom<T>::kPasses]) {
+  typedef LineGeom<T> G;
+#pragma unroll
+  for (int it = 0; it < G::kPasses; ++it) q[it] = load16<kStream>(first + p.off + (long)(it * G::kRowsPerPass) * L);
+#pragma unroll
+  for (int it = 0; it < G::kPasses; ++it) q[it] = p.ok ? q[it] : zero4();
+}
+
+template <bool kStream, class T>
+__device__ __forceinline__ void pack_lds_to_global(const unsigned char* img, T* first, long L, const PackLane& p,
+                                                   int lane) {
+  typedef LineGeom<T> G;
+#pragma unroll
+  for (int it = 0; it < G::kPasses; ++it) {
+    const uint4 v = *reinterpret_cast<const uint4*>(
+        img + swz<G::kRowBytes>(it * G::kRowsPerPass + lane / G::kChunks, lane & (G::kChunks - 1)));
+    if (p.ok) store16<kStream>(first + p.off + (long)(it * G::kRowsPerPass) * L, v);
+  }
+}
+
 // ---- rows of any length and alignment (prompt prefill) --------------------------------------
 // The same slab movement for rows whose start is only element-aligned (L not a multiple of 8) and
 // whose last elements may stop anywhere. Under-aligned 16-byte accesses are served by the hardware
@@ -606,6 +655,16 @@ __device__ __forceinline__ SpanCoord span_coord(long span, int spans_per_row, in
   return c;
 }
 
+// Packed rows (see pack_lane): the wavefront's first row and how many steps of its image are rows
+__device__ __forceinline__ SpanCoord pack_coord(long span, int pack, long rows, int L) {
+  SpanCoord c;
+  c.row = span * pack;
+  c.sp = 0;
+  c.s0 = 0;
+  c.nvalid = (int)min((long)pack, rows - c.row) * L;
+  return c;
+}
+
 // Workgroup index -> first span. Workgroups are dealt round-robin to the 8 XCDs, each with its own L2. With
 // kRemap an XCD instead gets runs of SPEAR_BTP_XCD_GROUP neighbouring workgroups (windows of 8 such runs sweep
 // the tensor, so the chip as a whole still walks memory front to back): the workgroup that reads a halo and the
@@ -645,6 +704,7 @@ struct Grid {
   long total_spans;
   bool stream;     // kStreamIn of the kernels
   bool lines;      // rows of several spans that do not end on a 128-byte line: kLines of the kernels that have it
+  int pack;        // rows of at most half a span: how many a wavefront takes (kPack of the kernels that have it), else 1
   int waves;       // wavefronts per workgroup
   unsigned blocks;
 };
@@ -658,12 +718,21 @@ inline Grid make_grid(long rows, int L, int waves_long = kWaves, int waves_short
   g.total_spans = rows * g.spans_per_row;
   g.stream = g.spans_per_row == 1;  // template argument kStreamIn of the kernels: rows of a single span
   g.lines = !g.stream && (L % 64) != 0 && SPEAR_BTP_WHOLE_LINES;
+  g.pack = SPEAR_BTP_PACK_SHORT_ROWS && L > 0 && 2 * L <= kSpan ? kSpan / L : 1;
   g.waves = g.stream ? waves_short : waves_long;
   g.blocks = (unsigned)((g.total_spans + g.waves - 1) / g.waves);
   return g;
 }
 
 inline bool stream_inputs(const Grid& g) { return g.stream; }
+
+// The same rows with `g.pack` of them to a wavefront (the kernels' kPack instances, which count rows where the
+// others count spans).
+inline Grid packed(Grid g, long rows) {
+  g.total_spans = rows;
+  g.blocks = (unsigned)(((rows + g.pack - 1) / g.pack + g.waves - 1) / g.waves);
+  return g;
+}
 
 // Whether a kernel instance reads its slabs with non-temporal loads, from the knob above and from
 // whether its rows are single spans (the kernels' template argument).

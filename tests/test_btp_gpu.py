@@ -415,6 +415,72 @@ def test_rows_of_several_spans_that_do_not_end_on_a_cache_line(B, H, L, offsets)
     assert_close(f64(carries)[:, :, : nb - 1], rck[:, :, : nb - 1], F32_ATOL, F32_RTOL, "checkpoint")
 
 
+@pytest.mark.parametrize("L", [16, 32, 48, 64])
+@pytest.mark.parametrize("B,H", [(1, 1), (1, 3), (2, 3), (1, 7), (5, 5), (8, 33)])
+def test_short_rows_packed_several_to_a_wavefront(B, H, L):
+    """Rows of at most 64 steps share a wavefront (128 // L of them side by side in its image; the last wavefront
+    takes what is left). Every instance against the oracle, nothing written outside the tensors, and every row of
+    the batch bit-identical to the same row run alone (where it sits first in its wavefront's image)."""
+    from spear_amd import _btp
+
+    coeff, x, dy = make_inputs(B, H, L, seed=700 + L + B * H, stress=1.5)
+    c = coeff.to(DEV)
+    gate = torch.log(c.float())
+    shape = (B, H, 16, L)
+    n = int(np.prod(shape))
+    ck = torch.empty(0, device=DEV, dtype=torch.float32)
+    xv, gv, gv32 = x.to(DEV), dy.to(DEV), dy.float().to(DEV)
+
+    def untouched(name, buf, off=8):
+        assert bool((buf[:off] == 7).all()) and bool((buf[off + n :] == 7).all()), f"{name}: bytes outside the tensor changed"
+
+    for k in (2, 1):
+        print(f"short rows B={B} H={H} L={L} k={k}", flush=True)
+        (by, yv), (bd, dxv) = _carve(shape, x.dtype, 8, 7.0), _carve(shape, x.dtype, 8, 7.0)
+        (by32, y32), (bd32, dx32) = _carve(shape, torch.float32, 8, 7.0), _carve(shape, torch.float32, 8, 7.0)
+        dA, dA32 = torch.full((B, H, L), float("nan"), device=DEV), torch.full((B, H, L), float("nan"), device=DEV)
+        _btp.forward(c, xv, yv, ck, k, 32, flags=0)
+        _btp.forward(c, xv, y32, ck, k, 32, flags=0)
+        _btp.backward(c, xv, gv, ck, dxv, dA, k, 32)
+        _btp.backward(c, xv, gv, ck, dx32, dA32, k, 32, flags=_btp.FLAG_DX_F32)
+        torch.cuda.synchronize()
+        for name, buf in (("y", by), ("y fp32", by32), ("dx", bd), ("dx fp32", bd32)):
+            untouched(name, buf)
+        assert torch.equal(yv, y32.to(x.dtype)) and torch.equal(dxv, dx32.to(x.dtype)) and torch.equal(dA, dA32)
+        ry = orc.forward(f64(coeff), f64(x), k=k)
+        rdx, rdA = orc.backward(f64(coeff), f64(x), f64(dy), k=k)
+        assert_close(f64(y32.cpu()), ry, F32_ATOL, F32_RTOL, "y fp32")
+        assert_close(f64(dx32.cpu()), rdx, F32_ATOL, F32_RTOL, "dx fp32")
+        assert_close(f64(dA.cpu()), rdA, F32_ATOL, F32_RTOL, "dA")
+
+        # fp32 dy with the same values; log-space gates
+        dx2, dA2 = torch.empty_like(dxv), torch.empty_like(dA)
+        _btp.backward(c, xv, gv32, ck, dx2, dA2, k, 32)
+        assert torch.equal(dx2, dxv) and torch.equal(dA2, dA)
+        y3, dx3, dgate = torch.empty_like(yv), torch.empty_like(dxv), torch.empty_like(dA)
+        _btp.forward_log(gate, xv, y3, k)
+        _btp.backward_log(gate, xv, gv, dx3, dgate, k)
+        assert_close(f64(y3.cpu()), ry, BF16_ATOL, BF16_RTOL, "y (log gates)")
+        assert_close(f64(dx3.cpu()), rdx, BF16_ATOL, BF16_RTOL, "dx (log gates)")
+        assert_close(f64(dgate.cpu()), rdA * f64(coeff), 2 * F32_ATOL, 2 * F32_RTOL, "dgate")
+
+        # rows alone
+        for b, h in {(0, 0), (B - 1, H - 1), (B // 2, H // 2), (0, H - 1)}:
+            c1, x1, g1 = (t[b : b + 1, h : h + 1].contiguous() for t in (c, xv, gv))
+            y1, d1, a1 = torch.empty_like(x1), torch.empty_like(x1), torch.empty(1, 1, L, device=DEV)
+            _btp.forward(c1, x1, y1, ck, k, 32, flags=0)
+            _btp.backward(c1, x1, g1, ck, d1, a1, k, 32)
+            assert torch.equal(y1, yv[b : b + 1, h : h + 1]) and torch.equal(d1, dxv[b : b + 1, h : h + 1])
+            assert torch.equal(a1, dA[b : b + 1, h : h + 1]), f"row ({b}, {h}) differs from the same row run alone"
+    # with the carry store the rows are not packed: same y, carries against the oracle
+    y_ck, carries = run_forward(coeff, x, k=2, checkpoint=True)
+    assert torch.equal(y_ck, run_forward(coeff, x, k=2))
+    nb = L // 16
+    if nb > 1:
+        rck = orc.forward(f64(coeff), f64(x), with_checkpoint=True)[1]
+        assert_close(f64(carries)[:, :, : nb - 1], rck[:, :, : nb - 1], F32_ATOL, F32_RTOL, "checkpoint")
+
+
 def test_kernels_match_the_reference_float64_path_vectors():
     """Forward and backward kernels against y, dx, dA computed by the reference's own float64 path and
     autograd (tests/golden/make_cpu_path_vectors.py)."""
