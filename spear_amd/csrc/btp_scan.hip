@@ -97,13 +97,14 @@ constexpr int kFwdLinesWaves = SPEAR_BTP_FWD_LINES_WAVES;
 
 // kLines: rows of several spans whose byte length is not a multiple of 128; x and y move as whole cache lines
 // (line_place in btp_staging.h), at the price of two more workgroup barriers.
-// kPack: rows of at most half a span, `pack` of them to a wavefront (pack_lane in btp_staging.h); `total_spans`
-// counts rows then.
+// kFlat: rows that leave a span partly empty; spans are cut from the block sequence of the whole tensor (flat_lane in
+// btp_staging.h). `spans_per_row` holds the blocks in a row and `total_spans` the blocks in the tensor then, and
+// kStreamIn says that no row straddles two spans.
 template <class E, class C, class OutT, bool kCheckpoint, bool kStreamIn, bool kLines = false,
-          int kW = kLines ? kFwdLinesWaves : kWaves, bool kPack = false>
+          int kW = kLines ? kFwdLinesWaves : kWaves, bool kFlat = false>
 __global__ __launch_bounds__(64 * kW) SPEAR_BTP_FWD_OCC void btp_fwd_scan_kernel(
     const typename C::elem* __restrict__ coeff, const uint16_t* __restrict__ x, OutT* __restrict__ y,
-    float* __restrict__ ckpt, int L, int spans_per_row, long total_spans, int k, int pack) {
+    float* __restrict__ ckpt, int L, int spans_per_row, long total_spans, int k) {
   constexpr bool kOutF32 = std::is_same<OutT, float>::value;
   constexpr int kImgBytes = kOutF32 ? 8192 : 4096;
   // kW: wavefronts in this workgroup (8 measured 1-3 % slower than 4 on rows of whole lines, unlike backward)
@@ -116,19 +117,19 @@ __global__ __launch_bounds__(64 * kW) SPEAR_BTP_FWD_OCC void btp_fwd_scan_kernel
   // added 12 % to the bytes fetched).
   constexpr bool kHandOver = SPEAR_BTP_HANDOVER && !kStreamIn && kW > 1;
   static_assert(!kLines || kHandOver, "whole-line staging is for rows of several spans");
-  static_assert(!kPack || (kStreamIn && !kCheckpoint), "packing is for rows of one span, without the carry store");
+  static_assert(!kFlat || (!kCheckpoint && !kLines), "flat spans: no carry store, no whole-line movement");
   __shared__ float left_state[kHandOver ? kW : 1][kChan];
 
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const long span = first_span_of_workgroup<(SPEAR_BTP_XCD_REMAP == 2) || (SPEAR_BTP_XCD_REMAP == 1 && !kStreamIn)>(kW) + wave;
-  if (kPack ? span * pack >= total_spans : span >= total_spans) {  // wave-uniform
+  if (kFlat ? span * (kSpan / kTile) >= total_spans : span >= total_spans) {  // wave-uniform
     // keep the barrier count equal for every wavefront
     if constexpr (kLines) __syncthreads();
     if constexpr (kHandOver) __syncthreads();
     if constexpr (kLines) __syncthreads();
     return;
   }
-  const SpanCoord sc = kPack ? pack_coord(span, pack, total_spans, L) : span_coord(span, spans_per_row, L);
+  const SpanCoord sc = kFlat ? flat_coord(span, spans_per_row, total_spans) : span_coord(span, spans_per_row, L);
 
   unsigned char* img = lds[wave];
   float* a_lds = reinterpret_cast<float*>(img + kImgBytes);
@@ -150,14 +151,15 @@ __global__ __launch_bounds__(64 * kW) SPEAR_BTP_FWD_OCC void btp_fwd_scan_kernel
     px = line_place(xrows, L, sc.sp, lane, wave == 0);
     line_global_to_regs<nt_loads(kStreamIn)>(xrows, L, sc.sp, px, lane, xin);
     if (tail) line_tail_global_to_regs(xrows, L, sc.sp, lane, xtail);
-  } else if constexpr (kPack) {
-    pack_global_to_regs<nt_loads(kStreamIn)>(xslab, L, pack_lane<uint16_t>(lane, L, sc.nvalid / L), xin);
+  } else if constexpr (kFlat) {
+    pack_global_to_regs<nt_loads(kStreamIn)>(xrows, L, flat_lane<uint16_t>(lane, L, spans_per_row, sc.sp, sc.nvalid), xin);
   } else {
     slab16_global_to_regs<nt_loads(kStreamIn)>(xslab, L, sc.nvalid, lane, xin);
   }
   const typename C::pair_t ain = coeff_global_to_reg<C>(arow, sc.nvalid, lane);
-  // packed rows: no carry enters a block with which a row starts (wave-uniform per lane group)
-  const bool startA = kPack && (32 * j) % L == 0, startB = kPack && (32 * j + 16) % L == 0;
+  // flat spans: no carry enters a block with which a row starts (the same for the 16 lanes of a group)
+  const bool startA = kFlat && (sc.sp + 2 * j) % spans_per_row == 0;
+  const bool startB = kFlat && (sc.sp + 2 * j + 1) % spans_per_row == 0;
 
   const bool needs_left = (k == 2) && (sc.sp > 0);            // wave-uniform
   const bool halo = needs_left && !(kHandOver && wave > 0);     // recompute from a halo read
@@ -249,9 +251,9 @@ __global__ __launch_bounds__(64 * kW) SPEAR_BTP_FWD_OCC void btp_fwd_scan_kernel
     const LinePlace py = line_place(yrows, L, sc.sp, lane, wave == 0);
     line_lds_to_global<kStreamOut>(img, kImgStride, yrows, L, py, lane);
     if (tail) line_tail_lds_to_global(img, yrows, L, sc.sp, lane);
-  } else if constexpr (kPack) {
+  } else if constexpr (kFlat) {
     wave_lds_handover();
-    pack_lds_to_global<kStreamOut>(img, yrows, L, pack_lane<Y>(lane, L, sc.nvalid / L), lane);
+    pack_lds_to_global<kStreamOut>(img, yrows, L, flat_lane<Y>(lane, L, spans_per_row, sc.sp, sc.nvalid), lane);
   } else {
     wave_lds_handover();
     if constexpr (kOutF32) slab32_lds_to_global<kStreamOut>(img, yrows + sc.s0, L, sc.nvalid, lane);
@@ -276,12 +278,12 @@ constexpr int bwd_waves() {
   return kStreamIn ? SPEAR_BTP_BWD_SHORT_ROW_WAVES : kWavesLong;
 }
 
-template <class E, class C, class GradT, class DxT, bool kStreamIn, int kW, bool kLines = false, bool kPack = false>
+template <class E, class C, class GradT, class DxT, bool kStreamIn, int kW, bool kLines = false, bool kFlat = false>
 __device__ __forceinline__ void btp_bwd_scan_body(
     unsigned char (*lds)[4096 + (std::is_same<GradT, float>::value ? 8192 : 4096) + kCoeffLdsBytes],
     const typename C::elem* __restrict__ coeff, const uint16_t* __restrict__ x, const GradT* __restrict__ dy,
     DxT* __restrict__ dx, float* __restrict__ dA, int L, int spans_per_row, long total_spans,
-    int k, int pack) {
+    int k) {
   constexpr bool kGradF32 = std::is_same<GradT, float>::value;
   constexpr bool kDxF32 = std::is_same<DxT, float>::value;  // check mode: dx leaves unrounded
   constexpr int kGradBytes = kGradF32 ? 8192 : 4096;
@@ -292,22 +294,22 @@ __device__ __forceinline__ void btp_bwd_scan_body(
   constexpr bool kHandOver = SPEAR_BTP_HANDOVER && !kStreamIn && kW > 1;
   // kLines: x, dy and dx move as whole cache lines (line_place in btp_staging.h); see the forward kernel
   static_assert(!kLines || (kHandOver && !kDxF32), "whole-line staging: 16-bit dx, rows of several spans");
-  // kPack: rows of at most half a span, `pack` of them to a wavefront; `total_spans` counts rows then
-  static_assert(!kPack || kStreamIn, "packing is for rows of one span");
+  // kFlat: spans cut from the tensor's block sequence; see the forward kernel
+  static_assert(!kFlat || !kLines, "flat spans move rows the plain way");
   constexpr int kImgStride = 4096 + kGradBytes + kCoeffLdsBytes;
   __shared__ float edge_state[kHandOver ? kW : 1][2][kChan];
 
   SPEAR_BTP_PRIO(3);
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
   const long span = first_span_of_workgroup<(SPEAR_BTP_XCD_REMAP == 2) || (SPEAR_BTP_XCD_REMAP == 1 && !kStreamIn)>(kW) + wave;
-  if (kPack ? span * pack >= total_spans : span >= total_spans) {  // wave-uniform
+  if (kFlat ? span * (kSpan / kTile) >= total_spans : span >= total_spans) {  // wave-uniform
     // keep the barrier count equal for every wavefront
     if constexpr (kLines) __syncthreads();
     if constexpr (kHandOver) __syncthreads();
     if constexpr (kLines) __syncthreads();
     return;
   }
-  const SpanCoord sc = kPack ? pack_coord(span, pack, total_spans, L) : span_coord(span, spans_per_row, L);
+  const SpanCoord sc = kFlat ? flat_coord(span, spans_per_row, total_spans) : span_coord(span, spans_per_row, L);
 
   unsigned char* img_x = lds[wave];
   unsigned char* img_g = img_x + 4096;
@@ -337,9 +339,9 @@ __device__ __forceinline__ void btp_bwd_scan_body(
       line_tail_global_to_regs(xrows, L, sc.sp, lane, xtail);
       line_tail_global_to_regs(grows, L, sc.sp, lane, gtail);
     }
-  } else if constexpr (kPack) {
-    pack_global_to_regs<nt_loads(kStreamIn)>(xslab, L, pack_lane<uint16_t>(lane, L, sc.nvalid / L), xin);
-    pack_global_to_regs<nt_loads(kStreamIn)>(dy + slab_off, L, pack_lane<GradT>(lane, L, sc.nvalid / L), gin);
+  } else if constexpr (kFlat) {
+    pack_global_to_regs<nt_loads(kStreamIn)>(xrows, L, flat_lane<uint16_t>(lane, L, spans_per_row, sc.sp, sc.nvalid), xin);
+    pack_global_to_regs<nt_loads(kStreamIn)>(grows, L, flat_lane<GradT>(lane, L, spans_per_row, sc.sp, sc.nvalid), gin);
   } else {
     slab16_global_to_regs<nt_loads(kStreamIn)>(xslab, L, sc.nvalid, lane, xin);
     if constexpr (kGradF32) {
@@ -351,9 +353,13 @@ __device__ __forceinline__ void btp_bwd_scan_body(
   const typename C::pair_t ain = coeff_global_to_reg<C>(arow, sc.nvalid, lane);
 
   const bool needs_left = (k == 2) && (sc.sp > 0);             // wave-uniform
-  const bool needs_right = (k == 2) && (sc.s0 + kSpan < L);    // wave-uniform
+  // (flat spans: the block after the span exists and belongs to the row of the span's last block)
+  const int after = sc.sp + kSpan / kTile;  // flat spans: where the block after the span lies, counted from the first row
+  const bool needs_right = (k == 2) && (kFlat ? ((span + 1) * (kSpan / kTile) < total_spans && after % spans_per_row != 0)
+                                              : (sc.s0 + kSpan < L));  // wave-uniform
   // the right neighbour is in this workgroup unless this is its last wavefront or the last span overall
-  const bool right_here = kHandOver && wave + 1 < kW && span + 1 < total_spans;
+  const bool right_here = kHandOver && wave + 1 < kW &&
+                          (kFlat ? (span + 1) * (kSpan / kTile) < total_spans : span + 1 < total_spans);
   const bool halo_left = needs_left && !(kHandOver && wave > 0);
   const bool halo_right = needs_right && !right_here;
   float c_halo = 0.0f, dc_halo = 0.0f;
@@ -372,15 +378,18 @@ __device__ __forceinline__ void btp_bwd_scan_body(
     // gradient carry sent by the block just right of the span: a_0 * A_0 of that block
     float ah[16], gh[16];
     C::load_block(arow + kSpan, ah);
+    // (flat spans: that block lies after / spans_per_row rows further on)
+    const long right_off = kFlat ? ((sc.row + after / spans_per_row) * kChan + d) * (long)L + (after % spans_per_row) * kTile
+                                 : slab_off + (long)d * L + kSpan;
     if constexpr (kGradF32) {
-      const float* gp = reinterpret_cast<const float*>(dy) + slab_off + (long)d * L + kSpan;
+      const float* gp = reinterpret_cast<const float*>(dy) + right_off;
 #pragma unroll
       for (int c = 0; c < 4; ++c) {
         const float4 q = *reinterpret_cast<const float4*>(gp + 4 * c);
         gh[4 * c + 0] = q.x; gh[4 * c + 1] = q.y; gh[4 * c + 2] = q.z; gh[4 * c + 3] = q.w;
       }
     } else {
-      const uint16_t* gp = reinterpret_cast<const uint16_t*>(dy) + slab_off + (long)d * L + kSpan;
+      const uint16_t* gp = reinterpret_cast<const uint16_t*>(dy) + right_off;
       unpack8<E>(*reinterpret_cast<const uint4*>(gp), gh);
       unpack8<E>(*reinterpret_cast<const uint4*>(gp + 8), gh + 8);
     }
@@ -464,9 +473,10 @@ __device__ __forceinline__ void btp_bwd_scan_body(
     if (needs_left && wave > 0 && j == 0) c_halo = edge_state[wave - 1][0][d];
     if (needs_right && right_here && j == 3) dc_halo = edge_state[wave + 1][1][d];
   }
-  // packed rows: no carry crosses from one row into the next (wave-uniform per lane group)
-  const bool startA = kPack && (32 * j) % L == 0, startB = kPack && (32 * j + 16) % L == 0;
-  const bool endB = kPack && (32 * j + 32) % L == 0;
+  // flat spans: no carry crosses from one row into the next (the same for the 16 lanes of a group)
+  const bool startA = kFlat && (sc.sp + 2 * j) % spans_per_row == 0;
+  const bool startB = kFlat && (sc.sp + 2 * j + 1) % spans_per_row == 0;
+  const bool endB = kFlat && (sc.sp + 2 * j + 2) % spans_per_row == 0;
   const float cA = (two && !startA) ? (j == 0 ? c_halo : from_left) : 0.0f;
   const float cB = (two && !startB) ? v[15] : 0.0f;
   const float dcA = (two && !startB) ? dcA_raw : 0.0f;
@@ -524,8 +534,11 @@ __device__ __forceinline__ void btp_bwd_scan_body(
     wave_lds_handover();
     lane_write32(img_x, j, d, dxv);
     wave_lds_handover();
-    if constexpr (kPack) pack_lds_to_global<kStreamOut>(img_x, dx + slab_off, L, pack_lane<float>(lane, L, sc.nvalid / L), lane);
-    else slab32_lds_to_global<kStreamOut>(img_x, dx + slab_off, L, sc.nvalid, lane);
+    if constexpr (kFlat) {
+      pack_lds_to_global<kStreamOut>(img_x, dx + rows_off, L, flat_lane<float>(lane, L, spans_per_row, sc.sp, sc.nvalid), lane);
+    } else {
+      slab32_lds_to_global<kStreamOut>(img_x, dx + slab_off, L, sc.nvalid, lane);
+    }
   } else {
     // dx goes back through the x image: every lane overwrites exactly the chunks it read
     lane_write16<E>(img_x, j, d, dxv);
@@ -535,9 +548,9 @@ __device__ __forceinline__ void btp_bwd_scan_body(
       const LinePlace pd = line_place(dxrows, L, sc.sp, lane, wave == 0);
       line_lds_to_global<kStreamOut>(img_x, kImgStride, dxrows, L, pd, lane);
       if (tail) line_tail_lds_to_global(img_x, dxrows, L, sc.sp, lane);
-    } else if constexpr (kPack) {
+    } else if constexpr (kFlat) {
       wave_lds_handover();
-      pack_lds_to_global<kStreamOut>(img_x, dx + slab_off, L, pack_lane<uint16_t>(lane, L, sc.nvalid / L), lane);
+      pack_lds_to_global<kStreamOut>(img_x, dx + rows_off, L, flat_lane<uint16_t>(lane, L, spans_per_row, sc.sp, sc.nvalid), lane);
     } else {
       wave_lds_handover();
       slab16_lds_to_global<kStreamOut>(img_x, dx + slab_off, L, sc.nvalid, lane);
@@ -547,54 +560,60 @@ __device__ __forceinline__ void btp_bwd_scan_body(
 
 // 16-bit dy and 16-bit coefficients (the reference's operands): the body fits 128 VGPRs, so four
 // waves per SIMD are requested explicitly.
-template <class E, class C, bool kStreamIn, int kW = bwd_waves<true, kStreamIn>(), bool kLines = false, bool kPack = false>
+template <class E, class C, bool kStreamIn, int kW = bwd_waves<true, kStreamIn>(), bool kLines = false, bool kFlat = false>
 __global__ __launch_bounds__((64 * kW)) SPEAR_BTP_BWD_OCC void btp_bwd_scan_kernel(
     const typename C::elem* __restrict__ coeff, const uint16_t* __restrict__ x, const uint16_t* __restrict__ dy,
-    uint16_t* __restrict__ dx, float* __restrict__ dA, int L, int spans_per_row, long total_spans, int k, int pack) {
+    uint16_t* __restrict__ dx, float* __restrict__ dA, int L, int spans_per_row, long total_spans, int k) {
   __shared__ __align__(16) unsigned char lds[kW][4096 + 4096 + kCoeffLdsBytes];
-  btp_bwd_scan_body<E, C, uint16_t, uint16_t, kStreamIn, kW, kLines, kPack>(lds, coeff, x, dy, dx, dA, L, spans_per_row,
-                                                                        total_spans, k, pack);
+  btp_bwd_scan_body<E, C, uint16_t, uint16_t, kStreamIn, kW, kLines, kFlat>(lds, coeff, x, dy, dx, dA, L, spans_per_row,
+                                                                        total_spans, k);
 }
 
 // fp32 dy (twice the staging registers and LDS), log-space gates (an exponential per coefficient)
 // and the fp32-dx check mode: occupancy is left to the compiler.
-template <class E, class C, class GradT, class DxT, bool kStreamIn, bool kLines = false, bool kPack = false>
+template <class E, class C, class GradT, class DxT, bool kStreamIn, bool kLines = false, bool kFlat = false>
 __global__ __launch_bounds__((64 * bwd_waves<false, kStreamIn>())) void btp_bwd_scan_kernel_relaxed(
     const typename C::elem* __restrict__ coeff, const uint16_t* __restrict__ x, const GradT* __restrict__ dy,
-    DxT* __restrict__ dx, float* __restrict__ dA, int L, int spans_per_row, long total_spans, int k, int pack) {
+    DxT* __restrict__ dx, float* __restrict__ dA, int L, int spans_per_row, long total_spans, int k) {
   constexpr int kGradBytes = std::is_same<GradT, float>::value ? 8192 : 4096;
   constexpr int kW = bwd_waves<false, kStreamIn>();
   __shared__ __align__(16) unsigned char lds[kW][4096 + kGradBytes + kCoeffLdsBytes];
-  btp_bwd_scan_body<E, C, GradT, DxT, kStreamIn, kW, kLines, kPack>(lds, coeff, x, dy, dx, dA, L, spans_per_row,
-                                                                    total_spans, k, pack);
+  btp_bwd_scan_body<E, C, GradT, DxT, kStreamIn, kW, kLines, kFlat>(lds, coeff, x, dy, dx, dA, L, spans_per_row,
+                                                                    total_spans, k);
 }
 
-template <class E, class C, class OutT, bool kCheckpoint, bool kStreamIn, bool kLines = false, bool kPack = false>
+template <class E, class C, class OutT, bool kCheckpoint, bool kStreamIn, bool kLines = false, bool kFlat = false>
 void launch_fwd_as(const FwdArgs& p, const Grid& g, hipStream_t s) {
   constexpr int kW = kLines ? kFwdLinesWaves : kWaves;
-  hipLaunchKernelGGL((btp_fwd_scan_kernel<E, C, OutT, kCheckpoint, kStreamIn, kLines, kW, kPack>), dim3(g.blocks),
+  hipLaunchKernelGGL((btp_fwd_scan_kernel<E, C, OutT, kCheckpoint, kStreamIn, kLines, kW, kFlat>), dim3(g.blocks),
                      dim3(64 * g.waves), 0, s, static_cast<const typename C::elem*>(p.coeff),
                      static_cast<const uint16_t*>(p.x), static_cast<OutT*>(p.y), p.checkpoint, p.L, g.spans_per_row,
-                     g.total_spans, p.k, g.pack);
+                     g.total_spans, p.k);
 }
 
 template <class E, class C, class OutT>
 hipError_t launch_fwd(const FwdArgs& p, hipStream_t s) {
   const long rows = (long)p.B * p.H;
-  const Grid g = make_grid(rows, p.L);
-  const bool ck = p.checkpoint != nullptr, st = stream_inputs(g);
-  if (g.lines) {  // rows of several spans that do not end on a cache line
-    const Grid gl = make_grid(rows, p.L, kFwdLinesWaves);
-    if (ck) launch_fwd_as<E, C, OutT, true, false, true>(p, gl, s);
-    else launch_fwd_as<E, C, OutT, false, false, true>(p, gl, s);
-  } else if (st && g.pack > 1 && !ck) {  // rows of at most half a span, several to a wavefront
-    launch_fwd_as<E, C, OutT, false, true, false, true>(p, packed(g, rows), s);
-  } else if (ck) {
-    if (st) launch_fwd_as<E, C, OutT, true, true>(p, g, s);
-    else launch_fwd_as<E, C, OutT, true, false>(p, g, s);
+  const bool ck = p.checkpoint != nullptr;
+  const Movement move = movement_for(p.L);
+  if (move == kMoveLines) {
+    const Grid g = make_grid(rows, p.L, kFwdLinesWaves);
+    if (ck) launch_fwd_as<E, C, OutT, true, false, true>(p, g, s);
+    else launch_fwd_as<E, C, OutT, false, false, true>(p, g, s);
+  } else if (move == kMoveFlat && !ck) {  // (the carry store keeps the per-row cut)
+    const Grid g = flat_grid(rows, p.L);
+    if (g.stream) launch_fwd_as<E, C, OutT, false, true, false, true>(p, g, s);
+    else launch_fwd_as<E, C, OutT, false, false, false, true>(p, g, s);
   } else {
-    if (st) launch_fwd_as<E, C, OutT, false, true>(p, g, s);
-    else launch_fwd_as<E, C, OutT, false, false>(p, g, s);
+    const Grid g = make_grid(rows, p.L);
+    const bool st = stream_inputs(g);
+    if (ck) {
+      if (st) launch_fwd_as<E, C, OutT, true, true>(p, g, s);
+      else launch_fwd_as<E, C, OutT, true, false>(p, g, s);
+    } else {
+      if (st) launch_fwd_as<E, C, OutT, false, true>(p, g, s);
+      else launch_fwd_as<E, C, OutT, false, false>(p, g, s);
+    }
   }
   return hipGetLastError();
 }
@@ -608,21 +627,16 @@ void launch_bwd_as(const BwdArgs& p, const Grid& g, hipStream_t s) {
   const auto* dy = static_cast<const GradT*>(p.dy);
   auto go = [&](auto kernel, auto* dx) {
     hipLaunchKernelGGL(kernel, dim3(g.blocks), dim3(64 * g.waves), 0, s, c, x, dy, dx, p.dA, p.L, g.spans_per_row,
-                       g.total_spans, p.k, g.pack);
+                       g.total_spans, p.k);
   };
   auto* dx16 = static_cast<uint16_t*>(p.dx);
-  const bool pack = kStreamIn && g.pack > 1;  // rows of at most half a span, several to a wavefront
-  if (p.dx_f32) {                             // fp32 check mode
+  if (p.dx_f32) {  // fp32 check mode
     auto* dx32 = static_cast<float*>(p.dx);
-    if constexpr (kStreamIn) {
-      if (pack) return go(btp_bwd_scan_kernel_relaxed<E, C, GradT, float, true, false, true>, dx32);
-    }
+    if (g.flat) return go(btp_bwd_scan_kernel_relaxed<E, C, GradT, float, kStreamIn, false, true>, dx32);
     return go(btp_bwd_scan_kernel_relaxed<E, C, GradT, float, kStreamIn>, dx32);
   }
   if constexpr (kGradF32 || C::kLog) {
-    if constexpr (kStreamIn) {
-      if (pack) return go(btp_bwd_scan_kernel_relaxed<E, C, GradT, uint16_t, true, false, true>, dx16);
-    }
+    if (g.flat) return go(btp_bwd_scan_kernel_relaxed<E, C, GradT, uint16_t, kStreamIn, false, true>, dx16);
     // Rows that do not end on a cache line: whole lines with 16-bit dy (log-space gates: +2-3 % on rows of 8 spans
     // and more). With an fp32 dy, whose rows are twice as long and at worst 64 bytes off the lines, it measured
     // the same on long rows and 5 % slower at L = 272 (two more barriers at this kernel's lower occupancy).
@@ -631,11 +645,15 @@ void launch_bwd_as(const BwdArgs& p, const Grid& g, hipStream_t s) {
     }
     return go(btp_bwd_scan_kernel_relaxed<E, C, GradT, uint16_t, kStreamIn>, dx16);
   } else if constexpr (kStreamIn) {
-    if (pack) return go(btp_bwd_scan_kernel<E, C, true, bwd_waves<true, true>(), false, true>, dx16);
+    if (g.flat) return go(btp_bwd_scan_kernel<E, C, true, bwd_waves<true, true>(), false, true>, dx16);
     return go(btp_bwd_scan_kernel<E, C, true>, dx16);
   } else {
     const bool small = g.waves == kWaves;  // rows of a few spans: the smaller workgroup
-    if (g.lines) {                         // rows that do not end on a cache line
+    if (g.flat) {
+      return small ? go(btp_bwd_scan_kernel<E, C, false, kWaves, false, true>, dx16)
+                   : go(btp_bwd_scan_kernel<E, C, false, kWavesLong, false, true>, dx16);
+    }
+    if (g.lines) {  // rows that do not end on a cache line
       return small ? go(btp_bwd_scan_kernel<E, C, false, kWaves, true>, dx16)
                    : go(btp_bwd_scan_kernel<E, C, false, kWavesLong, true>, dx16);
     }
@@ -645,7 +663,8 @@ void launch_bwd_as(const BwdArgs& p, const Grid& g, hipStream_t s) {
 
 template <class E, class C, class GradT>
 hipError_t launch_bwd(const BwdArgs& p, hipStream_t s) {
-  constexpr bool kLeanIo = !(std::is_same<GradT, float>::value || C::kLog);
+  constexpr bool kGradF32 = std::is_same<GradT, float>::value;
+  constexpr bool kLeanIo = !(kGradF32 || C::kLog);
   const bool lean = kLeanIo && !p.dx_f32;  // the kernel launch_bwd_as picks
   const long rows = (long)p.B * p.H;
   // Workgroups of kWavesLong wavefronts hand more carries over in LDS and read fewer halos; with the workgroups
@@ -654,9 +673,14 @@ hipError_t launch_bwd(const BwdArgs& p, hipStream_t s) {
   // from 16 spans on the two are within +-2 % of each other either way.
   int long_row_waves = (p.L + kSpan - 1) / kSpan <= 8 ? kWaves : bwd_waves<true, false>();
   if (SPEAR_BTP_BWD_LINES_WAVES && (p.L % 64) != 0) long_row_waves = SPEAR_BTP_BWD_LINES_WAVES;
-  const Grid g = lean ? make_grid(rows, p.L, long_row_waves, bwd_waves<true, true>())
-                      : make_grid(rows, p.L, bwd_waves<false, false>(), bwd_waves<false, true>());
-  if (stream_inputs(g)) launch_bwd_as<E, C, GradT, true>(p, g.pack > 1 ? packed(g, rows) : g, s);
+  const int waves_long = lean ? long_row_waves : bwd_waves<false, false>();
+  const int waves_short = lean ? bwd_waves<true, true>() : bwd_waves<false, true>();
+  Movement move = movement_for(p.L);
+  // whole lines are not taken with an fp32 dy or in the check mode (launch_bwd_as): those rows go flat or plain
+  if (move == kMoveLines && (kGradF32 || p.dx_f32)) move = SPEAR_BTP_FLAT_SPANS ? kMoveFlat : kMovePlain;
+  Grid g = move == kMoveFlat ? flat_grid(rows, p.L, waves_long, waves_short) : make_grid(rows, p.L, waves_long, waves_short);
+  if (move != kMoveLines) g.lines = false;
+  if (stream_inputs(g)) launch_bwd_as<E, C, GradT, true>(p, g, s);
   else launch_bwd_as<E, C, GradT, false>(p, g, s);
   return hipGetLastError();
 }

@@ -23,8 +23,8 @@
 #ifndef SPEAR_BTP_WHOLE_LINES    // 1: rows of several spans that do not end on a 128-byte line move as whole lines
 #define SPEAR_BTP_WHOLE_LINES 1
 #endif
-#ifndef SPEAR_BTP_PACK_SHORT_ROWS  // 1: rows of at most half a span are packed several to a wavefront
-#define SPEAR_BTP_PACK_SHORT_ROWS 1
+#ifndef SPEAR_BTP_FLAT_SPANS      // 1: rows that leave a span partly empty are cut from the tensor's block sequence
+#define SPEAR_BTP_FLAT_SPANS 1
 #endif
 #ifndef SPEAR_BTP_STREAM_STORES  // 0: never, 1: always
 #define SPEAR_BTP_STREAM_STORES 1
@@ -350,27 +350,31 @@ __device__ __forceinline__ void line_tail_lds_to_global(const unsigned char* img
   }
 }
 
-// ---- rows of at most half a span ---------------------------------------------------------------
-// A wavefront works on a [16 channel x 128 step] image. A row of L <= 64 steps fills at most half of it, and with
-// one row per wavefront a launch at L = 64 / 32 / 16 moved 0.63 / 0.39 / 0.21 of the peak rate. Such rows are
-// therefore packed: a wavefront takes floor(128 / L) consecutive (batch, head) rows, whose slabs follow each other
-// in memory, and lays them side by side in its image (row q of the pack at steps [q L, (q + 1) L)). Coefficients,
-// dA and the carry arithmetic see 128 consecutive steps as before; the kernels only have to drop the carries at
-// the steps where a new row starts.
+// ---- rows that do not fill whole spans ---------------------------------------------------------
+// A wavefront works on a [16 channel x 128 step] image. With spans cut per row, a row of L <= 64 steps fills at
+// most half of one (a launch at L = 64 / 32 / 16 moved 0.63 / 0.39 / 0.21 of the peak rate) and the last span of
+// a row of 192 steps is half empty. The kFlat instances of the kernels cut spans from the block sequence of the
+// whole tensor instead: span s is blocks [8 s, 8 s + 8) of all rows' blocks in order, so only the tensor's very
+// last span can be short. The coefficients and dA of a span are 128 consecutive values (their rows follow each
+// other in memory); x, dy, y and dx come from one slab per row the span touches, side by side in the image. The
+// arithmetic is unchanged except that no carry crosses the steps where a new row starts.
 struct PackLane {
-  long off;  // of the lane's chunk in pass 0, in elements from the slab of the pack's first row
-  bool ok;   // the chunk exists (its row is one of the pack's)
+  long off;  // of the lane's chunk in pass 0, in elements from the slab of the span's first row
+  bool ok;   // the chunk exists
 };
 
+// `nb` = blocks in a row, `b0` = which block of its row the span's first block is, `nvalid` = steps in the span
 template <class T>
-__device__ __forceinline__ PackLane pack_lane(int lane, int L, int rows_here) {
+__device__ __forceinline__ PackLane flat_lane(int lane, int L, int nb, int b0, int nvalid) {
   typedef LineGeom<T> G;
+  constexpr int kPerBlockShift = 4 - G::kStepsShift;  // log2 of the chunks in a block
   const int lp = lane & (G::kChunks - 1), lr = lane / G::kChunks;
-  const int per_row = L >> G::kStepsShift;           // chunks of one row
-  const int q = lp / per_row, cw = lp - q * per_row;  // which row of the pack, which chunk of it
+  const int blk = lp >> kPerBlockShift, part = lp & ((1 << kPerBlockShift) - 1);
+  const int q = (b0 + blk) / nb, b = b0 + blk - q * nb;  // rows after the span's first one, block inside that row
   PackLane p;
-  p.ok = q < rows_here;
-  p.off = p.ok ? (long)(q * kChan + lr) * L + (cw << G::kStepsShift) : (long)lr * L;  // else: a chunk that is always there
+  p.ok = kTile * blk < nvalid;
+  p.off = p.ok ? (long)(q * kChan + lr) * L + kTile * b + (part << G::kStepsShift)
+               : (long)lr * L + kTile * b0;  // else the span's first chunk, which is always there
   return p;
 }
 
@@ -655,13 +659,14 @@ __device__ __forceinline__ SpanCoord span_coord(long span, int spans_per_row, in
   return c;
 }
 
-// Packed rows (see pack_lane): the wavefront's first row and how many steps of its image are rows
-__device__ __forceinline__ SpanCoord pack_coord(long span, int pack, long rows, int L) {
+// Spans cut from the tensor's block sequence (see flat_lane): `sp` is which block of its row the span starts with
+__device__ __forceinline__ SpanCoord flat_coord(long span, int nb, long total_blocks) {
   SpanCoord c;
-  c.row = span * pack;
-  c.sp = 0;
-  c.s0 = 0;
-  c.nvalid = (int)min((long)pack, rows - c.row) * L;
+  const long first = span * (kSpan / kTile);
+  c.row = first / nb;
+  c.sp = (int)(first - c.row * nb);
+  c.s0 = c.sp * kTile;
+  c.nvalid = (int)min((long)(kSpan / kTile), total_blocks - first) * kTile;
   return c;
 }
 
@@ -699,12 +704,44 @@ __device__ __forceinline__ long first_span_of_workgroup(int waves = kWaves) {
   }
 }
 
+// How the rows of a launch are cut into spans and moved:
+//   kMovePlain  per row, a span's own 256 bytes of each channel row (rows of whole spans: the benchmark shapes; rows
+//               of 65..127 steps, whose slabs are one contiguous run each)
+//   kMoveLines  per row, whole cache lines (rows of several spans that do not end on a 128-byte line)
+//   kMoveFlat   from the tensor's block sequence (rows that leave a span partly empty); Grid::stream then says
+//               that no row straddles two spans (L = 16, 32, 64)
+// A row of L steps fills L / (128 ceil(L / 128)) of its spans. Flat spans have no empty lanes but move rows the
+// plain way: 0.80 of peak on rows of whole lines (L % 64 == 0), 0.75 when the rows lie 64 bytes off the lines
+// (L % 64 == 32) and 0.65-0.69 when they lie 32 bytes off. Whole lines keep the per-row cut and reach 0.72-0.78
+// on rows that fill their spans well. Measured over 23 lengths from 144 to 1168 at 8 Mi (token, head) units, whole
+// lines win from the fill percentages below on (SPEAR_BTP_LINES_MIN_FILL, and ..._HALF for L % 64 == 32), within 3 %.
+// Below a span, rows of at most 64 steps go flat (0.73-0.82 against 0.21-0.63) and longer ones stay plain
+// (0.73-0.78 against 0.67-0.76 flat).
+#ifndef SPEAR_BTP_LINES_MIN_FILL
+#define SPEAR_BTP_LINES_MIN_FILL 65
+#endif
+#ifndef SPEAR_BTP_LINES_MIN_FILL_HALF
+#define SPEAR_BTP_LINES_MIN_FILL_HALF 80
+#endif
+enum Movement : int { kMovePlain = 0, kMoveLines = 1, kMoveFlat = 2 };
+
+inline Movement movement_for(int L) {
+  if (L <= 0 || L % kSpan == 0) return kMovePlain;
+  if (L < kSpan) return SPEAR_BTP_FLAT_SPANS && 2 * L <= kSpan ? kMoveFlat : kMovePlain;
+  const int spans = (L + kSpan - 1) / kSpan;
+  const bool off_lines = L % 64 != 0 && SPEAR_BTP_WHOLE_LINES;
+  const long min_fill = L % 64 == 32 ? SPEAR_BTP_LINES_MIN_FILL_HALF : SPEAR_BTP_LINES_MIN_FILL;
+  if (off_lines && 100L * L >= min_fill * spans * kSpan) return kMoveLines;
+  return SPEAR_BTP_FLAT_SPANS ? kMoveFlat : (off_lines ? kMoveLines : kMovePlain);
+}
+
 struct Grid {
   int spans_per_row;
   long total_spans;
   bool stream;     // kStreamIn of the kernels
   bool lines;      // rows of several spans that do not end on a 128-byte line: kLines of the kernels that have it
-  int pack;        // rows of at most half a span: how many a wavefront takes (kPack of the kernels that have it), else 1
+  bool flat;       // spans cut from the tensor's block sequence (kFlat of the kernels that have it); then
+                   // spans_per_row holds the blocks in a row and total_spans the blocks in the tensor
   int waves;       // wavefronts per workgroup
   unsigned blocks;
 };
@@ -717,8 +754,8 @@ inline Grid make_grid(long rows, int L, int waves_long = kWaves, int waves_short
   g.spans_per_row = (L + kSpan - 1) / kSpan;
   g.total_spans = rows * g.spans_per_row;
   g.stream = g.spans_per_row == 1;  // template argument kStreamIn of the kernels: rows of a single span
-  g.lines = !g.stream && (L % 64) != 0 && SPEAR_BTP_WHOLE_LINES;
-  g.pack = SPEAR_BTP_PACK_SHORT_ROWS && L > 0 && 2 * L <= kSpan ? kSpan / L : 1;
+  g.lines = movement_for(L) == kMoveLines;
+  g.flat = false;
   g.waves = g.stream ? waves_short : waves_long;
   g.blocks = (unsigned)((g.total_spans + g.waves - 1) / g.waves);
   return g;
@@ -726,11 +763,17 @@ inline Grid make_grid(long rows, int L, int waves_long = kWaves, int waves_short
 
 inline bool stream_inputs(const Grid& g) { return g.stream; }
 
-// The same rows with `g.pack` of them to a wavefront (the kernels' kPack instances, which count rows where the
-// others count spans).
-inline Grid packed(Grid g, long rows) {
-  g.total_spans = rows;
-  g.blocks = (unsigned)(((rows + g.pack - 1) / g.pack + g.waves - 1) / g.waves);
+// The grid of the kFlat instances for the same rows.
+inline Grid flat_grid(long rows, int L, int waves_long = kWaves, int waves_short = kWaves) {
+  Grid g;
+  g.spans_per_row = L / kTile;
+  g.total_spans = rows * g.spans_per_row;
+  g.stream = (kSpan / kTile) % g.spans_per_row == 0;  // no row straddles two spans
+  g.lines = false;
+  g.flat = true;
+  g.waves = g.stream ? waves_short : waves_long;
+  const long spans = (g.total_spans + kSpan / kTile - 1) / (kSpan / kTile);
+  g.blocks = (unsigned)((spans + g.waves - 1) / g.waves);
   return g;
 }
 

@@ -342,8 +342,9 @@ def _carve(shape, dtype, offset, fill):
 @pytest.mark.parametrize("offsets", [(0, 0, 0, 0), (8, 16, 24, 40), (56, 8, 0, 32)], ids=["on_lines", "offsets_a", "offsets_b"])
 @pytest.mark.parametrize("B,H,L", [(2, 3, 144), (1, 2, 272), (3, 5, 400), (2, 2, 1040), (1, 3, 2032), (5, 1, 2000), (7, 3, 272)])
 def test_rows_of_several_spans_that_do_not_end_on_a_cache_line(B, H, L, offsets):
-    """Rows of several spans with L % 64 != 0 start at different offsets inside their 128-byte lines; forward and
-    backward then move whole lines and hand the ends of the rows from wavefront to wavefront (16-bit and fp32 y, 16-bit
+    """Rows of several spans with L % 64 != 0 start at different offsets inside their 128-byte lines; where such rows
+    fill their spans well (all lengths here but 144, which goes the way of the next test) forward and backward move
+    whole lines and hand the ends of the rows from wavefront to wavefront (16-bit and fp32 y, 16-bit
     dy, linear and log-space gates; an fp32 dy and the fp32-dx check mode keep the plain movement). Tensors are placed at
     16-byte steps off the line grid (x, dy, y and dx each at their own), so every row start 0..7 chunks into a line
     occurs. Results against the oracle; the 16-bit results equal the rounded fp32 ones (y: another instance of the
@@ -415,12 +416,13 @@ def test_rows_of_several_spans_that_do_not_end_on_a_cache_line(B, H, L, offsets)
     assert_close(f64(carries)[:, :, : nb - 1], rck[:, :, : nb - 1], F32_ATOL, F32_RTOL, "checkpoint")
 
 
-@pytest.mark.parametrize("L", [16, 32, 48, 64])
+@pytest.mark.parametrize("L", [16, 32, 48, 64, 144, 160, 192, 288, 320, 576])
 @pytest.mark.parametrize("B,H", [(1, 1), (1, 3), (2, 3), (1, 7), (5, 5), (8, 33)])
-def test_short_rows_packed_several_to_a_wavefront(B, H, L):
-    """Rows of at most 64 steps share a wavefront (128 // L of them side by side in its image; the last wavefront
-    takes what is left). Every instance against the oracle, nothing written outside the tensors, and every row of
-    the batch bit-identical to the same row run alone (where it sits first in its wavefront's image)."""
+def test_spans_cut_from_the_block_sequence_of_the_tensor(B, H, L):
+    """Rows that would leave a span partly empty (at most 64 steps; a few spans with little in the last one) have
+    their spans cut from the blocks of all rows in order: short rows share a wavefront, longer ones start anywhere
+    in one, and carries stop at the row starts. Every instance against the oracle, nothing written outside the
+    tensors, and every row of the batch bit-identical to the same row run alone (where it starts its first span)."""
     from spear_amd import _btp
 
     coeff, x, dy = make_inputs(B, H, L, seed=700 + L + B * H, stress=1.5)
@@ -435,7 +437,7 @@ def test_short_rows_packed_several_to_a_wavefront(B, H, L):
         assert bool((buf[:off] == 7).all()) and bool((buf[off + n :] == 7).all()), f"{name}: bytes outside the tensor changed"
 
     for k in (2, 1):
-        print(f"short rows B={B} H={H} L={L} k={k}", flush=True)
+        print(f"flat spans B={B} H={H} L={L} k={k}", flush=True)
         (by, yv), (bd, dxv) = _carve(shape, x.dtype, 8, 7.0), _carve(shape, x.dtype, 8, 7.0)
         (by32, y32), (bd32, dx32) = _carve(shape, torch.float32, 8, 7.0), _carve(shape, torch.float32, 8, 7.0)
         dA, dA32 = torch.full((B, H, L), float("nan"), device=DEV), torch.full((B, H, L), float("nan"), device=DEV)
@@ -472,7 +474,7 @@ def test_short_rows_packed_several_to_a_wavefront(B, H, L):
             _btp.backward(c1, x1, g1, ck, d1, a1, k, 32)
             assert torch.equal(y1, yv[b : b + 1, h : h + 1]) and torch.equal(d1, dxv[b : b + 1, h : h + 1])
             assert torch.equal(a1, dA[b : b + 1, h : h + 1]), f"row ({b}, {h}) differs from the same row run alone"
-    # with the carry store the rows are not packed: same y, carries against the oracle
+    # with the carry store the spans are cut per row: same y, carries against the oracle
     y_ck, carries = run_forward(coeff, x, k=2, checkpoint=True)
     assert torch.equal(y_ck, run_forward(coeff, x, k=2))
     nb = L // 16
