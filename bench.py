@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the BTP hot path: forward + backward at B=1024, L=128, dim=512 (H=32) bf16.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c3|c4|c5] [--no-cpu-baseline] [--no-other-configs]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c3|c4|c5|r2032|r64|r192] [--no-cpu-baseline] [--no-other-configs]
 
 A step is one forward plus one backward launch through the C ABI on one batch of synthetic
 input that is already resident in HBM. Buffers rotate over several independent sets so that a
@@ -73,6 +73,10 @@ CONFIGS = {
     # not one of the reference's benchmark shapes: c5's size with rows of 4064 bytes, which do not end on a 128-byte
     # cache line (the stand-alone kernels move such rows as whole lines and pass row ends between wavefronts)
     "r2032": (64, 128, 2032, 1237, 0.25, "sigmoid"),
+    # rows that would leave a span of 128 steps partly empty: the kernels cut spans from the blocks of all rows in order
+    # (rows of 64 steps share a wavefront two by two; rows of 192 steps start anywhere in one)
+    "r64": (2048, 32, 64, 1238, 0.25, "sigmoid"),
+    "r192": (1024, 32, 192, 1239, 0.25, "sigmoid"),
 }
 LAYER_LAYOUT_CONFIGS = ("c3", "c4", "c5")  # the fused kernels' rows are feature vectors: L does not change their alignment
 
@@ -718,7 +722,8 @@ def main() -> int:
     streaming = None if args.no_streaming else guarded(streaming_leg)
 
     # The other full-size configurations (long rows: B=16 H=64 L=8192; log-space stress: B=64 H=128 L=2048; rows that
-    # do not end on a cache line: B=64 H=128 L=2032), each timed in this same run: stand-alone forward, backward and forward+backward step, and the fused layer-layout
+    # do not end on a cache line: B=64 H=128 L=2032; rows that do not fill whole spans: L=64 and L=192), each timed
+    # in this same run: stand-alone forward, backward and forward+backward step, and the fused layer-layout
     # forward / backward on tensors of the same size. Three rotating buffer sets (2.3-12 GiB: nothing is served
     # from the 256 MiB memory-side cache), inputs drawn on the device with the configurations' distributions
     # (values do not change the time), HIP events on the launch stream.
