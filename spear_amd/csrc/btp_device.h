@@ -56,7 +56,12 @@ struct Fp16 {
   static __device__ __forceinline__ float hi(uint32_t w) {
     return (float)__builtin_bit_cast(halfx2_t, w)[1];
   }
+  // Round-to-nearest-even of the fp32 values. The empty asm keeps the conversion apart from the arithmetic before it:
+  // folded into a mixed-precision FMA (v_fma_mixlo_f16) the value would be rounded once from the exact sum, which
+  // differs from the rounded fp32 result where that lies exactly between two fp16 values, and the compiler folds
+  // in some kernel instances and not in others.
   static __device__ __forceinline__ uint32_t pack2(float a, float b) {
+    asm("" : "+v"(a), "+v"(b));
     halfx2_t h = {(_Float16)a, (_Float16)b};
     return __builtin_bit_cast(uint32_t, h);
   }
