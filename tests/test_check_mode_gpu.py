@@ -163,3 +163,22 @@ def test_fused_results_fp32_match_oracle_to_1e4(B, L, H, Hkv, qkv):
     assert torch.equal(out16, out32.to(out16.dtype))
     for name, lo, hi in zip(("da/dgate", "db/dk", "dc/dq", "dv"), g16, g32):
         assert torch.equal(lo, hi.to(lo.dtype)), name
+
+
+@pytest.mark.parametrize("qkv", [False, True], ids=["layer", "qkv_gate"])
+@pytest.mark.parametrize("B,L,H,Hkv", [(2, 48, 8, 8), (3, 128, 8, 2), (2, 272, 12, 3), (16, 256, 16, 16)])
+def test_fused_fp16_results_are_the_rounded_fp32_results(B, L, H, Hkv, qkv):
+    """fp16 tensors through the fused kernels: every 16-bit result is the fp32 result of the check mode rounded to
+    nearest even (the conversion is not folded into the arithmetic before it, where a single rounding from the exact
+    sum would differ at ties)."""
+    ins = _mix_inputs(B, L, H, Hkv, seed=1700 + L + H, qkv=qkv)
+    ins = tuple(t.half() if t.dtype == torch.bfloat16 else t for t in ins)
+    print(f"fused fp16 B={B} L={L} H={H} Hkv={Hkv} qkv={qkv}", flush=True)
+    out32, g32 = _mix_run(ins, H, Hkv, qkv, f32=True)
+    out16, g16 = _mix_run(ins, H, Hkv, qkv, f32=False)
+    assert out16.dtype == torch.float16
+    assert torch.equal(out16, out32.to(out16.dtype))
+    for name, lo, hi in zip(("da/dgate", "db/dk", "dc/dq", "dv"), g16, g32):
+        assert torch.equal(lo, hi.to(lo.dtype)), name
+    ref_out, ref_g = _mix_oracle(ins, H, Hkv, qkv)
+    assert_close(f64(out32), ref_out, F32_ATOL, F32_RTOL, "out fp32")
