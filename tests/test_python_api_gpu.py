@@ -305,18 +305,19 @@ def test_torch_compile_of_the_added_ops():
     assert torch.equal(o_c, phalanx_mix(a, b, c, v, 4))
 
 
-def test_entry_points_can_be_captured_in_a_hip_graph():
+@pytest.mark.parametrize("L", [256, 64, 192, 400], ids=["whole_spans", "short_rows", "partly_empty_span", "off_the_lines"])
+def test_entry_points_can_be_captured_in_a_hip_graph(L):
     """The C-ABI calls allocate nothing and launch on the given stream, so they can be recorded into
     a graph and replayed. Every replay is checked against the eager result, with eager work and
-    synchronisation between replays."""
+    synchronisation between replays. One row length for each way the kernels cut and move rows."""
     from spear_amd import _btp
 
-    coeff, x, dy = make_inputs(4, 8, 256, seed=77)
+    coeff, x, dy = make_inputs(4, 8, L, seed=77)
     c, xx, g = coeff.to(DEV), x.to(DEV), dy.to(DEV)
-    y = torch.empty(4, 8, 16, 256, device=DEV, dtype=torch.bfloat16)
+    y = torch.empty(4, 8, 16, L, device=DEV, dtype=torch.bfloat16)
     dx = torch.empty_like(xx)
-    dA = torch.empty(4, 8, 256, device=DEV)
-    ck = torch.empty(4, 8, 16, 16, device=DEV)
+    dA = torch.empty(4, 8, L, device=DEV)
+    ck = torch.empty(4, 8, L // 16, 16, device=DEV)
 
     def launch():
         _btp.forward(c, xx, y, ck, 2, 32, flags=0)
