@@ -31,6 +31,11 @@
 //     halo read), so workgroups are fully independent: no flags, no look-back, no second kernel,
 //     and the carry is never dropped at a launch-shape boundary (the reference drops it at
 //     cluster boundaries, btp-forward.cu:359-366).
+//   * Row lengths other than whole spans get one of two more instances of each kernel (movement_for in
+//     btp_staging.h picks): kFlat cuts spans from the blocks of all rows in order, for rows that would leave a span
+//     partly empty (short rows then share a wavefront, and no carry crosses a row start); kLines moves whole
+//     128-byte lines for rows of several spans that do not end on a line, wavefronts passing the row ends to each
+//     other through LDS. The arithmetic is the same in all three.
 //
 // Backward uses, per block i with local index r (g = dy, c = carry into the block,
 // dC = carry of the gradient coming back from block i+1):
